@@ -1,0 +1,169 @@
+/*
+ * rmi_oracle.h — CPU restatement of rust-model-inference's quantized matrix
+ * products.  TEST INFRASTRUCTURE ONLY: this library is the checker that the
+ * HIP kernels are compared against and the CPU baseline that is timed beside
+ * them.  Nothing in the shipped GPU path links, loads or calls it.
+ *
+ * Every function follows one reference function in arithmetic order; the
+ * reference file:line is cited at each declaration (paths are relative to the
+ * reference repository root).  Three f32 accumulation orders exist in the
+ * reference for the same Q8_0 GEMV (scalar, AVX2, NEON); each is restated
+ * separately because they differ in the last bits.
+ *
+ * Pinned by reference-held known-answer vectors (see tests/test_oracle_*.py);
+ * functions for which no reference vector exists are cross-pinned against an
+ * independent formulation (brute-force integer dots, f64 dequantised dots,
+ * numpy.float16, the intrinsics twin in rmi_oracle_avx2.c).
+ */
+#ifndef RMI_ORACLE_H
+#define RMI_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    RMI_REF_SCALAR = 0, /* portable scalar kernels                        */
+    RMI_REF_AVX2 = 1,   /* x86-64 production kernels (AVX2+FMA order)     */
+    RMI_REF_NEON = 2    /* aarch64 production kernels (fused sequential)  */
+};
+
+/* src/ops/float.rs:177-207 — IEEE binary16 <-> binary32, round-to-nearest-even */
+float rmi_ref_f16_to_f32(uint16_t bits);
+uint16_t rmi_ref_f32_to_f16(float v);
+
+/* src/ops/quant/q8_0.rs:49-71 (scalar), :176-230 (AVX2), :75-164 (NEON).
+ * q8[n] int8 bit patterns, scales[n/32] f32 holding f16-rounded values. */
+void rmi_ref_quantize_q8_0(const float *input, size_t n, uint8_t *q8,
+                           float *scales, int variant);
+
+/* src/ops/kernel/q8_0/scalar.rs:31-58, avx2.rs:53-174, neon.rs:49-73.
+ * output[0] is row_start (the pre-sliced convention of dispatch.rs:36). */
+void rmi_ref_matmul_q8_0_quantized_range(const uint8_t *weight,
+                                         const uint8_t *input_q8,
+                                         const float *input_scales,
+                                         float *output, size_t n_in,
+                                         size_t row_start, size_t row_end,
+                                         int variant);
+
+/* src/ops/kernel/q8_0/parallel.rs:102-139 — full-length output, writes only
+ * rows [ith*ceil(n_out/nth), ...). */
+void rmi_ref_matmul_q8_0_quantized_parallel_rows(
+    const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
+    float *output, size_t n_in, size_t n_out, size_t ith, size_t nth,
+    int variant);
+
+/* The "per-block int32 dot" of scalar.rs:49-53: dots[row*n_in/32 + block]. */
+void rmi_ref_block_dots_q8_0(const uint8_t *weight, const uint8_t *input_q8,
+                             int32_t *dots, size_t n_in, size_t n_out);
+
+/* src/ops/kernel/q8_0/scalar.rs:3-29 (variant SCALAR) and avx2.rs:180-217
+ * (variant AVX2): the f32-activation `matmul_q8_0` of parallel.rs:317-341. */
+void rmi_ref_matmul_q8_0_f32(const uint8_t *weight, const float *input,
+                             float *output, size_t n_in, size_t n_out,
+                             int variant);
+
+/* src/ops/kernel/trait_.rs:59-109 — Kernel::forward / forward_batched for a
+ * Q8_0 weight: quantize each token row, one GEMV per token, token-major out. */
+void rmi_ref_q8_0_forward_batched(const uint8_t *weight, const float *input,
+                                  float *output, size_t n_in, size_t n_out,
+                                  size_t n_tokens, int variant);
+
+/* src/ops/quant/fuse.rs:25-64 — byte concat of two row-stacked weights.
+ * Returns fused row count, or 0 when the per-row byte lengths differ
+ * (the reference's `None`).  `fused` must hold a_len+b_len bytes. */
+size_t rmi_ref_fuse_vstack(const uint8_t *a, size_t a_len, size_t a_rows,
+                           const uint8_t *b, size_t b_len, size_t b_rows,
+                           uint8_t *fused);
+
+/* src/ops/quant/mod.rs:75-122 (scalar), :140-200 (AVX2).  SoA output:
+ * d[n/256], qs[n], bsums[n/16]. */
+void rmi_ref_quantize_row_q8_k(const float *x, size_t n, float *d, int8_t *qs,
+                               int16_t *bsums, int variant);
+
+/* src/ops/quant/mod.rs:25-33 */
+void rmi_ref_get_scale_min_k4(int j, const uint8_t *scales12, uint8_t *sc,
+                              uint8_t *mn);
+/* the kmask unpack of src/ops/quant/mod.rs:237-258: out[0..8)=scales,
+ * out[8..16)=mins */
+void rmi_ref_unpack_scales_kmask(const uint8_t *scales12, uint8_t *out16);
+
+/* src/ops/quant/mod.rs:210-289 (scalar) and :701-799 (AVX2). */
+float rmi_ref_vec_dot_q4k_q8k(const uint8_t *q4k_row, size_t n_blocks,
+                              const float *d, const int8_t *qs,
+                              const int16_t *bsums, int variant);
+
+/* Exact integers per super-block of the same dot: isum[b] = sum_l aux32[l]
+ * (scale-weighted q4*q8 products), msum[b] = sum_j bsums[j]*mins[j/2]. */
+void rmi_ref_q4k_q8k_block_ints(const uint8_t *q4k_row, size_t n_blocks,
+                                const int8_t *qs, const int16_t *bsums,
+                                int32_t *isum, int32_t *msum);
+
+/* src/ops/quant/mod.rs:456-490, 492-508 */
+void rmi_ref_dequantize_row_q4_k(const uint8_t *blocks, float *output,
+                                 size_t n);
+
+/* src/ops/kernel/q4_k.rs:56-93 — Q4_KKernel::forward_prepared over a Q8_K
+ * activation; rows [ith*ceil(n_out/nth), ...) of the full output. */
+void rmi_ref_q4k_forward_prepared(const uint8_t *weight, const float *d,
+                                  const int8_t *qs, const int16_t *bsums,
+                                  float *output, size_t n_in, size_t n_out,
+                                  size_t ith, size_t nth, int variant);
+
+/* src/ops/kernel/q4_k.rs:20-54 — Q4_KKernel::forward_prequantized: rebuild
+ * f32 x from (q8, scales), dequantise each row, sequential f32 dot. */
+void rmi_ref_q4k_forward_prequantized(const uint8_t *weight,
+                                      const uint8_t *input_q8,
+                                      const float *input_scales,
+                                      float *output, size_t n_in,
+                                      size_t n_out, size_t ith, size_t nth);
+
+/* src/core/model.rs:65-85 — QuantizedLinear::forward_dequant: whole-weight
+ * Q4_K dequant, then sequential f32 GEMV with the raw f32 input. */
+void rmi_ref_quantized_linear_forward(const uint8_t *weight,
+                                      const float *input, float *output,
+                                      size_t in_features,
+                                      size_t out_features);
+
+/* ---- rmi_oracle_avx2.c: the same AVX2 kernels written with the same
+ * intrinsics the reference uses; bit-identical to the RMI_REF_AVX2 variants
+ * above on any AVX2+FMA host.  Used to cross-check the order emulation and
+ * as the timed CPU baseline. ---- */
+int rmi_ref_have_avx2(void);
+void rmi_ref_x86_quantize_q8_0(const float *input, size_t n, uint8_t *q8,
+                               float *scales);
+void rmi_ref_x86_matmul_q8_0_range(const uint8_t *weight,
+                                   const uint8_t *input_q8,
+                                   const float *input_scales, float *output,
+                                   size_t n_in, size_t row_start,
+                                   size_t row_end);
+float rmi_ref_x86_vec_dot_q4k_q8k(const uint8_t *q4k_row, size_t n_blocks,
+                                  const float *d, const int8_t *qs,
+                                  const int16_t *bsums);
+void rmi_ref_x86_quantize_row_q8_k(const float *x, size_t n, float *d,
+                                   int8_t *qs, int16_t *bsums);
+
+/* Threaded baseline: the (ith,nth) row partition of parallel.rs:124-138 over
+ * persistent threads with a spin barrier per matmul (the shape of
+ * ComputePool::compute, src/core/thread_pool.rs:119-161). */
+typedef struct rmi_ref_pool rmi_ref_pool;
+rmi_ref_pool *rmi_ref_pool_create(int n_threads);
+void rmi_ref_pool_destroy(rmi_ref_pool *pool);
+int rmi_ref_pool_threads(const rmi_ref_pool *pool);
+/* y[t] = W x[t] for t < n_tokens, AVX2 kernels, rows split over the pool. */
+void rmi_ref_pool_matmul_q8_0(rmi_ref_pool *pool, const uint8_t *weight,
+                              const uint8_t *input_q8,
+                              const float *input_scales, float *output,
+                              size_t n_in, size_t n_out, size_t n_tokens);
+void rmi_ref_pool_matmul_q4k_q8k(rmi_ref_pool *pool, const uint8_t *weight,
+                                 const float *d, const int8_t *qs,
+                                 const int16_t *bsums, float *output,
+                                 size_t n_in, size_t n_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RMI_ORACLE_H */
