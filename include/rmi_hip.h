@@ -1,0 +1,169 @@
+/*
+ * rmi_hip.h — C ABI of the MI355X (gfx950) back end for rust-model-inference's
+ * quantized-weight matrix products.
+ *
+ * This is what the crate's `hip` op back end binds over FFI.  Every entry
+ * point names the reference interface it stands in for (paths relative to the
+ * reference repository).  Conventions:
+ *   - plain pointers and sizes only; weights live behind opaque handles;
+ *   - functions returning int give 0 on success and a negative RMI_HIP_E_*
+ *     code on failure, never abort or throw; rmi_hip_last_error() returns the
+ *     message of the calling thread's last failure;
+ *   - "host" entry points take caller-owned host slices that are valid only
+ *     for the call (the `&[u8]` / `&mut [f32]` of the Kernel trait);
+ *     "_dev" entry points take device pointers and a hipStream_t (as void*),
+ *     enqueue work and return without synchronising;
+ *   - re-entrant: the Kernel trait is Send + Sync and is called concurrently
+ *     by all pool threads; every host thread gets its own stream and staging.
+ *
+ * f32 results of the Q8_0 GEMV and the Q4_K x Q8_K GEMV reproduce the
+ * accumulation order of the reference's x86-64 production kernels
+ * (avx2.rs:71-173, quant/mod.rs:701-799) bit for bit; the MFMA GEMM
+ * reproduces the fused sequential order of neon.rs:49-73.
+ */
+#ifndef RMI_HIP_H
+#define RMI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RMI_HIP_OK 0
+#define RMI_HIP_E_INVALID (-1)   /* bad argument / shape mismatch            */
+#define RMI_HIP_E_RUNTIME (-2)   /* HIP runtime error (message has details)  */
+#define RMI_HIP_E_NOT_INIT (-3)  /* rmi_hip_init has not succeeded           */
+#define RMI_HIP_E_NO_DEVICE (-4) /* no gfx950 device visible                 */
+
+#define RMI_HIP_DTYPE_Q8_0 8
+#define RMI_HIP_DTYPE_Q4_K 12
+
+/* Activation rounding of quantize_q8_0_into: the reference picks it per host
+ * architecture (src/ops/quant/q8_0.rs:3-24). */
+#define RMI_HIP_ROUND_HALF_AWAY 0 /* scalar path, :49-71: 1/d, round()        */
+#define RMI_HIP_ROUND_TIES_EVEN 1 /* AVX2 path, :176-230: 127/amax, rint()    */
+
+typedef struct rmi_hip_weight rmi_hip_weight;
+
+/* ---- context: replaces the lazy OnceLock GPU context of src/ops/float.rs:44-58.
+ * A failing init is the "fall back to CPU" signal of float.rs:51-57. */
+int rmi_hip_init(int device);
+void rmi_hip_shutdown(void);
+const char *rmi_hip_last_error(void);
+/* name/arch of the bound device, compute units, bytes of HBM */
+int rmi_hip_device_info(char *name, size_t name_len, int *compute_units, size_t *hbm_bytes);
+
+/* ---- weights: replace the borrowed `&[u8]` of QuantizedTensor::from_bytes /
+ * Q8Kernel::new / Q4_KKernel::new (src/ops/kernel/quantized_tensor.rs:120-138,
+ * q8_0/mod.rs:21-31, q4_k.rs:13-17).  The bytes are copied to HBM and repacked
+ * once; the host slice may be dropped afterwards.  NULL on failure. */
+rmi_hip_weight *rmi_hip_upload_q8_0(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
+rmi_hip_weight *rmi_hip_upload_q4_k(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
+/* QTensorOwned::fuse_vstack (src/ops/kernel/qtensor_owned.rs:138-164) and
+ * fuse_vstack_q8_0 / _q4_k (src/ops/quant/fuse.rs:25-64): rows of a then rows
+ * of b.  NULL (the reference's None) when dtype or n_in differ. */
+rmi_hip_weight *rmi_hip_fuse_vstack(const rmi_hip_weight *a, const rmi_hip_weight *b);
+void rmi_hip_free_weight(rmi_hip_weight *w);
+uint32_t rmi_hip_weight_n_in(const rmi_hip_weight *w);
+uint32_t rmi_hip_weight_n_out(const rmi_hip_weight *w);
+int rmi_hip_weight_dtype(const rmi_hip_weight *w);
+/* bytes this weight occupies in HBM after repacking */
+size_t rmi_hip_weight_device_bytes(const rmi_hip_weight *w);
+
+/* ---- Q8_0, host slices ---------------------------------------------------*/
+
+/* Kernel::forward_prequantized for Q8Kernel (src/ops/kernel/q8_0/mod.rs:33-55)
+ * = matmul_q8_0_quantized_parallel_rows (q8_0/parallel.rs:102-139): `output`
+ * is the FULL n_out-long slice; only rows of partition (ith, nth) are written. */
+int rmi_hip_q8_0_forward_prequantized(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth);
+/* matmul_q8_0_quantized_range (q8_0/dispatch.rs:27-108), the slot the Vulkan
+ * hook occupies (:36-52): `output` is PRE-SLICED, output[0] = row_start. */
+int rmi_hip_matmul_q8_0_quantized_range(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                        float *output, uint32_t n_in, uint32_t row_start, uint32_t row_end);
+/* n_tokens prequantized activations in one call: input_q8[n_tokens][n_in],
+ * input_scales[n_tokens][n_in/32], output[n_tokens][n_out] token-major
+ * (the layout of Kernel::forward_batched, trait_.rs:78-109). */
+int rmi_hip_matmul_q8_0_quantized_batch(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                        float *output, uint32_t n_in, uint32_t n_out, uint32_t n_tokens);
+/* Kernel::forward / forward_batched with f32 input (trait_.rs:59-109):
+ * quantize each token row on the device (rounding as given), then GEMV
+ * (n_tokens < gemm_min_tokens) or the MFMA GEMM. */
+int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens, int rounding);
+/* quantize_q8_0_into (src/ops/quant/q8_0.rs:3-24) run on the device. */
+int rmi_hip_quantize_q8_0(const float *input, uint32_t n, uint8_t *q8, float *scales, int rounding);
+/* The per-block int32 dots of scalar.rs:49-53, dots[n_out][n_in/32], computed
+ * from the repacked HBM copy (debug / parity entry point). */
+int rmi_hip_block_dots_q8_0(const rmi_hip_weight *w, const uint8_t *input_q8, int32_t *dots);
+/* ops::matmul_q8_0 (q8_0/parallel.rs:317-341): f32 activations used as they
+ * are, no activation quantisation. */
+int rmi_hip_matmul_q8_0_f32(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in, uint32_t n_out);
+
+/* ---- Q4_K, host slices ---------------------------------------------------*/
+
+/* Q4_KKernel::forward_prepared (src/ops/kernel/q4_k.rs:56-93) with the Q8_K
+ * activation passed as three arrays (BlockQ8K has no repr(C),
+ * src/ops/quant/mod.rs:35-40): d[n_in/256], qs[n_in], bsums[n_in/16]. */
+int rmi_hip_q4_k_forward_prepared(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                                  const int16_t *q8k_bsums, float *output, uint32_t n_in, uint32_t n_out, uint32_t ith,
+                                  uint32_t nth);
+/* Same with f32 input: quantize_row_q8_k on the device (quant/mod.rs:140-200),
+ * the `q8_k == None` branch of q4_k.rs:77-84; n_tokens rows, token-major out. */
+int rmi_hip_q4_k_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens);
+/* quantize_row_q8_k (quant/mod.rs:42-59) run on the device. */
+int rmi_hip_quantize_row_q8_k(const float *input, uint32_t n, float *d, int8_t *qs, int16_t *bsums);
+/* Q4_KKernel::forward_prequantized (q4_k.rs:20-54): dequantise-and-dot with
+ * the Q8_0 activation turned back into f32. */
+int rmi_hip_q4_k_forward_prequantized(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth);
+/* QuantizedLinear::forward / forward_dequant (src/core/model.rs:65-91): f32
+ * input, Q4_K weight dequantised in registers, no scratch needed. */
+int rmi_hip_quantized_linear_forward(const rmi_hip_weight *w, const float *input, float *output, uint32_t in_features,
+                                     uint32_t out_features);
+/* Exact integers of the Q4_K x Q8_K dot per super-block (parity entry point):
+ * isum/msum[n_out][n_in/256] as in vec_dot_q4k_q8k_scalar, quant/mod.rs:260-284. */
+int rmi_hip_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *q8k_qs, const int16_t *q8k_bsums, int32_t *isum,
+                            int32_t *msum);
+
+/* ---- device-resident entry points (activations stay in HBM) ---------------*/
+
+void *rmi_hip_malloc(size_t nbytes);
+void rmi_hip_free(void *dptr);
+int rmi_hip_memcpy_h2d(void *dst, const void *src, size_t nbytes);
+int rmi_hip_memcpy_d2h(void *dst, const void *src, size_t nbytes);
+int rmi_hip_synchronize(void);
+
+/* y[t][row] for rows [row_start,row_end) of n_tokens (1..8) activations.
+ * y has row stride 1 and token stride y_stride floats; y[t][0] is row 0. */
+int rmi_hip_gemv_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, void *stream);
+int rmi_hip_quantize_q8_0_dev(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
+                              int rounding, void *stream);
+/* Y[t][:] = W . Q8_0(X[t][:]) for n_tokens >= 1 through int8 MFMA. */
+int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                          uint32_t n_tokens, uint32_t y_stride, void *stream);
+int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                              const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride,
+                              uint32_t row_start, uint32_t row_end, void *stream);
+int rmi_hip_quantize_row_q8_k_dev(const float *x, float *d, int8_t *qs, int16_t *bsums, uint32_t n_tokens,
+                                  uint32_t n_in, void *stream);
+
+/* A fixed list of independent Q8_0 GEMVs (a token-step's projection set, or
+ * the q/k/v and gate/up pairs that share an input) run as ONE launch.  The
+ * reference issues them one after another inside one pool.compute closure
+ * (src/models/qwen3.rs:738-774, 991-1019). */
+typedef struct rmi_hip_gemv_group rmi_hip_gemv_group;
+rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip_weight *const *weights,
+                                              const int8_t *const *x_q8, const float *const *x_scales,
+                                              float *const *y, uint32_t n_tokens);
+void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g);
+int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RMI_HIP_H */

@@ -1,0 +1,192 @@
+// extern "C" entry points for Q4_K weights (Q4_KKernel and QuantizedLinear).
+#include "rmi_internal.h"
+
+namespace {
+
+int check_q4k(const rmi_hip_weight *w, uint32_t n_in, uint32_t n_out) {
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_K) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_K weight handle");
+    if (w->n_in != n_in || w->n_out != n_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "weight is %u x %u, call says %u x %u", w->n_out, w->n_in, n_out, n_in);
+    return RMI_HIP_OK;
+}
+
+// q4_k.rs:30-35: per_thread = ceil(n_out / nth)
+bool partition(uint32_t n_out, uint32_t ith, uint32_t nth, uint32_t *start, uint32_t *end) {
+    if (nth == 0) nth = 1;
+    const uint32_t per_thread = (n_out + nth - 1) / nth;
+    const uint64_t s = uint64_t(ith) * per_thread;
+    if (s >= n_out) return false;
+    *start = uint32_t(s);
+    *end = *start + per_thread < n_out ? *start + per_thread : n_out;
+    return *start < *end;
+}
+
+int fetch(RmiThreadCtx *c, void *host, const void *dev, size_t nbytes, int pin_slot) {
+    if (nbytes == 0) return RMI_HIP_OK;
+    void *pin = rmi_pin_buf(c, pin_slot, nbytes);
+    if (!pin) return RMI_HIP_E_RUNTIME;
+    RMI_HIP_CHECK(hipMemcpyAsync(pin, dev, nbytes, hipMemcpyDeviceToHost, c->stream));
+    RMI_HIP_CHECK(hipStreamSynchronize(c->stream));
+    memcpy(host, pin, nbytes);
+    return RMI_HIP_OK;
+}
+
+// host bytes -> device slot via pinned slot (same index)
+void *push(RmiThreadCtx *c, int slot, const void *host, size_t nbytes) {
+    void *pin = rmi_pin_buf(c, slot, nbytes);
+    void *dev = rmi_dev_buf(c, slot, nbytes);
+    if (!pin || !dev) return nullptr;
+    memcpy(pin, host, nbytes);
+    if (hipMemcpyAsync(dev, pin, nbytes, hipMemcpyHostToDevice, c->stream) != hipSuccess) {
+        rmi_set_error("hipMemcpyAsync H2D failed");
+        return nullptr;
+    }
+    return dev;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rmi_hip_q4_k_forward_prepared(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                                  const int16_t *q8k_bsums, float *output, uint32_t n_in, uint32_t n_out, uint32_t ith,
+                                  uint32_t nth) {
+    RMI_REQUIRE_INIT();
+    int rc = check_q4k(w, n_in, n_out);
+    if (rc != RMI_HIP_OK) return rc;
+    uint32_t start, end;
+    if (!partition(n_out, ith, nth, &start, &end)) return RMI_HIP_OK;
+    if (!q8k_d || !q8k_qs || !q8k_bsums || !output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const float *d_d = static_cast<const float *>(push(c, 0, q8k_d, size_t(n_in / 256) * 4));
+    const int8_t *d_qs = static_cast<const int8_t *>(push(c, 2, q8k_qs, n_in));
+    const int16_t *d_bs = static_cast<const int16_t *>(push(c, 3, q8k_bsums, size_t(n_in / 16) * 2));
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(end - start) * 4));
+    if (!d_d || !d_qs || !d_bs || !d_y) return RMI_HIP_E_RUNTIME;
+    rc = rmi_launch_gemv_q4_k(w, d_d, d_qs, d_bs, d_y - start, 1, end - start, start, end, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, output + start, d_y, size_t(end - start) * 4, 1);
+}
+
+int rmi_hip_q4_k_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens) {
+    RMI_REQUIRE_INIT();
+    int rc = check_q4k(w, n_in, n_out);
+    if (rc != RMI_HIP_OK) return rc;
+    if (n_tokens == 0 || n_out == 0) return RMI_HIP_OK;
+    if (!input || !output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const size_t n_x = size_t(n_tokens) * n_in;
+    const float *d_x = static_cast<const float *>(push(c, 0, input, n_x * 4));
+    int8_t *d_qs = static_cast<int8_t *>(rmi_dev_buf(c, 2, n_x));
+    int16_t *d_bs = static_cast<int16_t *>(rmi_dev_buf(c, 3, n_x / 16 * 2));
+    float *d_d = static_cast<float *>(rmi_dev_buf(c, 4, n_x / 256 * 4));
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(n_tokens) * n_out * 4));
+    if (!d_x || !d_qs || !d_bs || !d_d || !d_y) return RMI_HIP_E_RUNTIME;
+    rc = rmi_launch_quantize_q8_k(d_x, d_d, d_qs, d_bs, n_tokens, n_in, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    rc = rmi_launch_gemv_q4_k(w, d_d, d_qs, d_bs, d_y, n_tokens, n_out, 0, n_out, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, output, d_y, size_t(n_tokens) * n_out * 4, 1);
+}
+
+int rmi_hip_quantize_row_q8_k(const float *input, uint32_t n, float *d, int8_t *qs, int16_t *bsums) {
+    RMI_REQUIRE_INIT();
+    if (n % 256 != 0) return rmi_fail(RMI_HIP_E_INVALID, "n=%u is not a multiple of 256", n);  // quant/mod.rs:144 asserts
+    if (n == 0) return RMI_HIP_OK;
+    if (!input || !d || !qs || !bsums) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const float *d_x = static_cast<const float *>(push(c, 0, input, size_t(n) * 4));
+    int8_t *d_qs = static_cast<int8_t *>(rmi_dev_buf(c, 2, n));
+    int16_t *d_bs = static_cast<int16_t *>(rmi_dev_buf(c, 3, size_t(n) / 16 * 2));
+    float *d_d = static_cast<float *>(rmi_dev_buf(c, 4, size_t(n) / 256 * 4));
+    if (!d_x || !d_qs || !d_bs || !d_d) return RMI_HIP_E_RUNTIME;
+    int rc = rmi_launch_quantize_q8_k(d_x, d_d, d_qs, d_bs, 1, n, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    rc = fetch(c, qs, d_qs, n, 1);
+    if (rc == RMI_HIP_OK) rc = fetch(c, bsums, d_bs, size_t(n) / 16 * 2, 1);
+    if (rc == RMI_HIP_OK) rc = fetch(c, d, d_d, size_t(n) / 256 * 4, 1);
+    return rc;
+}
+
+int rmi_hip_q4_k_forward_prequantized(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth) {
+    RMI_REQUIRE_INIT();
+    int rc = check_q4k(w, n_in, n_out);
+    if (rc != RMI_HIP_OK) return rc;
+    uint32_t start, end;
+    if (!partition(n_out, ith, nth, &start, &end)) return RMI_HIP_OK;
+    if (!input_q8 || !input_scales || !output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const int8_t *d_q8 = static_cast<const int8_t *>(push(c, 0, input_q8, n_in));
+    const float *d_sc = static_cast<const float *>(push(c, 2, input_scales, size_t(n_in / 32) * 4));
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(end - start) * 4));
+    if (!d_q8 || !d_sc || !d_y) return RMI_HIP_E_RUNTIME;
+    rc = rmi_launch_q4_k_dequant_dot(w, nullptr, d_q8, d_sc, d_y - start, start, end, 0, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, output + start, d_y, size_t(end - start) * 4, 1);
+}
+
+int rmi_hip_quantized_linear_forward(const rmi_hip_weight *w, const float *input, float *output, uint32_t in_features,
+                                     uint32_t out_features) {
+    RMI_REQUIRE_INIT();
+    int rc = check_q4k(w, in_features, out_features);
+    if (rc != RMI_HIP_OK) return rc;
+    if (out_features == 0) return RMI_HIP_OK;
+    if (!input || !output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const float *d_x = static_cast<const float *>(push(c, 0, input, size_t(in_features) * 4));
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(out_features) * 4));
+    if (!d_x || !d_y) return RMI_HIP_E_RUNTIME;
+    rc = rmi_launch_q4_k_dequant_dot(w, d_x, nullptr, nullptr, d_y, 0, out_features, 1, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, output, d_y, size_t(out_features) * 4, 1);
+}
+
+int rmi_hip_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *q8k_qs, const int16_t *q8k_bsums, int32_t *isum,
+                            int32_t *msum) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_K) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_K weight handle");
+    const size_t n = size_t(w->n_out) * w->n_units;
+    if (n == 0) return RMI_HIP_OK;
+    if (!q8k_qs || !q8k_bsums || !isum || !msum) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const int8_t *d_qs = static_cast<const int8_t *>(push(c, 0, q8k_qs, w->n_in));
+    const int16_t *d_bs = static_cast<const int16_t *>(push(c, 2, q8k_bsums, size_t(w->n_in / 16) * 2));
+    int32_t *d_out = static_cast<int32_t *>(rmi_dev_buf(c, 1, n * 8));
+    if (!d_qs || !d_bs || !d_out) return RMI_HIP_E_RUNTIME;
+    int rc = rmi_launch_block_ints_q4_k(w, d_qs, d_bs, d_out, d_out + n, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    rc = fetch(c, isum, d_out, n * 4, 1);
+    if (rc == RMI_HIP_OK) rc = fetch(c, msum, d_out + n, n * 4, 1);
+    return rc;
+}
+
+int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                              const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride,
+                              uint32_t row_start, uint32_t row_end, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_K) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_K weight handle");
+    if (row_start >= row_end || n_tokens == 0) return RMI_HIP_OK;
+    if (row_end > w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) exceed n_out=%u", row_start, row_end, w->n_out);
+    if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
+    if (!q8k_d || !q8k_qs || !q8k_bsums || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    return rmi_launch_gemv_q4_k(w, q8k_d, q8k_qs, q8k_bsums, y, n_tokens, y_stride, row_start, row_end,
+                                static_cast<hipStream_t>(stream));
+}
+
+int rmi_hip_quantize_row_q8_k_dev(const float *x, float *d, int8_t *qs, int16_t *bsums, uint32_t n_tokens,
+                                  uint32_t n_in, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (n_in % 256 != 0) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u is not a multiple of 256", n_in);
+    if (!x || !d || !qs || !bsums) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    return rmi_launch_quantize_q8_k(x, d, qs, bsums, n_tokens, n_in, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,350 @@
+// extern "C" entry points for Q8_0 weights: the host-slice calls that stand in
+// for the Kernel trait methods, the device-resident calls, and GEMV groups.
+#include <vector>
+
+#include "rmi_internal.h"
+
+namespace {
+
+// GEMV launches take at most 8 tokens; at or above this many the MFMA GEMM runs.
+constexpr uint32_t kGemmMinTokens = 16;
+
+int check_q8(const rmi_hip_weight *w, uint32_t n_in, uint32_t n_out) {
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (w->n_in != n_in || w->n_out != n_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "weight is %u x %u, call says %u x %u", w->n_out, w->n_in, n_out, n_in);
+    return RMI_HIP_OK;
+}
+
+RmiGemvProblem make_problem(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                            uint32_t y_stride, uint32_t row_start, uint32_t row_end) {
+    RmiGemvProblem p{};
+    p.w = w->data;
+    p.x_q8 = x_q8;
+    p.x_scales = x_scales;
+    p.y = y;
+    p.n_in = w->n_in;
+    p.n_oct = w->n_units;
+    p.y_stride = y_stride;
+    p.row_start = row_start;
+    p.row_end = row_end;
+    p.tile0 = row_start / kTileRows;
+    p.n_tiles = row_end > row_start ? (row_end + kTileRows - 1) / kTileRows - p.tile0 : 0;
+    p.cost_begin = 0;
+    return p;
+}
+
+// tokens per GEMV launch so that the LDS staging fits
+uint32_t gemv_chunk(const rmi_hip_weight *w) {
+    const size_t per_token = size_t(w->n_units) * 288;
+    uint32_t c = per_token ? uint32_t((64 * 1024) / per_token) : 8;
+    return c > 8 ? 8 : c;
+}
+
+// device pointers in, rows [row_start,row_end) of n_tokens tokens
+int gemv_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
+                uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s) {
+    const uint32_t chunk = gemv_chunk(w);
+    if (chunk == 0) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u is too long for the GEMV staging", w->n_in);
+    const uint32_t nb = w->n_in / 32;
+    for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
+        const uint32_t nt = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
+        RmiGemvProblem p = make_problem(w, x_q8 + size_t(t0) * w->n_in, x_scales + size_t(t0) * nb,
+                                        y + size_t(t0) * y_stride, y_stride, row_start, row_end);
+        int rc = rmi_launch_gemv_q8_0_single(p, nt, s);
+        if (rc != RMI_HIP_OK) return rc;
+    }
+    return RMI_HIP_OK;
+}
+
+// host activation (q8 + scales) -> one pinned + one device buffer
+struct StagedX {
+    int8_t *d_q8;
+    float *d_scales;
+};
+int stage_x(RmiThreadCtx *c, const uint8_t *q8, const float *scales, size_t n_q8, size_t n_scales, StagedX *out) {
+    const size_t q_bytes = (n_q8 + 15) & ~size_t(15);
+    const size_t total = q_bytes + n_scales * 4;
+    uint8_t *pin = static_cast<uint8_t *>(rmi_pin_buf(c, 0, total));
+    uint8_t *dev = static_cast<uint8_t *>(rmi_dev_buf(c, 0, total));
+    if (!pin || !dev) return RMI_HIP_E_RUNTIME;
+    memcpy(pin, q8, n_q8);
+    memcpy(pin + q_bytes, scales, n_scales * 4);
+    RMI_HIP_CHECK(hipMemcpyAsync(dev, pin, total, hipMemcpyHostToDevice, c->stream));
+    out->d_q8 = reinterpret_cast<int8_t *>(dev);
+    out->d_scales = reinterpret_cast<float *>(dev + q_bytes);
+    return RMI_HIP_OK;
+}
+
+int fetch(RmiThreadCtx *c, void *host, const void *dev, size_t nbytes, int pin_slot) {
+    if (nbytes == 0) return RMI_HIP_OK;
+    void *pin = rmi_pin_buf(c, pin_slot, nbytes);
+    if (!pin) return RMI_HIP_E_RUNTIME;
+    RMI_HIP_CHECK(hipMemcpyAsync(pin, dev, nbytes, hipMemcpyDeviceToHost, c->stream));
+    RMI_HIP_CHECK(hipStreamSynchronize(c->stream));
+    memcpy(host, pin, nbytes);
+    return RMI_HIP_OK;
+}
+
+int host_gemv_range(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales, float *out_row_start,
+                    uint32_t n_tokens, uint32_t out_stride, uint32_t row_start, uint32_t row_end) {
+    if (row_start >= row_end) return RMI_HIP_OK;
+    if (row_end > w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) exceed n_out=%u", row_start, row_end, w->n_out);
+    if (!input_q8 || !input_scales || !out_row_start) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    StagedX x;
+    int rc = stage_x(c, input_q8, input_scales, size_t(n_tokens) * w->n_in, size_t(n_tokens) * (w->n_in / 32), &x);
+    if (rc != RMI_HIP_OK) return rc;
+    const uint32_t n_rows = row_end - row_start;
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(n_tokens) * n_rows * 4));
+    if (!d_y) return RMI_HIP_E_RUNTIME;
+    // device y holds only the row slice: y[t][row - row_start]
+    rc = gemv_tokens(w, x.d_q8, x.d_scales, d_y - row_start, n_tokens, n_rows, row_start, row_end, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    if (out_stride == n_rows) return fetch(c, out_row_start, d_y, size_t(n_tokens) * n_rows * 4, 1);
+    float *pin = static_cast<float *>(rmi_pin_buf(c, 1, size_t(n_tokens) * n_rows * 4));
+    if (!pin) return RMI_HIP_E_RUNTIME;
+    RMI_HIP_CHECK(hipMemcpyAsync(pin, d_y, size_t(n_tokens) * n_rows * 4, hipMemcpyDeviceToHost, c->stream));
+    RMI_HIP_CHECK(hipStreamSynchronize(c->stream));
+    for (uint32_t t = 0; t < n_tokens; t++)
+        memcpy(out_row_start + size_t(t) * out_stride, pin + size_t(t) * n_rows, size_t(n_rows) * 4);
+    return RMI_HIP_OK;
+}
+
+}  // namespace
+
+struct rmi_hip_gemv_group {
+    RmiGemvProblem *d_list = nullptr;
+    uint32_t n_problems = 0;
+    uint32_t total_cost = 0;
+    uint32_t total_tiles = 0;
+    uint32_t max_n_oct = 0;
+    uint32_t n_tokens = 0;
+};
+
+extern "C" {
+
+int rmi_hip_matmul_q8_0_quantized_range(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                        float *output, uint32_t n_in, uint32_t row_start, uint32_t row_end) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (w->n_in != n_in) return rmi_fail(RMI_HIP_E_INVALID, "weight has n_in=%u, call says %u", w->n_in, n_in);
+    return host_gemv_range(w, input_q8, input_scales, output, 1, row_end > row_start ? row_end - row_start : 0,
+                           row_start, row_end);
+}
+
+int rmi_hip_q8_0_forward_prequantized(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth) {
+    RMI_REQUIRE_INIT();
+    int rc = check_q8(w, n_in, n_out);
+    if (rc != RMI_HIP_OK) return rc;
+    uint32_t start = 0, end = n_out;
+    if (nth > 1 && n_out != 0) {  // parallel.rs:114-138
+        const uint32_t per_thread = (n_out + nth - 1) / nth;
+        const uint64_t s64 = uint64_t(ith) * per_thread;
+        if (s64 >= n_out) return RMI_HIP_OK;
+        start = uint32_t(s64);
+        end = start + per_thread < n_out ? start + per_thread : n_out;
+    }
+    if (start >= end) return RMI_HIP_OK;
+    if (!output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    return host_gemv_range(w, input_q8, input_scales, output + start, 1, end - start, start, end);
+}
+
+int rmi_hip_matmul_q8_0_quantized_batch(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                        float *output, uint32_t n_in, uint32_t n_out, uint32_t n_tokens) {
+    RMI_REQUIRE_INIT();
+    int rc = check_q8(w, n_in, n_out);
+    if (rc != RMI_HIP_OK) return rc;
+    if (n_tokens == 0 || n_out == 0) return RMI_HIP_OK;
+    return host_gemv_range(w, input_q8, input_scales, output, n_tokens, n_out, 0, n_out);
+}
+
+int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens, int rounding) {
+    RMI_REQUIRE_INIT();
+    int rc = check_q8(w, n_in, n_out);
+    if (rc != RMI_HIP_OK) return rc;
+    if (n_tokens == 0 || n_out == 0) return RMI_HIP_OK;
+    if (!input || !output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const size_t n_x = size_t(n_tokens) * n_in;
+    float *pin = static_cast<float *>(rmi_pin_buf(c, 0, n_x * 4));
+    float *d_x = static_cast<float *>(rmi_dev_buf(c, 0, n_x * 4));
+    int8_t *d_q8 = static_cast<int8_t *>(rmi_dev_buf(c, 2, n_x));
+    float *d_sc = static_cast<float *>(rmi_dev_buf(c, 3, n_x / 32 * 4));
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(n_tokens) * n_out * 4));
+    if (!pin || !d_x || !d_q8 || !d_sc || !d_y) return RMI_HIP_E_RUNTIME;
+    memcpy(pin, input, n_x * 4);
+    RMI_HIP_CHECK(hipMemcpyAsync(d_x, pin, n_x * 4, hipMemcpyHostToDevice, c->stream));
+    rc = rmi_launch_quantize_q8_0(d_x, d_q8, d_sc, n_tokens, n_in, rounding, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    if (n_tokens >= kGemmMinTokens)
+        rc = rmi_launch_gemm_q8_0(w, d_q8, d_sc, d_y, n_tokens, n_out, c->stream);
+    else
+        rc = gemv_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, output, d_y, size_t(n_tokens) * n_out * 4, 1);
+}
+
+int rmi_hip_quantize_q8_0(const float *input, uint32_t n, uint8_t *q8, float *scales, int rounding) {
+    RMI_REQUIRE_INIT();
+    const uint32_t blocks = n / 32;  // a ragged tail is left untouched, as in q8_0.rs:4
+    if (blocks == 0) return RMI_HIP_OK;
+    if (!input || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const size_t n_x = size_t(blocks) * 32;
+    float *pin = static_cast<float *>(rmi_pin_buf(c, 0, n_x * 4));
+    float *d_x = static_cast<float *>(rmi_dev_buf(c, 0, n_x * 4));
+    const size_t q_bytes = (n_x + 15) & ~size_t(15);
+    uint8_t *d_out = static_cast<uint8_t *>(rmi_dev_buf(c, 2, q_bytes + size_t(blocks) * 4));
+    if (!pin || !d_x || !d_out) return RMI_HIP_E_RUNTIME;
+    memcpy(pin, input, n_x * 4);
+    RMI_HIP_CHECK(hipMemcpyAsync(d_x, pin, n_x * 4, hipMemcpyHostToDevice, c->stream));
+    int rc = rmi_launch_quantize_q8_0(d_x, reinterpret_cast<int8_t *>(d_out), reinterpret_cast<float *>(d_out + q_bytes),
+                                      1, blocks * 32, rounding, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    uint8_t *pout = static_cast<uint8_t *>(rmi_pin_buf(c, 1, q_bytes + size_t(blocks) * 4));
+    if (!pout) return RMI_HIP_E_RUNTIME;
+    RMI_HIP_CHECK(hipMemcpyAsync(pout, d_out, q_bytes + size_t(blocks) * 4, hipMemcpyDeviceToHost, c->stream));
+    RMI_HIP_CHECK(hipStreamSynchronize(c->stream));
+    memcpy(q8, pout, n_x);
+    memcpy(scales, pout + q_bytes, size_t(blocks) * 4);
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_block_dots_q8_0(const rmi_hip_weight *w, const uint8_t *input_q8, int32_t *dots) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    const size_t n = size_t(w->n_out) * (w->n_in / 32);
+    if (n == 0) return RMI_HIP_OK;
+    if (!input_q8 || !dots) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    uint8_t *pin = static_cast<uint8_t *>(rmi_pin_buf(c, 0, w->n_in));
+    int8_t *d_x = static_cast<int8_t *>(rmi_dev_buf(c, 0, w->n_in));
+    int32_t *d_dots = static_cast<int32_t *>(rmi_dev_buf(c, 1, n * 4));
+    if (!pin || !d_x || !d_dots) return RMI_HIP_E_RUNTIME;
+    memcpy(pin, input_q8, w->n_in);
+    RMI_HIP_CHECK(hipMemcpyAsync(d_x, pin, w->n_in, hipMemcpyHostToDevice, c->stream));
+    int rc = rmi_launch_block_dots_q8_0(w, d_x, d_dots, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, dots, d_dots, n * 4, 1);
+}
+
+int rmi_hip_matmul_q8_0_f32(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in, uint32_t n_out) {
+    RMI_REQUIRE_INIT();
+    int rc = check_q8(w, n_in, n_out);
+    if (rc != RMI_HIP_OK) return rc;
+    if (n_out == 0) return RMI_HIP_OK;
+    if (!input || !output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    float *pin = static_cast<float *>(rmi_pin_buf(c, 0, size_t(n_in) * 4));
+    float *d_x = static_cast<float *>(rmi_dev_buf(c, 0, size_t(n_in) * 4));
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(n_out) * 4));
+    if (!pin || !d_x || !d_y) return RMI_HIP_E_RUNTIME;
+    memcpy(pin, input, size_t(n_in) * 4);
+    RMI_HIP_CHECK(hipMemcpyAsync(d_x, pin, size_t(n_in) * 4, hipMemcpyHostToDevice, c->stream));
+    rc = rmi_launch_matmul_q8_0_f32(w, d_x, d_y, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, output, d_y, size_t(n_out) * 4, 1);
+}
+
+// ------------------------------------------------------ device-resident
+
+int rmi_hip_gemv_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (row_start >= row_end || n_tokens == 0) return RMI_HIP_OK;
+    if (row_end > w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) exceed n_out=%u", row_start, row_end, w->n_out);
+    if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
+    if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    return gemv_tokens(w, x_q8, x_scales, y, n_tokens, y_stride, row_start, row_end, static_cast<hipStream_t>(stream));
+}
+
+int rmi_hip_quantize_q8_0_dev(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
+                              int rounding, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (n_in % 32 != 0) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u is not a multiple of 32", n_in);
+    if (!x || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    return rmi_launch_quantize_q8_0(x, q8, scales, n_tokens, n_in, rounding, static_cast<hipStream_t>(stream));
+}
+
+int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                          uint32_t n_tokens, uint32_t y_stride, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
+    if (y_stride < w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < n_out=%u", y_stride, w->n_out);
+    if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    return rmi_launch_gemm_q8_0(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
+}
+
+rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip_weight *const *weights,
+                                              const int8_t *const *x_q8, const float *const *x_scales,
+                                              float *const *y, uint32_t n_tokens) {
+    if (!rmi_ready()) {
+        rmi_set_error("rmi_hip_init has not succeeded");
+        return nullptr;
+    }
+    if (n_problems == 0 || n_tokens == 0 || n_tokens > 8 || !weights || !x_q8 || !x_scales || !y) {
+        rmi_set_error("gemv group needs >=1 problem and 1..8 tokens");
+        return nullptr;
+    }
+    if (!rmi_thread_ctx()) return nullptr;
+    std::vector<RmiGemvProblem> list(n_problems);
+    rmi_hip_gemv_group *g = new rmi_hip_gemv_group();
+    g->n_problems = n_problems;
+    g->n_tokens = n_tokens;
+    uint64_t cost = 0;
+    for (uint32_t i = 0; i < n_problems; i++) {
+        const rmi_hip_weight *w = weights[i];
+        if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0 || !x_q8[i] || !x_scales[i] || !y[i]) {
+            rmi_set_error("gemv group problem %u: bad weight handle or null pointer", i);
+            delete g;
+            return nullptr;
+        }
+        list[i] = make_problem(w, x_q8[i], x_scales[i], y[i], w->n_out, 0, w->n_out);
+        list[i].cost_begin = uint32_t(cost);
+        cost += uint64_t(list[i].n_tiles) * list[i].n_oct;
+        g->total_tiles += list[i].n_tiles;
+        if (w->n_units > g->max_n_oct) g->max_n_oct = w->n_units;
+    }
+    if (cost > 0xffffffffull || size_t(n_tokens) * g->max_n_oct * 288 > 64 * 1024) {
+        rmi_set_error("gemv group too large (cost %llu, %u tokens x %u octets)", (unsigned long long)cost, n_tokens,
+                      g->max_n_oct);
+        delete g;
+        return nullptr;
+    }
+    g->total_cost = uint32_t(cost);
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&g->d_list), sizeof(RmiGemvProblem) * n_problems);
+    if (e == hipSuccess)
+        e = hipMemcpy(g->d_list, list.data(), sizeof(RmiGemvProblem) * n_problems, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        rmi_set_error("gemv group upload failed: %s", hipGetErrorString(e));
+        if (g->d_list) hipFree(g->d_list);
+        delete g;
+        return nullptr;
+    }
+    return g;
+}
+
+void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g) {
+    if (!g) return;
+    if (g->d_list) hipFree(g->d_list);
+    delete g;
+}
+
+int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!g) return rmi_fail(RMI_HIP_E_INVALID, "null group");
+    return rmi_launch_gemv_q8_0_group(g->d_list, g->n_problems, g->total_cost, g->total_tiles, g->max_n_oct,
+                                      g->n_tokens, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

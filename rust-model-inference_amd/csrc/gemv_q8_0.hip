@@ -1,0 +1,302 @@
+// Q8_0 x Q8_0 decode GEMV (1..8 tokens) over the HBM tile stream, the per-block
+// integer dots, the device activation quantizer and the f32-activation GEMV.
+//
+// Arithmetic order of the GEMV = matmul_q8_0_vs_q8_0_avx2
+// (src/ops/kernel/q8_0/avx2.rs:71-173): eight f32 accumulators per row, lane L
+// taking fma(f32(wd)*xs[b], float(sum_{k=4L..4L+3} w*x), acc_L) block after
+// block, then hsum_ps (src/ops/dot.rs:447-456).  Eight GPU lanes hold the eight
+// accumulators of one row, so results match that kernel bit for bit.
+#include "rmi_internal.h"
+
+namespace {
+
+__device__ __forceinline__ float h2f(uint32_t bits16) {
+    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
+}
+
+// lane L of 8: ((l0+l4)+(l1+l5)) + ((l2+l6)+(l3+l7)), valid in lane 0 of the group
+__device__ __forceinline__ float hsum8_lanes(float a) {
+    a = a + __shfl_xor(a, 4, 64);
+    a = a + __shfl_xor(a, 1, 64);
+    a = a + __shfl_xor(a, 2, 64);
+    return a;
+}
+
+__device__ __forceinline__ void block_fma(float &acc, uint32_t w_bits, float xs, int wq, int xq) {
+    const float s = h2f(w_bits) * xs;  // one rounding, as _mm_mul_ps(cvtph, set1(bd))
+    const int p = __builtin_amdgcn_sdot4(wq, xq, 0, false);
+    acc = __builtin_fmaf(s, float(p), acc);
+}
+
+// One wave per workgroup.  The wave walks a contiguous range of 8-row tiles
+// (possibly across several problems of a group) and keeps the activation of
+// the current problem in LDS, permuted to the weight's quad order.
+template <int B>
+__global__ __launch_bounds__(64) void gemv_q8_0_kernel(RmiGemvProblem single,
+                                                        const RmiGemvProblem *__restrict__ list, uint32_t n_problems,
+                                                        uint32_t total_cost, uint32_t n_waves) {
+    extern __shared__ uint4 lds[];
+    const uint32_t lane = threadIdx.x, r = lane >> 3, L = lane & 7;
+    const uint64_t c0 = uint64_t(total_cost) * blockIdx.x / n_waves;
+    const uint64_t c1 = uint64_t(total_cost) * (blockIdx.x + 1) / n_waves;
+    if (c0 >= c1) return;
+
+    // problem that holds cost position c0
+    uint32_t pi = 0;
+    if (list) {
+        uint32_t lo = 0, hi = n_problems;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (list[mid].cost_begin <= c0) lo = mid; else hi = mid;
+        }
+        pi = lo;
+    }
+    RmiGemvProblem p = list ? list[pi] : single;
+    // first tile whose start cost is >= c0
+    uint32_t k = uint32_t((c0 - p.cost_begin + p.n_oct - 1) / p.n_oct);
+    bool staged = false;
+
+    for (;;) {
+        if (k >= p.n_tiles) {
+            pi++;
+            if (!list || pi >= n_problems) break;
+            p = list[pi];
+            k = 0;
+            staged = false;
+            continue;
+        }
+        if (uint64_t(p.cost_begin) + uint64_t(k) * p.n_oct >= c1) break;
+
+        const uint32_t n_oct = p.n_oct;
+        const uint32_t tok_u4 = n_oct * 18;  // per token: 16 uint4 of quants + 2 of scales per octet
+        if (!staged) {
+            __syncthreads();  // earlier reads of the previous activation are done
+            const uint32_t nb = p.n_in >> 5;
+            uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
+            for (int t = 0; t < B; t++) {
+                const uint32_t *xq = reinterpret_cast<const uint32_t *>(p.x_q8 + size_t(t) * p.n_in);
+                const float *xs = p.x_scales + size_t(t) * nb;
+                uint32_t *dq = lds_dw + t * tok_u4 * 4;
+                for (uint32_t i = lane; i < n_oct * 64; i += 64) {
+                    const uint32_t b = i >> 3, l = i & 7;
+                    dq[(b >> 2) * 32 + l * 4 + (b & 3)] = b < nb ? xq[i] : 0u;
+                }
+                float *ds = reinterpret_cast<float *>(dq + n_oct * 64);
+                for (uint32_t i = lane; i < n_oct * 8; i += 64) ds[i] = i < nb ? xs[i] : 0.0f;
+            }
+            __syncthreads();
+            staged = true;
+        }
+
+        const uint4 *tile = reinterpret_cast<const uint4 *>(p.w + size_t(p.tile0 + k) * n_oct * kOctetBytes);
+        const uint4 *sc_ptr = tile + r;
+        const uint4 *q_ptr = tile + n_oct * 8 + lane;
+
+        float acc[B];
+#pragma unroll
+        for (int t = 0; t < B; t++) acc[t] = 0.0f;
+
+        for (uint32_t o0 = 0; o0 < n_oct; o0 += 4) {
+            uint4 sc[4], qa[4], qb[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (o0 + i < n_oct) {
+                    sc[i] = sc_ptr[(o0 + i) * 8];
+                    qa[i] = q_ptr[(2 * (o0 + i)) * 64];
+                    qb[i] = q_ptr[(2 * (o0 + i) + 1) * 64];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (o0 + i < n_oct) {
+                    const uint32_t o = o0 + i;
+#pragma unroll
+                    for (int t = 0; t < B; t++) {
+                        const uint4 *xt = lds + t * tok_u4;
+                        const uint4 xa = xt[(2 * o) * 8 + L];
+                        const uint4 xb = xt[(2 * o + 1) * 8 + L];
+                        const float4 s0 = reinterpret_cast<const float4 *>(xt + n_oct * 16)[2 * o];
+                        const float4 s1 = reinterpret_cast<const float4 *>(xt + n_oct * 16)[2 * o + 1];
+                        float a = acc[t];
+                        block_fma(a, sc[i].x & 0xffffu, s0.x, int(qa[i].x), int(xa.x));
+                        block_fma(a, sc[i].x >> 16, s0.y, int(qa[i].y), int(xa.y));
+                        block_fma(a, sc[i].y & 0xffffu, s0.z, int(qa[i].z), int(xa.z));
+                        block_fma(a, sc[i].y >> 16, s0.w, int(qa[i].w), int(xa.w));
+                        block_fma(a, sc[i].z & 0xffffu, s1.x, int(qb[i].x), int(xb.x));
+                        block_fma(a, sc[i].z >> 16, s1.y, int(qb[i].y), int(xb.y));
+                        block_fma(a, sc[i].w & 0xffffu, s1.z, int(qb[i].z), int(xb.z));
+                        block_fma(a, sc[i].w >> 16, s1.w, int(qb[i].w), int(xb.w));
+                        acc[t] = a;
+                    }
+                }
+            }
+        }
+
+        const uint32_t row = (p.tile0 + k) * kTileRows + r;
+#pragma unroll
+        for (int t = 0; t < B; t++) {
+            const float y = hsum8_lanes(acc[t]);
+            if (L == 0 && row >= p.row_start && row < p.row_end) p.y[size_t(t) * p.y_stride + row] = y;
+        }
+        k++;
+    }
+}
+
+template <int B>
+int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, uint32_t n_problems, uint32_t total_cost,
+                uint32_t total_tiles, uint32_t max_n_oct, hipStream_t s) {
+    const size_t lds_bytes = size_t(B) * max_n_oct * 288;
+    if (lds_bytes > 64 * 1024)
+        return rmi_fail(RMI_HIP_E_INVALID, "activation of %d tokens x %u elements does not fit the LDS staging", B,
+                        max_n_oct * 256);
+    uint32_t n_waves = uint32_t(rmi_device_cus()) * 16;
+    if (n_waves > total_tiles) n_waves = total_tiles;
+    RmiGemvProblem dummy{};
+    hipLaunchKernelGGL(gemv_q8_0_kernel<B>, dim3(n_waves), dim3(64), lds_bytes, s, single ? *single : dummy, d_list,
+                       n_problems, total_cost, n_waves);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int dispatch_gemv(uint32_t n_tokens, const RmiGemvProblem *single, const RmiGemvProblem *d_list, uint32_t n_problems,
+                  uint32_t total_cost, uint32_t total_tiles, uint32_t max_n_oct, hipStream_t s) {
+    if (total_tiles == 0 || total_cost == 0) return RMI_HIP_OK;
+    switch (n_tokens) {
+        case 1: return launch_gemv<1>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        case 2: return launch_gemv<2>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        case 3: return launch_gemv<3>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        case 4: return launch_gemv<4>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        case 5: return launch_gemv<5>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        case 6: return launch_gemv<6>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        case 7: return launch_gemv<7>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        case 8: return launch_gemv<8>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        default: return rmi_fail(RMI_HIP_E_INVALID, "gemv takes 1..8 tokens per launch, got %u", n_tokens);
+    }
+}
+
+// ---- per-block integer dots from the repacked stream ----
+__global__ __launch_bounds__(256) void block_dots_q8_0_kernel(const uint8_t *__restrict__ w,
+                                                               const int8_t *__restrict__ x_q8,
+                                                               int32_t *__restrict__ dots, uint32_t n_out, uint32_t nb,
+                                                               uint32_t n_oct) {
+    const uint64_t total = uint64_t(n_out) * nb;
+    for (uint64_t i = blockIdx.x * uint64_t(blockDim.x) + threadIdx.x; i < total;
+         i += uint64_t(gridDim.x) * blockDim.x) {
+        const uint32_t row = uint32_t(i / nb), b = uint32_t(i % nb);
+        const uint8_t *tile = w + size_t(row >> 3) * n_oct * kOctetBytes;
+        const uint32_t *quad =
+            reinterpret_cast<const uint32_t *>(tile + size_t(n_oct) * 128 + size_t(b >> 2) * 1024 + (row & 7) * 128);
+        const uint32_t *xq = reinterpret_cast<const uint32_t *>(x_q8 + size_t(b) * 32);
+        int acc = 0;
+        for (uint32_t L = 0; L < 8; L++) acc = __builtin_amdgcn_sdot4(int(quad[L * 4 + (b & 3)]), int(xq[L]), acc, false);
+        dots[i] = acc;
+    }
+}
+
+// ---- quantize_q8_0_into on the device: 8 lanes per 32-element block ----
+__global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restrict__ x, int8_t *__restrict__ q8,
+                                                             float *__restrict__ scales, uint32_t n_blocks,
+                                                             int rounding) {
+    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t b = gid >> 3, l = gid & 7;
+    if (b >= n_blocks) return;  // whole 8-lane groups leave together
+    const float4 v = reinterpret_cast<const float4 *>(x)[size_t(b) * 8 + l];
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    const float d = amax == 0.0f ? 0.0f : amax / 127.0f;
+    float r0, r1, r2, r3;
+    if (rounding == RMI_HIP_ROUND_TIES_EVEN) {
+        const float id = amax == 0.0f ? 0.0f : 127.0f / amax;
+        r0 = rintf(v.x * id);
+        r1 = rintf(v.y * id);
+        r2 = rintf(v.z * id);
+        r3 = rintf(v.w * id);
+    } else {
+        const float inv = d == 0.0f ? 0.0f : 1.0f / d;
+        r0 = roundf(v.x * inv);
+        r1 = roundf(v.y * inv);
+        r2 = roundf(v.z * inv);
+        r3 = roundf(v.w * inv);
+    }
+    // NaN: the AVX2 clamp max_ps(r,-128) yields -128, Rust's clamp + `as i8` yields 0
+    const bool even = rounding == RMI_HIP_ROUND_TIES_EVEN;
+    const int i0 = (r0 != r0 && !even) ? 0 : int(fminf(fmaxf(r0, -128.0f), 127.0f));
+    const int i1 = (r1 != r1 && !even) ? 0 : int(fminf(fmaxf(r1, -128.0f), 127.0f));
+    const int i2 = (r2 != r2 && !even) ? 0 : int(fminf(fmaxf(r2, -128.0f), 127.0f));
+    const int i3 = (r3 != r3 && !even) ? 0 : int(fminf(fmaxf(r3, -128.0f), 127.0f));
+    reinterpret_cast<uint32_t *>(q8)[size_t(b) * 8 + l] =
+        uint32_t(i0 & 0xff) | (uint32_t(i1 & 0xff) << 8) | (uint32_t(i2 & 0xff) << 16) | (uint32_t(i3 & 0xff) << 24);
+    if (l == 0) scales[b] = float(_Float16(d));
+}
+
+// ---- ops::matmul_q8_0 with f32 activations, AVX2 order (avx2.rs:180-217):
+// two 8-lane accumulators; elements 0-7 and 16-23 of a block feed acc0, 8-15
+// and 24-31 feed acc1, each as fma(d*float(q), x, acc); y = hsum(acc0+acc1).
+// Lane i of 8 holds acc0[i] and acc1[i]; one 8-lane group per row. ----
+__global__ __launch_bounds__(64) void matmul_q8_0_f32_kernel(const uint8_t *__restrict__ w,
+                                                              const float *__restrict__ x, float *__restrict__ y,
+                                                              uint32_t n_out, uint32_t nb, uint32_t n_oct) {
+    const uint32_t lane = threadIdx.x, r = lane >> 3, i = lane & 7;
+    const uint32_t tile_idx = blockIdx.x;
+    const uint8_t *tile = w + size_t(tile_idx) * n_oct * kOctetBytes;
+    const uint8_t *quants = tile + size_t(n_oct) * 128;
+    float acc0 = 0.0f, acc1 = 0.0f;
+    for (uint32_t b = 0; b < nb; b++) {
+        const float d = h2f(reinterpret_cast<const uint16_t *>(tile + size_t(b >> 3) * 128 + r * 16)[b & 7]);
+        const uint8_t *quad = quants + size_t(b >> 2) * 1024 + r * 128 + (b & 3) * 4;
+        // element e of the block sits in the slice of lane e/4 at byte e%4
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t e = g * 8 + i;
+            const float q = float(int(int8_t(quad[(e >> 2) * 16 + (e & 3)])));
+            const float wq = d * q;
+            const float xv = x[size_t(b) * 32 + e];
+            if (g & 1) acc1 = __builtin_fmaf(wq, xv, acc1); else acc0 = __builtin_fmaf(wq, xv, acc0);
+        }
+    }
+    const float s = hsum8_lanes(acc0 + acc1);
+    const uint32_t row = tile_idx * kTileRows + r;
+    if (i == 0 && row < n_out) y[row] = s;
+}
+
+}  // namespace
+
+int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s) {
+    return dispatch_gemv(n_tokens, &p, nullptr, 1, p.n_tiles * p.n_oct, p.n_tiles, p.n_oct, s);
+}
+
+int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, uint32_t n_problems, uint32_t total_cost,
+                               uint32_t total_tiles, uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s) {
+    return dispatch_gemv(n_tokens, nullptr, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+}
+
+int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s) {
+    const uint64_t total = uint64_t(w->n_out) * (w->n_in / 32);
+    if (total == 0) return RMI_HIP_OK;
+    const uint32_t grid = uint32_t(total / 256 + 1 < 65535 ? total / 256 + 1 : 65535);
+    hipLaunchKernelGGL(block_dots_q8_0_kernel, dim3(grid), dim3(256), 0, s, w->data, x_q8, dots, w->n_out,
+                       w->n_in / 32, w->n_units);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int rmi_launch_quantize_q8_0(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
+                             int rounding, hipStream_t s) {
+    const uint64_t n_blocks = uint64_t(n_tokens) * (n_in / 32);
+    if (n_blocks == 0) return RMI_HIP_OK;
+    if (n_blocks * 8 > 0xffffffffull) return rmi_fail(RMI_HIP_E_INVALID, "activation too large for one launch");
+    const uint32_t grid = uint32_t((n_blocks * 8 + 255) / 256);
+    hipLaunchKernelGGL(quantize_q8_0_kernel, dim3(grid), dim3(256), 0, s, x, q8, scales, uint32_t(n_blocks), rounding);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int rmi_launch_matmul_q8_0_f32(const rmi_hip_weight *w, const float *x, float *y, hipStream_t s) {
+    if (w->n_tiles == 0) return RMI_HIP_OK;
+    hipLaunchKernelGGL(matmul_q8_0_f32_kernel, dim3(w->n_tiles), dim3(64), 0, s, w->data, x, y, w->n_out,
+                       w->n_in / 32, w->n_units);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}

@@ -1,0 +1,128 @@
+// Internal declarations shared by the translation units of librmi_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/rmi_hip.h"
+
+// ---------------------------------------------------------------- layouts
+//
+// Q8_0 weights in HBM ("tile stream").  Rows are grouped in tiles of 8, the
+// blocks of a row in octets of 8 (256 elements).  One tile is contiguous:
+//
+//   [ scales : n_oct x (8 rows x 8 f16)           ]  n_oct x 128 B
+//   [ quants : 2*n_oct quads x (8 rows x 8 L x 16) ]  n_oct x 2048 B
+//
+// A quad is 4 consecutive blocks; inside it, for row r and lane L (0..7) the
+// 16 bytes are the 4-byte slices k = 4L..4L+3 of blocks 4q+0..4q+3.  A wave
+// (8 rows x 8 lanes) therefore reads one quad with a single fully coalesced
+// 1 KiB load, and lane L owns exactly the elements that lane L of the
+// reference's 8-lane f32 accumulator sums (avx2.rs:128-147).  Rows beyond
+// n_out and blocks beyond n_in/32 are zero (scale 0, quants 0).  The stream
+// carries 34 bytes per block, the same as the source format.
+constexpr uint32_t kTileRows = 8;
+constexpr uint32_t kOctetBytes = 128 + 2048;  // per tile per octet
+
+// Q4_K weights in HBM.  Tiles of 8 rows; per tile and super-block:
+//
+//   [ header : 8 rows x 16 B ]  f16 d, f16 dmin, the 12 packed scale bytes
+//   [ quants : 8 rows x 8 L x 16 B ]  1024 B
+//
+// The 16 bytes of (row r, lane L) are four dwords, one per 32-byte group g of
+// the 128 nibble bytes: bytes 32g+4L..32g+4L+3, i.e. elements 64g+4L.. (low
+// nibbles, sub-block 2g) and 64g+32+4L.. (high nibbles, sub-block 2g+1).  Lane
+// L thus owns what lane L of the reference's 8-lane integer accumulator sums
+// (quant/mod.rs:770-790), and a wave reads a super-block of 8 rows with one
+// coalesced 1 KiB load.  144 bytes per super-block, as in the source format.
+constexpr uint32_t kQ4KSuperBytes = 8 * 16 + 1024;  // per tile per super-block
+
+struct rmi_hip_weight {
+    int dtype;
+    uint32_t n_in;
+    uint32_t n_out;
+    uint32_t n_tiles;   // ceil(n_out / 8)
+    uint32_t n_units;   // Q8_0: octets per row; Q4_K: super-blocks per row
+    size_t tile_bytes;  // bytes of one tile
+    size_t nbytes;      // device allocation
+    uint8_t *data;      // device pointer
+};
+
+// ------------------------------------------------------------------ errors
+void rmi_set_error(const char *fmt, ...);
+int rmi_fail(int code, const char *fmt, ...);
+bool rmi_ready();
+
+#define RMI_HIP_CHECK(expr)                                                                        \
+    do {                                                                                           \
+        hipError_t _e = (expr);                                                                    \
+        if (_e != hipSuccess)                                                                      \
+            return rmi_fail(RMI_HIP_E_RUNTIME, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, \
+                            __LINE__);                                                             \
+    } while (0)
+
+#define RMI_REQUIRE_INIT()                                                             \
+    do {                                                                               \
+        if (!rmi_ready()) return rmi_fail(RMI_HIP_E_NOT_INIT, "rmi_hip_init has not succeeded"); \
+    } while (0)
+
+// ---------------------------------------------------- per-thread staging
+// One per calling host thread: its own stream plus device and pinned host
+// buffers that grow on demand, so concurrent Kernel calls never share state.
+struct RmiThreadCtx {
+    hipStream_t stream = nullptr;
+    void *dev[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    size_t dev_cap[6] = {0, 0, 0, 0, 0, 0};
+    void *pin[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    size_t pin_cap[6] = {0, 0, 0, 0, 0, 0};
+};
+RmiThreadCtx *rmi_thread_ctx();
+// slot buffers, grown to at least nbytes; nullptr on failure (error is set)
+void *rmi_dev_buf(RmiThreadCtx *c, int slot, size_t nbytes);
+void *rmi_pin_buf(RmiThreadCtx *c, int slot, size_t nbytes);
+int rmi_device_cus();
+
+// ------------------------------------------------- launchers (device ptrs)
+int rmi_launch_repack_q8_0(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
+int rmi_launch_repack_q4_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
+int rmi_launch_copy_rows(const rmi_hip_weight *src, rmi_hip_weight *dst, uint32_t dst_row0, hipStream_t s);
+
+struct RmiGemvProblem {
+    const uint8_t *w;      // tile stream
+    const int8_t *x_q8;    // [n_tokens][n_in]
+    const float *x_scales; // [n_tokens][n_in/32]
+    float *y;              // y[t*y_stride + row]
+    uint32_t n_in;
+    uint32_t n_oct;
+    uint32_t y_stride;
+    uint32_t row_start;    // rows written: [row_start, row_end)
+    uint32_t row_end;
+    uint32_t tile0;        // first tile touched
+    uint32_t n_tiles;      // tiles touched
+    uint32_t cost_begin;   // prefix sum of n_tiles*n_oct over earlier problems
+};
+int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
+int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, uint32_t n_problems, uint32_t total_cost,
+                               uint32_t total_tiles, uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s);
+int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s);
+int rmi_launch_quantize_q8_0(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
+                             int rounding, hipStream_t s);
+int rmi_launch_matmul_q8_0_f32(const rmi_hip_weight *w, const float *x, float *y, hipStream_t s);
+int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                         uint32_t n_tokens, uint32_t y_stride, hipStream_t s);
+
+int rmi_launch_quantize_q8_k(const float *x, float *d, int8_t *qs, int16_t *bsums, uint32_t n_tokens, uint32_t n_in,
+                             hipStream_t s);
+int rmi_launch_gemv_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
+                         uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s);
+int rmi_launch_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *qs, const int16_t *bsums, int32_t *isum,
+                               int32_t *msum, hipStream_t s);
+// mode 0: x = q8 * scale rebuilt per element (Q4_KKernel::forward_prequantized)
+// mode 1: raw f32 x (QuantizedLinear::forward_dequant)
+int rmi_launch_q4_k_dequant_dot(const rmi_hip_weight *w, const float *x_f32, const int8_t *x_q8,
+                                const float *x_scales, float *y, uint32_t row_start, uint32_t row_end, int mode,
+                                hipStream_t s);

@@ -1,0 +1,304 @@
+// Context, error reporting, per-thread staging, weight upload / fusion.
+#include <mutex>
+#include <vector>
+
+#include "rmi_internal.h"
+
+namespace {
+
+thread_local char t_error[512] = "";
+int g_device = -1;
+int g_cus = 0;
+size_t g_hbm = 0;
+char g_name[128] = "";
+std::mutex g_mutex;
+std::vector<RmiThreadCtx *> g_ctxs;
+thread_local RmiThreadCtx *t_ctx = nullptr;
+
+}  // namespace
+
+void rmi_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_error, sizeof(t_error), fmt, ap);
+    va_end(ap);
+}
+
+int rmi_fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_error, sizeof(t_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool rmi_ready() { return g_device >= 0; }
+int rmi_device_cus() { return g_cus; }
+
+RmiThreadCtx *rmi_thread_ctx() {
+    if (t_ctx) return t_ctx;
+    if (hipSetDevice(g_device) != hipSuccess) {
+        rmi_set_error("hipSetDevice(%d) failed", g_device);
+        return nullptr;
+    }
+    RmiThreadCtx *c = new RmiThreadCtx();
+    // default priority: mixed-priority streams are not used anywhere
+    if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
+        rmi_set_error("hipStreamCreate failed");
+        delete c;
+        return nullptr;
+    }
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        g_ctxs.push_back(c);
+    }
+    t_ctx = c;
+    return c;
+}
+
+void *rmi_dev_buf(RmiThreadCtx *c, int slot, size_t nbytes) {
+    if (nbytes == 0) nbytes = 16;
+    if (c->dev_cap[slot] >= nbytes) return c->dev[slot];
+    if (c->dev[slot]) {
+        // the stream may still read the old buffer
+        hipStreamSynchronize(c->stream);
+        hipFree(c->dev[slot]);
+        c->dev[slot] = nullptr;
+        c->dev_cap[slot] = 0;
+    }
+    size_t cap = (nbytes + 4095) & ~size_t(4095);
+    if (hipMalloc(&c->dev[slot], cap) != hipSuccess) {
+        rmi_set_error("hipMalloc(%zu) for staging failed", cap);
+        return nullptr;
+    }
+    c->dev_cap[slot] = cap;
+    return c->dev[slot];
+}
+
+void *rmi_pin_buf(RmiThreadCtx *c, int slot, size_t nbytes) {
+    if (nbytes == 0) nbytes = 16;
+    if (c->pin_cap[slot] >= nbytes) return c->pin[slot];
+    if (c->pin[slot]) {
+        hipStreamSynchronize(c->stream);
+        hipHostFree(c->pin[slot]);
+        c->pin[slot] = nullptr;
+        c->pin_cap[slot] = 0;
+    }
+    size_t cap = (nbytes + 4095) & ~size_t(4095);
+    if (hipHostMalloc(&c->pin[slot], cap, hipHostMallocDefault) != hipSuccess) {
+        rmi_set_error("hipHostMalloc(%zu) for staging failed", cap);
+        return nullptr;
+    }
+    c->pin_cap[slot] = cap;
+    return c->pin[slot];
+}
+
+extern "C" {
+
+const char *rmi_hip_last_error(void) { return t_error; }
+
+int rmi_hip_init(int device) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_device >= 0) {
+        if (g_device == device) return RMI_HIP_OK;
+        return rmi_fail(RMI_HIP_E_INVALID, "already initialised on device %d", g_device);
+    }
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0)
+        return rmi_fail(RMI_HIP_E_NO_DEVICE, "no HIP device visible (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+    if (device < 0 || device >= count) return rmi_fail(RMI_HIP_E_INVALID, "device %d out of range (have %d)", device, count);
+    hipDeviceProp_t prop;
+    RMI_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return rmi_fail(RMI_HIP_E_NO_DEVICE, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
+    RMI_HIP_CHECK(hipSetDevice(device));
+    g_cus = prop.multiProcessorCount;
+    g_hbm = prop.totalGlobalMem;
+    snprintf(g_name, sizeof(g_name), "%s (%s)", prop.name, prop.gcnArchName);
+    g_device = device;
+    return RMI_HIP_OK;
+}
+
+void rmi_hip_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_device < 0) return;
+    hipDeviceSynchronize();
+    for (RmiThreadCtx *c : g_ctxs) {
+        for (int i = 0; i < 6; i++) {
+            if (c->dev[i]) hipFree(c->dev[i]);
+            if (c->pin[i]) hipHostFree(c->pin[i]);
+            c->dev[i] = nullptr;
+            c->pin[i] = nullptr;
+            c->dev_cap[i] = c->pin_cap[i] = 0;
+        }
+        if (c->stream) hipStreamDestroy(c->stream);
+        c->stream = nullptr;
+    }
+    // contexts stay allocated: their owning threads may still hold the pointer
+    g_device = -1;
+}
+
+int rmi_hip_device_info(char *name, size_t name_len, int *compute_units, size_t *hbm_bytes) {
+    RMI_REQUIRE_INIT();
+    if (name && name_len) snprintf(name, name_len, "%s", g_name);
+    if (compute_units) *compute_units = g_cus;
+    if (hbm_bytes) *hbm_bytes = g_hbm;
+    return RMI_HIP_OK;
+}
+
+void *rmi_hip_malloc(size_t nbytes) {
+    if (!rmi_ready()) {
+        rmi_set_error("rmi_hip_init has not succeeded");
+        return nullptr;
+    }
+    if (!rmi_thread_ctx()) return nullptr;
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, nbytes ? nbytes : 16);
+    if (e != hipSuccess) {
+        rmi_set_error("hipMalloc(%zu) failed: %s", nbytes, hipGetErrorString(e));
+        return nullptr;
+    }
+    return p;
+}
+
+void rmi_hip_free(void *dptr) {
+    if (dptr) hipFree(dptr);
+}
+
+int rmi_hip_memcpy_h2d(void *dst, const void *src, size_t nbytes) {
+    RMI_REQUIRE_INIT();
+    if (!rmi_thread_ctx()) return RMI_HIP_E_RUNTIME;
+    RMI_HIP_CHECK(hipMemcpy(dst, src, nbytes, hipMemcpyHostToDevice));
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_memcpy_d2h(void *dst, const void *src, size_t nbytes) {
+    RMI_REQUIRE_INIT();
+    if (!rmi_thread_ctx()) return RMI_HIP_E_RUNTIME;
+    RMI_HIP_CHECK(hipMemcpy(dst, src, nbytes, hipMemcpyDeviceToHost));
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_synchronize(void) {
+    RMI_REQUIRE_INIT();
+    if (!rmi_thread_ctx()) return RMI_HIP_E_RUNTIME;
+    RMI_HIP_CHECK(hipDeviceSynchronize());
+    return RMI_HIP_OK;
+}
+
+// ------------------------------------------------------------------ weights
+
+static rmi_hip_weight *alloc_weight(int dtype, uint32_t n_in, uint32_t n_out) {
+    rmi_hip_weight *w = new rmi_hip_weight();
+    w->dtype = dtype;
+    w->n_in = n_in;
+    w->n_out = n_out;
+    w->n_tiles = (n_out + kTileRows - 1) / kTileRows;
+    if (dtype == RMI_HIP_DTYPE_Q8_0) {
+        w->n_units = (n_in / 32 + 7) / 8;
+        w->tile_bytes = size_t(w->n_units) * kOctetBytes;
+    } else {
+        w->n_units = n_in / 256;
+        w->tile_bytes = size_t(w->n_units) * kQ4KSuperBytes;
+    }
+    w->nbytes = size_t(w->n_tiles) * w->tile_bytes;
+    w->data = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->data), w->nbytes ? w->nbytes : 16);
+    if (e != hipSuccess) {
+        rmi_set_error("hipMalloc(%zu) for a weight failed: %s", w->nbytes, hipGetErrorString(e));
+        delete w;
+        return nullptr;
+    }
+    return w;
+}
+
+static rmi_hip_weight *upload(int dtype, const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {
+    if (!rmi_ready()) {
+        rmi_set_error("rmi_hip_init has not succeeded");
+        return nullptr;
+    }
+    const uint32_t block_elems = dtype == RMI_HIP_DTYPE_Q8_0 ? 32 : 256;
+    const size_t block_bytes = dtype == RMI_HIP_DTYPE_Q8_0 ? 34 : 144;
+    if (n_in == 0 || n_in % block_elems != 0) {
+        rmi_set_error("n_in=%u is not a positive multiple of %u", n_in, block_elems);
+        return nullptr;
+    }
+    const size_t want = size_t(n_out) * (n_in / block_elems) * block_bytes;
+    if (nbytes < want || (!blocks && want)) {
+        rmi_set_error("weight slice holds %zu bytes, %u x %u needs %zu", nbytes, n_out, n_in, want);
+        return nullptr;
+    }
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return nullptr;
+    rmi_hip_weight *w = alloc_weight(dtype, n_in, n_out);
+    if (!w) return nullptr;
+    if (want == 0) return w;
+    uint8_t *staging = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&staging), want);
+    if (e == hipSuccess) e = hipMemcpyAsync(staging, blocks, want, hipMemcpyHostToDevice, c->stream);
+    int rc = RMI_HIP_OK;
+    if (e == hipSuccess)
+        rc = dtype == RMI_HIP_DTYPE_Q8_0 ? rmi_launch_repack_q8_0(staging, w, c->stream)
+                                         : rmi_launch_repack_q4_k(staging, w, c->stream);
+    if (e == hipSuccess && rc == RMI_HIP_OK) e = hipStreamSynchronize(c->stream);
+    if (staging) hipFree(staging);
+    if (e != hipSuccess || rc != RMI_HIP_OK) {
+        if (e != hipSuccess) rmi_set_error("weight upload failed: %s", hipGetErrorString(e));
+        rmi_hip_free_weight(w);
+        return nullptr;
+    }
+    return w;
+}
+
+rmi_hip_weight *rmi_hip_upload_q8_0(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {
+    return upload(RMI_HIP_DTYPE_Q8_0, blocks, nbytes, n_in, n_out);
+}
+
+rmi_hip_weight *rmi_hip_upload_q4_k(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {
+    return upload(RMI_HIP_DTYPE_Q4_K, blocks, nbytes, n_in, n_out);
+}
+
+rmi_hip_weight *rmi_hip_fuse_vstack(const rmi_hip_weight *a, const rmi_hip_weight *b) {
+    if (!rmi_ready()) {
+        rmi_set_error("rmi_hip_init has not succeeded");
+        return nullptr;
+    }
+    if (!a || !b || a->dtype != b->dtype || a->n_in != b->n_in) {
+        rmi_set_error("fuse_vstack: dtype or n_in differ");
+        return nullptr;
+    }
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return nullptr;
+    rmi_hip_weight *w = alloc_weight(a->dtype, a->n_in, a->n_out + b->n_out);
+    if (!w) return nullptr;
+    hipError_t e = hipSuccess;
+    int rc = RMI_HIP_OK;
+    if (w->nbytes) {
+        // whole tiles of `a` move as bytes; a ragged last tile and all of `b`
+        // when it starts inside a tile go through the row copier
+        e = hipMemsetAsync(w->data, 0, w->nbytes, c->stream);
+        if (e == hipSuccess) rc = rmi_launch_copy_rows(a, w, 0, c->stream);
+        if (e == hipSuccess && rc == RMI_HIP_OK) rc = rmi_launch_copy_rows(b, w, a->n_out, c->stream);
+        if (e == hipSuccess && rc == RMI_HIP_OK) e = hipStreamSynchronize(c->stream);
+    }
+    if (e != hipSuccess || rc != RMI_HIP_OK) {
+        if (e != hipSuccess) rmi_set_error("fuse_vstack failed: %s", hipGetErrorString(e));
+        rmi_hip_free_weight(w);
+        return nullptr;
+    }
+    return w;
+}
+
+void rmi_hip_free_weight(rmi_hip_weight *w) {
+    if (!w) return;
+    if (w->data) hipFree(w->data);
+    delete w;
+}
+
+uint32_t rmi_hip_weight_n_in(const rmi_hip_weight *w) { return w ? w->n_in : 0; }
+uint32_t rmi_hip_weight_n_out(const rmi_hip_weight *w) { return w ? w->n_out : 0; }
+int rmi_hip_weight_dtype(const rmi_hip_weight *w) { return w ? w->dtype : 0; }
+size_t rmi_hip_weight_device_bytes(const rmi_hip_weight *w) { return w ? w->nbytes : 0; }
+
+}  // extern "C"

@@ -1,0 +1,159 @@
+"""ctypes binding of ``librmi_hip.so`` (the C ABI declared in ``include/rmi_hip.h``).
+
+This is the only way Python reaches the GPU path: there is no CPU fallback, and
+loading fails loudly when the library has not been built.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librmi_hip.so")
+
+DTYPE_Q8_0 = 8
+DTYPE_Q4_K = 12
+ROUND_HALF_AWAY = 0
+ROUND_TIES_EVEN = 1
+
+_u8p = C.POINTER(C.c_uint8)
+_i8p = C.POINTER(C.c_int8)
+_i16p = C.POINTER(C.c_int16)
+_i32p = C.POINTER(C.c_int32)
+_f32p = C.POINTER(C.c_float)
+_vp = C.c_void_p
+_u32 = C.c_uint32
+_sz = C.c_size_t
+
+# name -> (restype, argtypes); must list every symbol of include/rmi_hip.h
+SIGNATURES = {
+    "rmi_hip_init": (C.c_int, [C.c_int]),
+    "rmi_hip_shutdown": (None, []),
+    "rmi_hip_last_error": (C.c_char_p, []),
+    "rmi_hip_device_info": (C.c_int, [C.c_char_p, _sz, C.POINTER(C.c_int), C.POINTER(_sz)]),
+    "rmi_hip_upload_q8_0": (_vp, [_u8p, _sz, _u32, _u32]),
+    "rmi_hip_upload_q4_k": (_vp, [_u8p, _sz, _u32, _u32]),
+    "rmi_hip_fuse_vstack": (_vp, [_vp, _vp]),
+    "rmi_hip_free_weight": (None, [_vp]),
+    "rmi_hip_weight_n_in": (_u32, [_vp]),
+    "rmi_hip_weight_n_out": (_u32, [_vp]),
+    "rmi_hip_weight_dtype": (C.c_int, [_vp]),
+    "rmi_hip_weight_device_bytes": (_sz, [_vp]),
+    "rmi_hip_q8_0_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
+    "rmi_hip_matmul_q8_0_quantized_range": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32]),
+    "rmi_hip_matmul_q8_0_quantized_batch": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32]),
+    "rmi_hip_q8_0_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32, C.c_int]),
+    "rmi_hip_quantize_q8_0": (C.c_int, [_f32p, _u32, _u8p, _f32p, C.c_int]),
+    "rmi_hip_block_dots_q8_0": (C.c_int, [_vp, _u8p, _i32p]),
+    "rmi_hip_matmul_q8_0_f32": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32]),
+    "rmi_hip_q4_k_forward_prepared": (C.c_int, [_vp, _f32p, _i8p, _i16p, _f32p, _u32, _u32, _u32, _u32]),
+    "rmi_hip_q4_k_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32]),
+    "rmi_hip_quantize_row_q8_k": (C.c_int, [_f32p, _u32, _f32p, _i8p, _i16p]),
+    "rmi_hip_q4_k_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
+    "rmi_hip_quantized_linear_forward": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32]),
+    "rmi_hip_block_ints_q4_k": (C.c_int, [_vp, _i8p, _i16p, _i32p, _i32p]),
+    "rmi_hip_malloc": (_vp, [_sz]),
+    "rmi_hip_free": (None, [_vp]),
+    "rmi_hip_memcpy_h2d": (C.c_int, [_vp, _vp, _sz]),
+    "rmi_hip_memcpy_d2h": (C.c_int, [_vp, _vp, _sz]),
+    "rmi_hip_synchronize": (C.c_int, []),
+    "rmi_hip_gemv_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "rmi_hip_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, _u32, C.c_int, _vp]),
+    "rmi_hip_gemm_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
+    "rmi_hip_gemv_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "rmi_hip_quantize_row_q8_k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
+    "rmi_hip_gemv_group_create": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u32]),
+    "rmi_hip_gemv_group_destroy": (None, [_vp]),
+    "rmi_hip_gemv_group_run_dev": (C.c_int, [_vp, _vp]),
+}
+
+
+class RmiHipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"rmi_hip error {code}: {message}")
+        self.code = code
+
+
+def load_library():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(hipcc, gfx950); there is no CPU fallback")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError names a missing export
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = load_library()
+
+
+def last_error():
+    return (lib.rmi_hip_last_error() or b"").decode()
+
+
+def check(rc):
+    if rc != 0:
+        raise RmiHipError(rc, last_error())
+
+
+def init(device=0):
+    check(lib.rmi_hip_init(device))
+
+
+def device_info():
+    name = C.create_string_buffer(128)
+    cus, hbm = C.c_int(), _sz()
+    check(lib.rmi_hip_device_info(name, 128, C.byref(cus), C.byref(hbm)))
+    return name.value.decode(), cus.value, hbm.value
+
+
+def ptr(a, ty):
+    return a.ctypes.data_as(ty)
+
+
+def as_u8(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype not in (np.uint8, np.int8):
+        raise TypeError("expected a byte array")
+    return a.view(np.uint8)
+
+
+def as_f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+class DeviceBuffer:
+    """A raw HBM allocation (for the device-resident entry points)."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        self.ptr = lib.rmi_hip_malloc(self.nbytes)
+        if not self.ptr:
+            raise RmiHipError(-2, last_error())
+
+    @classmethod
+    def from_array(cls, a):
+        a = np.ascontiguousarray(a)
+        buf = cls(a.nbytes)
+        check(lib.rmi_hip_memcpy_h2d(buf.ptr, a.ctypes.data, a.nbytes))
+        return buf
+
+    def to_array(self, dtype, shape):
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes
+        check(lib.rmi_hip_memcpy_d2h(out.ctypes.data, self.ptr, out.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            lib.rmi_hip_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
