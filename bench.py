@@ -1,0 +1,329 @@
+#!/usr/bin/env python3
+"""Benchmark of the Q8_0 decode GEMV path on one MI355X.
+
+A "step" is one token-step of the Qwen3-0.6B projection set at decode batch B:
+(q, k, v, o, gate, up, down) x 28 layers + the tied 151936-row lm_head = 197
+Q8_0 x Q8_0 GEMVs over 633 MB of distinct weights (more than the 256 MB
+Infinity Cache, so every step streams from HBM).  Weights and quantized
+activations are resident in HBM before the timed region starts.
+
+  --mode grouped     (default) the whole projection set in ONE launch of the GEMV kernel
+  --mode per_matmul  197 launches per step, one per matrix (the call pattern of the Kernel trait)
+  --mode layer       113 launches per step: [q,k,v] [o] [gate,up] [down] per layer + lm_head,
+                     the grouping a dependent decode step allows
+
+Prints one JSON line.  `value` = algorithmic bytes per step / wall time per step.
+`roofline` prices the GEMV kernel alone from HIP events recorded on the launch
+stream around every step.  `cpu_baseline` times the restated reference CPU path
+(the checker's AVX2 kernels over a persistent-thread row partition) on the same
+weights and activations in this process.
+"""
+import argparse
+import ctypes as C
+import importlib
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class HipEvents:
+    """hipEvent timing on a given stream (the null stream here), via libamdhip64."""
+
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+
+    def create(self):
+        ev = C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(ev)) == 0
+        return ev
+
+    def record(self, ev, stream=None):
+        assert self.hip.hipEventRecord(ev, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.hip.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.hip.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return ms.value
+
+
+def physical_cores():
+    try:
+        seen = set()
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("physical id"):
+                phys = line.split(":")[1].strip()
+            elif line.startswith("core id"):
+                core = line.split(":")[1].strip()
+            elif not line.strip():
+                if phys is not None and core is not None:
+                    seen.add((phys, core))
+                phys = core = None
+        if seen:
+            return len(seen)
+    except OSError:
+        pass
+    return os.cpu_count() or 1
+
+
+def build_projection_set(pkg, batch, keep_host):
+    """Uploads the 197 weights and their quantized activations; returns problem records."""
+    synth, K, H = pkg.synth, pkg.kernel, pkg.hip
+    shapes = []
+    for layer in range(synth.QWEN3_0_6B_LAYERS):
+        for name, n_out, n_in in synth.QWEN3_0_6B_LAYER:
+            shapes.append((f"blk.{layer}.{name}", n_out, n_in, layer))
+    name, n_out, n_in = synth.QWEN3_0_6B_LM_HEAD
+    shapes.append((name, n_out, n_in, -1))
+    problems = []
+    t0 = time.time()
+    for i, (name, n_out, n_in, layer) in enumerate(shapes):
+        w = synth.q8_0_weight(synth.seed_for(1, i), n_out, n_in)
+        x = synth.activations(synth.seed_for(1, 0x8000 + i), batch, n_in)
+        kernel = K.Q8Kernel(w, n_in, n_out)
+        d_x = H.DeviceBuffer.from_array(x)
+        d_q8 = H.DeviceBuffer(batch * n_in)
+        d_sc = H.DeviceBuffer(batch * (n_in // 32) * 4)
+        d_y = H.DeviceBuffer(batch * n_out * 4)
+        # the activation is quantized by the device quantizer (x86-64 rounding), as a decode step would
+        H.check(H.lib.rmi_hip_quantize_q8_0_dev(d_x.ptr, d_q8.ptr, d_sc.ptr, batch, n_in, H.ROUND_TIES_EVEN, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        rec = dict(name=name, n_out=n_out, n_in=n_in, layer=layer, kernel=kernel, d_q8=d_q8, d_sc=d_sc, d_y=d_y)
+        if keep_host:
+            rec["w"] = w
+            rec["q8"] = d_q8.to_array(np.uint8, (batch, n_in))
+            rec["sc"] = d_sc.to_array(np.float32, (batch, n_in // 32))
+        d_x.free()
+        problems.append(rec)
+    log(f"[bench] uploaded {len(problems)} weights in {time.time() - t0:.1f}s")
+    return problems
+
+
+def make_group(H, recs, batch):
+    n = len(recs)
+    arr = lambda vals: (C.c_void_p * n)(*vals)  # noqa: E731
+    g = H.lib.rmi_hip_gemv_group_create(n, arr([r["kernel"].w.handle for r in recs]), arr([r["d_q8"].ptr for r in recs]),
+                                        arr([r["d_sc"].ptr for r in recs]), arr([r["d_y"].ptr for r in recs]), batch)
+    if not g:
+        raise RuntimeError(H.last_error())
+    return g
+
+
+def layer_groups(H, problems, batch):
+    """[q,k,v] [o] [gate,up] [down] per layer, then lm_head: what a dependent decode step can fuse."""
+    groups = []
+    by_layer = {}
+    for r in problems:
+        by_layer.setdefault(r["layer"], []).append(r)
+    for layer in sorted(k for k in by_layer if k >= 0):
+        rs = {r["name"].split(".")[-1]: r for r in by_layer[layer]}
+        for names in (("attn_q", "attn_k", "attn_v"), ("attn_output",), ("ffn_gate", "ffn_up"), ("ffn_down",)):
+            groups.append(make_group(H, [rs[n] for n in names], batch))
+    groups.append(make_group(H, by_layer[-1], batch))
+    return groups
+
+
+def cpu_baseline(problems, batch, alg_bytes):
+    """The restated reference CPU path on the same weights: 10 warm-ups, 15 samples, median
+    (the reference's methodology, src/bin/micro_bench.rs:32-33, 94-152)."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import rmi_oracle as oracle
+
+    if not oracle.have_avx2():
+        return None
+    cores = min(16, physical_cores())
+    pool = oracle.Pool(cores)
+    outs = [np.zeros((batch, r["n_out"]), np.float32) for r in problems]
+
+    def step():
+        for r, out in zip(problems, outs):
+            pool.matmul_q8_0(r["w"], r["q8"], r["sc"], out, r["n_in"], r["n_out"], batch)
+
+    t_budget = time.time()
+    for _ in range(10):
+        step()
+        if time.time() - t_budget > 20:
+            break
+    samples = []
+    for _ in range(15):
+        t0 = time.perf_counter()
+        step()
+        samples.append(time.perf_counter() - t0)
+        if time.time() - t_budget > 40:
+            break
+    pool.close()
+    med = statistics.median(samples)
+    return {
+        "value": round(alg_bytes / med / 1e9, 2),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{len(samples)} full token-steps (197 GEMVs, {alg_bytes / 1e6:.0f} MB each) after warm-up, median; "
+                  f"restated reference AVX2 kernels, (ith,nth) row partition over {cores} persistent threads",
+        "ms_per_step": round(med * 1e3, 3),
+        "token_steps_per_s": round(1.0 / med, 2),
+    }, outs
+
+
+def read_traffic(mode):
+    """HBM bytes per launch measured with rocprofv3 --pmc, recorded under profiles/."""
+    path = os.path.join(ROOT, "profiles", f"gemv_q8_0_{mode}_qwen3_0.6b_pmc.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
+    ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the untimed secondary launch modes")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across GPUs", file=sys.stderr)
+        sys.exit(2)
+
+    pkg = importlib.import_module("rust-model-inference_amd")
+    H, synth = pkg.hip, pkg.synth
+    pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
+    dev_name, cus, hbm = H.device_info()
+    batch = args.batch
+    want_cpu = not args.no_cpu_baseline
+    problems = build_projection_set(pkg, batch, keep_host=want_cpu)
+    alg_bytes = sum(synth.q8_0_gemv_bytes(r["n_out"], r["n_in"], batch) for r in problems)
+    flops = sum(2 * r["n_out"] * r["n_in"] * batch for r in problems)
+    ev = HipEvents()
+
+    group_all = make_group(H, problems, batch)
+    groups_layer = layer_groups(H, problems, batch)
+
+    def step_grouped():
+        H.check(H.lib.rmi_hip_gemv_group_run_dev(group_all, None))
+
+    def step_per_matmul():
+        for r in problems:
+            H.check(H.lib.rmi_hip_gemv_q8_0_dev(r["kernel"].w.handle, r["d_q8"].ptr, r["d_sc"].ptr, r["d_y"].ptr, batch,
+                                                r["n_out"], 0, r["n_out"], None))
+
+    def step_layer():
+        for g in groups_layer:
+            H.check(H.lib.rmi_hip_gemv_group_run_dev(g, None))
+
+    modes = {"grouped": (step_grouped, 1), "per_matmul": (step_per_matmul, len(problems)),
+             "layer": (step_layer, len(groups_layer))}
+
+    def measure(mode, steps, warmup):
+        fn, launches = modes[mode]
+        for _ in range(warmup):
+            fn()
+        starts = [ev.create() for _ in range(steps)]
+        stops = [ev.create() for _ in range(steps)]
+        H.check(H.lib.rmi_hip_synchronize())
+        t0 = time.perf_counter()
+        for i in range(steps):
+            ev.record(starts[i])
+            fn()
+            ev.record(stops[i])
+        H.check(H.lib.rmi_hip_synchronize())
+        wall = (time.perf_counter() - t0) / steps
+        dev_ms = [ev.elapsed_ms(a, b) for a, b in zip(starts, stops)]
+        return wall, statistics.mean(dev_ms), launches
+
+    wall, dev_ms, launches = measure(args.mode, args.steps, args.warmup)
+    value = alg_bytes / wall / 1e9
+    achieved = alg_bytes / (dev_ms * 1e-3) / 1e9  # bytes per launch / average launch duration, summed over the step
+    result = {
+        "metric": "Q8_0 GEMV HBM GB/s, Qwen3-0.6B shapes, 1 GPU",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 dot4 -> f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"Qwen3-0.6B per-token projection set (7x28 + lm_head = 197 Q8_0 GEMVs, 633 MB of weights), "
+                        f"decode batch {batch}, launch mode {args.mode}",
+            "batch": batch,
+            "launches_per_step": launches,
+            "algorithmic_bytes_per_step": alg_bytes,
+            "flops_per_step": flops,
+            "device": dev_name.strip(),
+            "compute_units": cus,
+        },
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "token_steps_per_s": round(1.0 / wall, 1),
+        "gflops": round(flops / wall / 1e9, 1),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gemv_q8_0_kernel<%d,%s>" % (batch, "true" if args.mode != "per_matmul" else "false"),
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
+            "algorithmic_bytes_per_launch": round(alg_bytes / launches),
+            "traffic": read_traffic(args.mode),
+        },
+    }
+
+    if not args.no_extra:
+        extra = {}
+        for mode in modes:
+            if mode == args.mode:
+                continue
+            w2, d2, l2 = measure(mode, max(5, args.steps // 5), 3)
+            extra[mode] = {"GB/s": round(alg_bytes / w2 / 1e9, 1), "ms_per_step": round(w2 * 1e3, 4),
+                           "device_ms_per_step": round(d2, 4), "launches_per_step": l2,
+                           "token_steps_per_s": round(1.0 / w2, 1)}
+        result["other_launch_modes"] = extra
+
+    if want_cpu:
+        got = cpu_baseline(problems, batch, alg_bytes)
+        if got:
+            result["cpu_baseline"], cpu_outs = got
+            # the timed GPU step and the CPU baseline computed the same numbers
+            step_grouped()
+            H.check(H.lib.rmi_hip_synchronize())
+            worst = 0
+            for r, ref in zip(problems, cpu_outs):
+                gpu = r["d_y"].to_array(np.float32, (batch, r["n_out"]))
+                worst = max(worst, int(np.count_nonzero(gpu.view(np.uint32) != ref.view(np.uint32))))
+            result["cpu_baseline"]["gpu_outputs_differing_from_cpu"] = worst
+        else:
+            result["cpu_baseline"] = None
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

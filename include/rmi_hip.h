@@ -137,6 +137,11 @@ int rmi_hip_memcpy_h2d(void *dst, const void *src, size_t nbytes);
 int rmi_hip_memcpy_d2h(void *dst, const void *src, size_t nbytes);
 int rmi_hip_synchronize(void);
 
+/* Plain device-to-device streaming copy kernel (nbytes a multiple of 16).  No
+ * counterpart in the reference: it is the known-size kernel against which
+ * hardware HBM-traffic counters are calibrated when profiling. */
+int rmi_hip_copy_dev(void *dst, const void *src, size_t nbytes, void *stream);
+
 /* y[t][row] for rows [row_start,row_end) of n_tokens (1..8) activations.
  * y has row stride 1 and token stride y_stride floats; y[t][0] is row 0. */
 int rmi_hip_gemv_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,

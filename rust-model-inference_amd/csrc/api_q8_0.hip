@@ -285,6 +285,12 @@ int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
     return rmi_launch_gemm_q8_0(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
 }
 
+int rmi_hip_copy_dev(void *dst, const void *src, size_t nbytes, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!dst || !src || nbytes % 16 != 0) return rmi_fail(RMI_HIP_E_INVALID, "copy needs non-null pointers and a multiple of 16 bytes");
+    return rmi_launch_copy(src, dst, nbytes, static_cast<hipStream_t>(stream));
+}
+
 rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip_weight *const *weights,
                                               const int8_t *const *x_q8, const float *const *x_scales,
                                               float *const *y, uint32_t n_tokens) {

@@ -31,10 +31,12 @@ __device__ __forceinline__ void block_fma(float &acc, uint32_t w_bits, float xs,
 // One wave per workgroup.  The wave walks a contiguous range of 8-row tiles
 // (possibly across several problems of a group) and keeps the activation of
 // the current problem in LDS, permuted to the weight's quad order.
-template <int B>
+// GROUPED = false: one matrix, described by the by-value `single` argument.
+template <int B, bool GROUPED>
 __global__ __launch_bounds__(64) void gemv_q8_0_kernel(RmiGemvProblem single,
-                                                        const RmiGemvProblem *__restrict__ list, uint32_t n_problems,
-                                                        uint32_t total_cost, uint32_t n_waves) {
+                                                        const RmiGemvProblem *__restrict__ list_arg,
+                                                        uint32_t n_problems, uint32_t total_cost, uint32_t n_waves) {
+    const RmiGemvProblem *__restrict__ list = GROUPED ? list_arg : nullptr;
     extern __shared__ uint4 lds[];
     const uint32_t lane = threadIdx.x, r = lane >> 3, L = lane & 7;
     const uint64_t c0 = uint64_t(total_cost) * blockIdx.x / n_waves;
@@ -151,9 +153,12 @@ int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, uint
                         max_n_oct * 256);
     uint32_t n_waves = uint32_t(rmi_device_cus()) * 16;
     if (n_waves > total_tiles) n_waves = total_tiles;
-    RmiGemvProblem dummy{};
-    hipLaunchKernelGGL(gemv_q8_0_kernel<B>, dim3(n_waves), dim3(64), lds_bytes, s, single ? *single : dummy, d_list,
-                       n_problems, total_cost, n_waves);
+    if (single)
+        hipLaunchKernelGGL((gemv_q8_0_kernel<B, false>), dim3(n_waves), dim3(64), lds_bytes, s, *single, d_list,
+                           n_problems, total_cost, n_waves);
+    else
+        hipLaunchKernelGGL((gemv_q8_0_kernel<B, true>), dim3(n_waves), dim3(64), lds_bytes, s, RmiGemvProblem{}, d_list,
+                           n_problems, total_cost, n_waves);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -261,7 +266,22 @@ __global__ __launch_bounds__(64) void matmul_q8_0_f32_kernel(const uint8_t *__re
     if (i == 0 && row < n_out) y[row] = s;
 }
 
+// plain streaming copy: the known-size kernel that HBM traffic counters are scaled against
+__global__ __launch_bounds__(256) void copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
+    for (size_t i = blockIdx.x * size_t(blockDim.x) + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x)
+        dst[i] = src[i];
+}
+
 }  // namespace
+
+int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s) {
+    const size_t n = nbytes / 16;
+    if (n == 0) return RMI_HIP_OK;
+    hipLaunchKernelGGL(copy_kernel, dim3(uint32_t(rmi_device_cus()) * 8), dim3(256), 0, s,
+                       static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), n);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
 
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s) {
     return dispatch_gemv(n_tokens, &p, nullptr, 1, p.n_tiles * p.n_oct, p.n_tiles, p.n_oct, s);

@@ -108,6 +108,7 @@ struct RmiGemvProblem {
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
 int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, uint32_t n_problems, uint32_t total_cost,
                                uint32_t total_tiles, uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s);
+int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s);
 int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s);
 int rmi_launch_quantize_q8_0(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
                              int rounding, hipStream_t s);

@@ -57,6 +57,7 @@ SIGNATURES = {
     "rmi_hip_memcpy_h2d": (C.c_int, [_vp, _vp, _sz]),
     "rmi_hip_memcpy_d2h": (C.c_int, [_vp, _vp, _sz]),
     "rmi_hip_synchronize": (C.c_int, []),
+    "rmi_hip_copy_dev": (C.c_int, [_vp, _vp, _sz, _vp]),
     "rmi_hip_gemv_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, _u32, C.c_int, _vp]),
     "rmi_hip_gemm_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),

@@ -1,0 +1,194 @@
+"""GPU parity of the Q4_K path (Q4_KKernel, QuantizedLinear), through the C ABI.
+
+Bars: Q8_K quantizer and per-super-block integers bit-exact; Q4_K x Q8_K GEMV
+f32 bit-exact against the restated x86-64 kernel (vec_dot_q4k_q8k_avx2 order)
+and within rel 1e-3 of the scalar one (the reference's own bound,
+src/ops/quant/mod.rs:1112-1162); dequantise-and-dot paths bit-exact against the
+restated sequential f32 sums.
+"""
+import numpy as np
+import pytest
+
+import gen
+from conftest import bits
+
+pytestmark = pytest.mark.gpu
+
+S, A = 0, 1
+
+
+def _same(a, b):
+    """Bit equality, with NaNs only required to coincide in position."""
+    na, nb = np.isnan(a), np.isnan(b)
+    return np.array_equal(na, nb) and np.array_equal(bits(a)[~na], bits(b)[~nb])
+
+
+def _q8k_blocks(K, d, qs, bs):
+    return [K.BlockQ8K(float(d[i]), qs[i * 256:(i + 1) * 256], bs[i * 16:(i + 1) * 16]) for i in range(d.size)]
+
+
+# ------------------------------------------------------------------ Q8_K quantizer
+
+def test_q8_k_quantizer_reference_kats(hip):
+    """tests/quantized_inference.rs:152-186."""
+    x = np.zeros(256, np.float32)
+    x[:5] = [-127.0, 0.5, 1.5, 2.5, -0.5]
+    blocks = hip.kernel.quantize_row_q8_k(x)
+    assert list(blocks[0].qs[:5]) == [-127, 0, 2, 2, 0]
+    x = np.array([(i - 127) * 0.03125 for i in range(256)], np.float32)
+    blocks = hip.kernel.quantize_row_q8_k(x)
+    assert len(blocks) == 1
+    assert int(blocks[0].bsums.astype(np.int32).sum()) == int(blocks[0].qs.astype(np.int32).sum())
+
+
+def test_q8_k_quantizer_bit_exact(hip, oracle):
+    rng = np.random.default_rng(50)
+    x = (rng.standard_normal(256 * 96) * rng.choice([1e-5, 1.0, 300.0], 256 * 96)).astype(np.float32)
+    x[:256] = 0
+    x[256:512] = -np.abs(x[256:512])
+    x[512:768] = 1.0                      # every element ties for the maximum: the first wins
+    x[768:1024] = np.tile([2.0, -2.0], 128)  # +max before -max
+    x[1024:1280] = np.tile([-2.0, 2.0], 128)  # -max before +max
+    x[1280:1536] = np.arange(256) - 127.5
+    H = hip.hip
+    d = np.zeros(x.size // 256, np.float32)
+    qs = np.zeros(x.size, np.int8)
+    bs = np.zeros(x.size // 16, np.int16)
+    H.check(H.lib.rmi_hip_quantize_row_q8_k(H.ptr(x, H._f32p), x.size, H.ptr(d, H._f32p), H.ptr(qs, H._i8p),
+                                            H.ptr(bs, H._i16p)))
+    for variant in (S, A):
+        rd, rq, rb = oracle.quantize_row_q8_k(x, variant)
+        assert np.array_equal(bits(d), bits(rd)) and np.array_equal(qs, rq) and np.array_equal(bs, rb)
+
+
+# ------------------------------------------------------------------ integer path
+
+@pytest.mark.parametrize("n_out,n_in", [(6144, 2048), (2048, 6144), (1, 256), (13, 512), (100, 1024)])
+def test_q4k_q8k_gemv_bit_exact(hip, oracle, n_out, n_in):
+    K = hip.kernel
+    w = hip.synth.q4_k_weight(60 + n_out, n_out, n_in)
+    x = hip.synth.activations(61 + n_in, 1, n_in)[0]
+    d, qs, bs = oracle.quantize_row_q8_k(x, A)
+    kernel = K.Q4_KKernel(w, n_in, n_out)
+    out = np.zeros(n_out, np.float32)
+    kernel.forward_prepared(x, None, None, _q8k_blocks(K, d, qs, bs), out, n_in, n_out, 0, 1)
+    ref = np.zeros(n_out, np.float32)
+    oracle.q4k_forward_prepared(w, d, qs, bs, ref, n_in, n_out, 0, 1, A)
+    assert np.array_equal(bits(out), bits(ref))
+    refs = np.zeros(n_out, np.float32)
+    oracle.q4k_forward_prepared(w, d, qs, bs, refs, n_in, n_out, 0, 1, S)
+    assert np.all(np.abs(out - refs) <= 1e-3 * np.maximum(np.abs(refs), 1.0))
+    # exact integers per super-block, read back from the repacked HBM copy
+    isum, msum = kernel.block_ints(_q8k_blocks(K, d, qs, bs))
+    rows = np.unique(np.linspace(0, n_out - 1, min(n_out, 40)).astype(int))
+    wr = w.reshape(n_out, -1)
+    for r in rows:
+        ri, rm = oracle.q4k_q8k_block_ints(wr[r], qs, bs)
+        assert np.array_equal(isum[r], ri) and np.array_equal(msum[r], rm)
+    # q8_k = None: the kernel quantizes input_f32 itself (q4_k.rs:77-84)
+    out2 = np.zeros(n_out, np.float32)
+    kernel.forward_prepared(x, None, None, None, out2, n_in, n_out, 0, 1)
+    assert np.array_equal(bits(out2), bits(out))
+
+
+def test_q4k_partition_and_fusion(hip, oracle):
+    """tests/fused_ffn_matmul_parity.rs:232-300 on make_qk_weight bytes (d/dmin may be inf/nan)."""
+    K = hip.kernel
+    n_in, n_per = 1024, 3584
+    row_bytes = n_in // 256 * 144
+    gate = gen.make_qk_weight(n_per * row_bytes, row_bytes, 0)
+    up = gen.make_qk_weight(n_per * row_bytes, row_bytes, 17)
+    d, qs, bs = oracle.quantize_row_q8_k(gen.ramp_input(n_in), A)
+    blocks = _q8k_blocks(K, d, qs, bs)
+    kg, ku = K.Q4_KKernel(gate, n_in, n_per), K.Q4_KKernel(up, n_in, n_per)
+
+    def run(kernel, rows, nth):
+        out = np.zeros(rows, np.float32)
+        for ith in range(nth):
+            kernel.forward_prepared(None, None, None, blocks, out, n_in, rows, ith, nth)
+        return out
+
+    g1, u1 = run(kg, n_per, 1), run(ku, n_per, 1)
+    rg, ru = np.zeros(n_per, np.float32), np.zeros(n_per, np.float32)
+    oracle.q4k_forward_prepared(gate, d, qs, bs, rg, n_in, n_per, 0, 1, A)
+    oracle.q4k_forward_prepared(up, d, qs, bs, ru, n_in, n_per, 0, 1, A)
+    assert _same(g1, rg) and _same(u1, ru)
+    assert _same(run(kg, n_per, 8), g1) and _same(run(ku, n_per, 3), u1)
+    fused = K.fuse_vstack(kg, ku)
+    f8 = run(fused, 2 * n_per, 8)
+    assert _same(f8[:n_per], g1) and _same(f8[n_per:], u1)
+    assert K.fuse_vstack(kg, K.Q8Kernel(gen.make_q8_0_weight(4, n_in, 0), n_in, 4)) is None
+
+
+@pytest.mark.parametrize("n_tokens", [1, 3, 8, 12])
+def test_q4k_forward_batched(hip, oracle, n_tokens):
+    n_out, n_in = 512, 2048
+    w = hip.synth.q4_k_weight(70, n_out, n_in)
+    x = hip.synth.activations(71, n_tokens, n_in)
+    out = np.zeros((n_tokens, n_out), np.float32)
+    hip.kernel.Q4_KKernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out)
+    for t in range(n_tokens):
+        d, qs, bs = oracle.quantize_row_q8_k(x[t], A)
+        ref = np.zeros(n_out, np.float32)
+        oracle.q4k_forward_prepared(w, d, qs, bs, ref, n_in, n_out, 0, 1, A)
+        assert np.array_equal(bits(out[t]), bits(ref)), t
+
+
+# ----------------------------------------------------------------- dequant paths
+
+def test_q4_k_kernel_multiplies_uniform_block(hip):
+    """tests/quantized_inference.rs:233-249."""
+    w = np.zeros(144, np.uint8)
+    w[0:2] = np.array([gen.f16_bits(1.0)], np.uint16).view(np.uint8)
+    w[4:16] = [1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1]
+    w[16:] = 0x11
+    out = np.zeros(1, np.float32)
+    hip.kernel.Q4_KKernel(w, 256, 1).forward_prequantized(np.ones(256, np.uint8), np.ones(8, np.float32), out, 256, 1,
+                                                         0, 1)
+    assert list(out) == [256.0]
+
+
+@pytest.mark.parametrize("n_out,n_in", [(6144, 2048), (2048, 6144), (5, 256), (77, 768)])
+def test_dequant_dot_paths_bit_exact(hip, oracle, n_out, n_in):
+    K = hip.kernel
+    w = hip.synth.q4_k_weight(80 + n_out, n_out, n_in)
+    x = hip.synth.activations(81 + n_in, 1, n_in)[0]
+    # QuantizedLinear::forward through the Layer interface
+    layer = K.QuantizedLinear.from_weight_slice(w, None, n_in, n_out, "ffn")
+    assert (layer.input_dim(), layer.output_dim(), layer.name()) == (n_in, n_out, "ffn")
+    out = np.zeros(n_out, np.float32)
+    layer.forward(x, out, K.ExecContext(scratch=np.zeros(0, np.float32)))
+    assert np.array_equal(bits(out), bits(oracle.quantized_linear_forward(w, x, n_in, n_out)))
+    # Q4_KKernel::forward_prequantized with a (ith, nth) slice
+    q8, sc = oracle.quantize_q8_0(x, A)
+    ref = np.zeros(n_out, np.float32)
+    oracle.q4k_forward_prequantized(w, q8, sc, ref, n_in, n_out, 0, 1)
+    got = np.zeros(n_out, np.float32)
+    for ith in range(3):
+        layer.kernel.forward_prequantized(q8, sc, got, n_in, n_out, ith, 3)
+    assert np.array_equal(bits(got), bits(ref))
+
+
+def test_model_graph_two_layers(hip, oracle):
+    """ModelGraph::forward_all ping-pong (src/core/model.rs:123-152)."""
+    K = hip.kernel
+    w1 = hip.synth.q4_k_weight(90, 512, 256)
+    w2 = hip.synth.q4_k_weight(91, 256, 512)
+    x = hip.synth.activations(92, 1, 256)[0]
+    graph = K.ModelGraph()
+    graph.add_layer(K.QuantizedLinear.from_weight_slice(w1, None, 256, 512, "a"))
+    graph.add_layer(K.QuantizedLinear.from_weight_slice(w2, None, 512, 256, "b"))
+    out = np.zeros(256, np.float32)
+    graph.forward_all(x, out, np.zeros(1024, np.float32), K.ExecContext(scratch=np.zeros(0, np.float32)))
+    h = oracle.quantized_linear_forward(w1, x, 256, 512)
+    assert np.array_equal(bits(out), bits(oracle.quantized_linear_forward(w2, h, 512, 256)))
+
+
+def test_q4k_errors(hip):
+    H, K = hip.hip, hip.kernel
+    with pytest.raises(H.RmiHipError):
+        K.Q4_KKernel(np.zeros(144, np.uint8), 128, 1)  # n_in not a multiple of 256
+    kernel = K.Q4_KKernel(np.zeros(144 * 2, np.uint8), 256, 2)
+    with pytest.raises(H.RmiHipError):
+        kernel.forward_prequantized(np.zeros(512, np.uint8), np.zeros(16, np.float32), np.zeros(2, np.float32), 512, 2,
+                                    0, 1)
