@@ -13,8 +13,8 @@ activations are resident in HBM before the timed region starts.
                      the grouping a dependent decode step allows
 
 Prints one JSON line.  `value` = algorithmic bytes per step / wall time per step.
-`roofline` prices the GEMV kernel alone from HIP events recorded on the launch
-stream around every step.  `cpu_baseline` times the restated reference CPU path
+`roofline` prices the GEMV kernel from two HIP events recorded on the launch
+stream at the two ends of the timed region (launch gaps included).  `cpu_baseline` times the restated reference CPU path
 (the checker's AVX2 kernels over a persistent-thread row partition) on the same
 weights and activations in this process.
 """
@@ -202,7 +202,7 @@ def main():
     ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
     ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extra", action="store_true", help="skip the untimed secondary launch modes")
+    ap.add_argument("--extra", action="store_true", help="also time the other launch modes, outside the timed region")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across GPUs", file=sys.stderr)
@@ -238,21 +238,20 @@ def main():
              "layer": (step_layer, len(groups_layer))}
 
     def measure(mode, steps, warmup):
+        """Returns (host wall s/step, device ms/step between two events on the launch stream, launches/step)."""
         fn, launches = modes[mode]
         for _ in range(warmup):
             fn()
-        starts = [ev.create() for _ in range(steps)]
-        stops = [ev.create() for _ in range(steps)]
+        ev_a, ev_b = ev.create(), ev.create()
         H.check(H.lib.rmi_hip_synchronize())
         t0 = time.perf_counter()
-        for i in range(steps):
-            ev.record(starts[i])
+        ev.record(ev_a)
+        for _ in range(steps):
             fn()
-            ev.record(stops[i])
+        ev.record(ev_b)
         H.check(H.lib.rmi_hip_synchronize())
         wall = (time.perf_counter() - t0) / steps
-        dev_ms = [ev.elapsed_ms(a, b) for a, b in zip(starts, stops)]
-        return wall, statistics.mean(dev_ms), launches
+        return wall, ev.elapsed_ms(ev_a, ev_b) / steps, launches
 
     wall, dev_ms, launches = measure(args.mode, args.steps, args.warmup)
     value = alg_bytes / wall / 1e9
@@ -296,7 +295,7 @@ def main():
         },
     }
 
-    if not args.no_extra:
+    if args.extra:
         extra = {}
         for mode in modes:
             if mode == args.mode:

@@ -30,7 +30,7 @@ RmiGemvProblem make_problem(const rmi_hip_weight *w, const int8_t *x_q8, const f
     p.row_end = row_end;
     p.tile0 = row_start / kTileRows;
     p.n_tiles = row_end > row_start ? (row_end + kTileRows - 1) / kTileRows - p.tile0 : 0;
-    p.cost_begin = 0;
+    p.reserved = 0;
     return p;
 }
 
@@ -116,9 +116,9 @@ int host_gemv_range(const rmi_hip_weight *w, const uint8_t *input_q8, const floa
 
 struct rmi_hip_gemv_group {
     RmiGemvProblem *d_list = nullptr;
+    uint4 *d_runs = nullptr;
     uint32_t n_problems = 0;
-    uint32_t total_cost = 0;
-    uint32_t total_tiles = 0;
+    uint32_t n_runs = 0;
     uint32_t max_n_oct = 0;
     uint32_t n_tokens = 0;
 };
@@ -307,7 +307,7 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
     rmi_hip_gemv_group *g = new rmi_hip_gemv_group();
     g->n_problems = n_problems;
     g->n_tokens = n_tokens;
-    uint64_t cost = 0;
+    uint64_t total_tiles = 0;
     for (uint32_t i = 0; i < n_problems; i++) {
         const rmi_hip_weight *w = weights[i];
         if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0 || !x_q8[i] || !x_scales[i] || !y[i]) {
@@ -316,24 +316,34 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
             return nullptr;
         }
         list[i] = make_problem(w, x_q8[i], x_scales[i], y[i], w->n_out, 0, w->n_out);
-        list[i].cost_begin = uint32_t(cost);
-        cost += uint64_t(list[i].n_tiles) * list[i].n_oct;
-        g->total_tiles += list[i].n_tiles;
+        total_tiles += list[i].n_tiles;
         if (w->n_units > g->max_n_oct) g->max_n_oct = w->n_units;
     }
-    if (cost > 0xffffffffull || size_t(n_tokens) * g->max_n_oct * 288 > 64 * 1024) {
-        rmi_set_error("gemv group too large (cost %llu, %u tokens x %u octets)", (unsigned long long)cost, n_tokens,
-                      g->max_n_oct);
+    if (total_tiles > 0x7fffffffull || size_t(n_tokens) * g->max_n_oct * 288 > 64 * 1024) {
+        rmi_set_error("gemv group too large (%llu tiles, %u tokens x %u octets)", (unsigned long long)total_tiles,
+                      n_tokens, g->max_n_oct);
         delete g;
         return nullptr;
     }
-    g->total_cost = uint32_t(cost);
+    // one run of consecutive tiles per wave, never across two matrices
+    std::vector<uint4> runs;
+    for (uint32_t i = 0; i < n_problems; i++) {
+        if (list[i].n_oct == 0) continue;
+        const uint32_t tpw = rmi_gemv_tiles_per_wave(list[i].n_oct, uint32_t(total_tiles));
+        for (uint32_t k = 0; k < list[i].n_tiles; k += tpw)
+            runs.push_back(make_uint4(i, k, list[i].n_tiles - k < tpw ? list[i].n_tiles - k : tpw, 0));
+    }
+    g->n_runs = uint32_t(runs.size());
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&g->d_list), sizeof(RmiGemvProblem) * n_problems);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&g->d_runs), sizeof(uint4) * (runs.size() + 1));
     if (e == hipSuccess)
         e = hipMemcpy(g->d_list, list.data(), sizeof(RmiGemvProblem) * n_problems, hipMemcpyHostToDevice);
+    if (e == hipSuccess && !runs.empty())
+        e = hipMemcpy(g->d_runs, runs.data(), sizeof(uint4) * runs.size(), hipMemcpyHostToDevice);
     if (e != hipSuccess) {
         rmi_set_error("gemv group upload failed: %s", hipGetErrorString(e));
         if (g->d_list) hipFree(g->d_list);
+        if (g->d_runs) hipFree(g->d_runs);
         delete g;
         return nullptr;
     }
@@ -343,14 +353,15 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
 void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g) {
     if (!g) return;
     if (g->d_list) hipFree(g->d_list);
+    if (g->d_runs) hipFree(g->d_runs);
     delete g;
 }
 
 int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream) {
     RMI_REQUIRE_INIT();
     if (!g) return rmi_fail(RMI_HIP_E_INVALID, "null group");
-    return rmi_launch_gemv_q8_0_group(g->d_list, g->n_problems, g->total_cost, g->total_tiles, g->max_n_oct,
-                                      g->n_tokens, static_cast<hipStream_t>(stream));
+    return rmi_launch_gemv_q8_0_group(g->d_list, g->d_runs, g->n_runs, g->max_n_oct, g->n_tokens,
+                                      static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

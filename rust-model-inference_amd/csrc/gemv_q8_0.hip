@@ -28,153 +28,165 @@ __device__ __forceinline__ void block_fma(float &acc, uint32_t w_bits, float xs,
     acc = __builtin_fmaf(s, float(p), acc);
 }
 
-// One wave per workgroup.  The wave walks a contiguous range of 8-row tiles
-// (possibly across several problems of a group) and keeps the activation of
-// the current problem in LDS, permuted to the weight's quad order.
-// GROUPED = false: one matrix, described by the by-value `single` argument.
+// Pointers that arrive inside a struct are generic; these casts tell the
+// compiler they are HBM addresses so that it emits global_load / global_store.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef const u32x4 __attribute__((address_space(1))) *gptr_u4;
+typedef const uint32_t __attribute__((address_space(1))) *gptr_u32;
+typedef const float __attribute__((address_space(1))) *gptr_f32;
+typedef float __attribute__((address_space(1))) *gptr_f32_w;
+template <typename T, typename U>
+__device__ __forceinline__ T as_global(U *p) {
+    return (T)(uintptr_t)p;
+}
+
+// The three 16-byte loads one lane issues for one octet of its row.
+struct OctetRegs {
+    u32x4 sc;  // 8 f16 block scales of the row (same for the 8 lanes of the row)
+    u32x4 qa;  // blocks 8o..8o+3, bytes 4L..4L+3 of each
+    u32x4 qb;  // blocks 8o+4..8o+7
+};
+
+__device__ __forceinline__ void load_octet(OctetRegs &g, gptr_u4 sc_ptr, gptr_u4 q_ptr, uint32_t o) {
+    g.sc = sc_ptr[o * 8];
+    g.qa = q_ptr[(2 * o) * 64];
+    g.qb = q_ptr[(2 * o + 1) * 64];
+}
+
+template <int B>
+__device__ __forceinline__ void octet_fma(float (&acc)[B], const OctetRegs &g, const uint4 *lds, uint32_t tok_u4,
+                                          uint32_t n_oct, uint32_t o, uint32_t L) {
+#pragma unroll
+    for (int t = 0; t < B; t++) {
+        const uint4 *xt = lds + t * tok_u4;
+        const uint4 xa = xt[(2 * o) * 8 + L];
+        const uint4 xb = xt[(2 * o + 1) * 8 + L];
+        const float4 s0 = reinterpret_cast<const float4 *>(xt + n_oct * 16)[2 * o];
+        const float4 s1 = reinterpret_cast<const float4 *>(xt + n_oct * 16)[2 * o + 1];
+        float a = acc[t];
+        block_fma(a, g.sc.x & 0xffffu, s0.x, int(g.qa.x), int(xa.x));
+        block_fma(a, g.sc.x >> 16, s0.y, int(g.qa.y), int(xa.y));
+        block_fma(a, g.sc.y & 0xffffu, s0.z, int(g.qa.z), int(xa.z));
+        block_fma(a, g.sc.y >> 16, s0.w, int(g.qa.w), int(xa.w));
+        block_fma(a, g.sc.z & 0xffffu, s1.x, int(g.qb.x), int(xb.x));
+        block_fma(a, g.sc.z >> 16, s1.y, int(g.qb.y), int(xb.y));
+        block_fma(a, g.sc.w & 0xffffu, s1.z, int(g.qb.z), int(xb.z));
+        block_fma(a, g.sc.w >> 16, s1.w, int(g.qb.w), int(xb.w));
+        acc[t] = a;
+    }
+}
+
+// One wave per workgroup; a wave owns a short run of consecutive 8-row tiles
+// of ONE matrix (about 16 KiB of weights).  A launch has far more waves than
+// fit on the chip at once: the dispatcher hands out runs as waves retire, which
+// balances the load and keeps the waves in flight reading one compact window of
+// HBM.  The activation of the matrix sits in LDS, permuted to quad order.
+// GROUPED = false: one matrix (`single`), run w starts at tile w * tiles_per_wave.
+// GROUPED = true: runs[w] = {problem index, first tile, tile count, -}.
 template <int B, bool GROUPED>
 __global__ __launch_bounds__(64) void gemv_q8_0_kernel(RmiGemvProblem single,
-                                                        const RmiGemvProblem *__restrict__ list_arg,
-                                                        uint32_t n_problems, uint32_t total_cost, uint32_t n_waves) {
-    const RmiGemvProblem *__restrict__ list = GROUPED ? list_arg : nullptr;
+                                                        const RmiGemvProblem *__restrict__ list,
+                                                        const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
     extern __shared__ uint4 lds[];
     const uint32_t lane = threadIdx.x, r = lane >> 3, L = lane & 7;
-    const uint64_t c0 = uint64_t(total_cost) * blockIdx.x / n_waves;
-    const uint64_t c1 = uint64_t(total_cost) * (blockIdx.x + 1) / n_waves;
-    if (c0 >= c1) return;
 
-    // problem that holds cost position c0
-    uint32_t pi = 0;
-    if (list) {
-        uint32_t lo = 0, hi = n_problems;
-        while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (list[mid].cost_begin <= c0) lo = mid; else hi = mid;
-        }
-        pi = lo;
+    RmiGemvProblem p;
+    uint32_t k, k_end;
+    if (GROUPED) {
+        const uint4 run = runs[blockIdx.x];
+        p = list[run.x];
+        k = run.y;
+        k_end = run.y + run.z;
+    } else {
+        p = single;
+        k = blockIdx.x * tiles_per_wave;
+        k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
     }
-    RmiGemvProblem p = list ? list[pi] : single;
-    // first tile whose start cost is >= c0
-    uint32_t k = uint32_t((c0 - p.cost_begin + p.n_oct - 1) / p.n_oct);
-    bool staged = false;
 
-    for (;;) {
-        if (k >= p.n_tiles) {
-            pi++;
-            if (!list || pi >= n_problems) break;
-            p = list[pi];
-            k = 0;
-            staged = false;
-            continue;
-        }
-        if (uint64_t(p.cost_begin) + uint64_t(k) * p.n_oct >= c1) break;
-
-        const uint32_t n_oct = p.n_oct;
-        const uint32_t tok_u4 = n_oct * 18;  // per token: 16 uint4 of quants + 2 of scales per octet
-        if (!staged) {
-            __syncthreads();  // earlier reads of the previous activation are done
-            const uint32_t nb = p.n_in >> 5;
-            uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
-            for (int t = 0; t < B; t++) {
-                const uint32_t *xq = reinterpret_cast<const uint32_t *>(p.x_q8 + size_t(t) * p.n_in);
-                const float *xs = p.x_scales + size_t(t) * nb;
-                uint32_t *dq = lds_dw + t * tok_u4 * 4;
-                for (uint32_t i = lane; i < n_oct * 64; i += 64) {
-                    const uint32_t b = i >> 3, l = i & 7;
-                    dq[(b >> 2) * 32 + l * 4 + (b & 3)] = b < nb ? xq[i] : 0u;
-                }
-                float *ds = reinterpret_cast<float *>(dq + n_oct * 64);
-                for (uint32_t i = lane; i < n_oct * 8; i += 64) ds[i] = i < nb ? xs[i] : 0.0f;
+    const uint32_t n_oct = p.n_oct;
+    const uint32_t tok_u4 = n_oct * 18;  // per token: 16 uint4 of quants + 2 of scales per octet
+    {
+        const uint32_t nb = p.n_in >> 5;
+        uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
+        for (int t = 0; t < B; t++) {
+            gptr_u32 xq = as_global<gptr_u32>(p.x_q8 + size_t(t) * p.n_in);
+            gptr_f32 xs = as_global<gptr_f32>(p.x_scales + size_t(t) * nb);
+            uint32_t *dq = lds_dw + t * tok_u4 * 4;
+            for (uint32_t i = lane; i < n_oct * 64; i += 64) {
+                const uint32_t b = i >> 3, l = i & 7;
+                dq[(b >> 2) * 32 + l * 4 + (b & 3)] = b < nb ? xq[i] : 0u;
             }
-            __syncthreads();
-            staged = true;
+            float *ds = reinterpret_cast<float *>(dq + n_oct * 64);
+            for (uint32_t i = lane; i < n_oct * 8; i += 64) ds[i] = i < nb ? xs[i] : 0.0f;
         }
+        __syncthreads();
+    }
 
-        const uint4 *tile = reinterpret_cast<const uint4 *>(p.w + size_t(p.tile0 + k) * n_oct * kOctetBytes);
-        const uint4 *sc_ptr = tile + r;
-        const uint4 *q_ptr = tile + n_oct * 8 + lane;
+    for (; k < k_end; k++) {
+        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * n_oct * kOctetBytes);
+        gptr_u4 sc_ptr = tile + r;
+        gptr_u4 q_ptr = tile + n_oct * 8 + lane;
 
         float acc[B];
 #pragma unroll
         for (int t = 0; t < B; t++) acc[t] = 0.0f;
 
-        for (uint32_t o0 = 0; o0 < n_oct; o0 += 4) {
-            uint4 sc[4], qa[4], qb[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                if (o0 + i < n_oct) {
-                    sc[i] = sc_ptr[(o0 + i) * 8];
-                    qa[i] = q_ptr[(2 * (o0 + i)) * 64];
-                    qb[i] = q_ptr[(2 * (o0 + i) + 1) * 64];
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                if (o0 + i < n_oct) {
-                    const uint32_t o = o0 + i;
-#pragma unroll
-                    for (int t = 0; t < B; t++) {
-                        const uint4 *xt = lds + t * tok_u4;
-                        const uint4 xa = xt[(2 * o) * 8 + L];
-                        const uint4 xb = xt[(2 * o + 1) * 8 + L];
-                        const float4 s0 = reinterpret_cast<const float4 *>(xt + n_oct * 16)[2 * o];
-                        const float4 s1 = reinterpret_cast<const float4 *>(xt + n_oct * 16)[2 * o + 1];
-                        float a = acc[t];
-                        block_fma(a, sc[i].x & 0xffffu, s0.x, int(qa[i].x), int(xa.x));
-                        block_fma(a, sc[i].x >> 16, s0.y, int(qa[i].y), int(xa.y));
-                        block_fma(a, sc[i].y & 0xffffu, s0.z, int(qa[i].z), int(xa.z));
-                        block_fma(a, sc[i].y >> 16, s0.w, int(qa[i].w), int(xa.w));
-                        block_fma(a, sc[i].z & 0xffffu, s1.x, int(qb[i].x), int(xb.x));
-                        block_fma(a, sc[i].z >> 16, s1.y, int(qb[i].y), int(xb.y));
-                        block_fma(a, sc[i].w & 0xffffu, s1.z, int(qb[i].z), int(xb.z));
-                        block_fma(a, sc[i].w >> 16, s1.w, int(qb[i].w), int(xb.w));
-                        acc[t] = a;
-                    }
-                }
-            }
+        // Software pipeline over the octets of the tile: while one pair of octets is
+        // multiplied, the loads of the next pair are in flight.  The accumulation
+        // order over blocks stays strictly ascending.
+        OctetRegs ra, rb, rc, rd;
+        load_octet(ra, sc_ptr, q_ptr, 0);
+        if (n_oct > 1) load_octet(rb, sc_ptr, q_ptr, 1);
+        for (uint32_t o = 0; o < n_oct; o += 4) {
+            if (o + 2 < n_oct) load_octet(rc, sc_ptr, q_ptr, o + 2);
+            if (o + 3 < n_oct) load_octet(rd, sc_ptr, q_ptr, o + 3);
+            octet_fma<B>(acc, ra, lds, tok_u4, n_oct, o, L);
+            if (o + 1 < n_oct) octet_fma<B>(acc, rb, lds, tok_u4, n_oct, o + 1, L);
+            if (o + 4 < n_oct) load_octet(ra, sc_ptr, q_ptr, o + 4);
+            if (o + 5 < n_oct) load_octet(rb, sc_ptr, q_ptr, o + 5);
+            if (o + 2 < n_oct) octet_fma<B>(acc, rc, lds, tok_u4, n_oct, o + 2, L);
+            if (o + 3 < n_oct) octet_fma<B>(acc, rd, lds, tok_u4, n_oct, o + 3, L);
         }
 
         const uint32_t row = (p.tile0 + k) * kTileRows + r;
+        gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
 #pragma unroll
         for (int t = 0; t < B; t++) {
             const float y = hsum8_lanes(acc[t]);
-            if (L == 0 && row >= p.row_start && row < p.row_end) p.y[size_t(t) * p.y_stride + row] = y;
+            if (L == 0 && row >= p.row_start && row < p.row_end) yp[size_t(t) * p.y_stride + row] = y;
         }
-        k++;
     }
 }
 
 template <int B>
-int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, uint32_t n_problems, uint32_t total_cost,
-                uint32_t total_tiles, uint32_t max_n_oct, hipStream_t s) {
+int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_waves,
+                uint32_t tiles_per_wave, uint32_t max_n_oct, hipStream_t s) {
     const size_t lds_bytes = size_t(B) * max_n_oct * 288;
     if (lds_bytes > 64 * 1024)
         return rmi_fail(RMI_HIP_E_INVALID, "activation of %d tokens x %u elements does not fit the LDS staging", B,
                         max_n_oct * 256);
-    uint32_t n_waves = uint32_t(rmi_device_cus()) * 16;
-    if (n_waves > total_tiles) n_waves = total_tiles;
     if (single)
-        hipLaunchKernelGGL((gemv_q8_0_kernel<B, false>), dim3(n_waves), dim3(64), lds_bytes, s, *single, d_list,
-                           n_problems, total_cost, n_waves);
+        hipLaunchKernelGGL((gemv_q8_0_kernel<B, false>), dim3(n_waves), dim3(64), lds_bytes, s, *single, d_list, d_runs,
+                           tiles_per_wave);
     else
         hipLaunchKernelGGL((gemv_q8_0_kernel<B, true>), dim3(n_waves), dim3(64), lds_bytes, s, RmiGemvProblem{}, d_list,
-                           n_problems, total_cost, n_waves);
+                           d_runs, tiles_per_wave);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
 
-int dispatch_gemv(uint32_t n_tokens, const RmiGemvProblem *single, const RmiGemvProblem *d_list, uint32_t n_problems,
-                  uint32_t total_cost, uint32_t total_tiles, uint32_t max_n_oct, hipStream_t s) {
-    if (total_tiles == 0 || total_cost == 0) return RMI_HIP_OK;
+int dispatch_gemv(uint32_t n_tokens, const RmiGemvProblem *single, const RmiGemvProblem *d_list, const uint4 *d_runs,
+                  uint32_t n_waves, uint32_t tiles_per_wave, uint32_t max_n_oct, hipStream_t s) {
+    if (n_waves == 0) return RMI_HIP_OK;
     switch (n_tokens) {
-        case 1: return launch_gemv<1>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
-        case 2: return launch_gemv<2>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
-        case 3: return launch_gemv<3>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
-        case 4: return launch_gemv<4>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
-        case 5: return launch_gemv<5>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
-        case 6: return launch_gemv<6>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
-        case 7: return launch_gemv<7>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
-        case 8: return launch_gemv<8>(single, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+        case 1: return launch_gemv<1>(single, d_list, d_runs, n_waves, tiles_per_wave, max_n_oct, s);
+        case 2: return launch_gemv<2>(single, d_list, d_runs, n_waves, tiles_per_wave, max_n_oct, s);
+        case 3: return launch_gemv<3>(single, d_list, d_runs, n_waves, tiles_per_wave, max_n_oct, s);
+        case 4: return launch_gemv<4>(single, d_list, d_runs, n_waves, tiles_per_wave, max_n_oct, s);
+        case 5: return launch_gemv<5>(single, d_list, d_runs, n_waves, tiles_per_wave, max_n_oct, s);
+        case 6: return launch_gemv<6>(single, d_list, d_runs, n_waves, tiles_per_wave, max_n_oct, s);
+        case 7: return launch_gemv<7>(single, d_list, d_runs, n_waves, tiles_per_wave, max_n_oct, s);
+        case 8: return launch_gemv<8>(single, d_list, d_runs, n_waves, tiles_per_wave, max_n_oct, s);
         default: return rmi_fail(RMI_HIP_E_INVALID, "gemv takes 1..8 tokens per launch, got %u", n_tokens);
     }
 }
@@ -274,6 +286,15 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4 *__restrict__ src
 
 }  // namespace
 
+// Tiles a wave takes in one run: about 8 tile-octets (17 KiB of weights), fewer
+// when the launch would otherwise have too few waves to fill the chip.
+uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles) {
+    uint32_t tpw = n_oct >= 8 ? 1 : 8 / (n_oct ? n_oct : 1);
+    const uint32_t fill = uint32_t(rmi_device_cus()) * 8;
+    while (tpw > 1 && launch_tiles / tpw < fill) tpw >>= 1;
+    return tpw ? tpw : 1;
+}
+
 int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s) {
     const size_t n = nbytes / 16;
     if (n == 0) return RMI_HIP_OK;
@@ -284,12 +305,14 @@ int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s) {
 }
 
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s) {
-    return dispatch_gemv(n_tokens, &p, nullptr, 1, p.n_tiles * p.n_oct, p.n_tiles, p.n_oct, s);
+    if (p.n_tiles == 0 || p.n_oct == 0) return RMI_HIP_OK;
+    const uint32_t tpw = rmi_gemv_tiles_per_wave(p.n_oct, p.n_tiles);
+    return dispatch_gemv(n_tokens, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, tpw, p.n_oct, s);
 }
 
-int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, uint32_t n_problems, uint32_t total_cost,
-                               uint32_t total_tiles, uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s) {
-    return dispatch_gemv(n_tokens, nullptr, d_list, n_problems, total_cost, total_tiles, max_n_oct, s);
+int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t max_n_oct,
+                               uint32_t n_tokens, hipStream_t s) {
+    return dispatch_gemv(n_tokens, nullptr, d_list, d_runs, n_runs, 0, max_n_oct, s);
 }
 
 int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s) {

@@ -103,11 +103,13 @@ struct RmiGemvProblem {
     uint32_t row_end;
     uint32_t tile0;        // first tile touched
     uint32_t n_tiles;      // tiles touched
-    uint32_t cost_begin;   // prefix sum of n_tiles*n_oct over earlier problems
+    uint32_t reserved;
 };
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
-int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, uint32_t n_problems, uint32_t total_cost,
-                               uint32_t total_tiles, uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s);
+// d_runs[w] = {problem index, first tile, tile count, 0}: the run of tiles wave w takes
+int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t max_n_oct,
+                               uint32_t n_tokens, hipStream_t s);
+uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles);
 int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s);
 int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s);
 int rmi_launch_quantize_q8_0(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
