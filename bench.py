@@ -202,6 +202,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
     ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration-mb", type=int, default=0,
+                    help="also launch the plain copy kernel on this many MiB, 5 times, outside the timed region "
+                         "(the known-size kernel that rocprofv3 --pmc traffic counters are scaled against)")
     ap.add_argument("--extra", action="store_true", help="also time the other launch modes, outside the timed region")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -252,6 +255,15 @@ def main():
         H.check(H.lib.rmi_hip_synchronize())
         wall = (time.perf_counter() - t0) / steps
         return wall, ev.elapsed_ms(ev_a, ev_b) / steps, launches
+
+    if args.copy_calibration_mb:
+        nbytes = args.copy_calibration_mb << 20
+        src, dst = H.DeviceBuffer(nbytes), H.DeviceBuffer(nbytes)
+        for _ in range(5):
+            H.check(H.lib.rmi_hip_copy_dev(dst.ptr, src.ptr, nbytes, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        src.free()
+        dst.free()
 
     wall, dev_ms, launches = measure(args.mode, args.steps, args.warmup)
     value = alg_bytes / wall / 1e9
