@@ -1,0 +1,196 @@
+//! `hip` op back end for rust-model-inference: binds librmi_hip.so (C ABI in
+//! include/rmi_hip.h) and implements the crate's existing `Kernel` and `Layer`
+//! traits on top of it.
+//!
+//! NOT COMPILED in the environment this back end was built in (no Rust
+//! toolchain there); it is the binding a maintainer drops into the crate as
+//! `src/hip.rs` behind `--features hip`, and it is kept thin so that it can be
+//! reviewed by eye: every method is one FFI call.
+//!
+//! Hook points in the crate:
+//!   * `QuantizedTensor::into_kernel` (src/ops/kernel/quantized_tensor.rs:167-190):
+//!     when `ops::hip_enabled()` return `Box::new(HipKernel::upload(..))` for
+//!     `Q8_0` / `Q4_K` instead of `Q8Kernel` / `Q4_KKernel`;
+//!   * `ops::enable_gpu` / the lazy context of src/ops/float.rs:44-58: call
+//!     `hip::init(0)`; on `Err` print and stay on the CPU kernels, as today;
+//!   * `matmul_q8_0_quantized_range` (src/ops/kernel/q8_0/dispatch.rs:36-52) is NOT
+//!     hooked: its weight argument is a borrowed byte slice with no handle.
+
+use std::ffi::{c_char, c_int, c_void, CStr};
+
+use crate::core::traits::{ExecContext, Layer};
+use crate::ops::kernel::Kernel;
+use crate::ops::quant::BlockQ8K;
+
+#[repr(C)]
+pub struct RmiHipWeight {
+    _private: [u8; 0],
+}
+
+#[link(name = "rmi_hip")]
+extern "C" {
+    fn rmi_hip_init(device: c_int) -> c_int;
+    fn rmi_hip_last_error() -> *const c_char;
+    fn rmi_hip_upload_q8_0(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
+    fn rmi_hip_upload_q4_k(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
+    fn rmi_hip_fuse_vstack(a: *const RmiHipWeight, b: *const RmiHipWeight) -> *mut RmiHipWeight;
+    fn rmi_hip_free_weight(w: *mut RmiHipWeight);
+    fn rmi_hip_q8_0_forward_prequantized(
+        w: *const RmiHipWeight, input_q8: *const u8, input_scales: *const f32, output: *mut f32,
+        n_in: u32, n_out: u32, ith: u32, nth: u32,
+    ) -> c_int;
+    fn rmi_hip_q8_0_forward_batched(
+        w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
+        rounding: c_int,
+    ) -> c_int;
+    fn rmi_hip_q4_k_forward_prepared(
+        w: *const RmiHipWeight, d: *const f32, qs: *const i8, bsums: *const i16, output: *mut f32,
+        n_in: u32, n_out: u32, ith: u32, nth: u32,
+    ) -> c_int;
+    fn rmi_hip_q4_k_forward_batched(
+        w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
+    ) -> c_int;
+    fn rmi_hip_q4_k_forward_prequantized(
+        w: *const RmiHipWeight, input_q8: *const u8, input_scales: *const f32, output: *mut f32,
+        n_in: u32, n_out: u32, ith: u32, nth: u32,
+    ) -> c_int;
+    fn rmi_hip_quantized_linear_forward(
+        w: *const RmiHipWeight, input: *const f32, output: *mut f32, in_features: u32, out_features: u32,
+    ) -> c_int;
+}
+
+const ROUND_TIES_EVEN: c_int = 1; // what quantize_q8_0_into does on x86-64 (src/ops/quant/q8_0.rs:5-12)
+
+fn last_error() -> String {
+    unsafe { CStr::from_ptr(rmi_hip_last_error()).to_string_lossy().into_owned() }
+}
+
+/// `Err` means "stay on the CPU kernels" (src/ops/float.rs:51-57).
+pub fn init(device: i32) -> Result<(), String> {
+    if unsafe { rmi_hip_init(device) } == 0 { Ok(()) } else { Err(last_error()) }
+}
+
+#[derive(Clone, Copy, PartialEq)]
+enum Dtype { Q8_0, Q4K }
+
+/// A weight resident in HBM.  `Kernel: Send + Sync`: the library gives every
+/// calling thread its own stream and staging, so `&self` calls may overlap.
+pub struct HipKernel {
+    handle: *mut RmiHipWeight,
+    dtype: Dtype,
+}
+unsafe impl Send for HipKernel {}
+unsafe impl Sync for HipKernel {}
+
+impl HipKernel {
+    pub fn upload_q8_0(weight: &[u8], n_in: usize, n_out: usize) -> Result<Self, String> {
+        let h = unsafe { rmi_hip_upload_q8_0(weight.as_ptr(), weight.len(), n_in as u32, n_out as u32) };
+        if h.is_null() { Err(last_error()) } else { Ok(Self { handle: h, dtype: Dtype::Q8_0 }) }
+    }
+    pub fn upload_q4_k(weight: &[u8], n_in: usize, n_out: usize) -> Result<Self, String> {
+        let h = unsafe { rmi_hip_upload_q4_k(weight.as_ptr(), weight.len(), n_in as u32, n_out as u32) };
+        if h.is_null() { Err(last_error()) } else { Ok(Self { handle: h, dtype: Dtype::Q4K }) }
+    }
+    /// `QTensorOwned::fuse_vstack` (src/ops/kernel/qtensor_owned.rs:138-164)
+    pub fn fuse_vstack(a: &Self, b: &Self) -> Option<Self> {
+        let h = unsafe { rmi_hip_fuse_vstack(a.handle, b.handle) };
+        if h.is_null() { None } else { Some(Self { handle: h, dtype: a.dtype }) }
+    }
+}
+
+impl Drop for HipKernel {
+    fn drop(&mut self) { unsafe { rmi_hip_free_weight(self.handle) } }
+}
+
+fn expect_ok(rc: c_int) {
+    if rc != 0 { panic!("GPU matmul failed: {}", last_error()); } // dispatch.rs:47-48
+}
+
+impl Kernel for HipKernel {
+    fn forward_prequantized(
+        &self, input_q8: &[u8], input_scales: &[f32], output: &mut [f32],
+        n_in: usize, n_out: usize, ith: usize, nth: usize,
+    ) {
+        let rc = unsafe {
+            match self.dtype {
+                Dtype::Q8_0 => rmi_hip_q8_0_forward_prequantized(
+                    self.handle, input_q8.as_ptr(), input_scales.as_ptr(), output.as_mut_ptr(),
+                    n_in as u32, n_out as u32, ith as u32, nth as u32),
+                Dtype::Q4K => rmi_hip_q4_k_forward_prequantized(
+                    self.handle, input_q8.as_ptr(), input_scales.as_ptr(), output.as_mut_ptr(),
+                    n_in as u32, n_out as u32, ith as u32, nth as u32),
+            }
+        };
+        expect_ok(rc);
+    }
+
+    fn forward_prepared(
+        &self, input_f32: &[f32], input_q8: &[u8], input_scales: &[f32], q8_k: Option<&[BlockQ8K]>,
+        output: &mut [f32], n_in: usize, n_out: usize, ith: usize, nth: usize,
+    ) {
+        if self.dtype == Dtype::Q8_0 {
+            return self.forward_prequantized(input_q8, input_scales, output, n_in, n_out, ith, nth);
+        }
+        // BlockQ8K has no repr(C) (src/ops/quant/mod.rs:35-40): pass three arrays.
+        let owned;
+        let blocks: &[BlockQ8K] = match q8_k {
+            Some(b) => b,
+            None => { owned = crate::ops::quant::quantize_row_q8_k(&input_f32[..n_in]); &owned } // q4_k.rs:77-84
+        };
+        let d: Vec<f32> = blocks.iter().map(|b| b.d).collect();
+        let qs: Vec<i8> = blocks.iter().flat_map(|b| b.qs.iter().copied()).collect();
+        let bs: Vec<i16> = blocks.iter().flat_map(|b| b.bsums.iter().copied()).collect();
+        expect_ok(unsafe {
+            rmi_hip_q4_k_forward_prepared(self.handle, d.as_ptr(), qs.as_ptr(), bs.as_ptr(), output.as_mut_ptr(),
+                                          n_in as u32, n_out as u32, ith as u32, nth as u32)
+        });
+    }
+
+    fn forward(&self, input: &[f32], output: &mut [f32], n_in: usize, n_out: usize) {
+        self.forward_batched(&input[..n_in], &mut output[..n_out], n_in, n_out);
+    }
+
+    fn forward_batched(&self, input: &[f32], output: &mut [f32], n_in: usize, n_out: usize) {
+        let n_tokens = (input.len() / n_in) as u32;
+        expect_ok(unsafe {
+            match self.dtype {
+                Dtype::Q8_0 => rmi_hip_q8_0_forward_batched(self.handle, input.as_ptr(), output.as_mut_ptr(),
+                                                            n_in as u32, n_out as u32, n_tokens, ROUND_TIES_EVEN),
+                Dtype::Q4K => rmi_hip_q4_k_forward_batched(self.handle, input.as_ptr(), output.as_mut_ptr(),
+                                                           n_in as u32, n_out as u32, n_tokens),
+            }
+        });
+    }
+}
+
+/// `QuantizedLinear` (src/core/model.rs:12-104) on the GPU: same constructor
+/// arguments, `ctx.scratch` is not used (the weight is dequantised in registers).
+pub struct HipLinear<'a> {
+    kernel: HipKernel,
+    in_features: usize,
+    out_features: usize,
+    layer_name: &'a str,
+}
+
+impl<'a> HipLinear<'a> {
+    pub fn from_weight_slice(weight: &[u8], _bias: Option<&[u8]>, in_features: usize, out_features: usize,
+                             name: &'a str) -> Result<Self, String> {
+        Ok(Self { kernel: HipKernel::upload_q4_k(weight, in_features, out_features)?, in_features, out_features,
+                  layer_name: name })
+    }
+}
+
+impl<'a> Layer for HipLinear<'a> {
+    fn forward(&self, input: &[f32], output: &mut [f32], _ctx: &mut ExecContext) {
+        expect_ok(unsafe {
+            rmi_hip_quantized_linear_forward(self.kernel.handle, input.as_ptr(), output.as_mut_ptr(),
+                                             self.in_features as u32, self.out_features as u32)
+        });
+    }
+    fn input_dim(&self) -> usize { self.in_features }
+    fn output_dim(&self) -> usize { self.out_features }
+    fn name(&self) -> &str { self.layer_name }
+}
+
+#[allow(dead_code)]
+fn _unused(_: *mut c_void) {}
