@@ -163,6 +163,48 @@ void rmi_ref_pool_matmul_q4k_q8k(rmi_ref_pool *pool, const uint8_t *weight,
                                  const int16_t *bsums, float *output,
                                  size_t n_in, size_t n_out);
 
+/* generic job on the pool: fn(arg, ith, nth) on every thread, then a barrier */
+void rmi_ref_pool_run(rmi_ref_pool *pool, void (*fn)(void *arg, int ith, int nth), void *arg);
+
+/* ---- rmi_qwen3.c: Qwen3Session::generate_inner (src/models/qwen3.rs:581-1158)
+ * restated for an all-Q8_0 model with F16 KV cache, NeoX RoPE, greedy sampling.
+ * Every quantized matmul goes through `matmul`, whose signature is that of
+ * Kernel::forward_prequantized with the weight as an opaque first argument, so
+ * the same loop runs on the restated CPU kernels or on any back end that is
+ * handed in from outside. ---- */
+typedef int (*rmi_ref_matmul_fn)(const void *weight, const uint8_t *input_q8, const float *input_scales,
+                                 float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth);
+
+typedef struct {
+    uint32_t n_embd, n_layer, n_head, n_head_kv, head_dim_k, head_dim_v, n_ff, vocab, n_ctx;
+    float eps, freq_base;
+    int32_t has_qk_norm;
+    int32_t quant_variant;        /* RMI_REF_SCALAR / RMI_REF_AVX2 activation quantizer */
+    const uint8_t *token_embd;    /* raw Q8_0 rows, for embedding_lookup_q8_0 */
+    const float *output_norm;
+    const void *output;           /* matmul weight of the (tied) lm_head */
+    const float *const *attn_norm, *const *ffn_norm, *const *q_norm, *const *k_norm; /* [n_layer] */
+    const void *const *wq, *const *wk, *const *wv, *const *wo, *const *w_gate, *const *w_up, *const *w_down;
+} rmi_ref_qwen3_model;
+
+/* weight argument for rmi_ref_cpu_matmul */
+typedef struct {
+    const uint8_t *blocks;
+    rmi_ref_pool *pool;
+} rmi_ref_cpu_weight;
+int rmi_ref_cpu_matmul(const void *weight, const uint8_t *input_q8, const float *input_scales, float *output,
+                       uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth);
+
+/* Runs n_prompt + max_new - 1 decoder steps (one token per step, prompt
+ * included).  Per step: FNV-1a hash of the logits' bytes, argmax, the two
+ * largest logits; full logits of the steps listed in dump_steps.  Returns the
+ * number of generated tokens, or -1 on error (non-finite logits, capacity). */
+int rmi_ref_qwen3_generate(const rmi_ref_qwen3_model *model, rmi_ref_matmul_fn matmul, rmi_ref_pool *pool,
+                           const uint32_t *prompt, uint32_t n_prompt, uint32_t max_new, uint32_t *generated,
+                           uint64_t *step_hash, uint32_t *step_argmax, float *step_top2,
+                           const uint32_t *dump_steps, uint32_t n_dump, float *dump_logits,
+                           double *seconds_total, double *seconds_matmul);
+
 #ifdef __cplusplus
 }
 #endif

@@ -299,3 +299,120 @@ class Pool:
 
     def __del__(self):
         self.close()
+
+
+# ---- restated Qwen3 decode loop with a pluggable matmul (rmi_qwen3.c) ----
+
+MATMUL_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, _u8p, _f32p, _f32p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32)
+_fpp = C.POINTER(_f32p)
+_vpp = C.POINTER(C.c_void_p)
+
+
+class Qwen3ModelStruct(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("n_embd", "n_layer", "n_head", "n_head_kv", "head_dim_k", "head_dim_v",
+                                          "n_ff", "vocab", "n_ctx")] + [
+        ("eps", C.c_float), ("freq_base", C.c_float), ("has_qk_norm", C.c_int32), ("quant_variant", C.c_int32),
+        ("token_embd", C.c_void_p), ("output_norm", _f32p), ("output", C.c_void_p),
+        ("attn_norm", _fpp), ("ffn_norm", _fpp), ("q_norm", _fpp), ("k_norm", _fpp),
+        ("wq", _vpp), ("wk", _vpp), ("wv", _vpp), ("wo", _vpp), ("w_gate", _vpp), ("w_up", _vpp), ("w_down", _vpp)]
+
+
+class CpuWeight(C.Structure):
+    _fields_ = [("blocks", C.c_void_p), ("pool", C.c_void_p)]
+
+
+lib.rmi_ref_cpu_matmul.restype = C.c_int
+lib.rmi_ref_qwen3_generate.restype = C.c_int
+lib.rmi_ref_qwen3_generate.argtypes = [C.POINTER(Qwen3ModelStruct), C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32),
+                                       C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint64),
+                                       C.POINTER(C.c_uint32), _f32p, C.POINTER(C.c_uint32), C.c_uint32, _f32p,
+                                       C.POINTER(C.c_double), C.POINTER(C.c_double)]
+
+_MATMUL_NAMES = ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down")
+_FIELD_OF = dict(zip(_MATMUL_NAMES, ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")))
+
+
+class Qwen3Decoder:
+    """The restated `Qwen3Session` over a GGUF-like tensor dict.
+
+    `weight_handle(name, bytes, n_in, n_out)` turns each Q8_0 matrix into the opaque
+    first argument of `matmul_fn` (a C function pointer with the signature of
+    Kernel::forward_prequantized).  With the defaults both are the restated CPU kernels.
+    """
+
+    def __init__(self, metadata, tensors, pool, matmul_fn=None, weight_handle=None, quant_variant=AVX2):
+        g = lambda k: int(metadata[f"qwen3.{k}"])  # noqa: E731
+        self.pool = pool
+        self._keep = []
+        m = Qwen3ModelStruct()
+        m.n_embd, m.n_layer, m.n_head, m.n_head_kv = g("embedding_length"), g("block_count"), g(
+            "attention.head_count"), g("attention.head_count_kv")
+        m.head_dim_k = int(metadata.get("qwen3.attention.key_length", m.n_embd // m.n_head))
+        m.head_dim_v = int(metadata.get("qwen3.attention.value_length", m.n_embd // m.n_head))
+        m.n_ff, m.n_ctx = g("feed_forward_length"), g("context_length")
+        m.vocab = int(metadata["qwen3.vocab_size"])
+        m.eps = float(metadata["qwen3.attention.layer_norm_rms_epsilon"])
+        m.freq_base = float(metadata.get("qwen3.rope.freq_base", 1e6))
+        m.has_qk_norm, m.quant_variant = 1, quant_variant
+        if weight_handle is None:
+            def weight_handle(name, data, n_in, n_out):
+                cw = CpuWeight(data.ctypes.data, pool._h)
+                self._keep.append(cw)
+                return C.addressof(cw)
+            matmul_fn = C.cast(lib.rmi_ref_cpu_matmul, C.c_void_p).value
+        self.matmul_fn = matmul_fn
+
+        def f32(name):
+            a = np.ascontiguousarray(tensors[name].view(np.float32))
+            self._keep.append(a)
+            return a.ctypes.data_as(_f32p)
+
+        def raw(name):
+            a = np.ascontiguousarray(tensors[name])
+            self._keep.append(a)
+            return a
+
+        embd = raw("token_embd.weight")
+        m.token_embd = embd.ctypes.data
+        m.output_norm = f32("output_norm.weight")
+        q_dim, kv_dim = m.n_head * m.head_dim_k, m.n_head_kv * m.head_dim_k
+        shapes = {"attn_q": (m.n_embd, q_dim), "attn_k": (m.n_embd, kv_dim), "attn_v": (m.n_embd, kv_dim),
+                  "attn_output": (m.n_head * m.head_dim_v, m.n_embd), "ffn_gate": (m.n_embd, m.n_ff),
+                  "ffn_up": (m.n_embd, m.n_ff), "ffn_down": (m.n_ff, m.n_embd)}
+        # tied lm_head: the embedding table is also the output matrix (qwen3.rs:283-287)
+        out_name = "output.weight" if "output.weight" in tensors else "token_embd.weight"
+        m.output = weight_handle(out_name, raw(out_name), m.n_embd, m.vocab)
+        for field in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+            gname = {"attn_norm": "attn_norm", "ffn_norm": "ffn_norm", "q_norm": "attn_q_norm", "k_norm": "attn_k_norm"}[field]
+            arr = (_f32p * m.n_layer)(*[f32(f"blk.{layer}.{gname}.weight") for layer in range(m.n_layer)])
+            self._keep.append(arr)
+            setattr(m, field, arr)
+        for name in _MATMUL_NAMES:
+            n_in, n_out = shapes[name]
+            arr = (C.c_void_p * m.n_layer)(*[weight_handle(f"blk.{layer}.{name}.weight",
+                                                           raw(f"blk.{layer}.{name}.weight"), n_in, n_out)
+                                             for layer in range(m.n_layer)])
+            self._keep.append(arr)
+            setattr(m, _FIELD_OF[name], arr)
+        self.model = m
+
+    def generate(self, prompt, max_new, dump_steps=()):
+        prompt = np.ascontiguousarray(prompt, np.uint32)
+        steps = prompt.size + max_new - 1
+        gen = np.zeros(max_new, np.uint32)
+        hashes = np.zeros(steps, np.uint64)
+        argmax = np.zeros(steps, np.uint32)
+        top2 = np.zeros((steps, 2), np.float32)
+        dump_steps = np.ascontiguousarray(dump_steps, np.uint32)
+        dump = np.zeros((max(dump_steps.size, 1), self.model.vocab), np.float32)
+        t_total, t_mm = C.c_double(), C.c_double()
+        u32p = C.POINTER(C.c_uint32)
+        n = lib.rmi_ref_qwen3_generate(C.byref(self.model), self.matmul_fn, self.pool._h, prompt.ctypes.data_as(u32p),
+                                       prompt.size, max_new, gen.ctypes.data_as(u32p),
+                                       hashes.ctypes.data_as(C.POINTER(C.c_uint64)), argmax.ctypes.data_as(u32p),
+                                       _p(top2, _f32p), dump_steps.ctypes.data_as(u32p), dump_steps.size,
+                                       _p(dump, _f32p), C.byref(t_total), C.byref(t_mm))
+        if n < 0:
+            raise RuntimeError("qwen3_generate failed (non-finite logits, capacity, or a failing matmul)")
+        return dict(tokens=gen[:n], hashes=hashes, argmax=argmax, top2=top2, dump=dump[:dump_steps.size],
+                    seconds=t_total.value, seconds_matmul=t_mm.value, steps=steps)

@@ -222,7 +222,7 @@ float rmi_ref_x86_vec_dot_q4k_q8k(const uint8_t *q4k, size_t nb, const float *d8
 
 /* ------------------------------------------------- persistent thread pool */
 
-enum { JOB_NONE = 0, JOB_Q8_0 = 1, JOB_Q4K = 2, JOB_EXIT = 3 };
+enum { JOB_NONE = 0, JOB_Q8_0 = 1, JOB_Q4K = 2, JOB_EXIT = 3, JOB_FN = 4 };
 
 struct rmi_ref_pool {
     int n_threads;
@@ -238,6 +238,8 @@ struct rmi_ref_pool {
     const int16_t *bsums;
     float *output;
     size_t n_in, n_out, n_tokens;
+    void (*fn)(void *, int, int);
+    void *fn_arg;
 };
 
 typedef struct {
@@ -246,6 +248,10 @@ typedef struct {
 } worker_arg;
 
 static void run_slice(rmi_ref_pool *p, int ith) {
+    if (p->job == JOB_FN) {
+        p->fn(p->fn_arg, ith, p->n_threads);
+        return;
+    }
     size_t nth = (size_t)p->n_threads;
     size_t per = (p->n_out + nth - 1) / nth;
     size_t start = (size_t)ith * per;
@@ -342,5 +348,12 @@ void rmi_ref_pool_matmul_q4k_q8k(rmi_ref_pool *p, const uint8_t *weight,
     p->n_in = n_in;
     p->n_out = n_out;
     p->n_tokens = 1;
+    pool_run(p);
+}
+
+void rmi_ref_pool_run(rmi_ref_pool *p, void (*fn)(void *arg, int ith, int nth), void *arg) {
+    p->job = JOB_FN;
+    p->fn = fn;
+    p->fn_arg = arg;
     pool_run(p);
 }

@@ -1,6 +1,7 @@
 """MI355X (gfx950) back end for rust-model-inference's quantized matrix products.
 
 ``synth``  seeded synthetic tensors of the benchmark shapes (numpy only)
+``gguf``   minimal GGUF v3 writer / mmap reader (synthetic Qwen3 file)
 ``hip``    ctypes binding of librmi_hip.so, the C ABI of include/rmi_hip.h
 ``kernel`` mirror of the reference's Kernel / Layer interface over that ABI
 
@@ -9,7 +10,7 @@ is missing; nothing here computes on the CPU.
 """
 import importlib
 
-from . import synth  # noqa: F401
+from . import gguf, synth  # noqa: F401
 
 _LAZY = ("hip", "kernel")
 
