@@ -194,33 +194,37 @@ def read_traffic(mode):
     return None
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
-    ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--copy-calibration-mb", type=int, default=0,
-                    help="also launch the plain copy kernel on this many MiB, 5 times, outside the timed region "
-                         "(the known-size kernel that rocprofv3 --pmc traffic counters are scaled against)")
-    ap.add_argument("--extra", action="store_true", help="also time the other launch modes, outside the timed region")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across GPUs", file=sys.stderr)
-        sys.exit(2)
+def time_region(H, ev, fn, steps, warmup):
+    """W untimed warm-up steps, then exactly K timed steps between a device synchronisation on both sides.
+    Returns (host wall seconds per step, device ms per step from two HIP events on the launch stream)."""
+    for _ in range(warmup):
+        fn()
+    ev_a, ev_b = ev.create(), ev.create()
+    H.check(H.lib.rmi_hip_synchronize())
+    t0 = time.perf_counter()
+    ev.record(ev_a)
+    for _ in range(steps):
+        fn()
+    ev.record(ev_b)
+    H.check(H.lib.rmi_hip_synchronize())
+    wall = (time.perf_counter() - t0) / steps
+    return wall, ev.elapsed_ms(ev_a, ev_b) / steps
 
-    pkg = importlib.import_module("rust-model-inference_amd")
+
+def base_result(args, metric, unit, value, wall, dtype, config):
+    return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(wall * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": dtype, "data": "synthetic", "config": config}
+
+
+def run_projection_set(args, pkg, ev):
     H, synth = pkg.hip, pkg.synth
-    pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
     dev_name, cus, hbm = H.device_info()
     batch = args.batch
     want_cpu = not args.no_cpu_baseline
     problems = build_projection_set(pkg, batch, keep_host=want_cpu)
     alg_bytes = sum(synth.q8_0_gemv_bytes(r["n_out"], r["n_in"], batch) for r in problems)
     flops = sum(2 * r["n_out"] * r["n_in"] * batch for r in problems)
-    ev = HipEvents()
 
     group_all = make_group(H, problems, batch)
     groups_layer = layer_groups(H, problems, batch)
@@ -240,22 +244,6 @@ def main():
     modes = {"grouped": (step_grouped, 1), "per_matmul": (step_per_matmul, len(problems)),
              "layer": (step_layer, len(groups_layer))}
 
-    def measure(mode, steps, warmup):
-        """Returns (host wall s/step, device ms/step between two events on the launch stream, launches/step)."""
-        fn, launches = modes[mode]
-        for _ in range(warmup):
-            fn()
-        ev_a, ev_b = ev.create(), ev.create()
-        H.check(H.lib.rmi_hip_synchronize())
-        t0 = time.perf_counter()
-        ev.record(ev_a)
-        for _ in range(steps):
-            fn()
-        ev.record(ev_b)
-        H.check(H.lib.rmi_hip_synchronize())
-        wall = (time.perf_counter() - t0) / steps
-        return wall, ev.elapsed_ms(ev_a, ev_b) / steps, launches
-
     if args.copy_calibration_mb:
         nbytes = args.copy_calibration_mb << 20
         src, dst = H.DeviceBuffer(nbytes), H.DeviceBuffer(nbytes)
@@ -265,32 +253,22 @@ def main():
         src.free()
         dst.free()
 
-    wall, dev_ms, launches = measure(args.mode, args.steps, args.warmup)
+    fn, launches = modes[args.mode]
+    wall, dev_ms = time_region(H, ev, fn, args.steps, args.warmup)
     value = alg_bytes / wall / 1e9
     achieved = alg_bytes / (dev_ms * 1e-3) / 1e9  # bytes per launch / average launch duration, summed over the step
-    result = {
-        "metric": "Q8_0 GEMV HBM GB/s, Qwen3-0.6B shapes, 1 GPU",
-        "value": round(value, 1),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(wall * 1e3, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "int8 dot4 -> f32",
-        "data": "synthetic",
-        "config": {
-            "workload": f"Qwen3-0.6B per-token projection set (7x28 + lm_head = 197 Q8_0 GEMVs, 633 MB of weights), "
-                        f"decode batch {batch}, launch mode {args.mode}",
-            "batch": batch,
-            "launches_per_step": launches,
-            "algorithmic_bytes_per_step": alg_bytes,
-            "flops_per_step": flops,
-            "device": dev_name.strip(),
-            "compute_units": cus,
-        },
+    result = base_result(args, "Q8_0 GEMV HBM GB/s, Qwen3-0.6B shapes, 1 GPU", "GB/s", round(value, 1), wall,
+                         "int8 dot4 -> f32", {
+        "workload": f"Qwen3-0.6B per-token projection set (7x28 + lm_head = 197 Q8_0 GEMVs, 633 MB of weights), "
+                    f"decode batch {batch}, launch mode {args.mode}",
+        "batch": batch,
+        "launches_per_step": launches,
+        "algorithmic_bytes_per_step": alg_bytes,
+        "flops_per_step": flops,
+        "device": dev_name.strip(),
+        "compute_units": cus,
+    })
+    result.update({
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "token_steps_per_s": round(1.0 / wall, 1),
         "gflops": round(flops / wall / 1e9, 1),
@@ -303,16 +281,16 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
             "algorithmic_bytes_per_launch": round(alg_bytes / launches),
-            "traffic": read_traffic(args.mode),
+            "traffic": read_traffic(args.mode) if batch == 1 else None,
         },
-    }
+    })
 
     if args.extra:
         extra = {}
-        for mode in modes:
+        for mode, (fn2, l2) in modes.items():
             if mode == args.mode:
                 continue
-            w2, d2, l2 = measure(mode, max(5, args.steps // 5), 3)
+            w2, d2 = time_region(H, ev, fn2, max(5, args.steps // 5), 3)
             extra[mode] = {"GB/s": round(alg_bytes / w2 / 1e9, 1), "ms_per_step": round(w2 * 1e3, 4),
                            "device_ms_per_step": round(d2, 4), "launches_per_step": l2,
                            "token_steps_per_s": round(1.0 / w2, 1)}
@@ -332,8 +310,169 @@ def main():
             result["cpu_baseline"]["gpu_outputs_differing_from_cpu"] = worst
         else:
             result["cpu_baseline"] = None
+    return result
 
-    print(json.dumps(result), flush=True)
+
+def run_gemm(args, pkg, ev):
+    """Prefill GEMM: X[M x 1024] . W[3072 x 1024]^T and X[M x 3072] . W[1024 x 3072]^T, Q8_0 both sides.
+    One step = both products on activations already quantized in HBM."""
+    H, synth, K = pkg.hip, pkg.synth, pkg.kernel
+    dev_name, cus, hbm = H.device_info()
+    M = args.tokens
+    recs = []
+    for i, (n_out, n_in) in enumerate([(3072, 1024), (1024, 3072)]):
+        w = synth.q8_0_weight(synth.seed_for(2, i), n_out, n_in)
+        x = synth.activations(synth.seed_for(2, 0x8000 + i), M, n_in)
+        k = K.Q8Kernel(w, n_in, n_out)
+        d_x = H.DeviceBuffer.from_array(x)
+        d_q8, d_sc, d_y = H.DeviceBuffer(M * n_in), H.DeviceBuffer(M * n_in // 32 * 4), H.DeviceBuffer(M * n_out * 4)
+        H.check(H.lib.rmi_hip_quantize_q8_0_dev(d_x.ptr, d_q8.ptr, d_sc.ptr, M, n_in, H.ROUND_TIES_EVEN, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        recs.append(dict(w=w, x=x, k=k, d_q8=d_q8, d_sc=d_sc, d_y=d_y, n_out=n_out, n_in=n_in))
+
+    def step():
+        for r in recs:
+            H.check(H.lib.rmi_hip_gemm_q8_0_dev(r["k"].w.handle, r["d_q8"].ptr, r["d_sc"].ptr, r["d_y"].ptr, M,
+                                                r["n_out"], None))
+
+    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
+    ops = sum(2.0 * M * r["n_in"] * r["n_out"] for r in recs)
+    value = ops / wall / 1e12
+    achieved = ops / (dev_ms * 1e-3) / 1e12
+    result = base_result(args, "Q8_0 prefill GEMM TOP/s (int8 MFMA), Qwen3-0.6B FFN shapes, 1 GPU", "TOP/s",
+                         round(value, 1), wall, "int8 MFMA -> f32", {
+        "workload": f"Q8_0 GEMM M={M} tokens: X[Mx1024].W[3072x1024]^T and X[Mx3072].W[1024x3072]^T, "
+                    f"per-block f32 rescale, 2 launches per step",
+        "tokens": M, "launches_per_step": 2, "ops_per_step": ops, "device": dev_name.strip(), "compute_units": cus})
+    result["roofline"] = {"bound": "mfma", "kernel": "gemm_q8_0_kernel", "achieved": round(achieved, 1), "peak": 5000.0,
+                          "unit": "TOP/s", "frac": round(achieved / 5000.0, 4),
+                          "avg_launch_us": round(dev_ms * 1e3 / 2, 3), "traffic": None}
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import rmi_oracle as oracle
+        if oracle.have_avx2():
+            cores = min(16, physical_cores())
+            pool = oracle.Pool(cores)
+            mt = min(M, 256)  # bounded sample: the first `mt` tokens of both products
+            outs, qs = [], []
+            for r in recs:
+                q8 = r["d_q8"].to_array(np.uint8, (M, r["n_in"]))[:mt].copy()
+                sc = r["d_sc"].to_array(np.float32, (M, r["n_in"] // 32))[:mt].copy()
+                qs.append((q8, sc))
+                outs.append(np.zeros((mt, r["n_out"]), np.float32))
+            samples = []
+            for it in range(4):
+                t0 = time.perf_counter()
+                for r, (q8, sc), out in zip(recs, qs, outs):
+                    pool.matmul_q8_0(r["w"], q8, sc, out, r["n_in"], r["n_out"], mt)
+                samples.append(time.perf_counter() - t0)
+            pool.close()
+            med = statistics.median(samples[1:])
+            step()
+            H.check(H.lib.rmi_hip_synchronize())
+            worst = 0.0
+            for r, out in zip(recs, outs):
+                gpu = r["d_y"].to_array(np.float32, (M, r["n_out"]))[:mt]
+                worst = max(worst, float(np.max(np.abs(gpu - out) / (1e-4 + 1e-4 * np.abs(out)))))
+            result["cpu_baseline"] = {
+                "value": round(ops * mt / M / med / 1e12, 4), "unit": "TOP/s", "cores": cores, "kind": "port",
+                "sample": f"first {mt} of {M} tokens of both products, one GEMV per token (the reference has no GEMM), "
+                          f"restated AVX2 kernels over {cores} threads, median of 3",
+                "max_err_over_tolerance": round(worst, 4)}
+    return result
+
+
+def run_q4k(args, pkg, ev):
+    """Q4_K x Q8_K decode GEMV at 1.7B-class FFN shapes (gate/up 6144x2048, down 2048x6144), 28 layers of
+    distinct weights (594 MB) so that every step streams from HBM; one launch per matrix."""
+    H, synth, K = pkg.hip, pkg.synth, pkg.kernel
+    dev_name, cus, hbm = H.device_info()
+    batch = args.batch
+    recs = []
+    shapes = [(6144, 2048), (6144, 2048), (2048, 6144)] * 28
+    for i, (n_out, n_in) in enumerate(shapes):
+        w = synth.q4_k_weight(synth.seed_for(3, i), n_out, n_in)
+        x = synth.activations(synth.seed_for(3, 0x8000 + i), batch, n_in)
+        k = K.Q4_KKernel(w, n_in, n_out)
+        d_x = H.DeviceBuffer.from_array(x)
+        d_d, d_q, d_b = H.DeviceBuffer(batch * n_in // 256 * 4), H.DeviceBuffer(batch * n_in), H.DeviceBuffer(batch * n_in // 16 * 2)
+        d_y = H.DeviceBuffer(batch * n_out * 4)
+        H.check(H.lib.rmi_hip_quantize_row_q8_k_dev(d_x.ptr, d_d.ptr, d_q.ptr, d_b.ptr, batch, n_in, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        d_x.free()
+        recs.append(dict(w=w if not args.no_cpu_baseline else None, k=k, d_d=d_d, d_q=d_q, d_b=d_b, d_y=d_y, n_out=n_out,
+                         n_in=n_in))
+
+    def step():
+        for r in recs:
+            H.check(H.lib.rmi_hip_gemv_q4_k_q8k_dev(r["k"].w.handle, r["d_d"].ptr, r["d_q"].ptr, r["d_b"].ptr,
+                                                    r["d_y"].ptr, batch, r["n_out"], 0, r["n_out"], None))
+
+    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
+    alg = sum(synth.q4_k_gemv_bytes(r["n_out"], r["n_in"], batch) for r in recs)
+    value = alg / wall / 1e9
+    achieved = alg / (dev_ms * 1e-3) / 1e9
+    result = base_result(args, "Q4_K x Q8_K GEMV HBM GB/s, 1.7B-class FFN shapes, 1 GPU", "GB/s", round(value, 1), wall,
+                         "int8 dot4 -> f32", {
+        "workload": f"Q4_K GEMV, 28 layers x (gate 6144x2048, up 6144x2048, down 2048x6144), decode batch {batch}, "
+                    f"one launch per matrix", "batch": batch, "launches_per_step": len(recs),
+        "algorithmic_bytes_per_step": alg, "device": dev_name.strip(), "compute_units": cus})
+    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_k_kernel<{batch}>", "achieved": round(achieved, 1),
+                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                          "avg_launch_us": round(dev_ms * 1e3 / len(recs), 3), "traffic": None}
+    if not args.no_cpu_baseline and batch == 1:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import rmi_oracle as oracle
+        if oracle.have_avx2():
+            cores = min(16, physical_cores())
+            pool = oracle.Pool(cores)
+            host = [(r["d_d"].to_array(np.float32, (r["n_in"] // 256,)), r["d_q"].to_array(np.int8, (r["n_in"],)),
+                     r["d_b"].to_array(np.int16, (r["n_in"] // 16,)), np.zeros(r["n_out"], np.float32)) for r in recs]
+            samples = []
+            for it in range(6):
+                t0 = time.perf_counter()
+                for r, (d, q, b, out) in zip(recs, host):
+                    pool.matmul_q4k_q8k(r["w"], d, q, b, out, r["n_in"], r["n_out"])
+                samples.append(time.perf_counter() - t0)
+            pool.close()
+            med = statistics.median(samples[1:])
+            step()
+            H.check(H.lib.rmi_hip_synchronize())
+            worst = max(int(np.count_nonzero(r["d_y"].to_array(np.float32, (r["n_out"],)).view(np.uint32)
+                                             != out.view(np.uint32))) for r, (_, _, _, out) in zip(recs, host))
+            result["cpu_baseline"] = {"value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                                      "sample": f"5 full steps (84 GEMVs, {alg / 1e6:.0f} MB), restated AVX2 "
+                                                f"vec_dot_q4k_q8k over {cores} threads, median",
+                                      "gpu_outputs_differing_from_cpu": worst}
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4k"], default="projection_set",
+                    help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
+                         "q4k: Q4_K x Q8_K decode GEMV")
+    ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
+    ap.add_argument("--tokens", type=int, default=2048, help="prefill tokens M for --workload gemm")
+    ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration-mb", type=int, default=0,
+                    help="also launch the plain copy kernel on this many MiB, 5 times, outside the timed region "
+                         "(the known-size kernel that rocprofv3 --pmc traffic counters are scaled against)")
+    ap.add_argument("--extra", action="store_true", help="also time the other launch modes, outside the timed region")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across GPUs", file=sys.stderr)
+        sys.exit(2)
+
+    pkg = importlib.import_module("rust-model-inference_amd")
+    pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
+    ev = HipEvents()
+    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4k": run_q4k}[args.workload]
+    print(json.dumps(run(args, pkg, ev)), flush=True)
 
 
 if __name__ == "__main__":
