@@ -384,7 +384,7 @@ def run_gemm(args, pkg, ev):
 
 def run_q4k(args, pkg, ev):
     """Q4_K x Q8_K decode GEMV at 1.7B-class FFN shapes (gate/up 6144x2048, down 2048x6144), 28 layers of
-    distinct weights (594 MB) so that every step streams from HBM; one launch per matrix."""
+    distinct weights (594 MB) so that every step streams from HBM; one grouped launch, or one per matrix with --mode per_matmul."""
     H, synth, K = pkg.hip, pkg.synth, pkg.kernel
     dev_name, cus, hbm = H.device_info()
     batch = args.batch
@@ -403,11 +403,26 @@ def run_q4k(args, pkg, ev):
         recs.append(dict(w=w if not args.no_cpu_baseline else None, k=k, d_d=d_d, d_q=d_q, d_b=d_b, d_y=d_y, n_out=n_out,
                          n_in=n_in))
 
-    def step():
+    n = len(recs)
+    arr = lambda vals: (C.c_void_p * n)(*vals)  # noqa: E731
+    group = H.lib.rmi_hip_gemv_group_create_q4_k(n, arr([r["k"].w.handle for r in recs]),
+                                                 arr([r["d_d"].ptr for r in recs]), arr([r["d_q"].ptr for r in recs]),
+                                                 arr([r["d_b"].ptr for r in recs]), arr([r["d_y"].ptr for r in recs]),
+                                                 batch)
+    if not group:
+        raise RuntimeError(H.last_error())
+
+    def step_per_matmul():
         for r in recs:
             H.check(H.lib.rmi_hip_gemv_q4_k_q8k_dev(r["k"].w.handle, r["d_d"].ptr, r["d_q"].ptr, r["d_b"].ptr,
                                                     r["d_y"].ptr, batch, r["n_out"], 0, r["n_out"], None))
 
+    def step_grouped():
+        H.check(H.lib.rmi_hip_gemv_group_run_dev(group, None))
+
+    grouped = args.mode != "per_matmul"
+    step = step_grouped if grouped else step_per_matmul
+    launches = 1 if grouped else n
     wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
     alg = sum(synth.q4_k_gemv_bytes(r["n_out"], r["n_in"], batch) for r in recs)
     value = alg / wall / 1e9
@@ -415,11 +430,13 @@ def run_q4k(args, pkg, ev):
     result = base_result(args, "Q4_K x Q8_K GEMV HBM GB/s, 1.7B-class FFN shapes, 1 GPU", "GB/s", round(value, 1), wall,
                          "int8 dot4 -> f32", {
         "workload": f"Q4_K GEMV, 28 layers x (gate 6144x2048, up 6144x2048, down 2048x6144), decode batch {batch}, "
-                    f"one launch per matrix", "batch": batch, "launches_per_step": len(recs),
+                    + ("one grouped launch" if grouped else "one launch per matrix"), "batch": batch,
+        "launches_per_step": launches,
         "algorithmic_bytes_per_step": alg, "device": dev_name.strip(), "compute_units": cus})
-    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_k_kernel<{batch}>", "achieved": round(achieved, 1),
-                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                          "avg_launch_us": round(dev_ms * 1e3 / len(recs), 3), "traffic": None}
+    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_k_kernel<{batch}, {'true' if grouped else 'false'}>",
+                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(achieved / HBM_PEAK_GBS, 4),
+                          "avg_launch_us": round(dev_ms * 1e3 / launches, 3), "traffic": None}
     if not args.no_cpu_baseline and batch == 1:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle

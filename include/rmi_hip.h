@@ -165,6 +165,11 @@ typedef struct rmi_hip_gemv_group rmi_hip_gemv_group;
 rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip_weight *const *weights,
                                               const int8_t *const *x_q8, const float *const *x_scales,
                                               float *const *y, uint32_t n_tokens);
+/* The same for Q4_K weights with Q8_K activations (three arrays per problem). */
+rmi_hip_gemv_group *rmi_hip_gemv_group_create_q4_k(uint32_t n_problems, const rmi_hip_weight *const *weights,
+                                                   const float *const *q8k_d, const int8_t *const *q8k_qs,
+                                                   const int16_t *const *q8k_bsums, float *const *y,
+                                                   uint32_t n_tokens);
 void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g);
 int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream);
 

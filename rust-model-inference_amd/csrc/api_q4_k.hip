@@ -1,4 +1,6 @@
 // extern "C" entry points for Q4_K weights (Q4_KKernel and QuantizedLinear).
+#include <vector>
+
 #include "rmi_internal.h"
 
 namespace {
@@ -179,6 +181,65 @@ int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
     if (!q8k_d || !q8k_qs || !q8k_bsums || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
     return rmi_launch_gemv_q4_k(w, q8k_d, q8k_qs, q8k_bsums, y, n_tokens, y_stride, row_start, row_end,
                                 static_cast<hipStream_t>(stream));
+}
+
+rmi_hip_gemv_group *rmi_hip_gemv_group_create_q4_k(uint32_t n_problems, const rmi_hip_weight *const *weights,
+                                                   const float *const *q8k_d, const int8_t *const *q8k_qs,
+                                                   const int16_t *const *q8k_bsums, float *const *y,
+                                                   uint32_t n_tokens) {
+    if (!rmi_ready()) {
+        rmi_set_error("rmi_hip_init has not succeeded");
+        return nullptr;
+    }
+    if (n_problems == 0 || n_tokens == 0 || n_tokens > 8 || !weights || !q8k_d || !q8k_qs || !q8k_bsums || !y) {
+        rmi_set_error("gemv group needs >=1 problem and 1..8 tokens");
+        return nullptr;
+    }
+    if (!rmi_thread_ctx()) return nullptr;
+    std::vector<RmiQ4kProblem> list(n_problems);
+    rmi_hip_gemv_group *g = new rmi_hip_gemv_group();
+    g->dtype = RMI_HIP_DTYPE_Q4_K;
+    g->n_problems = n_problems;
+    g->n_tokens = n_tokens;
+    uint64_t total_tiles = 0;
+    for (uint32_t i = 0; i < n_problems; i++) {
+        const rmi_hip_weight *w = weights[i];
+        if (!w || w->dtype != RMI_HIP_DTYPE_Q4_K || !q8k_d[i] || !q8k_qs[i] || !q8k_bsums[i] || !y[i]) {
+            rmi_set_error("gemv group problem %u: bad weight handle or null pointer", i);
+            delete g;
+            return nullptr;
+        }
+        list[i] = rmi_make_q4k_problem(w, q8k_d[i], q8k_qs[i], q8k_bsums[i], y[i], w->n_out, 0, w->n_out);
+        total_tiles += list[i].n_tiles;
+        if (w->n_units > g->max_units) g->max_units = w->n_units;
+    }
+    if (total_tiles > 0x7fffffffull || size_t(n_tokens) * g->max_units * 304 > 64 * 1024) {
+        rmi_set_error("gemv group too large (%llu tiles, %u tokens x %u super-blocks)", (unsigned long long)total_tiles,
+                      n_tokens, g->max_units);
+        delete g;
+        return nullptr;
+    }
+    std::vector<uint4> runs;
+    for (uint32_t i = 0; i < n_problems; i++) {
+        if (list[i].n_sb == 0) continue;
+        const uint32_t tpw = rmi_q4k_tiles_per_wave(list[i].n_sb, uint32_t(total_tiles), n_tokens);
+        for (uint32_t k = 0; k < list[i].n_tiles; k += tpw)
+            runs.push_back(make_uint4(i, k, list[i].n_tiles - k < tpw ? list[i].n_tiles - k : tpw, 0));
+    }
+    g->n_runs = uint32_t(runs.size());
+    hipError_t e = hipMalloc(&g->d_list, sizeof(RmiQ4kProblem) * n_problems);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&g->d_runs), sizeof(uint4) * (runs.size() + 1));
+    if (e == hipSuccess) e = hipMemcpy(g->d_list, list.data(), sizeof(RmiQ4kProblem) * n_problems, hipMemcpyHostToDevice);
+    if (e == hipSuccess && !runs.empty())
+        e = hipMemcpy(g->d_runs, runs.data(), sizeof(uint4) * runs.size(), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        rmi_set_error("gemv group upload failed: %s", hipGetErrorString(e));
+        if (g->d_list) hipFree(g->d_list);
+        if (g->d_runs) hipFree(g->d_runs);
+        delete g;
+        return nullptr;
+    }
+    return g;
 }
 
 int rmi_hip_quantize_row_q8_k_dev(const float *x, float *d, int8_t *qs, int16_t *bsums, uint32_t n_tokens,

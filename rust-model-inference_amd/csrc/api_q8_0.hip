@@ -114,15 +114,6 @@ int host_gemv_range(const rmi_hip_weight *w, const uint8_t *input_q8, const floa
 
 }  // namespace
 
-struct rmi_hip_gemv_group {
-    RmiGemvProblem *d_list = nullptr;
-    uint4 *d_runs = nullptr;
-    uint32_t n_problems = 0;
-    uint32_t n_runs = 0;
-    uint32_t max_n_oct = 0;
-    uint32_t n_tokens = 0;
-};
-
 extern "C" {
 
 int rmi_hip_matmul_q8_0_quantized_range(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
@@ -305,6 +296,7 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
     if (!rmi_thread_ctx()) return nullptr;
     std::vector<RmiGemvProblem> list(n_problems);
     rmi_hip_gemv_group *g = new rmi_hip_gemv_group();
+    g->dtype = RMI_HIP_DTYPE_Q8_0;
     g->n_problems = n_problems;
     g->n_tokens = n_tokens;
     uint64_t total_tiles = 0;
@@ -317,11 +309,11 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
         }
         list[i] = make_problem(w, x_q8[i], x_scales[i], y[i], w->n_out, 0, w->n_out);
         total_tiles += list[i].n_tiles;
-        if (w->n_units > g->max_n_oct) g->max_n_oct = w->n_units;
+        if (w->n_units > g->max_units) g->max_units = w->n_units;
     }
-    if (total_tiles > 0x7fffffffull || size_t(n_tokens) * g->max_n_oct * 288 > 64 * 1024) {
+    if (total_tiles > 0x7fffffffull || size_t(n_tokens) * g->max_units * 288 > 64 * 1024) {
         rmi_set_error("gemv group too large (%llu tiles, %u tokens x %u octets)", (unsigned long long)total_tiles,
-                      n_tokens, g->max_n_oct);
+                      n_tokens, g->max_units);
         delete g;
         return nullptr;
     }
@@ -329,12 +321,12 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
     std::vector<uint4> runs;
     for (uint32_t i = 0; i < n_problems; i++) {
         if (list[i].n_oct == 0) continue;
-        const uint32_t tpw = rmi_gemv_tiles_per_wave(list[i].n_oct, uint32_t(total_tiles));
+        const uint32_t tpw = rmi_gemv_tiles_per_wave(list[i].n_oct, uint32_t(total_tiles), n_tokens);
         for (uint32_t k = 0; k < list[i].n_tiles; k += tpw)
             runs.push_back(make_uint4(i, k, list[i].n_tiles - k < tpw ? list[i].n_tiles - k : tpw, 0));
     }
     g->n_runs = uint32_t(runs.size());
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&g->d_list), sizeof(RmiGemvProblem) * n_problems);
+    hipError_t e = hipMalloc(&g->d_list, sizeof(RmiGemvProblem) * n_problems);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&g->d_runs), sizeof(uint4) * (runs.size() + 1));
     if (e == hipSuccess)
         e = hipMemcpy(g->d_list, list.data(), sizeof(RmiGemvProblem) * n_problems, hipMemcpyHostToDevice);
@@ -360,8 +352,11 @@ void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g) {
 int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream) {
     RMI_REQUIRE_INIT();
     if (!g) return rmi_fail(RMI_HIP_E_INVALID, "null group");
-    return rmi_launch_gemv_q8_0_group(g->d_list, g->d_runs, g->n_runs, g->max_n_oct, g->n_tokens,
-                                      static_cast<hipStream_t>(stream));
+    if (g->dtype == RMI_HIP_DTYPE_Q4_K)
+        return rmi_launch_gemv_q4_k_group(static_cast<const RmiQ4kProblem *>(g->d_list), g->d_runs, g->n_runs,
+                                          g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
+    return rmi_launch_gemv_q8_0_group(static_cast<const RmiGemvProblem *>(g->d_list), g->d_runs, g->n_runs,
+                                      g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

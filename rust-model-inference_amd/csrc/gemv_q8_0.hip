@@ -22,9 +22,14 @@ __device__ __forceinline__ float hsum8_lanes(float a) {
     return a;
 }
 
+// signed 4 x int8 dot (v_dot4c_i32_i8 into a cleared register)
+__device__ __forceinline__ int dot4_i8(int a, int b) {
+    return __builtin_amdgcn_sdot4(a, b, 0, false);
+}
+
 __device__ __forceinline__ void block_fma(float &acc, uint32_t w_bits, float xs, int wq, int xq) {
     const float s = h2f(w_bits) * xs;  // one rounding, as _mm_mul_ps(cvtph, set1(bd))
-    const int p = __builtin_amdgcn_sdot4(wq, xq, 0, false);
+    const int p = dot4_i8(wq, xq);
     acc = __builtin_fmaf(s, float(p), acc);
 }
 
@@ -286,10 +291,13 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4 *__restrict__ src
 
 }  // namespace
 
-// Tiles a wave takes in one run: about 8 tile-octets (17 KiB of weights), fewer
-// when the launch would otherwise have too few waves to fill the chip.
-uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles) {
-    uint32_t tpw = n_oct >= 8 ? 1 : 8 / (n_oct ? n_oct : 1);
+// Tiles a wave takes in one run: about 8 tile-octets (17 KiB of weights) per
+// token of the batch, so that staging the activation (n_in bytes per token) stays
+// small against the weights read; fewer when the launch would otherwise have too
+// few waves to fill the chip.
+uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles, uint32_t n_tokens) {
+    const uint32_t target = 8 * (n_tokens ? n_tokens : 1);
+    uint32_t tpw = n_oct >= target ? 1 : target / (n_oct ? n_oct : 1);
     const uint32_t fill = uint32_t(rmi_device_cus()) * 8;
     while (tpw > 1 && launch_tiles / tpw < fill) tpw >>= 1;
     return tpw ? tpw : 1;
@@ -306,7 +314,7 @@ int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s) {
 
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s) {
     if (p.n_tiles == 0 || p.n_oct == 0) return RMI_HIP_OK;
-    const uint32_t tpw = rmi_gemv_tiles_per_wave(p.n_oct, p.n_tiles);
+    const uint32_t tpw = rmi_gemv_tiles_per_wave(p.n_oct, p.n_tiles, n_tokens);
     return dispatch_gemv(n_tokens, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, tpw, p.n_oct, s);
 }
 

@@ -22,6 +22,10 @@ __device__ __forceinline__ float hsum8_lanes(float a) {
     return a;
 }
 
+__device__ __forceinline__ int dot4_i8(int a, int b) {  // signed 4 x int8 dot
+    return __builtin_amdgcn_sdot4(a, b, 0, false);
+}
+
 // the kmask unpack of quant/mod.rs:237-258: sm.x,.y = 8 scales, sm.z,.w = 8 mins
 __device__ __forceinline__ uint4 unpack_scales(uint32_t u0, uint32_t u1, uint32_t u2) {
     const uint32_t kmask1 = 0x3f3f3f3fu, kmask2 = 0x0f0f0f0fu, kmask3 = 0x03030303u;
@@ -92,79 +96,130 @@ __global__ __launch_bounds__(64) void quantize_q8_k_kernel(const float *__restri
 // 1 dword d (+3 pad) = 76 dwords.
 constexpr uint32_t kSbDwords = 76;
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef const u32x4 __attribute__((address_space(1))) *gptr_u4;
+typedef const uint32_t __attribute__((address_space(1))) *gptr_u32;
+typedef const int16_t __attribute__((address_space(1))) *gptr_i16;
+typedef const float __attribute__((address_space(1))) *gptr_f32;
+typedef float __attribute__((address_space(1))) *gptr_f32_w;
+template <typename T, typename U>
+__device__ __forceinline__ T as_global(U *p) {
+    return (T)(uintptr_t)p;
+}
+
+struct SuperRegs {
+    u32x4 hdr;  // f16 d, f16 dmin, 12 packed scale bytes of the row
+    u32x4 qv;   // dwords 32g+4T (g = 0..3) of the row's nibble bytes
+};
+
+__device__ __forceinline__ void load_super(SuperRegs &g, gptr_u4 tile, uint32_t sb, uint32_t r, uint32_t lane) {
+    gptr_u4 chunk = tile + size_t(sb) * (kQ4KSuperBytes / 16);
+    g.hdr = chunk[r];
+    g.qv = chunk[8 + lane];
+}
+
 template <int B>
-__global__ __launch_bounds__(64) void gemv_q4_k_kernel(const uint8_t *__restrict__ w, const float *__restrict__ q8d,
-                                                        const int8_t *__restrict__ q8qs,
-                                                        const int16_t *__restrict__ q8bs, float *__restrict__ y,
-                                                        uint32_t n_in, uint32_t n_sb, uint32_t y_stride,
-                                                        uint32_t row_start, uint32_t row_end, uint32_t tile0,
-                                                        uint32_t n_tiles, uint32_t n_waves) {
+__device__ __forceinline__ void super_fma(float (&acc)[B], float (&acc_m)[B], const SuperRegs &g,
+                                          const uint32_t *lds_dw, uint32_t n_sb, uint32_t sb, uint32_t T) {
+    const float wd = h2f(g.hdr.x & 0xffffu), wdmin = h2f(g.hdr.x >> 16);
+    const uint4 sm = unpack_scales(g.hdr.y, g.hdr.z, g.hdr.w);
+    const uint32_t qd[4] = {g.qv.x, g.qv.y, g.qv.z, g.qv.w};
+    const int mn0 = int(byte_of(sm.z, sm.w, (2 * T) & 7)), mn1 = int(byte_of(sm.z, sm.w, (2 * T + 1) & 7));
+#pragma unroll
+    for (int t = 0; t < B; t++) {
+        const uint32_t *xs = lds_dw + (size_t(t) * n_sb + sb) * kSbDwords;
+        const uint4 xa = reinterpret_cast<const uint4 *>(xs + T * 8)[0];
+        const uint4 xb = reinterpret_cast<const uint4 *>(xs + T * 8)[1];
+        const uint32_t xd[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+        int sumi = 0;
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++) {
+            const int lo = int(qd[gg] & 0x0f0f0f0fu), hi = int((qd[gg] >> 4) & 0x0f0f0f0fu);
+            const int dl = dot4_i8(lo, int(xd[2 * gg]));
+            const int dh = dot4_i8(hi, int(xd[2 * gg + 1]));
+            sumi += int(byte_of(sm.x, sm.y, 2 * gg)) * dl + int(byte_of(sm.x, sm.y, 2 * gg + 1)) * dh;
+        }
+        const float d8 = __uint_as_float(xs[72]);
+        const float dd = wd * d8;
+        const float dm = (-wdmin) * d8;
+        acc[t] = __builtin_fmaf(dd, float(sumi), acc[t]);
+        const int s0 = int(xs[64 + ((2 * T) & 7)]), s1 = int(xs[64 + ((2 * T + 1) & 7)]);
+        const int prod = mn0 * s0 + mn1 * s1;
+        acc_m[t] = __builtin_fmaf(dm, float(prod), acc_m[t]);
+    }
+}
+
+// One wave per workgroup; a wave owns a short run of consecutive 8-row tiles of one
+// matrix, and a launch has far more waves than fit on the chip (see gemv_q8_0.hip).
+// GROUPED = false: one matrix (`single`), run w starts at tile w * tiles_per_wave.
+// GROUPED = true: runs[w] = {problem index, first tile, tile count, -}.
+template <int B, bool GROUPED>
+__global__ __launch_bounds__(64) void gemv_q4_k_kernel(RmiQ4kProblem single, const RmiQ4kProblem *__restrict__ list,
+                                                        const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
     extern __shared__ uint4 lds[];
     const uint32_t lane = threadIdx.x, r = lane >> 3, T = lane & 7;
+    RmiQ4kProblem p;
+    uint32_t k, k_end;
+    if (GROUPED) {
+        const uint4 run = runs[blockIdx.x];
+        p = list[run.x];
+        k = run.y;
+        k_end = run.y + run.z;
+    } else {
+        p = single;
+        k = blockIdx.x * tiles_per_wave;
+        k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
+    }
+    const uint32_t n_sb = p.n_sb, n_in = n_sb * 256;
     uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
     for (int t = 0; t < B; t++) {
         uint32_t *dst = lds_dw + size_t(t) * n_sb * kSbDwords;
-        const uint32_t *xq = reinterpret_cast<const uint32_t *>(q8qs + size_t(t) * n_in);
+        gptr_u32 xq = as_global<gptr_u32>(p.q8qs + size_t(t) * n_in);
         for (uint32_t i = lane; i < n_sb * 64; i += 64) {
             // source dword i of the row: super-block sb, element offset 4*(i%64) = 64g + 32*hi + 4T'
             const uint32_t sb = i >> 6, e = i & 63;
             const uint32_t g = e >> 4, hi = (e >> 3) & 1, tq = e & 7;
             dst[sb * kSbDwords + tq * 8 + g * 2 + hi] = xq[i];
         }
-        const int16_t *bs = q8bs + size_t(t) * (n_in / 16);
+        gptr_i16 bs = as_global<gptr_i16>(p.q8bs + size_t(t) * (n_in / 16));
         for (uint32_t i = lane; i < n_sb * 8; i += 64) {
             const uint32_t sb = i >> 3, j = i & 7;
             const int16_t s = int16_t(bs[sb * 16 + 2 * j] + bs[sb * 16 + 2 * j + 1]);
             dst[sb * kSbDwords + 64 + j] = uint32_t(int32_t(s));
         }
-        for (uint32_t i = lane; i < n_sb; i += 64) dst[i * kSbDwords + 72] = __float_as_uint(q8d[size_t(t) * n_sb + i]);
+        gptr_f32 dptr = as_global<gptr_f32>(p.q8d + size_t(t) * n_sb);
+        for (uint32_t i = lane; i < n_sb; i += 64) dst[i * kSbDwords + 72] = __float_as_uint(dptr[i]);
     }
     __syncthreads();
 
-    for (uint32_t k = blockIdx.x; k < n_tiles; k += n_waves) {
-        const uint8_t *tile = w + size_t(tile0 + k) * n_sb * kQ4KSuperBytes;
+    for (; k < k_end; k++) {
+        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * n_sb * kQ4KSuperBytes);
         float acc[B], acc_m[B];
 #pragma unroll
         for (int t = 0; t < B; t++) acc[t] = acc_m[t] = 0.0f;
-        for (uint32_t sb = 0; sb < n_sb; sb++) {
-            const uint8_t *chunk = tile + size_t(sb) * kQ4KSuperBytes;
-            const uint4 hdr = reinterpret_cast<const uint4 *>(chunk)[r];
-            const uint4 qv = reinterpret_cast<const uint4 *>(chunk + 128)[lane];
-            const float wd = h2f(hdr.x & 0xffffu), wdmin = h2f(hdr.x >> 16);
-            const uint4 sm = unpack_scales(hdr.y, hdr.z, hdr.w);
-            const uint32_t qd[4] = {qv.x, qv.y, qv.z, qv.w};
-            const int mn0 = int(byte_of(sm.z, sm.w, (2 * T) & 7)), mn1 = int(byte_of(sm.z, sm.w, (2 * T + 1) & 7));
-#pragma unroll
-            for (int t = 0; t < B; t++) {
-                const uint32_t *xs = lds_dw + (size_t(t) * n_sb + sb) * kSbDwords;
-                const uint4 xa = reinterpret_cast<const uint4 *>(xs + T * 8)[0];
-                const uint4 xb = reinterpret_cast<const uint4 *>(xs + T * 8)[1];
-                const uint32_t xd[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
-                int sumi = 0;
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int lo = int(qd[g] & 0x0f0f0f0fu), hi = int((qd[g] >> 4) & 0x0f0f0f0fu);
-                    const int dl = __builtin_amdgcn_sdot4(lo, int(xd[2 * g]), 0, false);
-                    const int dh = __builtin_amdgcn_sdot4(hi, int(xd[2 * g + 1]), 0, false);
-                    sumi += int(byte_of(sm.x, sm.y, 2 * g)) * dl + int(byte_of(sm.x, sm.y, 2 * g + 1)) * dh;
-                }
-                const float d8 = __uint_as_float(xs[72]);
-                const float dd = wd * d8;
-                const float dm = (-wdmin) * d8;
-                acc[t] = __builtin_fmaf(dd, float(sumi), acc[t]);
-                const int s0 = int(xs[64 + ((2 * T) & 7)]), s1 = int(xs[64 + ((2 * T + 1) & 7)]);
-                const int prod = mn0 * s0 + mn1 * s1;
-                acc_m[t] = __builtin_fmaf(dm, float(prod), acc_m[t]);
-            }
+        // software pipeline over super-blocks, two pairs deep; ascending order is kept
+        SuperRegs ra, rb, rc, rd;
+        load_super(ra, tile, 0, r, lane);
+        if (n_sb > 1) load_super(rb, tile, 1, r, lane);
+        for (uint32_t sb = 0; sb < n_sb; sb += 4) {
+            if (sb + 2 < n_sb) load_super(rc, tile, sb + 2, r, lane);
+            if (sb + 3 < n_sb) load_super(rd, tile, sb + 3, r, lane);
+            super_fma<B>(acc, acc_m, ra, lds_dw, n_sb, sb, T);
+            if (sb + 1 < n_sb) super_fma<B>(acc, acc_m, rb, lds_dw, n_sb, sb + 1, T);
+            if (sb + 4 < n_sb) load_super(ra, tile, sb + 4, r, lane);
+            if (sb + 5 < n_sb) load_super(rb, tile, sb + 5, r, lane);
+            if (sb + 2 < n_sb) super_fma<B>(acc, acc_m, rc, lds_dw, n_sb, sb + 2, T);
+            if (sb + 3 < n_sb) super_fma<B>(acc, acc_m, rd, lds_dw, n_sb, sb + 3, T);
         }
-        const uint32_t row = (tile0 + k) * kTileRows + r;
+        const uint32_t row = (p.tile0 + k) * kTileRows + r;
+        gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
 #pragma unroll
         for (int t = 0; t < B; t++) {
             const float main_val = hsum8_lanes(acc[t]);
             float m = acc_m[t];  // lanes T<4 hold acc_m[T]
             m = m + __shfl_xor(m, 2, 64);
             m = m + __shfl_xor(m, 1, 64);
-            if (T == 0 && row >= row_start && row < row_end) y[size_t(t) * y_stride + row] = main_val + m;
+            if (T == 0 && row >= p.row_start && row < p.row_end) yp[size_t(t) * p.y_stride + row] = main_val + m;
         }
     }
 }
@@ -248,19 +303,36 @@ __global__ __launch_bounds__(64) void q4_k_dequant_dot_kernel(const uint8_t *__r
 }
 
 template <int B>
-int launch_gemv_q4k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
-                    uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s) {
-    const uint32_t tile0 = row_start / kTileRows;
-    const uint32_t n_tiles = (row_end + kTileRows - 1) / kTileRows - tile0;
-    const size_t lds_bytes = size_t(B) * w->n_units * kSbDwords * 4;
+int launch_gemv_q4k(const RmiQ4kProblem *single, const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_waves,
+                    uint32_t tiles_per_wave, uint32_t max_n_sb, hipStream_t s) {
+    const size_t lds_bytes = size_t(B) * max_n_sb * kSbDwords * 4;
     if (lds_bytes > 64 * 1024)
-        return rmi_fail(RMI_HIP_E_INVALID, "activation of %d tokens x %u elements does not fit the LDS staging", B, w->n_in);
-    uint32_t n_waves = uint32_t(rmi_device_cus()) * 16;
-    if (n_waves > n_tiles) n_waves = n_tiles;
-    hipLaunchKernelGGL(gemv_q4_k_kernel<B>, dim3(n_waves), dim3(64), lds_bytes, s, w->data, d, qs, bsums, y, w->n_in,
-                       w->n_units, y_stride, row_start, row_end, tile0, n_tiles, n_waves);
+        return rmi_fail(RMI_HIP_E_INVALID, "activation of %d tokens x %u elements does not fit the LDS staging", B,
+                        max_n_sb * 256);
+    if (single)
+        hipLaunchKernelGGL((gemv_q4_k_kernel<B, false>), dim3(n_waves), dim3(64), lds_bytes, s, *single, d_list, d_runs,
+                           tiles_per_wave);
+    else
+        hipLaunchKernelGGL((gemv_q4_k_kernel<B, true>), dim3(n_waves), dim3(64), lds_bytes, s, RmiQ4kProblem{}, d_list,
+                           d_runs, tiles_per_wave);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
+}
+
+int dispatch_q4k(uint32_t nt, const RmiQ4kProblem *single, const RmiQ4kProblem *d_list, const uint4 *d_runs,
+                 uint32_t n_waves, uint32_t tpw, uint32_t max_n_sb, hipStream_t s) {
+    if (n_waves == 0) return RMI_HIP_OK;
+    switch (nt) {
+        case 1: return launch_gemv_q4k<1>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        case 2: return launch_gemv_q4k<2>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        case 3: return launch_gemv_q4k<3>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        case 4: return launch_gemv_q4k<4>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        case 5: return launch_gemv_q4k<5>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        case 6: return launch_gemv_q4k<6>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        case 7: return launch_gemv_q4k<7>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        case 8: return launch_gemv_q4k<8>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        default: return rmi_fail(RMI_HIP_E_INVALID, "gemv takes 1..8 tokens per launch, got %u", nt);
+    }
 }
 
 }  // namespace
@@ -275,6 +347,32 @@ int rmi_launch_quantize_q8_k(const float *x, float *d, int8_t *qs, int16_t *bsum
     return RMI_HIP_OK;
 }
 
+// Tiles a wave takes in one run: about 16 tile-super-blocks (18 KiB of weights) per token.
+uint32_t rmi_q4k_tiles_per_wave(uint32_t n_sb, uint32_t launch_tiles, uint32_t n_tokens) {
+    const uint32_t target = 16 * (n_tokens ? n_tokens : 1);
+    uint32_t tpw = n_sb >= target ? 1 : target / (n_sb ? n_sb : 1);
+    const uint32_t fill = uint32_t(rmi_device_cus()) * 8;
+    while (tpw > 1 && launch_tiles / tpw < fill) tpw >>= 1;
+    return tpw ? tpw : 1;
+}
+
+RmiQ4kProblem rmi_make_q4k_problem(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums,
+                                   float *y, uint32_t y_stride, uint32_t row_start, uint32_t row_end) {
+    RmiQ4kProblem p{};
+    p.w = w->data;
+    p.q8d = d;
+    p.q8qs = qs;
+    p.q8bs = bsums;
+    p.y = y;
+    p.n_sb = w->n_units;
+    p.y_stride = y_stride;
+    p.row_start = row_start;
+    p.row_end = row_end;
+    p.tile0 = row_start / kTileRows;
+    p.n_tiles = row_end > row_start ? (row_end + kTileRows - 1) / kTileRows - p.tile0 : 0;
+    return p;
+}
+
 int rmi_launch_gemv_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s) {
     if (row_start >= row_end || n_tokens == 0 || w->n_units == 0) return RMI_HIP_OK;
@@ -285,24 +383,19 @@ int rmi_launch_gemv_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *
     const uint32_t n_sb = w->n_units;
     for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
         const uint32_t nt = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
-        const float *dt = d + size_t(t0) * n_sb;
-        const int8_t *qt = qs + size_t(t0) * w->n_in;
-        const int16_t *bt = bsums + size_t(t0) * (w->n_in / 16);
-        float *yt = y + size_t(t0) * y_stride;
-        int rc;
-        switch (nt) {
-            case 1: rc = launch_gemv_q4k<1>(w, dt, qt, bt, yt, y_stride, row_start, row_end, s); break;
-            case 2: rc = launch_gemv_q4k<2>(w, dt, qt, bt, yt, y_stride, row_start, row_end, s); break;
-            case 3: rc = launch_gemv_q4k<3>(w, dt, qt, bt, yt, y_stride, row_start, row_end, s); break;
-            case 4: rc = launch_gemv_q4k<4>(w, dt, qt, bt, yt, y_stride, row_start, row_end, s); break;
-            case 5: rc = launch_gemv_q4k<5>(w, dt, qt, bt, yt, y_stride, row_start, row_end, s); break;
-            case 6: rc = launch_gemv_q4k<6>(w, dt, qt, bt, yt, y_stride, row_start, row_end, s); break;
-            case 7: rc = launch_gemv_q4k<7>(w, dt, qt, bt, yt, y_stride, row_start, row_end, s); break;
-            default: rc = launch_gemv_q4k<8>(w, dt, qt, bt, yt, y_stride, row_start, row_end, s); break;
-        }
+        RmiQ4kProblem p = rmi_make_q4k_problem(w, d + size_t(t0) * n_sb, qs + size_t(t0) * w->n_in,
+                                               bsums + size_t(t0) * (w->n_in / 16), y + size_t(t0) * y_stride, y_stride,
+                                               row_start, row_end);
+        const uint32_t tpw = rmi_q4k_tiles_per_wave(n_sb, p.n_tiles, nt);
+        int rc = dispatch_q4k(nt, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, tpw, n_sb, s);
         if (rc != RMI_HIP_OK) return rc;
     }
     return RMI_HIP_OK;
+}
+
+int rmi_launch_gemv_q4_k_group(const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t max_n_sb,
+                               uint32_t n_tokens, hipStream_t s) {
+    return dispatch_q4k(n_tokens, nullptr, d_list, d_runs, n_runs, 0, max_n_sb, s);
 }
 
 int rmi_launch_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *qs, const int16_t *bsums, int32_t *isum,

@@ -109,7 +109,7 @@ int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipS
 // d_runs[w] = {problem index, first tile, tile count, 0}: the run of tiles wave w takes
 int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t max_n_oct,
                                uint32_t n_tokens, hipStream_t s);
-uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles);
+uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles, uint32_t n_tokens);
 int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s);
 int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s);
 int rmi_launch_quantize_q8_0(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
@@ -120,6 +120,24 @@ int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const floa
 
 int rmi_launch_quantize_q8_k(const float *x, float *d, int8_t *qs, int16_t *bsums, uint32_t n_tokens, uint32_t n_in,
                              hipStream_t s);
+struct RmiQ4kProblem {
+    const uint8_t *w;     // Q4_K tile stream
+    const float *q8d;     // Q8_K activation: d[n_tokens][n_sb]
+    const int8_t *q8qs;   //                  qs[n_tokens][n_in]
+    const int16_t *q8bs;  //                  bsums[n_tokens][n_in/16]
+    float *y;             // y[t*y_stride + row]
+    uint32_t n_sb;
+    uint32_t y_stride;
+    uint32_t row_start;
+    uint32_t row_end;
+    uint32_t tile0;
+    uint32_t n_tiles;
+};
+RmiQ4kProblem rmi_make_q4k_problem(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums,
+                                   float *y, uint32_t y_stride, uint32_t row_start, uint32_t row_end);
+uint32_t rmi_q4k_tiles_per_wave(uint32_t n_sb, uint32_t launch_tiles, uint32_t n_tokens);
+int rmi_launch_gemv_q4_k_group(const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t max_n_sb,
+                               uint32_t n_tokens, hipStream_t s);
 int rmi_launch_gemv_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s);
 int rmi_launch_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *qs, const int16_t *bsums, int32_t *isum,
@@ -129,3 +147,14 @@ int rmi_launch_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *qs, const 
 int rmi_launch_q4_k_dequant_dot(const rmi_hip_weight *w, const float *x_f32, const int8_t *x_q8,
                                 const float *x_scales, float *y, uint32_t row_start, uint32_t row_end, int mode,
                                 hipStream_t s);
+
+// A fixed list of independent GEMVs (Q8_0 or Q4_K) launched as one kernel.
+struct rmi_hip_gemv_group {
+    int dtype = 0;
+    void *d_list = nullptr;  // RmiGemvProblem[] or RmiQ4kProblem[]
+    uint4 *d_runs = nullptr;
+    uint32_t n_problems = 0;
+    uint32_t n_runs = 0;
+    uint32_t max_units = 0;
+    uint32_t n_tokens = 0;
+};

@@ -136,6 +136,47 @@ def test_q4k_forward_batched(hip, oracle, n_tokens):
 
 # ----------------------------------------------------------------- dequant paths
 
+def test_q4k_grouped_launch_bit_exact(hip, oracle):
+    """One launch over a list of independent Q4_K x Q8_K GEMVs of mixed shapes, 1, 3 and 8 tokens."""
+    H, K = hip.hip, hip.kernel
+    shapes = [(1536, 1024), (1024, 1536), (37, 256), (6144, 2048), (2048, 6144), (9, 512)]
+    for n_tokens in (1, 3, 8):
+        kernels, bufs, refs = [], [], []
+        for i, (n_out, n_in) in enumerate(shapes):
+            w = hip.synth.q4_k_weight(300 + i, n_out, n_in)
+            x = hip.synth.activations(320 + 10 * n_tokens + i, n_tokens, n_in)
+            q = [oracle.quantize_row_q8_k(x[t], A) for t in range(n_tokens)]
+            ref = np.zeros((n_tokens, n_out), np.float32)
+            for t, (d, qs, bs) in enumerate(q):
+                oracle.q4k_forward_prepared(w, d, qs, bs, ref[t], n_in, n_out, 0, 1, A)
+            refs.append(ref)
+            kernels.append(K.Q4_KKernel(w, n_in, n_out))
+            bufs.append((H.DeviceBuffer.from_array(np.stack([t[0] for t in q])),
+                         H.DeviceBuffer.from_array(np.stack([t[1] for t in q])),
+                         H.DeviceBuffer.from_array(np.stack([t[2] for t in q])),
+                         H.DeviceBuffer(n_tokens * n_out * 4)))
+        n = len(shapes)
+        arr = lambda vals: (H.C.c_void_p * n)(*vals)  # noqa: E731
+        g = H.lib.rmi_hip_gemv_group_create_q4_k(n, arr([k.w.handle for k in kernels]), arr([b[0].ptr for b in bufs]),
+                                                 arr([b[1].ptr for b in bufs]), arr([b[2].ptr for b in bufs]),
+                                                 arr([b[3].ptr for b in bufs]), n_tokens)
+        assert g, H.last_error()
+        for _ in range(2):
+            H.check(H.lib.rmi_hip_gemv_group_run_dev(g, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        for i, (n_out, _) in enumerate(shapes):
+            got = bufs[i][3].to_array(np.float32, (n_tokens, n_out))
+            assert np.array_equal(bits(got), bits(refs[i])), (n_tokens, i)
+        H.lib.rmi_hip_gemv_group_destroy(g)
+    # a Q8_0 handle in a Q4_K group is refused
+    k8 = K.Q8Kernel(gen.make_q8_0_weight(4, 256, 0), 256, 4)
+    one = lambda v: (H.C.c_void_p * 1)(v)  # noqa: E731
+    p = bufs[0]
+    assert not H.lib.rmi_hip_gemv_group_create_q4_k(1, one(k8.w.handle), one(p[0].ptr), one(p[1].ptr), one(p[2].ptr),
+                                                    one(p[3].ptr), 1)
+    assert "bad weight handle" in H.last_error()
+
+
 def test_q4_k_kernel_multiplies_uniform_block(hip):
     """tests/quantized_inference.rs:233-249."""
     w = np.zeros(144, np.uint8)
