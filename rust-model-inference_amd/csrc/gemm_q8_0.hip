@@ -1,152 +1,159 @@
-// Q8_0 x Q8_0 prefill GEMM on int8 MFMA: Y[t][n] = sum_b (f32(wd[n][b]) * xs[t][b]) * dot_b(W[n], X[t]).
+// Q8_0 x Q8_0 prefill GEMM on the matrix cores: Y[t][n] = sum_b (f32(wd[n][b]) * xs[t][b]) * dot_b(W[n], X[t]).
 //
-// One 32x32x32 MFMA is one Q8_0 block (K = 32) of a 32-token x 32-row tile, so
-// the int32 accumulator is the per-block dot and starts from zero every block.
-// f32 order: acc = fma(float(dot), wd*xs, acc), blocks in sequence — the order
-// of matmul_q8_0_vs_q8_0_neon (src/ops/kernel/q8_0/neon.rs:49-73).
+// One 32x32x32 int8 MFMA is one Q8_0 block (K = 32) of a 32-token x 32-row
+// tile, so its int32 result is the per-block dot and starts from zero every
+// block.  The f32 scale products wd*xs of the same tile are a rank-1 outer
+// product, which v_mfma_f32_32x32x1_2b_f32 delivers in the accumulator layout
+// of the int8 result, two blocks per instruction (lanes 0-31 feed the first
+// block, lanes 32-63 the second); a single product plus zero is the correctly
+// rounded f32 product, subnormals included.  What is left for the VALU is
+// acc = fma(float(dot), scale, acc) with the blocks in sequence: the order of
+// matmul_q8_0_vs_q8_0_neon (src/ops/kernel/q8_0/neon.rs:49-73), bit for bit.
 //
 // Workgroup = 4 waves (2 x 2); wave (wn, wt) owns NTW x TTW MFMA tiles, i.e.
-// 32*NTW weight rows x 32*TTW tokens.  The launcher picks the largest tile that
-// still gives every SIMD about two waves.  Per quad (4 blocks,
-// 128 k) the workgroup stages into LDS, through registers so that the global
-// loads of the next DEPTH quads fly while quad q is multiplied:
-//   Ws  128 rows x 128 B, straight from the GEMV tile stream (quad order),
-//   Xs  TILE_T tokens x 128 B in natural order,
-//   wd  128 rows x 4 f32, xs 4 blocks x TILE_T f32 in accumulator order.
-// MFMA lane (c, h) supplies 16 of the 32 k values of its row/column; which 16
-// is free as long as both operands agree.  The 64 bytes at Ws[row][64h..] hold
-// the slices L = 4h..4h+3 of the row's quad: dword j of each 16-byte piece is
-// k = 16h+4L'..+3 of block j, i.e. bytes 16h..16h+15 of that block in the
-// natural activation order, which is what Xs[token][32j+16h..] holds.  Rows of
-// both LDS tiles are 144 B apart so that 16-byte reads of 8 consecutive lanes
-// fall into 8 different bank groups.
+// 32*NTW weight rows x 32*TTW tokens.  Per quad (4 blocks, 128 k) the
+// workgroup stages both int8 operands into LDS in the natural k order, 128
+// bytes a row, rows 144 bytes apart so that the 16-byte reads of 8 consecutive
+// lanes fall into 8 different bank groups.  Weights come from the GEMV tile
+// stream, whose 16-byte pieces hold the 4-byte slice L of blocks 0..3: each
+// piece is written back as four dwords, one into each block of the row.  LDS is
+// double-buffered (one barrier per quad) and the global loads of the next quad
+// stay in registers while the current one is multiplied.  MFMA lane (c, h)
+// reads bytes 16h..16h+15 of block j of its row / token for both operands.
+// The scales go from global memory straight into the lanes that feed the
+// outer-product MFMA.
 //
-// The f32 rescale is 3 VALU instructions per output per block (convert,
-// scale product, fma) against 32 MFMA cycles per 1024 outputs: the kernel is
-// bound by the VALU at about 1/6 of the int8 MFMA peak.
+// Per 32x32 tile and block the VALU issues 32 instructions (convert, fma;
+// 128 cycles) and the f32 outer product, which unlike the int8 MFMA does not
+// overlap with VALU work, holds the SIMD for about 32 more: the rescale bounds
+// the kernel at roughly a fifth of the int8 MFMA peak (measured: 958 TOP/s for
+// the multiply loop alone, with operands held in registers).
 #include "rmi_internal.h"
 
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v32f __attribute__((ext_vector_type(32)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kRowStride = 144;  // bytes between rows of Ws / Xs
+constexpr int kRowStride = 144;  // bytes between rows of the LDS tiles
 
 __device__ __forceinline__ float h2f(uint32_t bits16) {
     return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
 }
 
-template <int NTW, int TTW>  // 32-row and 32-token sub-tiles per wave
+// NTW x TTW 32x32 sub-tiles per wave, WN x WT waves per workgroup
+template <int NTW, int TTW, int WN, int WT>
 struct GemmSmem {
-    static constexpr int kTileN = 64 * NTW;
-    static constexpr int kTileT = 64 * TTW;
-    alignas(16) uint8_t ws[kTileN * kRowStride];
-    alignas(16) uint8_t xs_q[kTileT * kRowStride];
-    alignas(16) float wd[kTileN * 4];
-    alignas(16) float xs[4 * kTileT];  // [block j][32-token tile][h][16]
+    static constexpr int kTileN = 32 * NTW * WN;
+    static constexpr int kTileT = 32 * TTW * WT;
+    alignas(16) uint8_t ws[2][kTileN * kRowStride];
+    alignas(16) uint8_t xq[2][kTileT * kRowStride];
 };
 
-// DEPTH = quads whose global loads are in flight (held in registers) ahead of the multiply
-template <int NTW, int TTW, int DEPTH>
-__global__ __launch_bounds__(256) void gemm_q8_0_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ x_q8,
+template <int NTW, int TTW, int WN, int WT, int DEPTH>
+__global__ __launch_bounds__(64 * WN * WT) void gemm_q8_0_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ x_q8,
                                                          const float *__restrict__ x_scales, float *__restrict__ y,
                                                          uint32_t n_out, uint32_t n_in, uint32_t n_oct,
                                                          uint32_t n_tiles, uint32_t n_tokens, uint32_t y_stride) {
-    constexpr int kTileN = 64 * NTW, kTileT = 64 * TTW;
-    constexpr int kWPieces = kTileN * 8 / 256;  // 16-byte pieces of Ws per thread
-    constexpr int kXPieces = kTileT * 8 / 256;  // 16-byte pieces of Xs per thread
-    __shared__ GemmSmem<NTW, TTW> sm;
+    constexpr int kThreads = 64 * WN * WT;
+    constexpr int kTileN = 32 * NTW * WN, kTileT = 32 * TTW * WT;
+    constexpr int kWPieces = kTileN * 8 / kThreads;  // 16-byte pieces of the weight tile per thread
+    constexpr int kXPieces = kTileT * 8 / kThreads;  // 16-byte pieces of the token tile per thread
+    static_assert(kWPieces * kThreads == kTileN * 8 && kXPieces * kThreads == kTileT * 8, "tile must split evenly");
+    __shared__ GemmSmem<NTW, TTW, WN, WT> sm;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 31, h = lane >> 5;
-    const uint32_t n_off = (wave & 1) * 32 * NTW, t_off = (wave >> 1) * 32 * TTW;
+    const uint32_t n_off = (wave % WN) * 32 * NTW, t_off = (wave / WN) * 32 * TTW;
     const uint32_t n0 = blockIdx.x * kTileN, t0 = blockIdx.y * kTileT;
     const uint32_t nb = n_in >> 5, n_quads = (nb + 3) >> 2;
 
-    // --- what this thread stages per quad
-    // Ws: pieces p = tid + 256 i -> row p>>3, piece p&7
-    const uint8_t *w_src[kWPieces];
-    uint32_t w_dst[kWPieces];
+    // --- int8 staging: pieces p = tid + kThreads i -> row p>>3, piece p&7
+    // Addresses are a workgroup-uniform base plus a 32-bit offset per thread.
+    const uint32_t tile_first = (n0 >> 3) < n_tiles ? (n0 >> 3) : n_tiles - 1;
+    const uint8_t *w_base = w + size_t(tile_first) * n_oct * kOctetBytes;
+    uint32_t w_off[kWPieces], w_dst[kWPieces];
 #pragma unroll
     for (int i = 0; i < kWPieces; i++) {
-        const uint32_t p = tid + 256 * i, row = p >> 3, L = p & 7;
+        const uint32_t p = tid + kThreads * i, row = p >> 3, L = p & 7;
         uint32_t tile = (n0 + row) >> 3;
         if (tile >= n_tiles) tile = n_tiles - 1;  // rows past the padded stream: stay in bounds, never stored
-        w_src[i] = w + size_t(tile) * n_oct * kOctetBytes + size_t(n_oct) * 128 + ((n0 + row) & 7) * 128 + L * 16;
-        w_dst[i] = row * kRowStride + L * 16;
+        w_off[i] = (tile - tile_first) * n_oct * kOctetBytes + n_oct * 128 + ((n0 + row) & 7) * 128 + L * 16;
+        w_dst[i] = row * kRowStride + L * 4;
     }
-    // Xs: pieces p -> token p>>3, piece p&7
-    const int8_t *x_src[kXPieces];
-    uint32_t x_dst[kXPieces];
-    bool x_ok[kXPieces];
+    // Tokens past n_tokens and, in the last quad, pieces past n_in are multiplied like the rest: their
+    // products meet zero weight quants or are never stored.  Only the addresses are kept inside the buffer.
+    const int8_t *x_base = x_q8 + size_t(t0) * n_in;
+    const uint64_t x_room = uint64_t(n_tokens - t0) * n_in - 16;
+    const uint32_t x_lim = x_room < 0xfffffff0ull ? uint32_t(x_room) : 0xfffffff0u;
+    uint32_t x_off[kXPieces], x_dst[kXPieces];
 #pragma unroll
     for (int i = 0; i < kXPieces; i++) {
-        const uint32_t p = tid + 256 * i, tok = p >> 3, piece = p & 7;
-        x_ok[i] = t0 + tok < n_tokens;
-        x_src[i] = x_q8 + size_t(x_ok[i] ? t0 + tok : 0) * n_in + piece * 16;
+        const uint32_t p = tid + kThreads * i, tok = p >> 3, piece = p & 7;
+        x_off[i] = tok * n_in + piece * 16;
         x_dst[i] = tok * kRowStride + piece * 16;
     }
-    // wd: threads 0..127, one row each (4 f16 of the quad)
-    const uint8_t *wd_src = nullptr;
-    if (tid < kTileN) {
-        uint32_t tile = (n0 + tid) >> 3;
-        if (tile >= n_tiles) tile = n_tiles - 1;
-        wd_src = w + size_t(tile) * n_oct * kOctetBytes + ((n0 + tid) & 7) * 16;
-    }
-    // xs: element e = tid + 256 i of 4*kTileT -> block j = e / kTileT, token e % kTileT
-    constexpr int kXsPer = 4 * kTileT / 256;
-    const float *xs_src[kXsPer];
-    uint32_t xs_dst[kXsPer], xs_j[kXsPer];
-    bool xs_ok[kXsPer];
+    // --- scales of this lane: blocks h and 2+h of the quad, of row / token c of each sub-tile
+    uint32_t wd_off[NTW];
 #pragma unroll
-    for (int i = 0; i < kXsPer; i++) {
-        const uint32_t e = tid + 256 * i, j = e / kTileT, tok = e % kTileT;
-        const uint32_t tt = tok >> 5, within = tok & 31;
-        const uint32_t hh = (within >> 2) & 1, idx = ((within >> 3) << 2) | (within & 3);
-        xs_ok[i] = t0 + tok < n_tokens;
-        xs_src[i] = x_scales + size_t(xs_ok[i] ? t0 + tok : 0) * nb;
-        xs_j[i] = j;
-        xs_dst[i] = ((j * (kTileT / 32) + tt) * 2 + hh) * 16 + idx;
+    for (int nt = 0; nt < NTW; nt++) {
+        const uint32_t row = n0 + n_off + nt * 32 + c;
+        uint32_t tile = row >> 3;
+        if (tile >= n_tiles) tile = n_tiles - 1;
+        wd_off[nt] = (tile - tile_first) * n_oct * kOctetBytes + (row & 7) * 16;
+    }
+    const float *xs_base = x_scales + size_t(t0) * nb;
+    uint32_t xs_off[TTW];
+#pragma unroll
+    for (int tt = 0; tt < TTW; tt++) {
+        const uint32_t tok = t_off + tt * 32 + c;
+        xs_off[tt] = (tok < n_tokens - t0 ? tok : n_tokens - t0 - 1) * nb;
     }
 
     struct Stage {
         u32x4 w[kWPieces], x[kXPieces];
-        u32x2 wd;
-        float xs[kXsPer];
     };
-    Stage st[DEPTH];
-
+    struct Scales {  // as loaded: the four f16 weight scales of the quad, the two f32 token scales of this lane
+        u32x2 wd[NTW];
+        float xs[TTW][2];
+    };
     auto load_quad = [&](Stage &g, uint32_t q) {
 #pragma unroll
-        for (int i = 0; i < kWPieces; i++) g.w[i] = *reinterpret_cast<const u32x4 *>(w_src[i] + size_t(q) * 1024);
+        for (int i = 0; i < kWPieces; i++) g.w[i] = *reinterpret_cast<const u32x4 *>(w_base + (w_off[i] + q * 1024));
 #pragma unroll
         for (int i = 0; i < kXPieces; i++) {
-            // the last quad of a row may hold fewer than 4 blocks: pieces beyond n_in read as zero
-            const bool in_row = q * 128 + (tid & 7) * 16 < n_in;
-            g.x[i] = (x_ok[i] && in_row) ? *reinterpret_cast<const u32x4 *>(x_src[i] + size_t(q) * 128) : u32x4{0, 0, 0, 0};
-        }
-        g.wd = u32x2{0, 0};
-        if (tid < kTileN) g.wd = *reinterpret_cast<const u32x2 *>(wd_src + size_t(q >> 1) * 128 + (q & 1) * 8);
-#pragma unroll
-        for (int i = 0; i < kXsPer; i++) {
-            const uint32_t b = q * 4 + xs_j[i];
-            g.xs[i] = (xs_ok[i] && b < nb) ? xs_src[i][b] : 0.0f;
+            const uint32_t off = x_off[i] + q * 128;
+            g.x[i] = *reinterpret_cast<const u32x4 *>(x_base + (off < x_lim ? off : x_lim));
         }
     };
-    auto store_quad = [&](const Stage &g) {
+    auto store_quad = [&](const Stage &g, uint32_t buf) {
 #pragma unroll
-        for (int i = 0; i < kWPieces; i++) *reinterpret_cast<u32x4 *>(sm.ws + w_dst[i]) = g.w[i];
-#pragma unroll
-        for (int i = 0; i < kXPieces; i++) *reinterpret_cast<u32x4 *>(sm.xs_q + x_dst[i]) = g.x[i];
-        if (tid < kTileN) {
-            float4 f = make_float4(h2f(g.wd.x & 0xffffu), h2f(g.wd.x >> 16), h2f(g.wd.y & 0xffffu), h2f(g.wd.y >> 16));
-            *reinterpret_cast<float4 *>(sm.wd + tid * 4) = f;
+        for (int i = 0; i < kWPieces; i++) {
+            uint8_t *dst = sm.ws[buf] + w_dst[i];
+            *reinterpret_cast<uint32_t *>(dst) = g.w[i].x;
+            *reinterpret_cast<uint32_t *>(dst + 32) = g.w[i].y;
+            *reinterpret_cast<uint32_t *>(dst + 64) = g.w[i].z;
+            *reinterpret_cast<uint32_t *>(dst + 96) = g.w[i].w;
         }
 #pragma unroll
-        for (int i = 0; i < kXsPer; i++) sm.xs[xs_dst[i]] = g.xs[i];
+        for (int i = 0; i < kXPieces; i++) *reinterpret_cast<u32x4 *>(sm.xq[buf] + x_dst[i]) = g.x[i];
+    };
+    auto load_scales = [&](Scales &sc, uint32_t q) {
+        // weight scales of padded blocks are zero in the stream; token scales beyond n_in/32 are not there
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) {
+            sc.wd[nt] = *reinterpret_cast<const u32x2 *>(w_base + (wd_off[nt] + (q >> 1) * 128 + (q & 1) * 8));
+        }
+#pragma unroll
+        for (int tt = 0; tt < TTW; tt++) {
+            // past n_in/32 the last scale of the row is read instead; the consumer replaces it by zero
+            const uint32_t b = q * 4 + h;
+            sc.xs[tt][0] = xs_base[xs_off[tt] + (b < nb ? b : nb - 1)];
+            sc.xs[tt][1] = xs_base[xs_off[tt] + (b + 2 < nb ? b + 2 : nb - 1)];
+        }
     };
 
     float acc[NTW][TTW][16];
@@ -157,67 +164,84 @@ __global__ __launch_bounds__(256) void gemm_q8_0_kernel(const uint8_t *__restric
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[nt][tt][i] = 0.0f;
 
+    // Rings of DEPTH quads: the global loads of quad k wait in registers slot k % DEPTH (scales for DEPTH
+    // iterations, int8 pieces for DEPTH - 1: they move to LDS one iteration before they are multiplied).
+    Stage st[DEPTH];
+    Scales sc[DEPTH];
+    if (n_quads > 0) {
+        load_quad(st[0], 0);
+        store_quad(st[0], 0);
+    }
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++)
-        if (uint32_t(d) < n_quads) load_quad(st[d], d);
+    for (int k = 0; k < DEPTH; k++)
+        if (uint32_t(k) < n_quads) load_scales(sc[k], k);
+#pragma unroll
+    for (int k = 1; k <= DEPTH; k++)
+        if (uint32_t(k) < n_quads) load_quad(st[k % DEPTH], k);
     for (uint32_t q0 = 0; q0 < n_quads; q0 += DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; d++) {
         const uint32_t q = q0 + d;
         if (q >= n_quads) break;
-        __syncthreads();  // everyone is done reading the previous quad
-        store_quad(st[d]);
-        __syncthreads();
-        if (q + DEPTH < n_quads) load_quad(st[d], q + DEPTH);
-
-        v4i wj[NTW][4];
-        float wdv[NTW][4];
+        const uint32_t buf = q & 1;
+        __syncthreads();  // quad q is in sm.*[buf]; nobody reads the other buffer any more
+        float wd_cur[NTW][2], xs_cur[TTW][2];
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++) {
-            const uint32_t row = n_off + nt * 32 + c;
-            const u32x4 *wp = reinterpret_cast<const u32x4 *>(sm.ws + row * kRowStride + h * 64);
-            const u32x4 u0 = wp[0], u1 = wp[1], u2 = wp[2], u3 = wp[3];
-            wj[nt][0] = v4i{int(u0.x), int(u1.x), int(u2.x), int(u3.x)};
-            wj[nt][1] = v4i{int(u0.y), int(u1.y), int(u2.y), int(u3.y)};
-            wj[nt][2] = v4i{int(u0.z), int(u1.z), int(u2.z), int(u3.z)};
-            wj[nt][3] = v4i{int(u0.w), int(u1.w), int(u2.w), int(u3.w)};
-            const float4 f = *reinterpret_cast<const float4 *>(sm.wd + row * 4);
-            wdv[nt][0] = f.x;
-            wdv[nt][1] = f.y;
-            wdv[nt][2] = f.z;
-            wdv[nt][3] = f.w;
+            wd_cur[nt][0] = h2f((sc[d].wd[nt].x >> (16 * h)) & 0xffffu);
+            wd_cur[nt][1] = h2f((sc[d].wd[nt].y >> (16 * h)) & 0xffffu);
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            // blocks past n_in/32 in the last quad are all-zero on both sides (scale 0, quants 0):
-            // fma(float(0), 0, acc) leaves acc unchanged, so they are multiplied like the rest
-            {
+        for (int tt = 0; tt < TTW; tt++) {
+            // a scale past n_in/32 must be a true zero: its block's dot is zero and the product must not be NaN
+            xs_cur[tt][0] = q * 4 + h < nb ? sc[d].xs[tt][0] : 0.0f;
+            xs_cur[tt][1] = q * 4 + h + 2 < nb ? sc[d].xs[tt][1] : 0.0f;
+        }
+        if (q + DEPTH < n_quads) load_scales(sc[d], q + DEPTH);
+        if (q + 1 < n_quads) {
+            store_quad(st[(d + 1) % DEPTH], buf ^ 1);
+            if (q + 1 + DEPTH < n_quads) load_quad(st[(d + 1) % DEPTH], q + 1 + DEPTH);
+        }
+        const uint8_t *wrow[NTW], *xrow[TTW];
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) wrow[nt] = sm.ws[buf] + (n_off + nt * 32 + c) * kRowStride + h * 16;
+#pragma unroll
+        for (int tt = 0; tt < TTW; tt++) xrow[tt] = sm.xq[buf] + (t_off + tt * 32 + c) * kRowStride + h * 16;
+#pragma unroll
+        for (int p = 0; p < 2; p++) {  // blocks 2p and 2p+1 of the quad
+            v4i wv[NTW][2], xv[TTW][2];
+#pragma unroll
+            for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const u32x4 u = *reinterpret_cast<const u32x4 *>(wrow[nt] + (2 * p + e) * 32);
+                    wv[nt][e] = v4i{int(u.x), int(u.y), int(u.z), int(u.w)};
+                }
+#pragma unroll
+            for (int tt = 0; tt < TTW; tt++)
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const u32x4 u = *reinterpret_cast<const u32x4 *>(xrow[tt] + (2 * p + e) * 32);
+                    xv[tt][e] = v4i{int(u.x), int(u.y), int(u.z), int(u.w)};
+                }
+#pragma unroll
+            for (int nt = 0; nt < NTW; nt++)
 #pragma unroll
                 for (int tt = 0; tt < TTW; tt++) {
-                    const uint32_t tok = t_off + tt * 32 + c;
-                    const u32x4 xv = *reinterpret_cast<const u32x4 *>(sm.xs_q + tok * kRowStride + j * 32 + h * 16);
-                    const v4i a = v4i{int(xv.x), int(xv.y), int(xv.z), int(xv.w)};
-                    const float4 *xs4 =
-                        reinterpret_cast<const float4 *>(sm.xs + ((j * (kTileT / 32) + (t_off >> 5) + tt) * 2 + h) * 16);
-                    float s[16];
+                    // blocks past n_in/32 in the last quad are zero on both sides (scale 0, quants 0):
+                    // fma(float(0), 0, acc) leaves acc unchanged, so they are multiplied like the rest
+                    v32f zero32;
 #pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        const float4 v = xs4[g];
-                        s[4 * g] = v.x;
-                        s[4 * g + 1] = v.y;
-                        s[4 * g + 2] = v.z;
-                        s[4 * g + 3] = v.w;
-                    }
+                    for (int i = 0; i < 32; i++) zero32[i] = 0.0f;
+                    const v32f s = __builtin_amdgcn_mfma_f32_32x32x1f32(xs_cur[tt][p], wd_cur[nt][p], zero32, 0, 0, 0);
+                    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    const v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xv[tt][0], wv[nt][0], zero16, 0, 0, 0);
+                    const v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(xv[tt][1], wv[nt][1], zero16, 0, 0, 0);
 #pragma unroll
-                    for (int nt = 0; nt < NTW; nt++) {
-                        v16i d = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                        d = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, wj[nt][j], d, 0, 0, 0);
+                    for (int i = 0; i < 16; i++) acc[nt][tt][i] = __builtin_fmaf(float(d0[i]), s[i], acc[nt][tt][i]);
 #pragma unroll
-                        for (int i = 0; i < 16; i++)
-                            acc[nt][tt][i] = __builtin_fmaf(float(d[i]), wdv[nt][j] * s[i], acc[nt][tt][i]);
-                    }
+                    for (int i = 0; i < 16; i++) acc[nt][tt][i] = __builtin_fmaf(float(d1[i]), s[16 + i], acc[nt][tt][i]);
                 }
-            }
         }
       }
     }
@@ -237,12 +261,13 @@ __global__ __launch_bounds__(256) void gemm_q8_0_kernel(const uint8_t *__restric
     }
 }
 
-template <int NTW, int TTW, int DEPTH>
-void launch_gemm(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
-                        uint32_t n_tokens, uint32_t y_stride, hipStream_t s) {
-    dim3 grid((w->n_out + 64 * NTW - 1) / (64 * NTW), (n_tokens + 64 * TTW - 1) / (64 * TTW));
-    hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, DEPTH>), grid, dim3(256), 0, s, w->data, x_q8, x_scales, y, w->n_out,
-                       w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride);
+template <int NTW, int TTW, int WN, int WT, int DEPTH>
+void launch_gemm(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
+                 uint32_t y_stride, hipStream_t s) {
+    constexpr uint32_t tile_n = 32 * NTW * WN, tile_t = 32 * TTW * WT;
+    dim3 grid((w->n_out + tile_n - 1) / tile_n, (n_tokens + tile_t - 1) / tile_t);
+    hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, DEPTH>), grid, dim3(64 * WN * WT), 0, s, w->data, x_q8, x_scales, y,
+                       w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride);
 }
 
 }  // namespace
@@ -250,17 +275,19 @@ void launch_gemm(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_sca
 int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                          uint32_t n_tokens, uint32_t y_stride, hipStream_t s) {
     if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
-    // the largest workgroup tile that still yields two workgroups (eight waves) per compute unit
-    const uint64_t want = uint64_t(rmi_device_cus()) * 2;
+    // Measured on MI355X: the 128x128 tile (4 waves, 2x2 sub-tiles each) is fastest once it yields two
+    // workgroups per compute unit; below that the 128x64 tile of 8 single-sub-tile waves, and for small
+    // problems the 64x64 tile of 4 waves, keep more SIMDs fed.  A deeper register ring (DEPTH > 1) did not pay.
+    const uint64_t cus = uint64_t(rmi_device_cus());
     auto groups = [&](uint32_t tn, uint32_t tt) {
         return uint64_t((w->n_out + tn - 1) / tn) * ((n_tokens + tt - 1) / tt);
     };
-    if (n_tokens > 64 && groups(128, 128) >= want)
-        launch_gemm<2, 2, 2>(w, x_q8, x_scales, y, n_tokens, y_stride, s);
-    else if (groups(128, 64) >= want)
-        launch_gemm<2, 1, 3>(w, x_q8, x_scales, y, n_tokens, y_stride, s);
+    if (groups(128, 128) >= 2 * cus)
+        launch_gemm<2, 2, 2, 2, 1>(w, x_q8, x_scales, y, n_tokens, y_stride, s);
+    else if (groups(128, 64) >= 2 * cus)
+        launch_gemm<1, 1, 4, 2, 1>(w, x_q8, x_scales, y, n_tokens, y_stride, s);
     else
-        launch_gemm<1, 1, 4>(w, x_q8, x_scales, y, n_tokens, y_stride, s);
+        launch_gemm<1, 1, 2, 2, 1>(w, x_q8, x_scales, y, n_tokens, y_stride, s);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }

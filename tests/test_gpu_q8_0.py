@@ -303,6 +303,44 @@ def test_gemm_mfma_parity(hip, oracle, n_tokens, n_out, n_in):
     assert np.all(np.abs(out - ref_a) <= TOL(ref_a))
 
 
+def test_gemm_special_scales(hip, oracle):
+    """Weight scales that are zero, negative zero, f16 subnormals, the largest f16, inf and NaN, against token
+    scales down to f32 subnormals: the scale products formed on the matrix cores must round like the f32 multiply."""
+    n_tokens, n_out, n_in = 96, 160, 320
+    rng = np.random.default_rng(77)
+    w = hip.synth.q8_0_weight(1234, n_out, n_in).reshape(n_out, n_in // 32, 34).copy()
+    special = np.array([0x0000, 0x8000, 0x0001, 0x83ff, 0x7bff, 0xfbff, 0x7c00, 0xfc00, 0x7e00, 0x0400, 0x3c00],
+                       np.uint16)
+    pick = rng.integers(0, special.size, (n_out, n_in // 32))
+    keep = rng.random((n_out, n_in // 32)) < 0.5
+    scales = w[:, :, :2].copy().view(np.uint16)[:, :, 0]
+    scales = np.where(keep, scales, special[pick]).astype(np.uint16)
+    w[:, :, :2] = scales[:, :, None].view(np.uint8)
+    w = np.ascontiguousarray(w).reshape(-1)
+    q8 = rng.integers(-127, 128, (n_tokens, n_in), dtype=np.int8)
+    sc = (rng.random((n_tokens, n_in // 32), dtype=np.float32) + 0.5) * \
+        np.float32(10.0) ** rng.integers(-44, 3, (n_tokens, n_in // 32)).astype(np.float32)
+    sc[rng.random(sc.shape) < 0.05] = 0.0
+    sc = sc.astype(np.float32)
+    H = hip.hip
+    kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
+    d_q8, d_sc = H.DeviceBuffer.from_array(q8), H.DeviceBuffer.from_array(sc)
+    d_y = H.DeviceBuffer(n_tokens * n_out * 4)
+    H.check(H.lib.rmi_hip_gemm_q8_0_dev(kernel.w.handle, d_q8.ptr, d_sc.ptr, d_y.ptr, n_tokens, n_out, None))
+    H.check(H.lib.rmi_hip_synchronize())
+    out = d_y.to_array(np.float32, (n_tokens, n_out))
+    with np.errstate(all="ignore"):
+        ref = np.stack([oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, N) for t in range(n_tokens)])
+    nan_o, nan_r = np.isnan(out), np.isnan(ref)
+    assert np.array_equal(nan_o, nan_r) and nan_r.any() and not nan_r.all()
+    assert np.array_equal(bits(out)[~nan_o], bits(ref)[~nan_r])
+    # subnormal scale products were exercised (f16 subnormal weight scale x tiny token scale)
+    wd = scales.view(np.float16).astype(np.float32)
+    with np.errstate(all="ignore"):
+        prod = wd[:, None, :] * sc[None, :, :]
+    assert np.count_nonzero((prod != 0) & (np.abs(prod) < 1.17549435e-38)) > 1000
+
+
 def test_gemm_full_size_properties(hip, oracle):
     """M=2048 x (3072 x 1024): rows sampled against the checker; every token row equals
     the same token run through a 64-token call (tile position must not change bits)."""
