@@ -182,9 +182,9 @@ def cpu_baseline(problems, batch, alg_bytes):
     }, outs
 
 
-def read_traffic(mode):
-    """HBM bytes per launch measured with rocprofv3 --pmc, recorded under profiles/."""
-    path = os.path.join(ROOT, "profiles", f"gemv_q8_0_{mode}_qwen3_0.6b_pmc.txt")
+def read_traffic(name):
+    """HBM bytes per launch measured with rocprofv3 --pmc, recorded under profiles/<name>_pmc.txt."""
+    path = os.path.join(ROOT, "profiles", f"{name}_pmc.txt")
     try:
         for line in open(path):
             if line.startswith("traffic_bytes_per_launch:"):
@@ -192,6 +192,19 @@ def read_traffic(mode):
     except OSError:
         pass
     return None
+
+
+def copy_calibration(H, args):
+    """A plain copy kernel of known size, five launches: what rocprofv3 --pmc traffic counters are scaled against."""
+    if not args.copy_calibration_mb:
+        return
+    nbytes = args.copy_calibration_mb << 20
+    src, dst = H.DeviceBuffer(nbytes), H.DeviceBuffer(nbytes)
+    for _ in range(5):
+        H.check(H.lib.rmi_hip_copy_dev(dst.ptr, src.ptr, nbytes, None))
+    H.check(H.lib.rmi_hip_synchronize())
+    src.free()
+    dst.free()
 
 
 def time_region(H, ev, fn, steps, warmup):
@@ -244,14 +257,7 @@ def run_projection_set(args, pkg, ev):
     modes = {"grouped": (step_grouped, 1), "per_matmul": (step_per_matmul, len(problems)),
              "layer": (step_layer, len(groups_layer))}
 
-    if args.copy_calibration_mb:
-        nbytes = args.copy_calibration_mb << 20
-        src, dst = H.DeviceBuffer(nbytes), H.DeviceBuffer(nbytes)
-        for _ in range(5):
-            H.check(H.lib.rmi_hip_copy_dev(dst.ptr, src.ptr, nbytes, None))
-        H.check(H.lib.rmi_hip_synchronize())
-        src.free()
-        dst.free()
+    copy_calibration(H, args)
 
     fn, launches = modes[args.mode]
     wall, dev_ms = time_region(H, ev, fn, args.steps, args.warmup)
@@ -281,7 +287,7 @@ def run_projection_set(args, pkg, ev):
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
             "algorithmic_bytes_per_launch": round(alg_bytes / launches),
-            "traffic": read_traffic(args.mode) if batch == 1 else None,
+            "traffic": read_traffic(f"gemv_q8_0_{args.mode}_qwen3_0.6b") if batch == 1 else None,
         },
     })
 
@@ -335,6 +341,7 @@ def run_gemm(args, pkg, ev):
             H.check(H.lib.rmi_hip_gemm_q8_0_dev(r["k"].w.handle, r["d_q8"].ptr, r["d_sc"].ptr, r["d_y"].ptr, M,
                                                 r["n_out"], None))
 
+    copy_calibration(H, args)
     wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
     ops = sum(2.0 * M * r["n_in"] * r["n_out"] for r in recs)
     value = ops / wall / 1e12
@@ -346,7 +353,8 @@ def run_gemm(args, pkg, ev):
         "tokens": M, "launches_per_step": 2, "ops_per_step": ops, "device": dev_name.strip(), "compute_units": cus})
     result["roofline"] = {"bound": "mfma", "kernel": "gemm_q8_0_kernel", "achieved": round(achieved, 1), "peak": 5000.0,
                           "unit": "TOP/s", "frac": round(achieved / 5000.0, 4),
-                          "avg_launch_us": round(dev_ms * 1e3 / 2, 3), "traffic": None}
+                          "avg_launch_us": round(dev_ms * 1e3 / 2, 3),
+                          "traffic": read_traffic(f"gemm_q8_0_m{M}_qwen3_0.6b_ffn")}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
@@ -423,6 +431,7 @@ def run_q4k(args, pkg, ev):
     grouped = args.mode != "per_matmul"
     step = step_grouped if grouped else step_per_matmul
     launches = 1 if grouped else n
+    copy_calibration(H, args)
     wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
     alg = sum(synth.q4_k_gemv_bytes(r["n_out"], r["n_in"], batch) for r in recs)
     value = alg / wall / 1e9
@@ -436,7 +445,8 @@ def run_q4k(args, pkg, ev):
     result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_k_kernel<{batch}, {'true' if grouped else 'false'}>",
                           "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(achieved / HBM_PEAK_GBS, 4),
-                          "avg_launch_us": round(dev_ms * 1e3 / launches, 3), "traffic": None}
+                          "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
+                          "traffic": read_traffic("gemv_q4_k_grouped_1.7b_ffn") if grouped and batch == 1 else None}
     if not args.no_cpu_baseline and batch == 1:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle

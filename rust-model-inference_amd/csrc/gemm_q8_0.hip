@@ -57,7 +57,8 @@ template <int NTW, int TTW, int WN, int WT, int DEPTH>
 __global__ __launch_bounds__(64 * WN * WT) void gemm_q8_0_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ x_q8,
                                                          const float *__restrict__ x_scales, float *__restrict__ y,
                                                          uint32_t n_out, uint32_t n_in, uint32_t n_oct,
-                                                         uint32_t n_tiles, uint32_t n_tokens, uint32_t y_stride) {
+                                                         uint32_t n_tiles, uint32_t n_tokens, uint32_t y_stride,
+                                                         uint32_t grid_n, uint32_t grid_t, uint32_t t_fastest) {
     constexpr int kThreads = 64 * WN * WT;
     constexpr int kTileN = 32 * NTW * WN, kTileT = 32 * TTW * WT;
     constexpr int kWPieces = kTileN * 8 / kThreads;  // 16-byte pieces of the weight tile per thread
@@ -68,7 +69,14 @@ __global__ __launch_bounds__(64 * WN * WT) void gemm_q8_0_kernel(const uint8_t *
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 31, h = lane >> 5;
     const uint32_t n_off = (wave % WN) * 32 * NTW, t_off = (wave / WN) * 32 * TTW;
-    const uint32_t n0 = blockIdx.x * kTileN, t0 = blockIdx.y * kTileT;
+    // Workgroups are handed to the 8 XCDs round-robin, each XCD with its own L2.  Renumber them so that the
+    // workgroups of one XCD are consecutive tiles, running fastest along the smaller operand: every XCD then
+    // fetches that operand whole and only its own eighth of the larger one.
+    const uint32_t n_groups = grid_n * grid_t, lin = blockIdx.x;
+    const uint32_t xcd = lin & 7, slot = lin >> 3;
+    const uint32_t tile_id = xcd * (n_groups >> 3) + (xcd < (n_groups & 7) ? xcd : (n_groups & 7)) + slot;
+    const uint32_t n0 = (t_fastest ? tile_id / grid_t : tile_id % grid_n) * kTileN;
+    const uint32_t t0 = (t_fastest ? tile_id % grid_t : tile_id / grid_n) * kTileT;
     const uint32_t nb = n_in >> 5, n_quads = (nb + 3) >> 2;
 
     // --- int8 staging: pieces p = tid + kThreads i -> row p>>3, piece p&7
@@ -265,9 +273,10 @@ template <int NTW, int TTW, int WN, int WT, int DEPTH>
 void launch_gemm(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
                  uint32_t y_stride, hipStream_t s) {
     constexpr uint32_t tile_n = 32 * NTW * WN, tile_t = 32 * TTW * WT;
-    dim3 grid((w->n_out + tile_n - 1) / tile_n, (n_tokens + tile_t - 1) / tile_t);
-    hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, DEPTH>), grid, dim3(64 * WN * WT), 0, s, w->data, x_q8, x_scales, y,
-                       w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride);
+    const uint32_t grid_n = (w->n_out + tile_n - 1) / tile_n, grid_t = (n_tokens + tile_t - 1) / tile_t;
+    hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, DEPTH>), dim3(grid_n * grid_t), dim3(64 * WN * WT), 0, s,
+                       w->data, x_q8, x_scales, y, w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride, grid_n,
+                       grid_t, n_tokens < w->n_out ? 1u : 0u);
 }
 
 }  // namespace
@@ -282,6 +291,7 @@ int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const floa
     auto groups = [&](uint32_t tn, uint32_t tt) {
         return uint64_t((w->n_out + tn - 1) / tn) * ((n_tokens + tt - 1) / tt);
     };
+    if (groups(64, 64) > 0x7fffffffull) return rmi_fail(RMI_HIP_E_INVALID, "GEMM too large for one launch");
     if (groups(128, 128) >= 2 * cus)
         launch_gemm<2, 2, 2, 2, 1>(w, x_q8, x_scales, y, n_tokens, y_stride, s);
     else if (groups(128, 64) >= 2 * cus)
