@@ -126,6 +126,13 @@ def make_group(H, recs, batch):
     return g
 
 
+def group_maxt(H, g):
+    """Third template argument of the kernel a group launches: 64 (one wave per workgroup) or 512."""
+    wg, waves = C.c_uint32(), C.c_uint32()
+    H.check(H.lib.rmi_hip_gemv_group_shape(g, C.byref(wg), C.byref(waves)))
+    return "64" if waves.value == 1 else "512"
+
+
 def layer_groups(H, problems, batch):
     """[q,k,v] [o] [gate,up] [down] per layer, then lm_head: what a dependent decode step can fuse."""
     groups = []
@@ -280,7 +287,8 @@ def run_projection_set(args, pkg, ev):
         "gflops": round(flops / wall / 1e9, 1),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_q8_0_kernel<%d,%s>" % (batch, "true" if args.mode != "per_matmul" else "false"),
+            "kernel": "gemv_q8_0_kernel<%d,%s,%s>" % (batch, "true" if args.mode != "per_matmul" else "false",
+                                                       group_maxt(H, group_all) if args.mode == "grouped" else "*"),
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -442,7 +450,7 @@ def run_q4k(args, pkg, ev):
                     + ("one grouped launch" if grouped else "one launch per matrix"), "batch": batch,
         "launches_per_step": launches,
         "algorithmic_bytes_per_step": alg, "device": dev_name.strip(), "compute_units": cus})
-    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_k_kernel<{batch}, {'true' if grouped else 'false'}>",
+    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_k_kernel<{batch},{'true' if grouped else 'false'},{group_maxt(H, group) if grouped else '*'}>",
                           "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(achieved / HBM_PEAK_GBS, 4),
                           "avg_launch_us": round(dev_ms * 1e3 / launches, 3),

@@ -172,6 +172,8 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create_q4_k(uint32_t n_problems, const rm
                                                    uint32_t n_tokens);
 void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g);
 int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream);
+/* Launch shape of a group, for profiling tools: workgroups per launch and waves per workgroup. */
+int rmi_hip_gemv_group_shape(const rmi_hip_gemv_group *g, uint32_t *n_workgroups, uint32_t *waves_per_workgroup);
 
 #ifdef __cplusplus
 }

@@ -219,12 +219,16 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create_q4_k(uint32_t n_problems, const rm
         delete g;
         return nullptr;
     }
+    g->wpg = rmi_gemv_waves_per_group(
+        size_t(n_tokens) * g->max_units * 304,
+        size_t(rmi_q4k_tiles_per_wave(g->max_units, uint32_t(total_tiles), n_tokens)) * g->max_units * kQ4KSuperBytes);
     std::vector<uint4> runs;
     for (uint32_t i = 0; i < n_problems; i++) {
         if (list[i].n_sb == 0) continue;
         const uint32_t tpw = rmi_q4k_tiles_per_wave(list[i].n_sb, uint32_t(total_tiles), n_tokens);
         for (uint32_t k = 0; k < list[i].n_tiles; k += tpw)
             runs.push_back(make_uint4(i, k, list[i].n_tiles - k < tpw ? list[i].n_tiles - k : tpw, 0));
+        while (runs.size() % g->wpg) runs.push_back(make_uint4(i, 0, 0, 0));
     }
     g->n_runs = uint32_t(runs.size());
     hipError_t e = hipMalloc(&g->d_list, sizeof(RmiQ4kProblem) * n_problems);

@@ -317,13 +317,17 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
         delete g;
         return nullptr;
     }
-    // one run of consecutive tiles per wave, never across two matrices
+    // one run of consecutive tiles per wave, never across two matrices; the waves of a workgroup share a matrix
+    g->wpg = rmi_gemv_waves_per_group(
+        size_t(n_tokens) * g->max_units * 288,
+        size_t(rmi_gemv_tiles_per_wave(g->max_units, uint32_t(total_tiles), n_tokens)) * g->max_units * kOctetBytes);
     std::vector<uint4> runs;
     for (uint32_t i = 0; i < n_problems; i++) {
         if (list[i].n_oct == 0) continue;
         const uint32_t tpw = rmi_gemv_tiles_per_wave(list[i].n_oct, uint32_t(total_tiles), n_tokens);
         for (uint32_t k = 0; k < list[i].n_tiles; k += tpw)
             runs.push_back(make_uint4(i, k, list[i].n_tiles - k < tpw ? list[i].n_tiles - k : tpw, 0));
+        while (runs.size() % g->wpg) runs.push_back(make_uint4(i, 0, 0, 0));
     }
     g->n_runs = uint32_t(runs.size());
     hipError_t e = hipMalloc(&g->d_list, sizeof(RmiGemvProblem) * n_problems);
@@ -342,6 +346,13 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
     return g;
 }
 
+int rmi_hip_gemv_group_shape(const rmi_hip_gemv_group *g, uint32_t *n_workgroups, uint32_t *waves_per_workgroup) {
+    if (!g) return rmi_fail(RMI_HIP_E_INVALID, "null gemv group");
+    if (n_workgroups) *n_workgroups = g->n_runs / g->wpg;
+    if (waves_per_workgroup) *waves_per_workgroup = g->wpg;
+    return RMI_HIP_OK;
+}
+
 void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g) {
     if (!g) return;
     if (g->d_list) hipFree(g->d_list);
@@ -354,9 +365,9 @@ int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream) {
     if (!g) return rmi_fail(RMI_HIP_E_INVALID, "null group");
     if (g->dtype == RMI_HIP_DTYPE_Q4_K)
         return rmi_launch_gemv_q4_k_group(static_cast<const RmiQ4kProblem *>(g->d_list), g->d_runs, g->n_runs,
-                                          g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
+                                          g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
     return rmi_launch_gemv_q8_0_group(static_cast<const RmiGemvProblem *>(g->d_list), g->d_runs, g->n_runs,
-                                      g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
+                                      g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -137,14 +137,15 @@ __device__ __forceinline__ void super_fma(float (&acc)[B], float (&acc_m)[B], co
             const int lo = int(qd[gg] & 0x0f0f0f0fu), hi = int((qd[gg] >> 4) & 0x0f0f0f0fu);
             const int dl = dot4_i8(lo, int(xd[2 * gg]));
             const int dh = dot4_i8(hi, int(xd[2 * gg + 1]));
-            sumi += int(byte_of(sm.x, sm.y, 2 * gg)) * dl + int(byte_of(sm.x, sm.y, 2 * gg + 1)) * dh;
+            // 6-bit scale x (4 products of a nibble and an int8): both factors fit 24 bits, full-rate multiply-add
+            sumi += __mul24(int(byte_of(sm.x, sm.y, 2 * gg)), dl) + __mul24(int(byte_of(sm.x, sm.y, 2 * gg + 1)), dh);
         }
         const float d8 = __uint_as_float(xs[72]);
         const float dd = wd * d8;
         const float dm = (-wdmin) * d8;
         acc[t] = __builtin_fmaf(dd, float(sumi), acc[t]);
         const int s0 = int(xs[64 + ((2 * T) & 7)]), s1 = int(xs[64 + ((2 * T + 1) & 7)]);
-        const int prod = mn0 * s0 + mn1 * s1;
+        const int prod = __mul24(mn0, s0) + __mul24(mn1, s1);  // 6-bit min x 16-bit pair sum
         acc_m[t] = __builtin_fmaf(dm, float(prod), acc_m[t]);
     }
 }
@@ -153,21 +154,23 @@ __device__ __forceinline__ void super_fma(float (&acc)[B], float (&acc_m)[B], co
 // matrix, and a launch has far more waves than fit on the chip (see gemv_q8_0.hip).
 // GROUPED = false: one matrix (`single`), run w starts at tile w * tiles_per_wave.
 // GROUPED = true: runs[w] = {problem index, first tile, tile count, -}.
-template <int B, bool GROUPED>
-__global__ __launch_bounds__(64) void gemv_q4_k_kernel(RmiQ4kProblem single, const RmiQ4kProblem *__restrict__ list,
+// MAXT = 64: one wave per workgroup; 512: up to eight waves sharing one staged activation
+template <int B, bool GROUPED, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_q4_k_kernel(RmiQ4kProblem single, const RmiQ4kProblem *__restrict__ list,
                                                         const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
     extern __shared__ uint4 lds[];
-    const uint32_t lane = threadIdx.x, r = lane >> 3, T = lane & 7;
+    const uint32_t lane = threadIdx.x & 63, r = lane >> 3, T = lane & 7;
+    const uint32_t w_idx = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     RmiQ4kProblem p;
     uint32_t k, k_end;
     if (GROUPED) {
-        const uint4 run = runs[blockIdx.x];
+        const uint4 run = runs[w_idx];
         p = list[run.x];
         k = run.y;
         k_end = run.y + run.z;
     } else {
         p = single;
-        k = blockIdx.x * tiles_per_wave;
+        k = w_idx * tiles_per_wave < p.n_tiles ? w_idx * tiles_per_wave : p.n_tiles;
         k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
     }
     const uint32_t n_sb = p.n_sb, n_in = n_sb * 256;
@@ -175,20 +178,20 @@ __global__ __launch_bounds__(64) void gemv_q4_k_kernel(RmiQ4kProblem single, con
     for (int t = 0; t < B; t++) {
         uint32_t *dst = lds_dw + size_t(t) * n_sb * kSbDwords;
         gptr_u32 xq = as_global<gptr_u32>(p.q8qs + size_t(t) * n_in);
-        for (uint32_t i = lane; i < n_sb * 64; i += 64) {
+        for (uint32_t i = threadIdx.x; i < n_sb * 64; i += blockDim.x) {
             // source dword i of the row: super-block sb, element offset 4*(i%64) = 64g + 32*hi + 4T'
             const uint32_t sb = i >> 6, e = i & 63;
             const uint32_t g = e >> 4, hi = (e >> 3) & 1, tq = e & 7;
             dst[sb * kSbDwords + tq * 8 + g * 2 + hi] = xq[i];
         }
         gptr_i16 bs = as_global<gptr_i16>(p.q8bs + size_t(t) * (n_in / 16));
-        for (uint32_t i = lane; i < n_sb * 8; i += 64) {
+        for (uint32_t i = threadIdx.x; i < n_sb * 8; i += blockDim.x) {
             const uint32_t sb = i >> 3, j = i & 7;
             const int16_t s = int16_t(bs[sb * 16 + 2 * j] + bs[sb * 16 + 2 * j + 1]);
             dst[sb * kSbDwords + 64 + j] = uint32_t(int32_t(s));
         }
         gptr_f32 dptr = as_global<gptr_f32>(p.q8d + size_t(t) * n_sb);
-        for (uint32_t i = lane; i < n_sb; i += 64) dst[i * kSbDwords + 72] = __float_as_uint(dptr[i]);
+        for (uint32_t i = threadIdx.x; i < n_sb; i += blockDim.x) dst[i * kSbDwords + 72] = __float_as_uint(dptr[i]);
     }
     __syncthreads();
 
@@ -304,33 +307,41 @@ __global__ __launch_bounds__(64) void q4_k_dequant_dot_kernel(const uint8_t *__r
 
 template <int B>
 int launch_gemv_q4k(const RmiQ4kProblem *single, const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_waves,
-                    uint32_t tiles_per_wave, uint32_t max_n_sb, hipStream_t s) {
+                    uint32_t wpg, uint32_t tiles_per_wave, uint32_t max_n_sb, hipStream_t s) {
     const size_t lds_bytes = size_t(B) * max_n_sb * kSbDwords * 4;
     if (lds_bytes > 64 * 1024)
         return rmi_fail(RMI_HIP_E_INVALID, "activation of %d tokens x %u elements does not fit the LDS staging", B,
                         max_n_sb * 256);
-    if (single)
-        hipLaunchKernelGGL((gemv_q4_k_kernel<B, false>), dim3(n_waves), dim3(64), lds_bytes, s, *single, d_list, d_runs,
+    const dim3 grid_single((n_waves + wpg - 1) / wpg), grid_group(n_waves / wpg), block(64 * wpg);
+    // the grouped run table is padded to whole workgroups
+    if (single && wpg == 1)
+        hipLaunchKernelGGL((gemv_q4_k_kernel<B, false, 64>), grid_single, block, lds_bytes, s, *single, d_list, d_runs,
+                           tiles_per_wave);
+    else if (single)
+        hipLaunchKernelGGL((gemv_q4_k_kernel<B, false, 512>), grid_single, block, lds_bytes, s, *single, d_list, d_runs,
+                           tiles_per_wave);
+    else if (wpg == 1)
+        hipLaunchKernelGGL((gemv_q4_k_kernel<B, true, 64>), grid_group, block, lds_bytes, s, RmiQ4kProblem{}, d_list, d_runs,
                            tiles_per_wave);
     else
-        hipLaunchKernelGGL((gemv_q4_k_kernel<B, true>), dim3(n_waves), dim3(64), lds_bytes, s, RmiQ4kProblem{}, d_list,
-                           d_runs, tiles_per_wave);
+        hipLaunchKernelGGL((gemv_q4_k_kernel<B, true, 512>), grid_group, block, lds_bytes, s, RmiQ4kProblem{}, d_list, d_runs,
+                           tiles_per_wave);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
 
 int dispatch_q4k(uint32_t nt, const RmiQ4kProblem *single, const RmiQ4kProblem *d_list, const uint4 *d_runs,
-                 uint32_t n_waves, uint32_t tpw, uint32_t max_n_sb, hipStream_t s) {
+                 uint32_t n_waves, uint32_t wpg, uint32_t tpw, uint32_t max_n_sb, hipStream_t s) {
     if (n_waves == 0) return RMI_HIP_OK;
     switch (nt) {
-        case 1: return launch_gemv_q4k<1>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
-        case 2: return launch_gemv_q4k<2>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
-        case 3: return launch_gemv_q4k<3>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
-        case 4: return launch_gemv_q4k<4>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
-        case 5: return launch_gemv_q4k<5>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
-        case 6: return launch_gemv_q4k<6>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
-        case 7: return launch_gemv_q4k<7>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
-        case 8: return launch_gemv_q4k<8>(single, d_list, d_runs, n_waves, tpw, max_n_sb, s);
+        case 1: return launch_gemv_q4k<1>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_sb, s);
+        case 2: return launch_gemv_q4k<2>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_sb, s);
+        case 3: return launch_gemv_q4k<3>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_sb, s);
+        case 4: return launch_gemv_q4k<4>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_sb, s);
+        case 5: return launch_gemv_q4k<5>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_sb, s);
+        case 6: return launch_gemv_q4k<6>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_sb, s);
+        case 7: return launch_gemv_q4k<7>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_sb, s);
+        case 8: return launch_gemv_q4k<8>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_sb, s);
         default: return rmi_fail(RMI_HIP_E_INVALID, "gemv takes 1..8 tokens per launch, got %u", nt);
     }
 }
@@ -347,9 +358,9 @@ int rmi_launch_quantize_q8_k(const float *x, float *d, int8_t *qs, int16_t *bsum
     return RMI_HIP_OK;
 }
 
-// Tiles a wave takes in one run: about 16 tile-super-blocks (18 KiB of weights) per token.
+// Tiles a wave takes in one run: about 16 tile-super-blocks (18 KiB of weights), 32 with more than one token.
 uint32_t rmi_q4k_tiles_per_wave(uint32_t n_sb, uint32_t launch_tiles, uint32_t n_tokens) {
-    const uint32_t target = 16 * (n_tokens ? n_tokens : 1);
+    const uint32_t target = n_tokens > 1 ? 32 : 16;  // measured best for 1 and for 2..8 tokens
     uint32_t tpw = n_sb >= target ? 1 : target / (n_sb ? n_sb : 1);
     const uint32_t fill = uint32_t(rmi_device_cus()) * 8;
     while (tpw > 1 && launch_tiles / tpw < fill) tpw >>= 1;
@@ -387,15 +398,17 @@ int rmi_launch_gemv_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *
                                                bsums + size_t(t0) * (w->n_in / 16), y + size_t(t0) * y_stride, y_stride,
                                                row_start, row_end);
         const uint32_t tpw = rmi_q4k_tiles_per_wave(n_sb, p.n_tiles, nt);
-        int rc = dispatch_q4k(nt, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, tpw, n_sb, s);
+        const uint32_t wpg =
+            rmi_gemv_waves_per_group(size_t(nt) * n_sb * kSbDwords * 4, size_t(tpw) * n_sb * kQ4KSuperBytes);
+        int rc = dispatch_q4k(nt, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, wpg, tpw, n_sb, s);
         if (rc != RMI_HIP_OK) return rc;
     }
     return RMI_HIP_OK;
 }
 
-int rmi_launch_gemv_q4_k_group(const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t max_n_sb,
-                               uint32_t n_tokens, hipStream_t s) {
-    return dispatch_q4k(n_tokens, nullptr, d_list, d_runs, n_runs, 0, max_n_sb, s);
+int rmi_launch_gemv_q4_k_group(const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,
+                               uint32_t max_n_sb, uint32_t n_tokens, hipStream_t s) {
+    return dispatch_q4k(n_tokens, nullptr, d_list, d_runs, n_runs, wpg, 0, max_n_sb, s);
 }
 
 int rmi_launch_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *qs, const int16_t *bsums, int32_t *isum,

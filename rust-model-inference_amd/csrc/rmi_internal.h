@@ -107,8 +107,11 @@ struct RmiGemvProblem {
 };
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
 // d_runs[w] = {problem index, first tile, tile count, 0}: the run of tiles wave w takes
-int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t max_n_oct,
-                               uint32_t n_tokens, hipStream_t s);
+// the run table holds n_runs entries, a multiple of wpg (waves per workgroup); the wpg runs of one
+// workgroup belong to one problem (count 0 pads)
+int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,
+                               uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s);
+uint32_t rmi_gemv_waves_per_group(size_t lds_bytes, size_t run_bytes);
 uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles, uint32_t n_tokens);
 int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s);
 int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s);
@@ -136,8 +139,8 @@ struct RmiQ4kProblem {
 RmiQ4kProblem rmi_make_q4k_problem(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums,
                                    float *y, uint32_t y_stride, uint32_t row_start, uint32_t row_end);
 uint32_t rmi_q4k_tiles_per_wave(uint32_t n_sb, uint32_t launch_tiles, uint32_t n_tokens);
-int rmi_launch_gemv_q4_k_group(const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t max_n_sb,
-                               uint32_t n_tokens, hipStream_t s);
+int rmi_launch_gemv_q4_k_group(const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,
+                               uint32_t max_n_sb, uint32_t n_tokens, hipStream_t s);
 int rmi_launch_gemv_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s);
 int rmi_launch_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *qs, const int16_t *bsums, int32_t *isum,
@@ -155,6 +158,7 @@ struct rmi_hip_gemv_group {
     uint4 *d_runs = nullptr;
     uint32_t n_problems = 0;
     uint32_t n_runs = 0;
+    uint32_t wpg = 1;  // waves per workgroup
     uint32_t max_units = 0;
     uint32_t n_tokens = 0;
 };

@@ -66,6 +66,7 @@ SIGNATURES = {
     "rmi_hip_gemv_group_create": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u32]),
     "rmi_hip_gemv_group_create_q4_k": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                              C.POINTER(_vp), _u32]),
+    "rmi_hip_gemv_group_shape": (C.c_int, [_vp, C.POINTER(_u32), C.POINTER(_u32)]),
     "rmi_hip_gemv_group_destroy": (None, [_vp]),
     "rmi_hip_gemv_group_run_dev": (C.c_int, [_vp, _vp]),
 }
