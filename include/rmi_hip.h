@@ -175,6 +175,74 @@ int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream);
 /* Launch shape of a group, for profiling tools: workgroups per launch and waves per workgroup. */
 int rmi_hip_gemv_group_shape(const rmi_hip_gemv_group *g, uint32_t *n_workgroups, uint32_t *waves_per_workgroup);
 
+/* ---------------------------------------------------------------------------
+ * Device-resident decode: Qwen3Session::generate_inner (src/models/qwen3.rs:581-1158)
+ * with every tensor in HBM between two token ids.  Embedding lookup
+ * (src/ops/embedding.rs:12-22), RMS norms (src/ops/norm.rs:3-19), the
+ * activation quantizer, NeoX RoPE (src/ops/rope.rs:21-37), attention over the
+ * F16 KV cache (qwen3.rs:876-933), SiLU (src/ops/activation/mod.rs:137-151) and
+ * greedy_token (qwen3.rs:172-191) run as kernels around the Q8_0 GEMVs.  All
+ * 2-D weights are Q8_0 blocks as in the GGUF file (dims [n_in, n_out],
+ * qwen3.rs:1297-1311); `output` NULL ties the head to token_embd (qwen3.rs:283-287).
+ * ------------------------------------------------------------------------- */
+typedef struct rmi_hip_qwen3 rmi_hip_qwen3;
+
+/* y[i] = exp(x[i]) as the decode kernels compute it: the bits of the platform libm's expf, which the
+ * reference's f32::exp resolves to (softmax src/ops/attention.rs:28-38, SiLU src/ops/activation/mod.rs:137-151).
+ * Device pointers; for parity tests of that function. */
+int rmi_hip_expf_dev(const float *x, float *y, size_t n, void *stream);
+
+typedef struct {
+    uint32_t n_embd, n_layer, n_head, n_head_kv, head_dim_k, head_dim_v, n_ff, vocab;
+    uint32_t capacity; /* positions the KV cache holds (prompt + generated) */
+    float eps, freq_base;
+    int32_t has_qk_norm;
+    int32_t rounding; /* RMI_HIP_ROUND_* of the activation quantizer */
+} rmi_hip_qwen3_config;
+
+typedef struct {
+    const uint8_t *token_embd; /* Q8_0 [vocab][n_embd] */
+    const uint8_t *output;     /* Q8_0 [vocab][n_embd] or NULL */
+    const float *output_norm;  /* [n_embd] */
+    /* per layer, [n_layer] pointers each */
+    const float *const *attn_norm, *const *ffn_norm, *const *q_norm, *const *k_norm;
+    const uint8_t *const *wq, *const *wk, *const *wv, *const *wo, *const *w_gate, *const *w_up, *const *w_down;
+} rmi_hip_qwen3_weights;
+
+/* The kernels of one step, on device pointers (what a host that keeps its own loop would call between
+ * the GEMVs).  None synchronises.
+ * x += residual (when not NULL), then rms_norm(x, weight) (src/ops/norm.rs:3-19) quantized as
+ * quantize_q8_0_into does (src/ops/quant/q8_0.rs); x keeps the sum.  n % 32 == 0. */
+int rmi_hip_rms_norm_quantize_q8_0_dev(float *x, const float *residual, const float *weight, uint32_t n, float eps,
+                                       int8_t *q8, float *scales, int rounding, void *stream);
+/* gate_up = [W_gate x ; W_up x] (2*n_ff): (W_up x) * silu(W_gate x), src/ops/activation/mod.rs:137-151
+ * as called at src/models/qwen3.rs:1016-1027, quantized to Q8_0. */
+int rmi_hip_silu_mul_quantize_q8_0_dev(const float *gate_up, uint32_t n_ff, int8_t *q8, float *scales, int rounding,
+                                       void *stream);
+/* qkv = [q ; k ; v] of one token: per-head RMS norm of q and k (NULL weights = none), rope_neox with the
+ * cos/sin of the position (head_dim_k/2 each, src/ops/rope.rs:21-37), rounding to f16: q to q16, k and v to
+ * their cache rows (src/models/qwen3.rs:826-875). */
+int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const float *k_norm, const float *cos_row,
+                                 const float *sin_row, uint16_t *q16, uint16_t *k_row, uint16_t *v_row, uint32_t n_head,
+                                 uint32_t n_head_kv, uint32_t head_dim_k, uint32_t head_dim_v, float eps, void *stream);
+/* Attention of one token over keys 0..n_keys-1 of an F16 cache [t][kv_stride] (src/models/qwen3.rs:876-933,
+ * dot_f16 src/ops/dot.rs:99-119, softmax src/ops/attention.rs:28-38); the output leaves quantized to Q8_0. */
+int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache,
+                                            uint32_t n_keys, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv,
+                                            uint32_t head_dim_k, uint32_t head_dim_v, int8_t *q8, float *scales,
+                                            int rounding, void *stream);
+
+/* Uploads and repacks the weights (host slices may be dropped afterwards), allocates the KV cache. */
+rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_hip_qwen3_weights *weights);
+void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s);
+/* Runs n_prompt + max_new - 1 steps, one token per step, positions 0.. (the prompt is fed token by
+ * token as generate_inner does), greedy sampling, no EOS.  Per step the argmax and the two largest
+ * logits; full logits of the steps listed in dump_steps.  One synchronisation at the end.
+ * Returns the number of generated tokens or a negative code (non-finite logits are an error). */
+int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_prompt, uint32_t max_new,
+                           uint32_t *generated, uint32_t *step_argmax, float *step_top2, const uint32_t *dump_steps,
+                           uint32_t n_dump, float *dump_logits, double *seconds);
+
 #ifdef __cplusplus
 }
 #endif

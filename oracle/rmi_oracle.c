@@ -652,3 +652,70 @@ void rmi_ref_quantized_linear_forward(const uint8_t *weight,
     }
     free(row);
 }
+
+/* ---- expf of the platform libm, restated (glibc >= 2.27, the FMA build that
+ * hosts with AVX2 select): x*32/ln2 = k + r in f64, 2^(k/32) from a table, a
+ * cubic in r; the reduction and the three polynomial steps are fused
+ * multiply-adds.  The reference's f32::exp (softmax, SiLU) resolves to that
+ * function; the GPU kernels carry the same formula.  rmi_ref_expf_mismatches
+ * compares it with this host's expf. ---- */
+static const uint64_t k_exp2f_tab[32] = {
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull,
+};
+
+float rmi_ref_expf_restated(float x) {
+    uint32_t ux, abstop;
+    memcpy(&ux, &x, 4);
+    abstop = (ux >> 20) & 0x7ff;
+    if (abstop >= (0x42b00000u >> 20)) { /* |x| >= 88 or NaN */
+        if (ux == 0xff800000u) return 0.0f;
+        if (abstop >= (0x7f800000u >> 20)) return x + x;
+        if (x > 0x1.62e42ep6f) return INFINITY;
+        if (x < -0x1.9fe368p6f) return 0.0f;
+    }
+    const double inv_ln2_n = 0x1.71547652b82fep+0 * 32, shift = 0x1.8p+52;
+    const double c0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, c1 = 0x1.ebfce50fac4f3p-3 / 32 / 32,
+                 c2 = 0x1.62e42ff0c52d6p-1 / 32;
+    double xd = (double)x, z = inv_ln2_n * xd, kd = z + shift, r, s, p, r2, y;
+    uint64_t ki, t;
+    memcpy(&ki, &kd, 8);
+    kd -= shift;
+    r = fma(inv_ln2_n, xd, -kd);
+    t = k_exp2f_tab[ki & 31] + (ki << 47);
+    memcpy(&s, &t, 8);
+    p = fma(c0, r, c1);
+    r2 = r * r;
+    y = fma(c2, r, 1.0);
+    y = fma(p, r2, y);
+    y = y * s;
+    return (float)y;
+}
+
+/* inputs with bit patterns first, first+stride, ... (count of them): how many differ from the host's expf */
+uint64_t rmi_ref_expf_mismatches(uint32_t first, uint32_t stride, uint64_t count) {
+    uint64_t bad = 0;
+    uint32_t b = first;
+    for (uint64_t i = 0; i < count; i++, b += stride) {
+        float x, a, m;
+        uint32_t ua, um;
+        memcpy(&x, &b, 4);
+        a = expf(x);
+        m = rmi_ref_expf_restated(x);
+        memcpy(&ua, &a, 4);
+        memcpy(&um, &m, 4);
+        if (ua != um && !(a != a && m != m)) bad++;
+    }
+    return bad;
+}
+
+/* y[i] = exp(x[i]): which = 0 the host's expf, 1 the restatement */
+void rmi_ref_expf_array(const float *x, float *y, size_t n, int which) {
+    for (size_t i = 0; i < n; i++) y[i] = which ? rmi_ref_expf_restated(x[i]) : expf(x[i]);
+}

@@ -35,6 +35,11 @@ enum {
 float rmi_ref_f16_to_f32(uint16_t bits);
 uint16_t rmi_ref_f32_to_f16(float v);
 
+/* expf of the platform libm restated (the formula the GPU kernels use), and a check against the host's expf */
+float rmi_ref_expf_restated(float x);
+uint64_t rmi_ref_expf_mismatches(uint32_t first, uint32_t stride, uint64_t count);
+void rmi_ref_expf_array(const float *x, float *y, size_t n, int which);
+
 /* src/ops/quant/q8_0.rs:49-71 (scalar), :176-230 (AVX2), :75-164 (NEON).
  * q8[n] int8 bit patterns, scales[n/32] f32 holding f16-rounded values. */
 void rmi_ref_quantize_q8_0(const float *input, size_t n, uint8_t *q8,
@@ -186,6 +191,14 @@ typedef struct {
     const float *const *attn_norm, *const *ffn_norm, *const *q_norm, *const *k_norm; /* [n_layer] */
     const void *const *wq, *const *wk, *const *wv, *const *wo, *const *w_gate, *const *w_up, *const *w_down;
 } rmi_ref_qwen3_model;
+
+/* the elementwise pieces of the loop, for per-kernel parity tests */
+void rmi_ref_rms_norm(const float *input, const float *weight, float *output, size_t n, float eps);
+void rmi_ref_rope_neox(float *x, size_t pos, size_t head_dim, float freq_base);
+void rmi_ref_rope_angles(size_t pos, size_t head_dim, float freq_base, float *cos_out, float *sin_out);
+void rmi_ref_silu_mul(const float *gate_out, float *up_out, size_t n);
+void rmi_ref_attention_f16(const float *q, const uint16_t *k_cache, const uint16_t *v_cache, size_t step,
+                           size_t kv_stride, size_t n_head, size_t n_head_kv, size_t hk, size_t hv, float *attn_out);
 
 /* weight argument for rmi_ref_cpu_matmul */
 typedef struct {

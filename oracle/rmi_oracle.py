@@ -91,6 +91,60 @@ def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
 
+lib.rmi_ref_expf_restated.restype = C.c_float
+lib.rmi_ref_expf_restated.argtypes = [C.c_float]
+lib.rmi_ref_expf_mismatches.restype = C.c_uint64
+lib.rmi_ref_expf_mismatches.argtypes = [C.c_uint32, C.c_uint32, C.c_uint64]
+
+
+def rms_norm(x, weight, eps):
+    x, weight = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(weight, np.float32)
+    out = np.empty_like(x)
+    lib.rmi_ref_rms_norm(_p(x, _f32p), _p(weight, _f32p), _p(out, _f32p), C.c_size_t(x.size), C.c_float(eps))
+    return out
+
+
+def rope_neox(x, pos, freq_base):
+    x = np.array(x, np.float32)
+    lib.rmi_ref_rope_neox(_p(x, _f32p), C.c_size_t(pos), C.c_size_t(x.size), C.c_float(freq_base))
+    return x
+
+
+def rope_angles(pos, head_dim, freq_base):
+    c, s = np.empty(head_dim // 2, np.float32), np.empty(head_dim // 2, np.float32)
+    lib.rmi_ref_rope_angles(C.c_size_t(pos), C.c_size_t(head_dim), C.c_float(freq_base), _p(c, _f32p), _p(s, _f32p))
+    return c, s
+
+
+def silu_mul(gate_out, up_out):
+    g, u = np.ascontiguousarray(gate_out, np.float32), np.array(up_out, np.float32)
+    lib.rmi_ref_silu_mul(_p(g, _f32p), _p(u, _f32p), C.c_size_t(g.size))
+    return u
+
+
+def attention_f16(q, k_cache, v_cache, step, kv_stride, n_head, n_head_kv, hk, hv):
+    q = np.ascontiguousarray(q, np.float32)
+    k_cache, v_cache = np.ascontiguousarray(k_cache, np.uint16), np.ascontiguousarray(v_cache, np.uint16)
+    out = np.zeros(n_head * hv, np.float32)
+    u16p = C.POINTER(C.c_uint16)
+    lib.rmi_ref_attention_f16(_p(q, _f32p), k_cache.ctypes.data_as(u16p), v_cache.ctypes.data_as(u16p),
+                              C.c_size_t(step), C.c_size_t(kv_stride), C.c_size_t(n_head), C.c_size_t(n_head_kv),
+                              C.c_size_t(hk), C.c_size_t(hv), _p(out, _f32p))
+    return out
+
+
+def expf_array(x, restated=False):
+    """exp of an f32 array through the host libm's expf, or through the restated formula"""
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty_like(x)
+    lib.rmi_ref_expf_array(_p(x, _f32p), _p(y, _f32p), C.c_size_t(x.size), int(restated))
+    return y
+
+
+def expf_restated(x):
+    return float(lib.rmi_ref_expf_restated(float(x)))
+
+
 def have_avx2():
     return bool(lib.rmi_ref_have_avx2())
 

@@ -139,6 +139,43 @@ static void attention_heads(void *argp, int ith, int nth) {
     }
 }
 
+/* ---- the elementwise pieces, exported for per-kernel parity tests ---- */
+void rmi_ref_rms_norm(const float *input, const float *weight, float *output, size_t n, float eps) {
+    rms_norm(input, weight, output, n, eps);
+}
+void rmi_ref_rope_neox(float *x, size_t pos, size_t head_dim, float freq_base) { rope_neox(x, pos, head_dim, freq_base); }
+void rmi_ref_rope_angles(size_t pos, size_t head_dim, float freq_base, float *cos_out, float *sin_out) {
+    float theta_scale = powf(freq_base, -2.0f / (float)head_dim), theta = (float)pos;
+    for (size_t i = 0; i < head_dim / 2; i++) {
+        cos_out[i] = cosf(theta);
+        sin_out[i] = sinf(theta);
+        theta *= theta_scale;
+    }
+}
+/* silu_mul_inplace(&gate_out, &mut up_out): up_out[i] *= gate_out[i] / (1 + exp(-gate_out[i])) */
+void rmi_ref_silu_mul(const float *gate_out, float *up_out, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float g = gate_out[i];
+        float s = g / (1.0f + expf(-g));
+        up_out[i] *= s;
+    }
+}
+/* attention of one token over keys 0..step of an F16 cache laid out [t][kv_stride] (qwen3.rs:876-933) */
+void rmi_ref_attention_f16(const float *q, const uint16_t *k_cache, const uint16_t *v_cache, size_t step,
+                           size_t kv_stride, size_t n_head, size_t n_head_kv, size_t hk, size_t hv, float *attn_out) {
+    rmi_ref_qwen3_model m;
+    memset(&m, 0, sizeof m);
+    m.n_head = (uint32_t)n_head;
+    m.n_head_kv = (uint32_t)n_head_kv;
+    m.head_dim_k = (uint32_t)hk;
+    m.head_dim_v = (uint32_t)hv;
+    size_t n_padded = (step + 1 + 255) / 256 * 256, score_stride = n_padded * 2 + 64;
+    float *scores = (float *)calloc(score_stride, 4);
+    attn_job job = {&m, q, attn_out, k_cache, v_cache, scores, score_stride, 0, kv_stride, step};
+    attention_heads(&job, 0, 1);
+    free(scores);
+}
+
 static uint64_t fnv1a(const void *data, size_t n) {
     const uint8_t *p = (const uint8_t *)data;
     uint64_t h = 1469598103934665603ull;

@@ -4,15 +4,16 @@
 ``gguf``   minimal GGUF v3 writer / mmap reader (synthetic Qwen3 file)
 ``hip``    ctypes binding of librmi_hip.so, the C ABI of include/rmi_hip.h
 ``kernel`` mirror of the reference's Kernel / Layer interface over that ABI
+``decode`` mirror of Qwen3Session over the device-resident decode entry points
 
-``hip`` and ``kernel`` load the compiled library on first use and raise if it
+``hip``, ``kernel`` and ``decode`` load the compiled library on first use and raise if it
 is missing; nothing here computes on the CPU.
 """
 import importlib
 
 from . import gguf, synth  # noqa: F401
 
-_LAZY = ("hip", "kernel")
+_LAZY = ("hip", "kernel", "decode")
 
 
 def __getattr__(name):

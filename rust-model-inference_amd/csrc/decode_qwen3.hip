@@ -1,0 +1,687 @@
+// Device-resident decode step of the Qwen3 text model: everything between two
+// token ids stays in HBM.  Follows Qwen3Session::generate_inner
+// (src/models/qwen3.rs:581-1158) for all-Q8_0 weights, F16 KV cache, NeoX RoPE,
+// per-head q/k RMS norm and greedy sampling:
+//   embedding_lookup_q8_0   src/ops/embedding.rs:12-22
+//   rms_norm                src/ops/norm.rs:3-19      (f64 sum of f32 squares)
+//   quantize_q8_0_into      src/ops/quant/q8_0.rs     (fused into the producer)
+//   rope_neox               src/ops/rope.rs:21-37     (cos/sin table from the host libm)
+//   attention, F16 cache    src/models/qwen3.rs:876-933, dot_f16 src/ops/dot.rs:99-119
+//   softmax                 src/ops/attention.rs:28-38
+//   silu_mul_inplace        src/ops/activation/mod.rs:137-151
+//   greedy_token            src/models/qwen3.rs:172-191
+// The quantized matmuls are the GEMV of gemv_q8_0.hip on q/k/v and gate/up
+// stacked into one weight each (src/ops/quant/fuse.rs:25-64).
+//
+// Every f32 rounding point of the reference is kept: products rounded to f32
+// before the f64 accumulation, f16 roundings of q, k, v and of the softmax
+// weights, the sequential f32 sum of softmax, one f32 division per weight, and
+// exp with the bits of the platform libm (device_math.h).  Only the f64 sums of
+// rms_norm run as a tree instead of in sequence; they hold f32 squares, so the
+// order can matter only when the f64 sum rounds differently in its last bits
+// and that flips the f32 rounding of the mean (about 2^-29 per norm).  A rounded
+// int8 quant that flips would move logits by 1e-2, so the step is held to
+// bit-identical logits against the CPU path, not to a tolerance.
+#include <chrono>
+#include <cmath>
+#include <vector>
+
+#include "device_math.h"
+#include "device_quant.h"
+#include "rmi_internal.h"
+
+namespace {
+
+__device__ __forceinline__ float h2f(uint32_t bits16) {
+    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
+}
+// f32 -> f16 of a value that has already been rounded to f32.  The empty asm keeps the compiler from folding
+// a preceding fma into v_fma_mixlo_f16, which rounds the exact result once; the reference rounds twice.
+__device__ __forceinline__ uint16_t f2h(float v) {
+    asm volatile("" : "+v"(v));
+    return __builtin_bit_cast(uint16_t, _Float16(v));
+}
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// x[e] = d * q of row `token` of a Q8_0 weight in the GEMV tile stream
+__global__ __launch_bounds__(256) void embed_q8_0_kernel(const uint8_t *__restrict__ w, uint32_t n_oct,
+                                                          const uint32_t *__restrict__ tok, uint32_t step,
+                                                          uint32_t vocab, float *__restrict__ x, uint32_t n_embd) {
+    uint32_t token = tok[step];
+    if (token >= vocab) token = vocab - 1;  // ids are validated on the host; never read outside the weight
+    const uint8_t *tile = w + size_t(token >> 3) * n_oct * kOctetBytes;
+    const uint32_t r = token & 7;
+    for (uint32_t e = threadIdx.x; e < n_embd; e += blockDim.x) {
+        const uint32_t b = e >> 5, k = e & 31;
+        const uint16_t dh = *reinterpret_cast<const uint16_t *>(tile + (b >> 3) * 128 + r * 16 + (b & 7) * 2);
+        const int8_t q = *reinterpret_cast<const int8_t *>(tile + size_t(n_oct) * 128 + size_t(b >> 2) * 1024 + r * 128 +
+                                                           (k >> 2) * 16 + (b & 3) * 4 + (k & 3));
+        x[e] = h2f(dh) * float(int(q));
+    }
+}
+
+// x += r (if r), then rms_norm(x, weight) quantized to Q8_0.  One workgroup of 256.
+__global__ __launch_bounds__(256) void add_rmsnorm_quant_kernel(float *__restrict__ x, const float *__restrict__ r,
+                                                                 const float *__restrict__ weight, uint32_t n, float eps,
+                                                                 int8_t *__restrict__ q8, float *__restrict__ scales,
+                                                                 int rounding) {
+    __shared__ double red[4];
+    const uint32_t tid = threadIdx.x;
+    double part = 0.0;
+    for (uint32_t i = tid * 4; i < n; i += 1024) {
+        float4 v = *reinterpret_cast<const float4 *>(x + i);
+        if (r) {
+            const float4 a = *reinterpret_cast<const float4 *>(r + i);
+            v.x += a.x;
+            v.y += a.y;
+            v.z += a.z;
+            v.w += a.w;
+            *reinterpret_cast<float4 *>(x + i) = v;
+        }
+        const float s0 = v.x * v.x, s1 = v.y * v.y, s2 = v.z * v.z, s3 = v.w * v.w;
+        part += double(s0);
+        part += double(s1);
+        part += double(s2);
+        part += double(s3);
+    }
+    part = wave_sum(part);
+    if ((tid & 63) == 0) red[tid >> 6] = part;
+    __syncthreads();
+    const double total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float mean_sq = float(total / double(n));
+    const float scale = 1.0f / sqrtf(mean_sq + eps);
+    for (uint32_t i = tid * 4; i < n; i += 1024) {
+        const float4 v = *reinterpret_cast<const float4 *>(x + i);
+        const float4 wv = *reinterpret_cast<const float4 *>(weight + i);
+        float4 o;
+        o.x = (v.x * scale) * wv.x;
+        o.y = (v.y * scale) * wv.y;
+        o.z = (v.z * scale) * wv.z;
+        o.w = (v.w * scale) * wv.w;
+        float sc;
+        reinterpret_cast<uint32_t *>(q8)[i >> 2] = rmi_quantize_block8(o, rounding, &sc);
+        if ((tid & 7) == 0) scales[i >> 5] = sc;
+    }
+}
+
+// Per head of the stacked q|k|v vector: q/k RMS norm, NeoX rotation, f16 rounding; k and v go to the cache row.
+__global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(const float *__restrict__ qkv,
+                                                                const float *__restrict__ q_norm,
+                                                                const float *__restrict__ k_norm,
+                                                                const float *__restrict__ cos_t,
+                                                                const float *__restrict__ sin_t, uint32_t pos,
+                                                                uint16_t *__restrict__ q16, uint16_t *__restrict__ k_row,
+                                                                uint16_t *__restrict__ v_row, uint32_t n_head,
+                                                                uint32_t n_head_kv, uint32_t hk, uint32_t hv, float eps) {
+    const uint32_t head = blockIdx.x, tid = threadIdx.x;
+    if (head >= n_head + n_head_kv) {  // v: rounding only
+        const uint32_t kvh = head - n_head - n_head_kv;
+        const float *src = qkv + size_t(n_head) * hk + size_t(n_head_kv) * hk + size_t(kvh) * hv;
+        for (uint32_t d = tid; d < hv; d += 64) v_row[kvh * hv + d] = f2h(src[d]);
+        return;
+    }
+    const bool is_q = head < n_head;
+    const uint32_t local = is_q ? head : head - n_head;
+    const float *src = qkv + (is_q ? size_t(local) * hk : size_t(n_head) * hk + size_t(local) * hk);
+    const float *nw = is_q ? q_norm : k_norm;
+    float scale = 1.0f;
+    if (nw) {
+        double part = 0.0;
+        for (uint32_t d = tid; d < hk; d += 64) {
+            const float sq = src[d] * src[d];
+            part += double(sq);
+        }
+        const double total = wave_sum(part);
+        const float mean_sq = float(total / double(hk));
+        scale = 1.0f / sqrtf(mean_sq + eps);
+    }
+    const uint32_t half = hk >> 1;
+    uint16_t *dst = is_q ? q16 + size_t(local) * hk : k_row + size_t(local) * hk;
+    for (uint32_t i = tid; i < half; i += 64) {
+        float x0 = src[i], x1 = src[i + half];
+        if (nw) {
+            x0 = (x0 * scale) * nw[i];
+            x1 = (x1 * scale) * nw[i + half];
+        }
+        const float cos_a = cos_t[size_t(pos) * half + i], sin_a = sin_t[size_t(pos) * half + i];
+        const float a = x1 * -sin_a;
+        const float b = x1 * cos_a;
+        dst[i] = f2h(__builtin_fmaf(x0, cos_a, a));
+        dst[i + half] = f2h(__builtin_fmaf(x0, sin_a, b));
+    }
+}
+
+// One workgroup per query head over keys 0..step of the F16 cache; the head's output leaves quantized to Q8_0.
+__global__ __launch_bounds__(256) void attention_quant_kernel(const uint16_t *__restrict__ q16,
+                                                              const uint16_t *__restrict__ k_cache,
+                                                              const uint16_t *__restrict__ v_cache, uint32_t step,
+                                                              uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv,
+                                                              uint32_t hk, uint32_t hv, int8_t *__restrict__ q8,
+                                                              float *__restrict__ scales, int rounding) {
+    extern __shared__ float lds_f[];
+    __shared__ float red_f[4];
+    const uint32_t head = blockIdx.x, tid = threadIdx.x;
+    const uint32_t kvh = head / (n_head / n_head_kv);
+    const uint32_t n_keys = step + 1;
+    float *scores = lds_f;                                                  // [n_keys]
+    float *outv = lds_f + ((n_keys + 3) & ~3u);                             // [hv]
+    uint16_t *w16 = reinterpret_cast<uint16_t *>(outv + hv);                // [n_keys]
+    uint16_t *qs = w16 + ((n_keys + 7) & ~7u);                              // [hk]
+    for (uint32_t d = tid; d < hk; d += 256) qs[d] = q16[size_t(head) * hk + d];
+    __syncthreads();
+    const float kq_scale = 1.0f / sqrtf(float(hk));
+    float my_max = -INFINITY;
+    for (uint32_t t = tid; t < n_keys; t += 256) {
+        const uint16_t *key = k_cache + size_t(t) * kv_stride + size_t(kvh) * hk;
+        double sum = 0.0;
+        for (uint32_t d = 0; d < hk; d += 8) {
+            const uint4 kk = *reinterpret_cast<const uint4 *>(key + d);
+            const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float p0 = h2f(qs[d + 2 * j]) * h2f(kw[j] & 0xffffu);
+                sum += double(p0);
+                const float p1 = h2f(qs[d + 2 * j + 1]) * h2f(kw[j] >> 16);
+                sum += double(p1);
+            }
+        }
+        const float s = float(sum) * kq_scale;
+        scores[t] = s;
+        my_max = fmaxf(my_max, s);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) my_max = fmaxf(my_max, __shfl_xor(my_max, off, 64));
+    if ((tid & 63) == 0) red_f[tid >> 6] = my_max;
+    __syncthreads();
+    const float max_val = fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3]));
+    __syncthreads();
+    for (uint32_t t = tid; t < n_keys; t += 256) scores[t] = rmi_expf(scores[t] - max_val);
+    __syncthreads();
+    if (tid == 0) {  // the reference adds the weights one after the other in f32
+        float acc = 0.0f;
+        for (uint32_t t = 0; t < n_keys; t++) acc += scores[t];
+        red_f[0] = acc;
+    }
+    __syncthreads();
+    const float sum = red_f[0];
+    for (uint32_t t = tid; t < n_keys; t += 256) {
+        const float e = scores[t];
+        w16[t] = f2h(sum > 0.0f ? e / sum : e);
+    }
+    __syncthreads();
+    for (uint32_t d = tid; d < hv; d += 256) {
+        const uint16_t *col = v_cache + size_t(kvh) * hv + d;
+        double acc = 0.0;
+        for (uint32_t t = 0; t < n_keys; t++) {
+            const float p = h2f(col[size_t(t) * kv_stride]) * h2f(w16[t]);
+            acc += double(p);
+        }
+        outv[d] = float(acc);
+    }
+    __syncthreads();
+    if (tid * 4 < hv) {  // hv is a multiple of 32: whole 8-lane groups
+        const float4 o = *reinterpret_cast<const float4 *>(outv + tid * 4);
+        float sc;
+        reinterpret_cast<uint32_t *>(q8)[(size_t(head) * hv >> 2) + tid] = rmi_quantize_block8(o, rounding, &sc);
+        if ((tid & 7) == 0) scales[(size_t(head) * hv >> 5) + (tid >> 3)] = sc;
+    }
+}
+
+// gu = [W_gate x ; W_up x]: h = (W_up x) * silu(W_gate x), quantized to Q8_0
+__global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float *__restrict__ gu, uint32_t n_ff,
+                                                             int8_t *__restrict__ q8, float *__restrict__ scales,
+                                                             int rounding) {
+    const uint32_t i = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n_ff) return;  // n_ff is a multiple of 32: whole 8-lane groups leave together
+    const float4 g = *reinterpret_cast<const float4 *>(gu + i);
+    const float4 u = *reinterpret_cast<const float4 *>(gu + n_ff + i);
+    float4 h;
+    h.x = u.x * (g.x / (1.0f + rmi_expf(-g.x)));
+    h.y = u.y * (g.y / (1.0f + rmi_expf(-g.y)));
+    h.z = u.z * (g.z / (1.0f + rmi_expf(-g.z)));
+    h.w = u.w * (g.w / (1.0f + rmi_expf(-g.w)));
+    float sc;
+    reinterpret_cast<uint32_t *>(q8)[i >> 2] = rmi_quantize_block8(h, rounding, &sc);
+    if ((threadIdx.x & 7) == 0) scales[i >> 5] = sc;
+}
+
+__global__ __launch_bounds__(256) void expf_kernel(const float *__restrict__ x, float *__restrict__ y, size_t n) {
+    for (size_t i = blockIdx.x * size_t(256) + threadIdx.x; i < n; i += size_t(gridDim.x) * 256) y[i] = rmi_expf(x[i]);
+}
+
+// greedy_token: the first strict maximum, the second largest value, and whether every logit is finite
+struct Top {
+    float best, second;
+    uint32_t id, finite;
+};
+__device__ __forceinline__ Top top_merge(const Top &a, const Top &b) {
+    Top r;
+    const bool a_first = a.best > b.best || (a.best == b.best && a.id < b.id);
+    const Top &hi = a_first ? a : b, &lo = a_first ? b : a;
+    r.best = hi.best;
+    r.id = hi.id;
+    r.second = fmaxf(fmaxf(hi.second, lo.second), lo.best);
+    r.finite = a.finite & b.finite;
+    return r;
+}
+__device__ __forceinline__ Top top_block_reduce(Top t, Top *sm) {
+    sm[threadIdx.x] = t;
+    __syncthreads();
+    for (uint32_t s = blockDim.x >> 1; s > 0; s >>= 1) {
+        if (threadIdx.x < s) sm[threadIdx.x] = top_merge(sm[threadIdx.x], sm[threadIdx.x + s]);
+        __syncthreads();
+    }
+    return sm[0];
+}
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__restrict__ logits, uint32_t n,
+                                                             Top *__restrict__ partial) {
+    __shared__ Top sm[256];
+    Top t{-INFINITY, -INFINITY, 0xffffffffu, 1u};
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+        const float l = logits[i];
+        if (!(fabsf(l) <= 3.4028234663852886e38f)) t.finite = 0;  // NaN or inf
+        if (l > t.best) {
+            t.second = t.best;
+            t.best = l;
+            t.id = i;
+        } else if (l > t.second) {
+            t.second = l;
+        }
+    }
+    const Top r = top_block_reduce(t, sm);
+    if (threadIdx.x == 0) partial[blockIdx.x] = r;
+}
+__global__ __launch_bounds__(256) void argmax_final_kernel(const Top *__restrict__ partial, uint32_t n_partial,
+                                                           uint32_t step, uint32_t n_prompt,
+                                                           uint32_t *__restrict__ tok, uint32_t *__restrict__ step_argmax,
+                                                           float *__restrict__ step_top2,
+                                                           uint32_t *__restrict__ nonfinite_steps) {
+    __shared__ Top sm[256];
+    Top t{-INFINITY, -INFINITY, 0xffffffffu, 1u};
+    for (uint32_t i = threadIdx.x; i < n_partial; i += 256) t = top_merge(t, partial[i]);
+    const Top r = top_block_reduce(t, sm);
+    if (threadIdx.x == 0) {
+        step_argmax[step] = r.id;
+        step_top2[2 * step] = r.best;
+        step_top2[2 * step + 1] = r.second;
+        if (!r.finite) atomicAdd(nonfinite_steps, 1u);
+        if (step + 1 >= n_prompt) tok[step + 1] = r.id;  // the next step reads its token here
+    }
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ session
+
+struct rmi_hip_qwen3 {
+    rmi_hip_qwen3_config cfg{};
+    uint32_t n_q = 0, n_k = 0, n_v = 0, n_attn = 0, kv_stride = 0, max_n_in = 0;
+    rmi_hip_weight *embd = nullptr, *head = nullptr;  // head == embd when tied
+    std::vector<rmi_hip_weight *> w_qkv, w_o, w_gu, w_down;
+    std::vector<float *> attn_norm, ffn_norm, q_norm, k_norm;
+    float *output_norm = nullptr;
+    float *cos_t = nullptr, *sin_t = nullptr;
+    uint16_t *k_cache = nullptr, *v_cache = nullptr, *q16 = nullptr;
+    float *x = nullptr, *resid = nullptr, *qkv = nullptr, *gu = nullptr, *logits = nullptr, *act_scales = nullptr;
+    int8_t *act_q8 = nullptr;
+    uint32_t *tok = nullptr, *step_argmax = nullptr, *nonfinite = nullptr;
+    float *step_top2 = nullptr;
+    void *partial = nullptr;
+    std::vector<void *> owned;  // every other device allocation, freed with the session
+};
+
+namespace {
+
+constexpr uint32_t kArgmaxGroups = 256;
+
+template <typename T>
+T *dev_alloc(rmi_hip_qwen3 *s, size_t count, bool zero = false) {
+    void *p = nullptr;
+    if (hipMalloc(&p, count * sizeof(T) ? count * sizeof(T) : sizeof(T)) != hipSuccess) {
+        rmi_set_error("hipMalloc of %zu bytes failed", count * sizeof(T));
+        return nullptr;
+    }
+    s->owned.push_back(p);
+    if (zero && hipMemset(p, 0, count * sizeof(T)) != hipSuccess) return nullptr;
+    return static_cast<T *>(p);
+}
+
+float *upload_f32(rmi_hip_qwen3 *s, const float *host, size_t n) {
+    float *d = dev_alloc<float>(s, n);
+    if (d && hipMemcpy(d, host, n * 4, hipMemcpyHostToDevice) != hipSuccess) {
+        rmi_set_error("hipMemcpy of a norm weight failed");
+        return nullptr;
+    }
+    return d;
+}
+
+rmi_hip_weight *upload_stack(const uint8_t *const *parts, const uint32_t *rows, int n_parts, uint32_t n_in) {
+    rmi_hip_weight *acc = nullptr;
+    for (int i = 0; i < n_parts; i++) {
+        rmi_hip_weight *w = rmi_hip_upload_q8_0(parts[i], size_t(rows[i]) * (n_in / 32) * 34, n_in, rows[i]);
+        if (!w) {
+            if (acc) rmi_hip_free_weight(acc);
+            return nullptr;
+        }
+        if (!acc) {
+            acc = w;
+            continue;
+        }
+        rmi_hip_weight *f = rmi_hip_fuse_vstack(acc, w);
+        rmi_hip_free_weight(acc);
+        rmi_hip_free_weight(w);
+        if (!f) {
+            rmi_set_error("stacking projection weights failed");
+            return nullptr;
+        }
+        acc = f;
+    }
+    return acc;
+}
+
+int gemv(const rmi_hip_weight *w, const int8_t *q8, const float *scales, float *y, hipStream_t st) {
+    RmiGemvProblem p{};
+    p.w = w->data;
+    p.x_q8 = q8;
+    p.x_scales = scales;
+    p.y = y;
+    p.n_in = w->n_in;
+    p.n_oct = w->n_units;
+    p.y_stride = w->n_out;
+    p.row_start = 0;
+    p.row_end = w->n_out;
+    p.tile0 = 0;
+    p.n_tiles = w->n_tiles;
+    return rmi_launch_gemv_q8_0_single(p, 1, st);
+}
+
+// one decoder step: token tok[step] at position `step`; leaves logits, argmax and the next token on the device
+int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, uint32_t n_prompt, hipStream_t st) {
+    const rmi_hip_qwen3_config &c = s->cfg;
+    const int rnd = c.rounding;
+    const size_t attn_lds = size_t((step + 1 + 3) & ~3u) * 4 + size_t(c.head_dim_v) * 4 +
+                            size_t((step + 1 + 7) & ~7u) * 2 + size_t(c.head_dim_k) * 2;
+    hipLaunchKernelGGL(embed_q8_0_kernel, dim3(1), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, step,
+                       c.vocab, s->x, c.n_embd);
+    const float *pending = nullptr;  // matmul output still to be added to the residual stream
+    for (uint32_t l = 0; l < c.n_layer; l++) {
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, pending, s->attn_norm[l], c.n_embd,
+                           c.eps, s->act_q8, s->act_scales, rnd);
+        int rc = gemv(s->w_qkv[l], s->act_q8, s->act_scales, s->qkv, st);
+        if (rc != RMI_HIP_OK) return rc;
+        const size_t row = (size_t(l) * c.capacity + step) * s->kv_stride;
+        hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv), dim3(64), 0, st, s->qkv,
+                           c.has_qk_norm ? s->q_norm[l] : nullptr, c.has_qk_norm ? s->k_norm[l] : nullptr, s->cos_t,
+                           s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv,
+                           c.head_dim_k, c.head_dim_v, c.eps);
+        const size_t layer_base = size_t(l) * c.capacity * s->kv_stride;
+        hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(256), attn_lds, st, s->q16,
+                           s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv,
+                           c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
+        rc = gemv(s->w_o[l], s->act_q8, s->act_scales, s->resid, st);
+        if (rc != RMI_HIP_OK) return rc;
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, s->resid, s->ffn_norm[l], c.n_embd,
+                           c.eps, s->act_q8, s->act_scales, rnd);
+        rc = gemv(s->w_gu[l], s->act_q8, s->act_scales, s->gu, st);
+        if (rc != RMI_HIP_OK) return rc;
+        hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((c.n_ff + 1023) / 1024), dim3(256), 0, st, s->gu, c.n_ff,
+                           s->act_q8, s->act_scales, rnd);
+        rc = gemv(s->w_down[l], s->act_q8, s->act_scales, s->resid, st);
+        if (rc != RMI_HIP_OK) return rc;
+        pending = s->resid;
+    }
+    hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, pending, s->output_norm, c.n_embd,
+                       c.eps, s->act_q8, s->act_scales, rnd);
+    int rc = gemv(s->head, s->act_q8, s->act_scales, s->logits, st);
+    if (rc != RMI_HIP_OK) return rc;
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxGroups), dim3(256), 0, st, s->logits, c.vocab,
+                       static_cast<Top *>(s->partial));
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, static_cast<const Top *>(s->partial),
+                       kArgmaxGroups, step, n_prompt, s->tok, s->step_argmax, s->step_top2, s->nonfinite);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rmi_hip_expf_dev(const float *x, float *y, size_t n, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (n == 0) return RMI_HIP_OK;
+    if (!x || !y) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
+    const size_t groups = (n + 255) / 256;
+    hipLaunchKernelGGL(expf_kernel, dim3(uint32_t(groups < 4096 ? groups : 4096)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), x, y, n);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_rms_norm_quantize_q8_0_dev(float *x, const float *residual, const float *weight, uint32_t n, float eps,
+                                       int8_t *q8, float *scales, int rounding, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (n == 0) return RMI_HIP_OK;
+    if (n % 32 != 0) return rmi_fail(RMI_HIP_E_INVALID, "n=%u is not a multiple of 32", n);
+    if (!x || !weight || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
+    hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), x, residual,
+                       weight, n, eps, q8, scales, rounding);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_silu_mul_quantize_q8_0_dev(const float *gate_up, uint32_t n_ff, int8_t *q8, float *scales, int rounding,
+                                       void *stream) {
+    RMI_REQUIRE_INIT();
+    if (n_ff == 0) return RMI_HIP_OK;
+    if (n_ff % 32 != 0) return rmi_fail(RMI_HIP_E_INVALID, "n_ff=%u is not a multiple of 32", n_ff);
+    if (!gate_up || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
+    hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((n_ff + 1023) / 1024), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       gate_up, n_ff, q8, scales, rounding);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const float *k_norm, const float *cos_row,
+                                 const float *sin_row, uint16_t *q16, uint16_t *k_row, uint16_t *v_row, uint32_t n_head,
+                                 uint32_t n_head_kv, uint32_t head_dim_k, uint32_t head_dim_v, float eps, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!qkv || !cos_row || !sin_row || !q16 || !k_row || !v_row) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
+    if (n_head == 0 || n_head_kv == 0 || head_dim_k % 2) return rmi_fail(RMI_HIP_E_INVALID, "bad head shape");
+    hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(n_head + 2 * n_head_kv), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), qkv, q_norm, k_norm, cos_row, sin_row, 0u, q16, k_row, v_row,
+                       n_head, n_head_kv, head_dim_k, head_dim_v, eps);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache,
+                                            uint32_t n_keys, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv,
+                                            uint32_t head_dim_k, uint32_t head_dim_v, int8_t *q8, float *scales,
+                                            int rounding, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!q16 || !k_cache || !v_cache || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
+    if (n_keys == 0 || n_head == 0 || n_head_kv == 0 || n_head % n_head_kv || head_dim_k % 32 || head_dim_v % 32 ||
+        head_dim_k == 0 || head_dim_v == 0 || kv_stride % 8)
+        return rmi_fail(RMI_HIP_E_INVALID, "bad attention shape");
+    const size_t lds = size_t((n_keys + 3) & ~3u) * 4 + size_t(head_dim_v) * 4 + size_t((n_keys + 7) & ~7u) * 2 +
+                       size_t(head_dim_k) * 2;
+    if (lds > 64 * 1024) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
+    hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(256), lds, static_cast<hipStream_t>(stream), q16,
+                       k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8, scales,
+                       rounding);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s) {
+    if (!s) return;
+    if (s->head && s->head != s->embd) rmi_hip_free_weight(s->head);
+    if (s->embd) rmi_hip_free_weight(s->embd);
+    for (auto *w : s->w_qkv) rmi_hip_free_weight(w);
+    for (auto *w : s->w_o) rmi_hip_free_weight(w);
+    for (auto *w : s->w_gu) rmi_hip_free_weight(w);
+    for (auto *w : s->w_down) rmi_hip_free_weight(w);
+    for (void *p : s->owned) hipFree(p);
+    delete s;
+}
+
+rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_hip_qwen3_weights *wt) {
+    if (!rmi_ready()) {
+        rmi_set_error("rmi_hip_init has not succeeded");
+        return nullptr;
+    }
+    if (!cfg || !wt || !wt->token_embd || !wt->output_norm) {
+        rmi_set_error("null configuration or weights");
+        return nullptr;
+    }
+    const rmi_hip_qwen3_config &c = *cfg;
+    if (c.n_embd == 0 || c.n_embd % 32 || c.n_ff == 0 || c.n_ff % 32 || c.n_layer == 0 || c.n_head == 0 ||
+        c.n_head_kv == 0 || c.n_head % c.n_head_kv || c.head_dim_k == 0 || c.head_dim_k % 32 || c.head_dim_v == 0 ||
+        c.head_dim_v % 32 || c.vocab == 0 || c.capacity == 0 ||
+        (c.rounding != RMI_HIP_ROUND_TIES_EVEN && c.rounding != RMI_HIP_ROUND_HALF_AWAY)) {
+        rmi_set_error("unsupported model shape");
+        return nullptr;
+    }
+    // attention keeps the scores of one head in LDS
+    if (size_t(c.capacity) * 6 + size_t(c.head_dim_v) * 4 + size_t(c.head_dim_k) * 2 + 64 > 64 * 1024) {
+        rmi_set_error("capacity %u exceeds what the attention kernel holds in LDS", c.capacity);
+        return nullptr;
+    }
+    if (!rmi_thread_ctx()) return nullptr;
+    rmi_hip_qwen3 *s = new rmi_hip_qwen3();
+    s->cfg = c;
+    s->n_q = c.n_head * c.head_dim_k;
+    s->n_k = c.n_head_kv * c.head_dim_k;
+    s->n_v = c.n_head_kv * c.head_dim_v;
+    s->n_attn = c.n_head * c.head_dim_v;
+    s->kv_stride = s->n_k > s->n_v ? s->n_k : s->n_v;
+    s->max_n_in = c.n_embd;
+    if (s->n_attn > s->max_n_in) s->max_n_in = s->n_attn;
+    if (c.n_ff > s->max_n_in) s->max_n_in = c.n_ff;
+    bool ok = true;
+    {
+        const uint32_t rows[1] = {c.vocab};
+        const uint8_t *parts[1] = {wt->token_embd};
+        ok = ok && (s->embd = upload_stack(parts, rows, 1, c.n_embd));
+        if (ok && wt->output) {
+            parts[0] = wt->output;
+            ok = ok && (s->head = upload_stack(parts, rows, 1, c.n_embd));
+        } else {
+            s->head = s->embd;
+        }
+    }
+    ok = ok && (s->output_norm = upload_f32(s, wt->output_norm, c.n_embd));
+    for (uint32_t l = 0; ok && l < c.n_layer; l++) {
+        const uint8_t *qkv[3] = {wt->wq[l], wt->wk[l], wt->wv[l]};
+        const uint32_t qkv_rows[3] = {s->n_q, s->n_k, s->n_v};
+        const uint8_t *gu[2] = {wt->w_gate[l], wt->w_up[l]};
+        const uint32_t gu_rows[2] = {c.n_ff, c.n_ff};
+        const uint8_t *o[1] = {wt->wo[l]}, *dn[1] = {wt->w_down[l]};
+        const uint32_t o_rows[1] = {c.n_embd};
+        rmi_hip_weight *w;
+        ok = ok && (w = upload_stack(qkv, qkv_rows, 3, c.n_embd));
+        if (ok) s->w_qkv.push_back(w);
+        ok = ok && (w = upload_stack(o, o_rows, 1, s->n_attn));
+        if (ok) s->w_o.push_back(w);
+        ok = ok && (w = upload_stack(gu, gu_rows, 2, c.n_embd));
+        if (ok) s->w_gu.push_back(w);
+        ok = ok && (w = upload_stack(dn, o_rows, 1, c.n_ff));
+        if (ok) s->w_down.push_back(w);
+        float *f;
+        ok = ok && (f = upload_f32(s, wt->attn_norm[l], c.n_embd));
+        if (ok) s->attn_norm.push_back(f);
+        ok = ok && (f = upload_f32(s, wt->ffn_norm[l], c.n_embd));
+        if (ok) s->ffn_norm.push_back(f);
+        if (ok && c.has_qk_norm) {
+            ok = ok && (f = upload_f32(s, wt->q_norm[l], c.head_dim_k));
+            if (ok) s->q_norm.push_back(f);
+            ok = ok && (f = upload_f32(s, wt->k_norm[l], c.head_dim_k));
+            if (ok) s->k_norm.push_back(f);
+        }
+    }
+    if (ok) {  // rope_neox angles, with the host libm as the reference's CPU path uses it (src/ops/rope.rs:21-37)
+        const uint32_t half = c.head_dim_k / 2;
+        std::vector<float> ct(size_t(c.capacity) * half), stv(size_t(c.capacity) * half);
+        const float theta_scale = powf(c.freq_base, -2.0f / float(c.head_dim_k));
+        for (uint32_t pos = 0; pos < c.capacity; pos++) {
+            float theta = float(pos);
+            for (uint32_t i = 0; i < half; i++) {
+                ct[size_t(pos) * half + i] = cosf(theta);
+                stv[size_t(pos) * half + i] = sinf(theta);
+                theta *= theta_scale;
+            }
+        }
+        ok = ok && (s->cos_t = upload_f32(s, ct.data(), ct.size())) && (s->sin_t = upload_f32(s, stv.data(), stv.size()));
+    }
+    const size_t cache = size_t(c.n_layer) * c.capacity * s->kv_stride;
+    ok = ok && (s->k_cache = dev_alloc<uint16_t>(s, cache, true)) && (s->v_cache = dev_alloc<uint16_t>(s, cache, true)) &&
+         (s->q16 = dev_alloc<uint16_t>(s, s->n_q)) && (s->x = dev_alloc<float>(s, c.n_embd)) &&
+         (s->resid = dev_alloc<float>(s, c.n_embd)) && (s->qkv = dev_alloc<float>(s, size_t(s->n_q) + s->n_k + s->n_v)) &&
+         (s->gu = dev_alloc<float>(s, size_t(2) * c.n_ff)) && (s->logits = dev_alloc<float>(s, c.vocab)) &&
+         (s->act_q8 = dev_alloc<int8_t>(s, s->max_n_in)) && (s->act_scales = dev_alloc<float>(s, s->max_n_in / 32)) &&
+         (s->tok = dev_alloc<uint32_t>(s, size_t(c.capacity) + 1, true)) &&
+         (s->step_argmax = dev_alloc<uint32_t>(s, c.capacity, true)) &&
+         (s->step_top2 = dev_alloc<float>(s, size_t(2) * c.capacity, true)) &&
+         (s->nonfinite = dev_alloc<uint32_t>(s, 1, true)) && (s->partial = dev_alloc<Top>(s, kArgmaxGroups));
+    if (!ok) {
+        rmi_hip_qwen3_destroy(s);
+        return nullptr;
+    }
+    return s;
+}
+
+int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_prompt, uint32_t max_new,
+                           uint32_t *generated, uint32_t *step_argmax, float *step_top2, const uint32_t *dump_steps,
+                           uint32_t n_dump, float *dump_logits, double *seconds) {
+    RMI_REQUIRE_INIT();
+    if (!s || !prompt || n_prompt == 0 || (max_new && !generated))
+        return rmi_fail(RMI_HIP_E_INVALID, "null session, prompt or output");
+    const rmi_hip_qwen3_config &c = s->cfg;
+    if (size_t(n_prompt) + max_new > c.capacity)
+        return rmi_fail(RMI_HIP_E_INVALID, "%u prompt + %u new tokens exceed the capacity %u", n_prompt, max_new,
+                        c.capacity);
+    for (uint32_t i = 0; i < n_prompt; i++)
+        if (prompt[i] >= c.vocab) return rmi_fail(RMI_HIP_E_INVALID, "token id %u outside the vocabulary", prompt[i]);
+    RmiThreadCtx *ctx = rmi_thread_ctx();
+    if (!ctx) return RMI_HIP_E_RUNTIME;
+    hipStream_t st = ctx->stream;
+    const uint32_t steps = n_prompt + max_new - 1;
+    float *d_dump = nullptr;
+    if (n_dump) {
+        if (!dump_steps || !dump_logits) return rmi_fail(RMI_HIP_E_INVALID, "null dump arrays");
+        RMI_HIP_CHECK(hipMalloc(reinterpret_cast<void **>(&d_dump), size_t(n_dump) * c.vocab * 4));
+    }
+    int rc = RMI_HIP_OK;
+    hipError_t e = hipMemcpyAsync(s->tok, prompt, size_t(n_prompt) * 4, hipMemcpyHostToDevice, st);
+    if (e == hipSuccess) e = hipMemsetAsync(s->nonfinite, 0, 4, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint32_t step = 0; e == hipSuccess && rc == RMI_HIP_OK && step < steps; step++) {
+        rc = enqueue_step(s, step, n_prompt, st);
+        for (uint32_t d = 0; rc == RMI_HIP_OK && d < n_dump; d++)
+            if (dump_steps[d] == step)
+                e = hipMemcpyAsync(d_dump + size_t(d) * c.vocab, s->logits, size_t(c.vocab) * 4, hipMemcpyDeviceToDevice, st);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (seconds) *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    uint32_t nonfinite = 0;
+    if (e == hipSuccess && rc == RMI_HIP_OK) {
+        if (max_new) e = hipMemcpy(generated, s->tok + n_prompt, size_t(max_new) * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess && step_argmax) e = hipMemcpy(step_argmax, s->step_argmax, size_t(steps) * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess && step_top2) e = hipMemcpy(step_top2, s->step_top2, size_t(steps) * 8, hipMemcpyDeviceToHost);
+        if (e == hipSuccess && n_dump) e = hipMemcpy(dump_logits, d_dump, size_t(n_dump) * c.vocab * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess) e = hipMemcpy(&nonfinite, s->nonfinite, 4, hipMemcpyDeviceToHost);
+    }
+    if (d_dump) hipFree(d_dump);
+    if (rc != RMI_HIP_OK) return rc;
+    if (e != hipSuccess) return rmi_fail(RMI_HIP_E_RUNTIME, "decode failed: %s", hipGetErrorString(e));
+    if (nonfinite) return rmi_fail(RMI_HIP_E_RUNTIME, "non-finite logits in %u steps", nonfinite);
+    return int(max_new);
+}
+
+}  // extern "C"

@@ -6,6 +6,7 @@
 // taking fma(f32(wd)*xs[b], float(sum_{k=4L..4L+3} w*x), acc_L) block after
 // block, then hsum_ps (src/ops/dot.rs:447-456).  Eight GPU lanes hold the eight
 // accumulators of one row, so results match that kernel bit for bit.
+#include "device_quant.h"
 #include "rmi_internal.h"
 
 namespace {
@@ -235,34 +236,9 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restr
     const uint32_t b = gid >> 3, l = gid & 7;
     if (b >= n_blocks) return;  // whole 8-lane groups leave together
     const float4 v = reinterpret_cast<const float4 *>(x)[size_t(b) * 8 + l];
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
-    const float d = amax == 0.0f ? 0.0f : amax / 127.0f;
-    float r0, r1, r2, r3;
-    if (rounding == RMI_HIP_ROUND_TIES_EVEN) {
-        const float id = amax == 0.0f ? 0.0f : 127.0f / amax;
-        r0 = rintf(v.x * id);
-        r1 = rintf(v.y * id);
-        r2 = rintf(v.z * id);
-        r3 = rintf(v.w * id);
-    } else {
-        const float inv = d == 0.0f ? 0.0f : 1.0f / d;
-        r0 = roundf(v.x * inv);
-        r1 = roundf(v.y * inv);
-        r2 = roundf(v.z * inv);
-        r3 = roundf(v.w * inv);
-    }
-    // NaN: the AVX2 clamp max_ps(r,-128) yields -128, Rust's clamp + `as i8` yields 0
-    const bool even = rounding == RMI_HIP_ROUND_TIES_EVEN;
-    const int i0 = (r0 != r0 && !even) ? 0 : int(fminf(fmaxf(r0, -128.0f), 127.0f));
-    const int i1 = (r1 != r1 && !even) ? 0 : int(fminf(fmaxf(r1, -128.0f), 127.0f));
-    const int i2 = (r2 != r2 && !even) ? 0 : int(fminf(fmaxf(r2, -128.0f), 127.0f));
-    const int i3 = (r3 != r3 && !even) ? 0 : int(fminf(fmaxf(r3, -128.0f), 127.0f));
-    reinterpret_cast<uint32_t *>(q8)[size_t(b) * 8 + l] =
-        uint32_t(i0 & 0xff) | (uint32_t(i1 & 0xff) << 8) | (uint32_t(i2 & 0xff) << 16) | (uint32_t(i3 & 0xff) << 24);
-    if (l == 0) scales[b] = float(_Float16(d));
+    float scale;
+    reinterpret_cast<uint32_t *>(q8)[size_t(b) * 8 + l] = rmi_quantize_block8(v, rounding, &scale);
+    if (l == 0) scales[b] = scale;
 }
 
 // ---- ops::matmul_q8_0 with f32 activations, AVX2 order (avx2.rs:180-217):

@@ -25,6 +25,26 @@ _vp = C.c_void_p
 _u32 = C.c_uint32
 _sz = C.c_size_t
 
+_u32p = C.POINTER(C.c_uint32)
+_f32pp = C.POINTER(_f32p)
+_u8pp = C.POINTER(_u8p)
+
+
+class Qwen3Config(C.Structure):
+    """rmi_hip_qwen3_config"""
+    _fields_ = [(n, C.c_uint32) for n in ("n_embd", "n_layer", "n_head", "n_head_kv", "head_dim_k", "head_dim_v", "n_ff",
+                                          "vocab", "capacity")] + [
+        ("eps", C.c_float), ("freq_base", C.c_float), ("has_qk_norm", C.c_int32), ("rounding", C.c_int32)]
+
+
+class Qwen3Weights(C.Structure):
+    """rmi_hip_qwen3_weights"""
+    _fields_ = [("token_embd", _u8p), ("output", _u8p), ("output_norm", _f32p),
+                ("attn_norm", _f32pp), ("ffn_norm", _f32pp), ("q_norm", _f32pp), ("k_norm", _f32pp),
+                ("wq", _u8pp), ("wk", _u8pp), ("wv", _u8pp), ("wo", _u8pp), ("w_gate", _u8pp), ("w_up", _u8pp),
+                ("w_down", _u8pp)]
+
+
 # name -> (restype, argtypes); must list every symbol of include/rmi_hip.h
 SIGNATURES = {
     "rmi_hip_init": (C.c_int, [C.c_int]),
@@ -66,6 +86,17 @@ SIGNATURES = {
     "rmi_hip_gemv_group_create": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u32]),
     "rmi_hip_gemv_group_create_q4_k": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                              C.POINTER(_vp), _u32]),
+    "rmi_hip_expf_dev": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "rmi_hip_rms_norm_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, C.c_float, _vp, _vp, C.c_int, _vp]),
+    "rmi_hip_silu_mul_quantize_q8_0_dev": (C.c_int, [_vp, _u32, _vp, _vp, C.c_int, _vp]),
+    "rmi_hip_qk_norm_rope_f16_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32,
+                                               C.c_float, _vp]),
+    "rmi_hip_attention_f16_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp,
+                                                          C.c_int, _vp]),
+    "rmi_hip_qwen3_create": (_vp, [C.POINTER(Qwen3Config), C.POINTER(Qwen3Weights)]),
+    "rmi_hip_qwen3_destroy": (None, [_vp]),
+    "rmi_hip_qwen3_generate": (C.c_int, [_vp, _u32p, _u32, _u32, _u32p, _u32p, _f32p, _u32p, _u32, _f32p,
+                                         C.POINTER(C.c_double)]),
     "rmi_hip_gemv_group_shape": (C.c_int, [_vp, C.POINTER(_u32), C.POINTER(_u32)]),
     "rmi_hip_gemv_group_destroy": (None, [_vp]),
     "rmi_hip_gemv_group_run_dev": (C.c_int, [_vp, _vp]),

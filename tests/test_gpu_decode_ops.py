@@ -1,0 +1,121 @@
+"""Per-kernel parity of the device-resident decode step, through the C ABI, bit for bit against the
+restated CPU pieces of Qwen3Session::generate_inner (rms_norm + quantizer, q/k norm + RoPE + f16
+rounding, F16-cache attention + quantizer, SiLU*up + quantizer).  Many random draws each: what can go
+wrong here is rare (a rounding tie, a last-bit difference before a rounding to int8 or f16)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+A = 1  # AVX2 rounding of the activation quantizer, as the x86-64 reference build
+
+
+def _quant(oracle, v):
+    q8, sc = oracle.quantize_q8_0(np.ascontiguousarray(v, np.float32), A)
+    return q8.view(np.int8), sc
+
+
+def _dev(H, a):
+    return H.DeviceBuffer.from_array(np.ascontiguousarray(a))
+
+
+@pytest.mark.parametrize("n", [1024, 512, 3072, 96])
+def test_rms_norm_quantize(hip, oracle, n):
+    H = hip.hip
+    rng = np.random.default_rng(n)
+    for trial in range(60):
+        x = (rng.normal(0, 1, n) * rng.choice([1e-3, 1.0, 30.0])).astype(np.float32)
+        x[rng.integers(0, n, 3)] *= 50.0  # outliers, as residual streams have
+        r = rng.normal(0, 0.5, n).astype(np.float32) if trial % 2 else None
+        w = (1.0 + 0.1 * rng.normal(0, 1, n)).astype(np.float32)
+        d_x, d_w = _dev(H, x), _dev(H, w)
+        d_r = _dev(H, r) if r is not None else None
+        d_q, d_s = H.DeviceBuffer(n), H.DeviceBuffer(n // 32 * 4)
+        H.check(H.lib.rmi_hip_rms_norm_quantize_q8_0_dev(d_x.ptr, d_r.ptr if d_r else None, d_w.ptr, n, 1e-6, d_q.ptr,
+                                                         d_s.ptr, A, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        xs = x + r if r is not None else x
+        assert np.array_equal(d_x.to_array(np.float32, (n,)).view(np.uint32), xs.view(np.uint32))
+        q_ref, s_ref = _quant(oracle, oracle.rms_norm(xs, w, 1e-6))
+        assert np.array_equal(d_q.to_array(np.int8, (n,)), q_ref), trial
+        assert np.array_equal(d_s.to_array(np.float32, (n // 32,)).view(np.uint32), s_ref.view(np.uint32)), trial
+        for b in (d_x, d_w, d_q, d_s) + ((d_r,) if d_r else ()):
+            b.free()
+
+
+def test_silu_mul_quantize(hip, oracle):
+    H = hip.hip
+    rng = np.random.default_rng(3)
+    n_ff = 3072
+    for trial in range(40):
+        gu = (rng.normal(0, 1, 2 * n_ff) * rng.choice([0.05, 1.0, 8.0, 40.0])).astype(np.float32)
+        d_gu, d_q, d_s = _dev(H, gu), H.DeviceBuffer(n_ff), H.DeviceBuffer(n_ff // 32 * 4)
+        H.check(H.lib.rmi_hip_silu_mul_quantize_q8_0_dev(d_gu.ptr, n_ff, d_q.ptr, d_s.ptr, A, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        q_ref, s_ref = _quant(oracle, oracle.silu_mul(gu[:n_ff], gu[n_ff:]))
+        assert np.array_equal(d_q.to_array(np.int8, (n_ff,)), q_ref), trial
+        assert np.array_equal(d_s.to_array(np.float32, (n_ff // 32,)).view(np.uint32), s_ref.view(np.uint32)), trial
+        for b in (d_gu, d_q, d_s):
+            b.free()
+
+
+@pytest.mark.parametrize("hk", [128, 64])
+def test_qk_norm_rope_f16(hip, oracle, hk):
+    H = hip.hip
+    rng = np.random.default_rng(hk)
+    n_head, n_kv, hv = 16, 8, hk
+    n_q, n_k, n_v = n_head * hk, n_kv * hk, n_kv * hv
+    for trial in range(40):
+        pos = int(rng.integers(0, 4000))
+        qkv = (rng.normal(0, 1, n_q + n_k + n_v) * rng.choice([0.1, 1.0, 20.0])).astype(np.float32)
+        qn = (1.0 + 0.2 * rng.normal(0, 1, hk)).astype(np.float32)
+        kn = (1.0 + 0.2 * rng.normal(0, 1, hk)).astype(np.float32)
+        with_norm = trial % 3 != 0
+        c, s = oracle.rope_angles(pos, hk, 1e6)
+        d = [_dev(H, a) for a in (qkv, qn, kn, c, s)]
+        d_q16, d_k, d_v = H.DeviceBuffer(n_q * 2), H.DeviceBuffer(n_k * 2), H.DeviceBuffer(n_v * 2)
+        H.check(H.lib.rmi_hip_qk_norm_rope_f16_dev(d[0].ptr, d[1].ptr if with_norm else None,
+                                                   d[2].ptr if with_norm else None, d[3].ptr, d[4].ptr, d_q16.ptr,
+                                                   d_k.ptr, d_v.ptr, n_head, n_kv, hk, hv, 1e-6, None))
+        H.check(H.lib.rmi_hip_synchronize())
+
+        def ref_heads(vec, n, w):
+            out = []
+            for h in range(n):
+                x = vec[h * hk:(h + 1) * hk]
+                if with_norm:
+                    x = oracle.rms_norm(x, w, 1e-6)
+                out.append(oracle.rope_neox(x, pos, 1e6))
+            return np.concatenate(out).astype(np.float16).view(np.uint16)
+
+        assert np.array_equal(d_q16.to_array(np.uint16, (n_q,)), ref_heads(qkv[:n_q], n_head, qn)), trial
+        assert np.array_equal(d_k.to_array(np.uint16, (n_k,)), ref_heads(qkv[n_q:n_q + n_k], n_kv, kn)), trial
+        assert np.array_equal(d_v.to_array(np.uint16, (n_v,)), qkv[n_q + n_k:].astype(np.float16).view(np.uint16))
+        for b in d + [d_q16, d_k, d_v]:
+            b.free()
+
+
+@pytest.mark.parametrize("hk,n_head,n_kv", [(128, 16, 8), (64, 8, 4)])
+def test_attention_f16_quantize(hip, oracle, hk, n_head, n_kv):
+    H = hip.hip
+    rng = np.random.default_rng(hk + 1)
+    hv = hk
+    kv_stride = n_kv * hk
+    for n_keys in [1, 2, 7, 8, 9, 36, 63, 64, 255, 256, 257, 640]:
+        for trial in range(3):
+            scale = rng.choice([0.3, 1.0, 3.0])
+            q = (rng.normal(0, 1, n_head * hk) * scale).astype(np.float32)
+            kc = (rng.normal(0, 1, (n_keys, kv_stride)) * scale).astype(np.float16).view(np.uint16)
+            vc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+            d_q, d_k, d_v = _dev(H, q.astype(np.float16).view(np.uint16)), _dev(H, kc), _dev(H, vc)
+            d_o, d_s = H.DeviceBuffer(n_head * hv), H.DeviceBuffer(n_head * hv // 32 * 4)
+            H.check(H.lib.rmi_hip_attention_f16_quantize_q8_0_dev(d_q.ptr, d_k.ptr, d_v.ptr, n_keys, kv_stride, n_head,
+                                                                  n_kv, hk, hv, d_o.ptr, d_s.ptr, A, None))
+            H.check(H.lib.rmi_hip_synchronize())
+            ref = oracle.attention_f16(q, kc, vc, n_keys - 1, kv_stride, n_head, n_kv, hk, hv)
+            q_ref, s_ref = _quant(oracle, ref)
+            assert np.array_equal(d_o.to_array(np.int8, (n_head * hv,)), q_ref), (n_keys, trial)
+            assert np.array_equal(d_s.to_array(np.float32, (n_head * hv // 32,)).view(np.uint32),
+                                  s_ref.view(np.uint32)), (n_keys, trial)
+            for b in (d_q, d_k, d_v, d_o, d_s):
+                b.free()

@@ -288,3 +288,15 @@ def test_legacy_f32_matmul_against_f64(oracle):
     for variant in (S, A):
         y = oracle.matmul_q8_0_f32(w, x, n_in, n_out, variant)
         assert np.all(np.abs(y - want) <= 2e-6 * terms)
+
+
+def test_expf_restatement_equals_host_libm(oracle):
+    """The formula the GPU kernels use for exp (glibc's expf, FMA build) against this host's expf: every 64th
+    float bit pattern (67 M inputs, all exponents, both signs, NaN/inf) plus the dense range softmax and
+    SiLU live in.  On all 2^32 patterns the count is 0 as well (a minute of CPU time, not run here)."""
+    assert oracle.lib.rmi_ref_expf_mismatches(0, 64, 1 << 26) == 0
+    lo = int(np.float32(-20.0).view(np.uint32))
+    assert oracle.lib.rmi_ref_expf_mismatches(lo - (1 << 22), 1, 1 << 22) == 0   # (-20, -10]
+    assert oracle.lib.rmi_ref_expf_mismatches(int(np.float32(1.0).view(np.uint32)), 1, 1 << 22) == 0  # [1, 1.5)
+    assert oracle.expf_restated(0.0) == 1.0 and oracle.expf_restated(-np.inf) == 0.0
+    assert np.isnan(oracle.expf_restated(np.nan)) and oracle.expf_restated(89.0) == np.inf
