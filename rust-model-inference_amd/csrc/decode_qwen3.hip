@@ -157,6 +157,14 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(const float *__r
 }
 
 // One workgroup per query head over keys 0..step of the F16 cache; the head's output leaves quantized to Q8_0.
+// The reference's sums are sequential (f64 over the head dimension for a score, f32 over the keys for the
+// softmax denominator, f64 over the keys for an output element); each is one dependent chain here too, fed
+// by loads that are issued a batch ahead.
+constexpr uint32_t kAttnBatch = 16;  // keys per batch of the value accumulation; w16 is padded to it
+__host__ __device__ inline size_t attn_lds_bytes(uint32_t n_keys, uint32_t hk, uint32_t hv) {
+    return size_t((n_keys + 3) & ~3u) * 4 + size_t(hv) * 4 + size_t((n_keys + kAttnBatch - 1) / kAttnBatch * kAttnBatch) * 2 +
+           size_t(hk) * 2;
+}
 __global__ __launch_bounds__(256) void attention_quant_kernel(const uint16_t *__restrict__ q16,
                                                               const uint16_t *__restrict__ k_cache,
                                                               const uint16_t *__restrict__ v_cache, uint32_t step,
@@ -168,10 +176,11 @@ __global__ __launch_bounds__(256) void attention_quant_kernel(const uint16_t *__
     const uint32_t head = blockIdx.x, tid = threadIdx.x;
     const uint32_t kvh = head / (n_head / n_head_kv);
     const uint32_t n_keys = step + 1;
-    float *scores = lds_f;                                                  // [n_keys]
-    float *outv = lds_f + ((n_keys + 3) & ~3u);                             // [hv]
-    uint16_t *w16 = reinterpret_cast<uint16_t *>(outv + hv);                // [n_keys]
-    uint16_t *qs = w16 + ((n_keys + 7) & ~7u);                              // [hk]
+    const uint32_t n_keys4 = (n_keys + 3) & ~3u, n_keys_b = (n_keys + kAttnBatch - 1) / kAttnBatch * kAttnBatch;
+    float *scores = lds_f;                                    // [n_keys4], zero beyond n_keys
+    float *outv = lds_f + n_keys4;                            // [hv]
+    uint16_t *w16 = reinterpret_cast<uint16_t *>(outv + hv);  // [n_keys_b], zero beyond n_keys
+    uint16_t *qs = w16 + n_keys_b;                            // [hk]
     for (uint32_t d = tid; d < hk; d += 256) qs[d] = q16[size_t(head) * hk + d];
     __syncthreads();
     const float kq_scale = 1.0f / sqrtf(float(hk));
@@ -179,15 +188,20 @@ __global__ __launch_bounds__(256) void attention_quant_kernel(const uint16_t *__
     for (uint32_t t = tid; t < n_keys; t += 256) {
         const uint16_t *key = k_cache + size_t(t) * kv_stride + size_t(kvh) * hk;
         double sum = 0.0;
-        for (uint32_t d = 0; d < hk; d += 8) {
-            const uint4 kk = *reinterpret_cast<const uint4 *>(key + d);
-            const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w};
+        for (uint32_t d = 0; d < hk; d += 32) {
+            uint4 kk[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float p0 = h2f(qs[d + 2 * j]) * h2f(kw[j] & 0xffffu);
-                sum += double(p0);
-                const float p1 = h2f(qs[d + 2 * j + 1]) * h2f(kw[j] >> 16);
-                sum += double(p1);
+            for (int c = 0; c < 4; c++) kk[c] = *reinterpret_cast<const uint4 *>(key + d + 8 * c);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint32_t kw[4] = {kk[c].x, kk[c].y, kk[c].z, kk[c].w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float p0 = h2f(qs[d + 8 * c + 2 * j]) * h2f(kw[j] & 0xffffu);
+                    sum += double(p0);
+                    const float p1 = h2f(qs[d + 8 * c + 2 * j + 1]) * h2f(kw[j] >> 16);
+                    sum += double(p1);
+                }
             }
         }
         const float s = float(sum) * kq_scale;
@@ -199,27 +213,45 @@ __global__ __launch_bounds__(256) void attention_quant_kernel(const uint16_t *__
     if ((tid & 63) == 0) red_f[tid >> 6] = my_max;
     __syncthreads();
     const float max_val = fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3]));
+    for (uint32_t t = tid; t < n_keys4; t += 256) scores[t] = t < n_keys ? rmi_expf(scores[t] - max_val) : 0.0f;
     __syncthreads();
-    for (uint32_t t = tid; t < n_keys; t += 256) scores[t] = rmi_expf(scores[t] - max_val);
-    __syncthreads();
-    if (tid == 0) {  // the reference adds the weights one after the other in f32
+    if (tid == 0) {  // the reference adds the weights one after the other in f32; adding the zeros changes nothing
         float acc = 0.0f;
-        for (uint32_t t = 0; t < n_keys; t++) acc += scores[t];
+        for (uint32_t t = 0; t < n_keys4; t += 4) {
+            const float4 e = *reinterpret_cast<const float4 *>(scores + t);
+            acc += e.x;
+            acc += e.y;
+            acc += e.z;
+            acc += e.w;
+        }
         red_f[0] = acc;
     }
     __syncthreads();
     const float sum = red_f[0];
-    for (uint32_t t = tid; t < n_keys; t += 256) {
-        const float e = scores[t];
-        w16[t] = f2h(sum > 0.0f ? e / sum : e);
+    for (uint32_t t = tid; t < n_keys_b; t += 256) {
+        const float e = t < n_keys ? scores[t] : 0.0f;
+        w16[t] = t < n_keys ? f2h(sum > 0.0f ? e / sum : e) : uint16_t(0);
     }
     __syncthreads();
     for (uint32_t d = tid; d < hv; d += 256) {
         const uint16_t *col = v_cache + size_t(kvh) * hv + d;
         double acc = 0.0;
-        for (uint32_t t = 0; t < n_keys; t++) {
-            const float p = h2f(col[size_t(t) * kv_stride]) * h2f(w16[t]);
-            acc += double(p);
+        uint16_t cur[kAttnBatch], nxt[kAttnBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kAttnBatch; j++) cur[j] = j < n_keys ? col[size_t(j) * kv_stride] : uint16_t(0);
+        for (uint32_t t0 = 0; t0 < n_keys; t0 += kAttnBatch) {
+#pragma unroll
+            for (uint32_t j = 0; j < kAttnBatch; j++) {  // the next batch is in flight while this one is added
+                const uint32_t t = t0 + kAttnBatch + j;
+                nxt[j] = t < n_keys ? col[size_t(t) * kv_stride] : uint16_t(0);
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < kAttnBatch; j++) {  // keys past n_keys add +0.0, as the reference's padding does
+                const float p = h2f(cur[j]) * h2f(w16[t0 + j]);
+                acc += double(p);
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < kAttnBatch; j++) cur[j] = nxt[j];
         }
         outv[d] = float(acc);
     }
@@ -404,8 +436,7 @@ int gemv(const rmi_hip_weight *w, const int8_t *q8, const float *scales, float *
 int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, uint32_t n_prompt, hipStream_t st) {
     const rmi_hip_qwen3_config &c = s->cfg;
     const int rnd = c.rounding;
-    const size_t attn_lds = size_t((step + 1 + 3) & ~3u) * 4 + size_t(c.head_dim_v) * 4 +
-                            size_t((step + 1 + 7) & ~7u) * 2 + size_t(c.head_dim_k) * 2;
+    const size_t attn_lds = attn_lds_bytes(step + 1, c.head_dim_k, c.head_dim_v);
     hipLaunchKernelGGL(embed_q8_0_kernel, dim3(1), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, step,
                        c.vocab, s->x, c.n_embd);
     const float *pending = nullptr;  // matmul output still to be added to the residual stream
@@ -508,8 +539,7 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     if (n_keys == 0 || n_head == 0 || n_head_kv == 0 || n_head % n_head_kv || head_dim_k % 32 || head_dim_v % 32 ||
         head_dim_k == 0 || head_dim_v == 0 || kv_stride % 8)
         return rmi_fail(RMI_HIP_E_INVALID, "bad attention shape");
-    const size_t lds = size_t((n_keys + 3) & ~3u) * 4 + size_t(head_dim_v) * 4 + size_t((n_keys + 7) & ~7u) * 2 +
-                       size_t(head_dim_k) * 2;
+    const size_t lds = attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
     if (lds > 64 * 1024) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
     hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(256), lds, static_cast<hipStream_t>(stream), q16,
                        k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8, scales,
@@ -548,7 +578,7 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
         return nullptr;
     }
     // attention keeps the scores of one head in LDS
-    if (size_t(c.capacity) * 6 + size_t(c.head_dim_v) * 4 + size_t(c.head_dim_k) * 2 + 64 > 64 * 1024) {
+    if (attn_lds_bytes(c.capacity, c.head_dim_k, c.head_dim_v) > 64 * 1024) {
         rmi_set_error("capacity %u exceeds what the attention kernel holds in LDS", c.capacity);
         return nullptr;
     }
