@@ -482,14 +482,86 @@ def run_q4k(args, pkg, ev):
     return result
 
 
+def run_decode(args, pkg, ev):
+    """End-to-end greedy decode, device-resident: a random-init Qwen3-0.6B-architecture model written as a
+    synthetic Q8_0 GGUF, 512 prompt tokens (fed one per step, as the reference's generate_inner does) plus 128
+    generated ones = 639 token-steps per generation.  One bench step = one generation."""
+    import tempfile
+    H = pkg.hip
+    dev_name, cus, hbm = H.device_info()
+    n_prompt, n_new = 512, 128
+    tmp = tempfile.mkdtemp(prefix="rmi_bench_")
+    path = os.path.join(tmp, "synthetic-qwen3-0.6b-q8_0.gguf")
+    pkg.gguf.write_synthetic_qwen3(path, seed=4)
+    f = pkg.gguf.GGUFFile(path)
+    tensors = {name: t[2] for name, t in f.tensors.items()}
+    sess = pkg.decode.Qwen3Session(f.metadata, tensors, capacity=n_prompt + n_new)
+    prompt = np.random.default_rng(7).integers(0, 151936, n_prompt, dtype=np.uint32)
+    token_steps = n_prompt + n_new - 1
+    last = {}
+
+    def step():
+        last.update(sess.generate(prompt, n_new))
+
+    for _ in range(args.warmup):
+        step()
+    H.check(H.lib.rmi_hip_synchronize())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()  # each generation ends with its own synchronisation
+    H.check(H.lib.rmi_hip_synchronize())
+    wall = (time.perf_counter() - t0) / args.steps
+    per_token = wall / token_steps
+    synth = pkg.synth
+    alg = sum(synth.q8_0_gemv_bytes(n_out, n_in) for _, n_out, n_in in synth.QWEN3_0_6B_LAYER) * 28 + \
+        synth.q8_0_gemv_bytes(151936, 1024)
+    result = base_result(args, "decode token-steps/s, Qwen3-0.6B Q8_0, 512 prompt + 128 greedy tokens, 1 GPU", "tok/s",
+                         round(token_steps / wall, 1), wall, "int8 dot4 -> f32 (F16 KV cache)", {
+        "workload": "device-resident greedy decode of a synthetic Q8_0 GGUF (Qwen3-0.6B architecture, 28 layers, "
+                    "vocab 151936), 639 token-steps per generation; one bench step = one generation",
+        "token_steps_per_generation": token_steps, "launches_per_token_step": 1 + 9 * 28 + 4,
+        "device": dev_name.strip(), "compute_units": cus})
+    result["ms_per_token_step"] = round(per_token * 1e3, 4)
+    achieved = alg / per_token / 1e9
+    result["roofline"] = {"bound": "hbm", "kernel": "gemv_q8_0_kernel<1,false,*> (113 GEMV launches per token-step)",
+                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(achieved / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_token_step": alg,
+                          "traffic": None,
+                          "note": "a token-step is 257 dependent launches of 3-6 us each; weights are read once per "
+                                  "step, so the step is launch-latency-bound, not HBM-bound"}
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import rmi_oracle as oracle
+        if oracle.have_avx2():
+            cores = min(16, physical_cores())
+            pool = oracle.Pool(cores)
+            cpu = oracle.Qwen3Decoder(f.metadata, tensors, pool).generate(prompt, n_new)
+            pool.close()
+            result["cpu_baseline"] = {
+                "value": round(token_steps / cpu["seconds"], 1), "unit": "tok/s", "cores": cores, "kind": "port",
+                "sample": f"one full generation ({token_steps} token-steps) of the restated Qwen3Session loop with the "
+                          f"restated AVX2 matmuls over {cores} threads",
+                "gpu_tokens_equal_cpu_tokens": bool(np.array_equal(cpu["tokens"], last["tokens"])),
+                "gpu_argmax_equal_cpu_argmax_all_steps": bool(np.array_equal(cpu["argmax"], last["argmax"]))}
+    sess.close()
+    del f, tensors
+    try:
+        os.remove(path)
+        os.rmdir(tmp)
+    except OSError:
+        pass
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4k"], default="projection_set",
+    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4k", "decode"], default="projection_set",
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
-                         "q4k: Q4_K x Q8_K decode GEMV")
+                         "q4k: Q4_K x Q8_K decode GEMV; decode: end-to-end device-resident greedy decode "
+                         "(one step = one 639-token-step generation)")
     ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill tokens M for --workload gemm")
     ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
@@ -506,7 +578,7 @@ def main():
     pkg = importlib.import_module("rust-model-inference_amd")
     pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
     ev = HipEvents()
-    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4k": run_q4k}[args.workload]
+    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4k": run_q4k, "decode": run_decode}[args.workload]
     print(json.dumps(run(args, pkg, ev)), flush=True)
 
 

@@ -156,68 +156,109 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(const float *__r
     }
 }
 
-// One workgroup per query head over keys 0..step of the F16 cache; the head's output leaves quantized to Q8_0.
-// The reference's sums are sequential (f64 over the head dimension for a score, f32 over the keys for the
-// softmax denominator, f64 over the keys for an output element); each is one dependent chain here too, fed
-// by loads that are issued a batch ahead.
-constexpr uint32_t kAttnBatch = 16;  // keys per batch of the value accumulation; w16 is padded to it
+// One workgroup of 1024 per query head over keys 0..step of the F16 cache; the head's output leaves quantized
+// to Q8_0.  The product of two f16 values is exact in f32, so the reference's "f32 product, f64 sum" is an f64
+// fma chain; those f64 sums are split over lanes and combined at the end (a different order can change a
+// result only when it flips the final rounding to f32, about once in 2^26 sums).  The f32 sum of the softmax
+// weights runs in sequence, as in the reference: there the order shows in the last bit.
+constexpr uint32_t kAttnThreads = 1024;
+constexpr uint32_t kAttnPad = 64;  // keys are padded to this in LDS
 __host__ __device__ inline size_t attn_lds_bytes(uint32_t n_keys, uint32_t hk, uint32_t hv) {
-    return size_t((n_keys + 3) & ~3u) * 4 + size_t(hv) * 4 + size_t((n_keys + kAttnBatch - 1) / kAttnBatch * kAttnBatch) * 2 +
-           size_t(hk) * 2;
+    const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
+    const size_t slices = kAttnThreads / hv ? kAttnThreads / hv : 1;
+    return n_pad * 8 + size_t(hk) * 8 + slices * hv * 8 + n_pad * 4 + size_t(hv) * 4;
 }
-__global__ __launch_bounds__(256) void attention_quant_kernel(const uint16_t *__restrict__ q16,
-                                                              const uint16_t *__restrict__ k_cache,
-                                                              const uint16_t *__restrict__ v_cache, uint32_t step,
-                                                              uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv,
-                                                              uint32_t hk, uint32_t hv, int8_t *__restrict__ q8,
-                                                              float *__restrict__ scales, int rounding) {
-    extern __shared__ float lds_f[];
-    __shared__ float red_f[4];
+__global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
+    const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
+    uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, uint32_t hk, uint32_t hv,
+    int8_t *__restrict__ q8, float *__restrict__ scales, int rounding) {
+    extern __shared__ double lds_d[];
+    __shared__ float red_f[kAttnThreads / 64];
     const uint32_t head = blockIdx.x, tid = threadIdx.x;
     const uint32_t kvh = head / (n_head / n_head_kv);
     const uint32_t n_keys = step + 1;
-    const uint32_t n_keys4 = (n_keys + 3) & ~3u, n_keys_b = (n_keys + kAttnBatch - 1) / kAttnBatch * kAttnBatch;
-    float *scores = lds_f;                                    // [n_keys4], zero beyond n_keys
-    float *outv = lds_f + n_keys4;                            // [hv]
-    uint16_t *w16 = reinterpret_cast<uint16_t *>(outv + hv);  // [n_keys_b], zero beyond n_keys
-    uint16_t *qs = w16 + n_keys_b;                            // [hk]
-    for (uint32_t d = tid; d < hk; d += 256) qs[d] = q16[size_t(head) * hk + d];
+    const uint32_t n_pad = (n_keys + kAttnPad - 1) / kAttnPad * kAttnPad;
+    const uint32_t n_slices = kAttnThreads / hv ? kAttnThreads / hv : 1;
+    double *wd = lds_d;                                          // [n_pad] softmax weights (f16 values), 0 beyond n_keys
+    double *qd = wd + n_pad;                                     // [hk]    the query (f16 values)
+    double *part = qd + hk;                                      // [n_slices][hv]
+    float *scores = reinterpret_cast<float *>(part + size_t(n_slices) * hv);  // [n_pad]
+    float *outv = scores + n_pad;                                // [hv]
+    for (uint32_t d = tid; d < hk; d += kAttnThreads) qd[d] = double(h2f(q16[size_t(head) * hk + d]));
+
+    // values: hv columns x n_slices ranges of keys.  The first loads of this thread's range go out now and
+    // arrive while the scores and the softmax are computed.
+    constexpr uint32_t kPre = 16;
+    const bool v_lane = tid < n_slices * hv;
+    const uint32_t vd = tid % hv, slice = tid / hv;
+    const uint32_t chunk = ((n_pad / 8 + n_slices - 1) / n_slices) * 8;  // keys per slice, a multiple of 8
+    const uint32_t t_begin = slice * chunk, t_end = t_begin + chunk < n_pad ? t_begin + chunk : n_pad;
+    const uint16_t *col = v_cache + size_t(kvh) * hv + (v_lane ? vd : 0);
+    uint32_t pre[kPre];  // one register each: 16-bit destinations would chain the loads
+#pragma unroll
+    for (uint32_t j = 0; j < kPre; j++) {
+        // unconditional loads (a guarded load would wait for itself): past the last key the row of the last key
+        // is read instead; its weight is zero or the element is skipped below
+        const uint32_t t = t_begin + j < n_keys ? t_begin + j : n_keys - 1;
+        pre[j] = col[size_t(t) * kv_stride];
+    }
+
     __syncthreads();
+
+    // scores: four lanes per key, a quarter of the head dimension each; the next round's key is loaded ahead
     const float kq_scale = 1.0f / sqrtf(float(hk));
+    const uint32_t quarter = hk >> 2, lane4 = tid & 3;
+    const double *qq = qd + lane4 * quarter;
     float my_max = -INFINITY;
-    for (uint32_t t = tid; t < n_keys; t += 256) {
-        const uint16_t *key = k_cache + size_t(t) * kv_stride + size_t(kvh) * hk;
+    for (uint32_t t0 = 0; t0 < n_keys; t0 += kAttnThreads / 4) {
+        const uint32_t t = t0 + (tid >> 2);
+        const bool live = t < n_keys;
+        const uint16_t *key = k_cache + size_t(live ? t : 0) * kv_stride + size_t(kvh) * hk + lane4 * quarter;
         double sum = 0.0;
-        for (uint32_t d = 0; d < hk; d += 32) {
+        if (quarter == 32) {  // head dimension 128: the four 16-byte loads of the lane go out together
             uint4 kk[4];
 #pragma unroll
-            for (int c = 0; c < 4; c++) kk[c] = *reinterpret_cast<const uint4 *>(key + d + 8 * c);
+            for (int c = 0; c < 4; c++) kk[c] = *reinterpret_cast<const uint4 *>(key + 8 * c);
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 const uint32_t kw[4] = {kk[c].x, kk[c].y, kk[c].z, kk[c].w};
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const float p0 = h2f(qs[d + 8 * c + 2 * j]) * h2f(kw[j] & 0xffffu);
-                    sum += double(p0);
-                    const float p1 = h2f(qs[d + 8 * c + 2 * j + 1]) * h2f(kw[j] >> 16);
-                    sum += double(p1);
+                    sum = __builtin_fma(double(h2f(kw[j] & 0xffffu)), qq[8 * c + 2 * j], sum);
+                    sum = __builtin_fma(double(h2f(kw[j] >> 16)), qq[8 * c + 2 * j + 1], sum);
+                }
+            }
+        } else {
+            for (uint32_t d = 0; d < quarter; d += 8) {
+                const uint4 kk = *reinterpret_cast<const uint4 *>(key + d);
+                const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    sum = __builtin_fma(double(h2f(kw[j] & 0xffffu)), qq[d + 2 * j], sum);
+                    sum = __builtin_fma(double(h2f(kw[j] >> 16)), qq[d + 2 * j + 1], sum);
                 }
             }
         }
-        const float s = float(sum) * kq_scale;
-        scores[t] = s;
-        my_max = fmaxf(my_max, s);
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        if (live) {
+            const float s = float(sum) * kq_scale;
+            if (lane4 == 0) scores[t] = s;
+            my_max = fmaxf(my_max, s);
+        }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) my_max = fmaxf(my_max, __shfl_xor(my_max, off, 64));
     if ((tid & 63) == 0) red_f[tid >> 6] = my_max;
     __syncthreads();
-    const float max_val = fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3]));
-    for (uint32_t t = tid; t < n_keys4; t += 256) scores[t] = t < n_keys ? rmi_expf(scores[t] - max_val) : 0.0f;
+    float max_val = red_f[0];
+#pragma unroll
+    for (uint32_t i = 1; i < kAttnThreads / 64; i++) max_val = fmaxf(max_val, red_f[i]);
+    for (uint32_t t = tid; t < n_pad; t += kAttnThreads) scores[t] = t < n_keys ? rmi_expf(scores[t] - max_val) : 0.0f;
     __syncthreads();
-    if (tid == 0) {  // the reference adds the weights one after the other in f32; adding the zeros changes nothing
+    if (tid == 0) {  // the reference adds the weights one after the other in f32; the padding zeros change nothing
         float acc = 0.0f;
-        for (uint32_t t = 0; t < n_keys4; t += 4) {
+        for (uint32_t t = 0; t < n_pad; t += 4) {
             const float4 e = *reinterpret_cast<const float4 *>(scores + t);
             acc += e.x;
             acc += e.y;
@@ -228,31 +269,30 @@ __global__ __launch_bounds__(256) void attention_quant_kernel(const uint16_t *__
     }
     __syncthreads();
     const float sum = red_f[0];
-    for (uint32_t t = tid; t < n_keys_b; t += 256) {
-        const float e = t < n_keys ? scores[t] : 0.0f;
-        w16[t] = t < n_keys ? f2h(sum > 0.0f ? e / sum : e) : uint16_t(0);
+    for (uint32_t t = tid; t < n_pad; t += kAttnThreads) {
+        const float e = scores[t];
+        wd[t] = t < n_keys ? double(h2f(f2h(sum > 0.0f ? e / sum : e))) : 0.0;
     }
     __syncthreads();
-    for (uint32_t d = tid; d < hv; d += 256) {
-        const uint16_t *col = v_cache + size_t(kvh) * hv + d;
+
+    if (v_lane) {
         double acc = 0.0;
-        uint16_t cur[kAttnBatch], nxt[kAttnBatch];
 #pragma unroll
-        for (uint32_t j = 0; j < kAttnBatch; j++) cur[j] = j < n_keys ? col[size_t(j) * kv_stride] : uint16_t(0);
-        for (uint32_t t0 = 0; t0 < n_keys; t0 += kAttnBatch) {
+        for (uint32_t j = 0; j < kPre; j++)  // keys past n_keys carry weight zero
+            if (t_begin + j < t_end) acc = __builtin_fma(double(h2f(pre[j])), wd[t_begin + j], acc);
+        for (uint32_t t0 = t_begin + kPre; t0 < t_end; t0 += 8) {
+            uint32_t cur[8];
 #pragma unroll
-            for (uint32_t j = 0; j < kAttnBatch; j++) {  // the next batch is in flight while this one is added
-                const uint32_t t = t0 + kAttnBatch + j;
-                nxt[j] = t < n_keys ? col[size_t(t) * kv_stride] : uint16_t(0);
-            }
+            for (uint32_t j = 0; j < 8; j++) cur[j] = col[size_t(t0 + j < n_keys ? t0 + j : n_keys - 1) * kv_stride];
 #pragma unroll
-            for (uint32_t j = 0; j < kAttnBatch; j++) {  // keys past n_keys add +0.0, as the reference's padding does
-                const float p = h2f(cur[j]) * h2f(w16[t0 + j]);
-                acc += double(p);
-            }
-#pragma unroll
-            for (uint32_t j = 0; j < kAttnBatch; j++) cur[j] = nxt[j];
+            for (uint32_t j = 0; j < 8; j++) acc = __builtin_fma(double(h2f(cur[j])), wd[t0 + j], acc);
         }
+        part[size_t(slice) * hv + vd] = acc;
+    }
+    __syncthreads();
+    for (uint32_t d = tid; d < hv; d += kAttnThreads) {
+        double acc = part[d];
+        for (uint32_t sl = 1; sl < n_slices; sl++) acc += part[size_t(sl) * hv + d];
         outv[d] = float(acc);
     }
     __syncthreads();
@@ -451,7 +491,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, uint32_t n_prompt, hipStream_t
                            s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv,
                            c.head_dim_k, c.head_dim_v, c.eps);
         const size_t layer_base = size_t(l) * c.capacity * s->kv_stride;
-        hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(256), attn_lds, st, s->q16,
+        hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(kAttnThreads), attn_lds, st, s->q16,
                            s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv,
                            c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
         rc = gemv(s->w_o[l], s->act_q8, s->act_scales, s->resid, st);
@@ -537,11 +577,11 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     RMI_REQUIRE_INIT();
     if (!q16 || !k_cache || !v_cache || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
     if (n_keys == 0 || n_head == 0 || n_head_kv == 0 || n_head % n_head_kv || head_dim_k % 32 || head_dim_v % 32 ||
-        head_dim_k == 0 || head_dim_v == 0 || kv_stride % 8)
+        head_dim_k == 0 || head_dim_v == 0 || head_dim_k > 1024 || head_dim_v > 1024 || kv_stride % 8)
         return rmi_fail(RMI_HIP_E_INVALID, "bad attention shape");
     const size_t lds = attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
     if (lds > 64 * 1024) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
-    hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(256), lds, static_cast<hipStream_t>(stream), q16,
+    hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream), q16,
                        k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8, scales,
                        rounding);
     RMI_HIP_CHECK(hipGetLastError());
@@ -572,7 +612,7 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
     const rmi_hip_qwen3_config &c = *cfg;
     if (c.n_embd == 0 || c.n_embd % 32 || c.n_ff == 0 || c.n_ff % 32 || c.n_layer == 0 || c.n_head == 0 ||
         c.n_head_kv == 0 || c.n_head % c.n_head_kv || c.head_dim_k == 0 || c.head_dim_k % 32 || c.head_dim_v == 0 ||
-        c.head_dim_v % 32 || c.vocab == 0 || c.capacity == 0 ||
+        c.head_dim_v % 32 || c.head_dim_k > 1024 || c.head_dim_v > 1024 || c.vocab == 0 || c.capacity == 0 ||
         (c.rounding != RMI_HIP_ROUND_TIES_EVEN && c.rounding != RMI_HIP_ROUND_HALF_AWAY)) {
         rmi_set_error("unsupported model shape");
         return nullptr;
