@@ -570,6 +570,8 @@ def main():
                     help="also launch the plain copy kernel on this many MiB, 5 times, outside the timed region "
                          "(the known-size kernel that rocprofv3 --pmc traffic counters are scaled against)")
     ap.add_argument("--extra", action="store_true", help="also time the other launch modes, outside the timed region")
+    ap.add_argument("--no-decode", action="store_true",
+                    help="projection_set only: skip the end-to-end decode figure that is attached to the JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across GPUs", file=sys.stderr)
@@ -579,7 +581,17 @@ def main():
     pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
     ev = HipEvents()
     run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4k": run_q4k, "decode": run_decode}[args.workload]
-    print(json.dumps(run(args, pkg, ev)), flush=True)
+    result = run(args, pkg, ev)
+    if args.workload == "projection_set" and not args.no_decode and args.batch == 1:
+        # the second half of the headline metric: end-to-end decode tok/s of the same model shape, measured
+        # after (and outside) the timed GEMV region
+        sub = argparse.Namespace(**vars(args))
+        sub.steps, sub.warmup = 2, 1
+        d = run_decode(sub, pkg, ev)
+        result["decode"] = {"value": d["value"], "unit": d["unit"], "ms_per_token_step": d["ms_per_token_step"],
+                            "workload": d["config"]["workload"], "generations_timed": sub.steps,
+                            "cpu_baseline": d.get("cpu_baseline")}
+    print(json.dumps(result), flush=True)
 
 
 if __name__ == "__main__":
