@@ -154,6 +154,11 @@ int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
 int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
                               const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride,
                               uint32_t row_start, uint32_t row_end, void *stream);
+/* Y[t][:] = vec_dot_q4k_q8k(W, Q8_K(X[t][:])) for many tokens through int8 MFMA (Kernel::forward_batched,
+ * src/ops/kernel/trait_.rs:78-109, on Q4_KKernel::forward_prepared, src/ops/kernel/q4_k.rs:56-93): exact
+ * integers, the f32 sums within rounding of the CPU kernels. */
+int rmi_hip_gemm_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                              const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride, void *stream);
 int rmi_hip_quantize_row_q8_k_dev(const float *x, float *d, int8_t *qs, int16_t *bsums, uint32_t n_tokens,
                                   uint32_t n_in, void *stream);
 

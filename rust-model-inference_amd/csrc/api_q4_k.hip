@@ -5,6 +5,8 @@
 
 namespace {
 
+constexpr uint32_t kGemmMinTokens = 16;
+
 int check_q4k(const rmi_hip_weight *w, uint32_t n_in, uint32_t n_out) {
     if (!w || w->dtype != RMI_HIP_DTYPE_Q4_K) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_K weight handle");
     if (w->n_in != n_in || w->n_out != n_out)
@@ -89,7 +91,9 @@ int rmi_hip_q4_k_forward_batched(const rmi_hip_weight *w, const float *input, fl
     if (!d_x || !d_qs || !d_bs || !d_d || !d_y) return RMI_HIP_E_RUNTIME;
     rc = rmi_launch_quantize_q8_k(d_x, d_d, d_qs, d_bs, n_tokens, n_in, c->stream);
     if (rc != RMI_HIP_OK) return rc;
-    rc = rmi_launch_gemv_q4_k(w, d_d, d_qs, d_bs, d_y, n_tokens, n_out, 0, n_out, c->stream);
+    // prefill: the matrix-core GEMM; a few tokens: the GEMV in the x86-64 kernel's order
+    rc = n_tokens >= kGemmMinTokens ? rmi_launch_gemm_q4_k(w, d_d, d_qs, d_bs, d_y, n_tokens, n_out, c->stream)
+                                    : rmi_launch_gemv_q4_k(w, d_d, d_qs, d_bs, d_y, n_tokens, n_out, 0, n_out, c->stream);
     if (rc != RMI_HIP_OK) return rc;
     return fetch(c, output, d_y, size_t(n_tokens) * n_out * 4, 1);
 }
@@ -181,6 +185,21 @@ int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
     if (!q8k_d || !q8k_qs || !q8k_bsums || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
     return rmi_launch_gemv_q4_k(w, q8k_d, q8k_qs, q8k_bsums, y, n_tokens, y_stride, row_start, row_end,
                                 static_cast<hipStream_t>(stream));
+}
+
+int rmi_hip_gemm_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                              const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_K) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_K weight handle");
+    if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
+    if (y_stride < w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < n_out=%u", y_stride, w->n_out);
+    if (!q8k_d || !q8k_qs || !q8k_bsums || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (w->n_units == 0) {
+        RMI_HIP_CHECK(hipMemset2DAsync(y, size_t(y_stride) * 4, 0, size_t(w->n_out) * 4, n_tokens,
+                                       static_cast<hipStream_t>(stream)));
+        return RMI_HIP_OK;
+    }
+    return rmi_launch_gemm_q4_k(w, q8k_d, q8k_qs, q8k_bsums, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
 }
 
 rmi_hip_gemv_group *rmi_hip_gemv_group_create_q4_k(uint32_t n_problems, const rmi_hip_weight *const *weights,

@@ -143,6 +143,8 @@ int rmi_launch_gemv_q4_k_group(const RmiQ4kProblem *d_list, const uint4 *d_runs,
                                uint32_t max_n_sb, uint32_t n_tokens, hipStream_t s);
 int rmi_launch_gemv_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s);
+int rmi_launch_gemm_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
+                         uint32_t n_tokens, uint32_t y_stride, hipStream_t s);
 int rmi_launch_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *qs, const int16_t *bsums, int32_t *isum,
                                int32_t *msum, hipStream_t s);
 // mode 0: x = q8 * scale rebuilt per element (Q4_KKernel::forward_prequantized)

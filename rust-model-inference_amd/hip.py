@@ -82,6 +82,7 @@ SIGNATURES = {
     "rmi_hip_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, _u32, C.c_int, _vp]),
     "rmi_hip_gemm_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "rmi_hip_gemm_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_quantize_row_q8_k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_group_create": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u32]),
     "rmi_hip_gemv_group_create_q4_k": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),

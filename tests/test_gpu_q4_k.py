@@ -134,6 +134,36 @@ def test_q4k_forward_batched(hip, oracle, n_tokens):
         assert np.array_equal(bits(out[t]), bits(ref)), t
 
 
+@pytest.mark.parametrize("n_tokens,n_out,n_in", [(64, 1000, 512), (37, 45, 256), (130, 6144, 2048), (300, 200, 6144),
+                                                  (16, 8, 256)])
+def test_q4k_gemm_mfma_parity(hip, oracle, n_tokens, n_out, n_in):
+    """Prefill (>= 16 tokens) goes through the matrix cores: the integers are exact, the f32 sums run in one
+    chain per output instead of the AVX2 kernel's lane chains.  Within 1e-4 + 1e-4*|ref| of the AVX2-order
+    result, within the reference's own 1e-3 of the scalar one, and within 2e-6 relative of the f64 sum over
+    the exact per-super-block integers."""
+    w = hip.synth.q4_k_weight(80 + n_tokens, n_out, n_in)
+    x = hip.synth.activations(81 + n_out, n_tokens, n_in)
+    out = np.zeros((n_tokens, n_out), np.float32)
+    hip.kernel.Q4_KKernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out)
+    wr = w.reshape(n_out, -1, 144)
+    wd = wr[:, :, 0:2].copy().view(np.float16)[:, :, 0].astype(np.float64)
+    wdmin = wr[:, :, 2:4].copy().view(np.float16)[:, :, 0].astype(np.float64)
+    rows = np.unique(np.linspace(0, n_out - 1, min(n_out, 24)).astype(int))
+    for t in np.unique(np.linspace(0, n_tokens - 1, min(n_tokens, 12)).astype(int)):
+        d, qs, bs = oracle.quantize_row_q8_k(x[t], A)
+        ref = np.zeros(n_out, np.float32)
+        oracle.q4k_forward_prepared(w, d, qs, bs, ref, n_in, n_out, 0, 1, A)
+        assert np.all(np.abs(out[t] - ref) <= 1e-4 + 1e-4 * np.abs(ref)), t
+        refs = np.zeros(n_out, np.float32)
+        oracle.q4k_forward_prepared(w, d, qs, bs, refs, n_in, n_out, 0, 1, S)
+        assert np.all(np.abs(out[t] - refs) <= 1e-3 * np.maximum(np.abs(refs), 1.0)), t
+        for r in rows:
+            isum, msum = oracle.q4k_q8k_block_ints(wr[r].reshape(-1), qs, bs)
+            exact = np.sum(wd[r] * d.astype(np.float64) * isum - wdmin[r] * d.astype(np.float64) * msum)
+            scale = np.sum(np.abs(wd[r] * d * isum) + np.abs(wdmin[r] * d * msum))
+            assert abs(float(out[t, r]) - exact) <= 2e-6 * scale + 1e-30, (t, r)
+
+
 # ----------------------------------------------------------------- dequant paths
 
 def test_q4k_grouped_launch_bit_exact(hip, oracle):
