@@ -174,6 +174,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
     int8_t *__restrict__ q8, float *__restrict__ scales, int rounding) {
     extern __shared__ double lds_d[];
     __shared__ float red_f[kAttnThreads / 64];
+    __shared__ uint64_t exp_tab[32];
     const uint32_t head = blockIdx.x, tid = threadIdx.x;
     const uint32_t kvh = head / (n_head / n_head_kv);
     const uint32_t n_keys = step + 1;
@@ -185,6 +186,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
     float *scores = reinterpret_cast<float *>(part + size_t(n_slices) * hv);  // [n_pad]
     float *outv = scores + n_pad;                                // [hv]
     for (uint32_t d = tid; d < hk; d += kAttnThreads) qd[d] = double(h2f(q16[size_t(head) * hk + d]));
+    if (tid < 32) exp_tab[tid] = kRmiExp2fTab[tid];
 
     // values: hv columns x n_slices ranges of keys.  The first loads of this thread's range go out now and
     // arrive while the scores and the softmax are computed.
@@ -203,22 +205,33 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
         pre[j] = col[size_t(t) * kv_stride];
     }
 
-    __syncthreads();
-
-    // scores: four lanes per key, a quarter of the head dimension each; the next round's key is loaded ahead
+    // scores: four lanes per key, a quarter of the head dimension each.  For head dimension 128 the first
+    // round's keys are loaded here, with the values above, so that one memory round trip covers all of them.
     const float kq_scale = 1.0f / sqrtf(float(hk));
     const uint32_t quarter = hk >> 2, lane4 = tid & 3;
     const double *qq = qd + lane4 * quarter;
-    float my_max = -INFINITY;
-    for (uint32_t t0 = 0; t0 < n_keys; t0 += kAttnThreads / 4) {
-        const uint32_t t = t0 + (tid >> 2);
-        const bool live = t < n_keys;
-        const uint16_t *key = k_cache + size_t(live ? t : 0) * kv_stride + size_t(kvh) * hk + lane4 * quarter;
-        double sum = 0.0;
-        if (quarter == 32) {  // head dimension 128: the four 16-byte loads of the lane go out together
-            uint4 kk[4];
+    uint4 kk0[4];
+    if (quarter == 32) {
+        const uint32_t t = (tid >> 2) < n_keys ? (tid >> 2) : 0;
+        const uint16_t *key = k_cache + size_t(t) * kv_stride + size_t(kvh) * hk + lane4 * quarter;
 #pragma unroll
-            for (int c = 0; c < 4; c++) kk[c] = *reinterpret_cast<const uint4 *>(key + 8 * c);
+        for (int c = 0; c < 4; c++) kk0[c] = *reinterpret_cast<const uint4 *>(key + 8 * c);
+    }
+    __syncthreads();
+
+    float my_max = -INFINITY;
+    if (quarter == 32) {  // head dimension 128: the keys of the next round are in flight while this one is summed
+        uint4 kk[4], kn[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) kk[c] = kk0[c];
+        for (uint32_t t0 = 0; t0 < n_keys; t0 += kAttnThreads / 4) {
+            const uint32_t t = t0 + (tid >> 2), tn = t + kAttnThreads / 4;
+            if (t0 + kAttnThreads / 4 < n_keys) {
+                const uint16_t *key = k_cache + size_t(tn < n_keys ? tn : 0) * kv_stride + size_t(kvh) * hk + lane4 * 32;
+#pragma unroll
+                for (int c = 0; c < 4; c++) kn[c] = *reinterpret_cast<const uint4 *>(key + 8 * c);
+            }
+            double sum = 0.0;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 const uint32_t kw[4] = {kk[c].x, kk[c].y, kk[c].z, kk[c].w};
@@ -228,7 +241,22 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
                     sum = __builtin_fma(double(h2f(kw[j] >> 16)), qq[8 * c + 2 * j + 1], sum);
                 }
             }
-        } else {
+            sum += __shfl_xor(sum, 1, 64);
+            sum += __shfl_xor(sum, 2, 64);
+            if (t < n_keys) {
+                const float s = float(sum) * kq_scale;
+                if (lane4 == 0) scores[t] = s;
+                my_max = fmaxf(my_max, s);
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++) kk[c] = kn[c];
+        }
+    } else {
+        for (uint32_t t0 = 0; t0 < n_keys; t0 += kAttnThreads / 4) {
+            const uint32_t t = t0 + (tid >> 2);
+            const bool live = t < n_keys;
+            const uint16_t *key = k_cache + size_t(live ? t : 0) * kv_stride + size_t(kvh) * hk + lane4 * quarter;
+            double sum = 0.0;
             for (uint32_t d = 0; d < quarter; d += 8) {
                 const uint4 kk = *reinterpret_cast<const uint4 *>(key + d);
                 const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w};
@@ -238,13 +266,13 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
                     sum = __builtin_fma(double(h2f(kw[j] >> 16)), qq[d + 2 * j + 1], sum);
                 }
             }
-        }
-        sum += __shfl_xor(sum, 1, 64);
-        sum += __shfl_xor(sum, 2, 64);
-        if (live) {
-            const float s = float(sum) * kq_scale;
-            if (lane4 == 0) scores[t] = s;
-            my_max = fmaxf(my_max, s);
+            sum += __shfl_xor(sum, 1, 64);
+            sum += __shfl_xor(sum, 2, 64);
+            if (live) {
+                const float s = float(sum) * kq_scale;
+                if (lane4 == 0) scores[t] = s;
+                my_max = fmaxf(my_max, s);
+            }
         }
     }
 #pragma unroll
@@ -254,7 +282,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
     float max_val = red_f[0];
 #pragma unroll
     for (uint32_t i = 1; i < kAttnThreads / 64; i++) max_val = fmaxf(max_val, red_f[i]);
-    for (uint32_t t = tid; t < n_pad; t += kAttnThreads) scores[t] = t < n_keys ? rmi_expf(scores[t] - max_val) : 0.0f;
+    for (uint32_t t = tid; t < n_pad; t += kAttnThreads) scores[t] = t < n_keys ? rmi_expf_tab(scores[t] - max_val, exp_tab) : 0.0f;
     __syncthreads();
     if (tid == 0) {  // the reference adds the weights one after the other in f32; the padding zeros change nothing
         float acc = 0.0f;
@@ -280,12 +308,24 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
 #pragma unroll
         for (uint32_t j = 0; j < kPre; j++)  // keys past n_keys carry weight zero
             if (t_begin + j < t_end) acc = __builtin_fma(double(h2f(pre[j])), wd[t_begin + j], acc);
-        for (uint32_t t0 = t_begin + kPre; t0 < t_end; t0 += 8) {
-            uint32_t cur[8];
+        if (t_begin + kPre < t_end) {  // longer ranges: batches of 8, the next one in flight while one is added
+            uint32_t cur[8], nxt[8];
 #pragma unroll
-            for (uint32_t j = 0; j < 8; j++) cur[j] = col[size_t(t0 + j < n_keys ? t0 + j : n_keys - 1) * kv_stride];
+            for (uint32_t j = 0; j < 8; j++) {
+                const uint32_t t = t_begin + kPre + j;
+                cur[j] = col[size_t(t < n_keys ? t : n_keys - 1) * kv_stride];
+            }
+            for (uint32_t t0 = t_begin + kPre; t0 < t_end; t0 += 8) {
 #pragma unroll
-            for (uint32_t j = 0; j < 8; j++) acc = __builtin_fma(double(h2f(cur[j])), wd[t0 + j], acc);
+                for (uint32_t j = 0; j < 8; j++) {
+                    const uint32_t t = t0 + 8 + j;
+                    nxt[j] = col[size_t(t < n_keys ? t : n_keys - 1) * kv_stride];
+                }
+#pragma unroll
+                for (uint32_t j = 0; j < 8; j++) acc = __builtin_fma(double(h2f(cur[j])), wd[t0 + j], acc);
+#pragma unroll
+                for (uint32_t j = 0; j < 8; j++) cur[j] = nxt[j];
+            }
         }
         part[size_t(slice) * hv + vd] = acc;
     }

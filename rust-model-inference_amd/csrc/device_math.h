@@ -12,9 +12,8 @@
 
 #include <cstdint>
 
-__device__ __forceinline__ float rmi_expf(float x) {
-    // 2^(i/32) as f64 bits, minus i << 47 so that adding k << 47 yields 2^(k/32)
-    static constexpr uint64_t kTab[32] = {
+// 2^(i/32) as f64 bits, minus i << 47 so that adding k << 47 yields 2^(k/32)
+__device__ static constexpr uint64_t kRmiExp2fTab[32] = {
     0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
     0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
     0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
@@ -23,7 +22,10 @@ __device__ __forceinline__ float rmi_expf(float x) {
     0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
     0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull,
-    };
+};
+
+// `tab` is kRmiExp2fTab or a copy of it in LDS (a kernel that calls this in a latency-bound phase copies it first)
+__device__ __forceinline__ float rmi_expf_tab(float x, const uint64_t *tab) {
     const uint32_t ux = __float_as_uint(x);
     const uint32_t abstop = (ux >> 20) & 0x7ff;
     if (abstop >= (0x42b00000u >> 20)) {  // |x| >= 88 or NaN
@@ -41,7 +43,7 @@ __device__ __forceinline__ float rmi_expf(float x) {
     const uint64_t ki = uint64_t(__double_as_longlong(kd));
     kd -= shift;
     const double r = __builtin_fma(inv_ln2_n, xd, -kd);
-    const uint64_t t = kTab[ki & 31] + (ki << 47);
+    const uint64_t t = tab[ki & 31] + (ki << 47);
     const double s = __longlong_as_double((long long)t);
     const double p = __builtin_fma(c0, r, c1);
     const double r2 = r * r;
@@ -50,3 +52,5 @@ __device__ __forceinline__ float rmi_expf(float x) {
     y = y * s;
     return float(y);
 }
+
+__device__ __forceinline__ float rmi_expf(float x) { return rmi_expf_tab(x, kRmiExp2fTab); }

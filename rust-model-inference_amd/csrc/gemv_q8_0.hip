@@ -114,6 +114,13 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
 
     const uint32_t n_oct = p.n_oct;
     const uint32_t tok_u4 = n_oct * 18;  // per token: 16 uint4 of quants + 2 of scales per octet
+    // The weight loads of the first tile go out before the activation is staged: the two round trips overlap.
+    OctetRegs ra, rb, rc, rd;
+    if (k < k_end) {
+        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * n_oct * kOctetBytes);
+        load_octet(ra, tile + r, tile + n_oct * 8 + lane, 0);
+        if (n_oct > 1) load_octet(rb, tile + r, tile + n_oct * 8 + lane, 1);
+    }
     {
         const uint32_t nb = p.n_in >> 5;
         uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
@@ -131,7 +138,7 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
         __syncthreads();
     }
 
-    for (; k < k_end; k++) {
+    for (bool first = true; k < k_end; k++, first = false) {
         gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * n_oct * kOctetBytes);
         gptr_u4 sc_ptr = tile + r;
         gptr_u4 q_ptr = tile + n_oct * 8 + lane;
@@ -143,9 +150,10 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
         // Software pipeline over the octets of the tile: while one pair of octets is
         // multiplied, the loads of the next pair are in flight.  The accumulation
         // order over blocks stays strictly ascending.
-        OctetRegs ra, rb, rc, rd;
-        load_octet(ra, sc_ptr, q_ptr, 0);
-        if (n_oct > 1) load_octet(rb, sc_ptr, q_ptr, 1);
+        if (!first) {
+            load_octet(ra, sc_ptr, q_ptr, 0);
+            if (n_oct > 1) load_octet(rb, sc_ptr, q_ptr, 1);
+        }
         for (uint32_t o = 0; o < n_oct; o += 4) {
             if (o + 2 < n_oct) load_octet(rc, sc_ptr, q_ptr, o + 2);
             if (o + 3 < n_oct) load_octet(rd, sc_ptr, q_ptr, o + 3);
