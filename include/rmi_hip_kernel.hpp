@@ -217,4 +217,36 @@ class QuantizedLinear : public Layer {
     std::string name_;
 };
 
+// Qwen3Session (src/models/qwen3.rs:581-1158) with the whole token step on the device.
+class Qwen3Session {
+  public:
+    Qwen3Session(const rmi_hip_qwen3_config &cfg, const rmi_hip_qwen3_weights &weights)
+        : cfg_(cfg), h_(rmi_hip_qwen3_create(&cfg, &weights)) {
+        if (!h_) throw HipError(RMI_HIP_E_RUNTIME, rmi_hip_last_error());
+    }
+    ~Qwen3Session() { rmi_hip_qwen3_destroy(h_); }
+    Qwen3Session(const Qwen3Session &) = delete;
+    Qwen3Session &operator=(const Qwen3Session &) = delete;
+    // greedy generation; per step the argmax and the two largest logits if the vectors are given
+    std::vector<uint32_t> generate(const std::vector<uint32_t> &prompt, uint32_t max_new,
+                                   std::vector<uint32_t> *step_argmax = nullptr, std::vector<float> *step_top2 = nullptr,
+                                   double *seconds = nullptr) {
+        const size_t steps = prompt.size() + max_new - 1;
+        std::vector<uint32_t> out(max_new);
+        if (step_argmax) step_argmax->assign(steps, 0);
+        if (step_top2) step_top2->assign(2 * steps, 0.0f);
+        const int n = rmi_hip_qwen3_generate(h_, prompt.data(), uint32_t(prompt.size()), max_new, out.data(),
+                                             step_argmax ? step_argmax->data() : nullptr,
+                                             step_top2 ? step_top2->data() : nullptr, nullptr, 0, nullptr, seconds);
+        check(n < 0 ? n : 0);
+        out.resize(size_t(n));
+        return out;
+    }
+    const rmi_hip_qwen3_config &config() const { return cfg_; }
+
+  private:
+    rmi_hip_qwen3_config cfg_;
+    rmi_hip_qwen3 *h_;
+};
+
 }  // namespace rmi

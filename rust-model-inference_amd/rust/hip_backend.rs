@@ -192,5 +192,61 @@ impl<'a> Layer for HipLinear<'a> {
     fn name(&self) -> &str { self.layer_name }
 }
 
-#[allow(dead_code)]
-fn _unused(_: *mut c_void) {}
+// ---------------------------------------------------------------- device-resident decode
+//
+// `Qwen3Session::generate_inner` (src/models/qwen3.rs:581-1158) with every tensor in HBM between two
+// token ids.  The two structs mirror rmi_hip_qwen3_config / rmi_hip_qwen3_weights of rmi_hip.h.
+
+#[repr(C)]
+pub struct RmiQwen3Config {
+    pub n_embd: u32, pub n_layer: u32, pub n_head: u32, pub n_head_kv: u32, pub head_dim_k: u32, pub head_dim_v: u32,
+    pub n_ff: u32, pub vocab: u32, pub capacity: u32,
+    pub eps: f32, pub freq_base: f32,
+    pub has_qk_norm: i32, pub rounding: i32,
+}
+
+#[repr(C)]
+pub struct RmiQwen3Weights {
+    pub token_embd: *const u8, pub output: *const u8, pub output_norm: *const f32,
+    pub attn_norm: *const *const f32, pub ffn_norm: *const *const f32,
+    pub q_norm: *const *const f32, pub k_norm: *const *const f32,
+    pub wq: *const *const u8, pub wk: *const *const u8, pub wv: *const *const u8, pub wo: *const *const u8,
+    pub w_gate: *const *const u8, pub w_up: *const *const u8, pub w_down: *const *const u8,
+}
+
+extern "C" {
+    fn rmi_hip_qwen3_create(cfg: *const RmiQwen3Config, weights: *const RmiQwen3Weights) -> *mut c_void;
+    fn rmi_hip_qwen3_destroy(s: *mut c_void);
+    fn rmi_hip_qwen3_generate(s: *mut c_void, prompt: *const u32, n_prompt: u32, max_new: u32, generated: *mut u32,
+                              step_argmax: *mut u32, step_top2: *mut f32, dump_steps: *const u32, n_dump: u32,
+                              dump_logits: *mut f32, seconds: *mut f64) -> c_int;
+}
+
+/// Owns the HBM copy of a model and its KV cache.  Built from the tensors `Qwen3Model::from_gguf`
+/// (src/models/qwen3.rs:263-420) borrows from the mmap; the slices may be dropped after `new`.
+pub struct HipQwen3Session { handle: *mut c_void }
+unsafe impl Send for HipQwen3Session {}
+
+impl HipQwen3Session {
+    pub fn new(cfg: &RmiQwen3Config, weights: &RmiQwen3Weights) -> Result<Self, String> {
+        let handle = unsafe { rmi_hip_qwen3_create(cfg, weights) };
+        if handle.is_null() { Err(last_error()) } else { Ok(Self { handle }) }
+    }
+
+    /// Greedy generation, the prompt fed one token per step as `generate_inner` does.
+    pub fn generate(&mut self, prompt: &[u32], max_new: usize) -> Result<Vec<u32>, String> {
+        let mut out = vec![0u32; max_new];
+        let n = unsafe {
+            rmi_hip_qwen3_generate(self.handle, prompt.as_ptr(), prompt.len() as u32, max_new as u32, out.as_mut_ptr(),
+                                   std::ptr::null_mut(), std::ptr::null_mut(), std::ptr::null(), 0,
+                                   std::ptr::null_mut(), std::ptr::null_mut())
+        };
+        if n < 0 { return Err(last_error()); }
+        out.truncate(n as usize);
+        Ok(out)
+    }
+}
+
+impl Drop for HipQwen3Session {
+    fn drop(&mut self) { unsafe { rmi_hip_qwen3_destroy(self.handle) } }
+}

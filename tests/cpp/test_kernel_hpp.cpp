@@ -131,6 +131,52 @@ int main() {
         }
         EXPECT(threw);
     }
+    {
+        // device-resident decode of a one-layer toy model: runs, is deterministic, and the tokens it
+        // generates are the argmax of the steps that produced them
+        const uint32_t n_embd = 64, n_head = 2, n_kv = 1, hd = 32, n_ff = 96, vocab = 40, cap = 24;
+        auto q8 = [](uint32_t rows, uint32_t cols, uint32_t seed) {
+            std::vector<uint8_t> w(size_t(rows) * (cols / 32) * 34);
+            uint32_t s = seed * 2654435761u + 1;
+            for (size_t b = 0; b < w.size() / 34; b++) {
+                w[b * 34] = 0x00;
+                w[b * 34 + 1] = 0x1c;  // f16 0x1c00 = 2^-8
+                for (int k = 0; k < 32; k++) {
+                    s = s * 1664525u + 1013904223u;
+                    w[b * 34 + 2 + k] = uint8_t(int8_t(int(s >> 24) % 100));
+                }
+            }
+            return w;
+        };
+        auto embd = q8(vocab, n_embd, 1), wq = q8(n_head * hd, n_embd, 2), wk = q8(n_kv * hd, n_embd, 3),
+             wv = q8(n_kv * hd, n_embd, 4), wo = q8(n_embd, n_head * hd, 5), wg = q8(n_ff, n_embd, 6),
+             wu = q8(n_ff, n_embd, 7), wd = q8(n_embd, n_ff, 8);
+        std::vector<float> ones(96, 1.0f);
+        const float *norm = ones.data();
+        const uint8_t *pq = wq.data(), *pk = wk.data(), *pv = wv.data(), *po = wo.data(), *pg = wg.data(),
+                      *pu = wu.data(), *pd = wd.data();
+        rmi_hip_qwen3_config cfg{n_embd, 1, n_head, n_kv, hd, hd, n_ff, vocab, cap, 1e-6f, 1e6f, 1, RMI_HIP_ROUND_TIES_EVEN};
+        rmi_hip_qwen3_weights wt{embd.data(), nullptr, norm, &norm, &norm, &norm, &norm, &pq, &pk, &pv, &po, &pg, &pu, &pd};
+        rmi::Qwen3Session sess(cfg, wt);
+        std::vector<uint32_t> prompt = {3, 17, 5, 39, 0, 8}, am1, am2;
+        std::vector<float> top;
+        auto a = sess.generate(prompt, 10, &am1, &top);
+        auto b = sess.generate(prompt, 10, &am2);
+        EXPECT(a.size() == 10 && a == b && am1 == am2 && am1.size() == 15);
+        bool greedy = true;
+        for (size_t i = 0; i < a.size(); i++) greedy = greedy && a[i] == am1[prompt.size() - 1 + i] && a[i] < vocab;
+        EXPECT(greedy);
+        bool ordered = true;
+        for (size_t i = 0; i < am1.size(); i++) ordered = ordered && top[2 * i] >= top[2 * i + 1];
+        EXPECT(ordered);
+        bool threw = false;
+        try {
+            sess.generate(prompt, 30);  // beyond the capacity
+        } catch (const rmi::HipError &e) {
+            threw = e.code == RMI_HIP_E_INVALID;
+        }
+        EXPECT(threw);
+    }
     std::printf(failures ? "%d FAILED\n" : "all C++ interface checks passed\n", failures);
     return failures ? 1 : 0;
 }
