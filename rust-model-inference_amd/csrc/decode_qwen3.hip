@@ -42,6 +42,14 @@ __device__ __forceinline__ uint16_t f2h(float v) {
     return __builtin_bit_cast(uint16_t, _Float16(v));
 }
 
+// Where the session's kernels read the step from: with it in HBM every launch of a token-step has the same
+// arguments at every step (replaying the step as a HIP graph was measured: 676 vs 678 token-steps/s, no gain,
+// so the launches stay eager).  A null pointer means "use the value argument".
+struct StepParams {
+    uint32_t step;      // position of the token being processed = row of the KV cache
+    uint32_t n_prompt;  // steps below n_prompt - 1 read their token from the prompt
+};
+
 __device__ __forceinline__ double wave_sum(double v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -50,9 +58,10 @@ __device__ __forceinline__ double wave_sum(double v) {
 
 // x[e] = d * q of row `token` of a Q8_0 weight in the GEMV tile stream
 __global__ __launch_bounds__(256) void embed_q8_0_kernel(const uint8_t *__restrict__ w, uint32_t n_oct,
-                                                          const uint32_t *__restrict__ tok, uint32_t step,
-                                                          uint32_t vocab, float *__restrict__ x, uint32_t n_embd) {
-    uint32_t token = tok[step];
+                                                          const uint32_t *__restrict__ tok,
+                                                          const StepParams *__restrict__ sp, uint32_t vocab,
+                                                          float *__restrict__ x, uint32_t n_embd) {
+    uint32_t token = tok[sp->step];
     if (token >= vocab) token = vocab - 1;  // ids are validated on the host; never read outside the weight
     const uint8_t *tile = w + size_t(token >> 3) * n_oct * kOctetBytes;
     const uint32_t r = token & 7;
@@ -117,8 +126,14 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(const float *__r
                                                                 const float *__restrict__ sin_t, uint32_t pos,
                                                                 uint16_t *__restrict__ q16, uint16_t *__restrict__ k_row,
                                                                 uint16_t *__restrict__ v_row, uint32_t n_head,
-                                                                uint32_t n_head_kv, uint32_t hk, uint32_t hv, float eps) {
+                                                                uint32_t n_head_kv, uint32_t hk, uint32_t hv, float eps,
+                                                                const StepParams *__restrict__ sp, uint32_t kv_stride) {
     const uint32_t head = blockIdx.x, tid = threadIdx.x;
+    if (sp) {  // session: position and cache row follow the step counter (k_row, v_row = the layer's cache)
+        pos = sp->step;
+        k_row += size_t(pos) * kv_stride;
+        v_row += size_t(pos) * kv_stride;
+    }
     if (head >= n_head + n_head_kv) {  // v: rounding only
         const uint32_t kvh = head - n_head - n_head_kv;
         const float *src = qkv + size_t(n_head) * hk + size_t(n_head_kv) * hk + size_t(kvh) * hv;
@@ -171,13 +186,13 @@ __host__ __device__ inline size_t attn_lds_bytes(uint32_t n_keys, uint32_t hk, u
 __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
     uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, uint32_t hk, uint32_t hv,
-    int8_t *__restrict__ q8, float *__restrict__ scales, int rounding) {
+    int8_t *__restrict__ q8, float *__restrict__ scales, int rounding, const StepParams *__restrict__ sp) {
     extern __shared__ double lds_d[];
     __shared__ float red_f[kAttnThreads / 64];
     __shared__ uint64_t exp_tab[32];
     const uint32_t head = blockIdx.x, tid = threadIdx.x;
     const uint32_t kvh = head / (n_head / n_head_kv);
-    const uint32_t n_keys = step + 1;
+    const uint32_t n_keys = (sp ? sp->step : step) + 1;
     const uint32_t n_pad = (n_keys + kAttnPad - 1) / kAttnPad * kAttnPad;
     const uint32_t n_slices = kAttnThreads / hv ? kAttnThreads / hv : 1;
     double *wd = lds_d;                                          // [n_pad] softmax weights (f16 values), 0 beyond n_keys
@@ -409,7 +424,7 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__rest
     if (threadIdx.x == 0) partial[blockIdx.x] = r;
 }
 __global__ __launch_bounds__(256) void argmax_final_kernel(const Top *__restrict__ partial, uint32_t n_partial,
-                                                           uint32_t step, uint32_t n_prompt,
+                                                           StepParams *__restrict__ sp,
                                                            uint32_t *__restrict__ tok, uint32_t *__restrict__ step_argmax,
                                                            float *__restrict__ step_top2,
                                                            uint32_t *__restrict__ nonfinite_steps) {
@@ -418,11 +433,13 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const Top *__restrict
     for (uint32_t i = threadIdx.x; i < n_partial; i += 256) t = top_merge(t, partial[i]);
     const Top r = top_block_reduce(t, sm);
     if (threadIdx.x == 0) {
+        const uint32_t step = sp->step, n_prompt = sp->n_prompt;
         step_argmax[step] = r.id;
         step_top2[2 * step] = r.best;
         step_top2[2 * step + 1] = r.second;
         if (!r.finite) atomicAdd(nonfinite_steps, 1u);
         if (step + 1 >= n_prompt) tok[step + 1] = r.id;  // the next step reads its token here
+        sp->step = step + 1;                             // last kernel of the step: the next one sees the new position
     }
 }
 
@@ -444,6 +461,7 @@ struct rmi_hip_qwen3 {
     uint32_t *tok = nullptr, *step_argmax = nullptr, *nonfinite = nullptr;
     float *step_top2 = nullptr;
     void *partial = nullptr;
+    void *params = nullptr;              // StepParams in HBM
     std::vector<void *> owned;  // every other device allocation, freed with the session
 };
 
@@ -512,28 +530,29 @@ int gemv(const rmi_hip_weight *w, const int8_t *q8, const float *scales, float *
     return rmi_launch_gemv_q8_0_single(p, 1, st);
 }
 
-// one decoder step: token tok[step] at position `step`; leaves logits, argmax and the next token on the device
-int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, uint32_t n_prompt, hipStream_t st) {
+// One decoder step: the token and the position come from the step counter in HBM, so every launch has the
+// same arguments at every step.  Leaves logits, argmax and the next token on the device and advances the counter.
+int enqueue_step(rmi_hip_qwen3 *s, hipStream_t st) {
     const rmi_hip_qwen3_config &c = s->cfg;
     const int rnd = c.rounding;
-    const size_t attn_lds = attn_lds_bytes(step + 1, c.head_dim_k, c.head_dim_v);
-    hipLaunchKernelGGL(embed_q8_0_kernel, dim3(1), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, step,
-                       c.vocab, s->x, c.n_embd);
+    StepParams *sp = static_cast<StepParams *>(s->params);
+    const size_t attn_lds = attn_lds_bytes(c.capacity, c.head_dim_k, c.head_dim_v);
+    hipLaunchKernelGGL(embed_q8_0_kernel, dim3(1), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, sp, c.vocab,
+                       s->x, c.n_embd);
     const float *pending = nullptr;  // matmul output still to be added to the residual stream
     for (uint32_t l = 0; l < c.n_layer; l++) {
         hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, pending, s->attn_norm[l], c.n_embd,
                            c.eps, s->act_q8, s->act_scales, rnd);
         int rc = gemv(s->w_qkv[l], s->act_q8, s->act_scales, s->qkv, st);
         if (rc != RMI_HIP_OK) return rc;
-        const size_t row = (size_t(l) * c.capacity + step) * s->kv_stride;
+        const size_t layer_base = size_t(l) * c.capacity * s->kv_stride;
         hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv), dim3(64), 0, st, s->qkv,
                            c.has_qk_norm ? s->q_norm[l] : nullptr, c.has_qk_norm ? s->k_norm[l] : nullptr, s->cos_t,
-                           s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv,
-                           c.head_dim_k, c.head_dim_v, c.eps);
-        const size_t layer_base = size_t(l) * c.capacity * s->kv_stride;
+                           s->sin_t, 0u, s->q16, s->k_cache + layer_base, s->v_cache + layer_base, c.n_head,
+                           c.n_head_kv, c.head_dim_k, c.head_dim_v, c.eps, sp, s->kv_stride);
         hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(kAttnThreads), attn_lds, st, s->q16,
-                           s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv,
-                           c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
+                           s->k_cache + layer_base, s->v_cache + layer_base, 0u, s->kv_stride, c.n_head, c.n_head_kv,
+                           c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd, sp);
         rc = gemv(s->w_o[l], s->act_q8, s->act_scales, s->resid, st);
         if (rc != RMI_HIP_OK) return rc;
         hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, s->resid, s->ffn_norm[l], c.n_embd,
@@ -553,7 +572,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, uint32_t n_prompt, hipStream_t
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxGroups), dim3(256), 0, st, s->logits, c.vocab,
                        static_cast<Top *>(s->partial));
     hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, static_cast<const Top *>(s->partial),
-                       kArgmaxGroups, step, n_prompt, s->tok, s->step_argmax, s->step_top2, s->nonfinite);
+                       kArgmaxGroups, sp, s->tok, s->step_argmax, s->step_top2, s->nonfinite);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -605,7 +624,7 @@ int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const fl
     if (n_head == 0 || n_head_kv == 0 || head_dim_k % 2) return rmi_fail(RMI_HIP_E_INVALID, "bad head shape");
     hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(n_head + 2 * n_head_kv), dim3(64), 0,
                        static_cast<hipStream_t>(stream), qkv, q_norm, k_norm, cos_row, sin_row, 0u, q16, k_row, v_row,
-                       n_head, n_head_kv, head_dim_k, head_dim_v, eps);
+                       n_head, n_head_kv, head_dim_k, head_dim_v, eps, static_cast<const StepParams *>(nullptr), 0u);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -623,7 +642,7 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     if (lds > 64 * 1024) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
     hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream), q16,
                        k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8, scales,
-                       rounding);
+                       rounding, static_cast<const StepParams *>(nullptr));
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -636,7 +655,7 @@ void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s) {
     for (auto *w : s->w_o) rmi_hip_free_weight(w);
     for (auto *w : s->w_gu) rmi_hip_free_weight(w);
     for (auto *w : s->w_down) rmi_hip_free_weight(w);
-    for (void *p : s->owned) hipFree(p);
+    for (void *p : s->owned) (void)hipFree(p);
     delete s;
 }
 
@@ -737,7 +756,8 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
          (s->tok = dev_alloc<uint32_t>(s, size_t(c.capacity) + 1, true)) &&
          (s->step_argmax = dev_alloc<uint32_t>(s, c.capacity, true)) &&
          (s->step_top2 = dev_alloc<float>(s, size_t(2) * c.capacity, true)) &&
-         (s->nonfinite = dev_alloc<uint32_t>(s, 1, true)) && (s->partial = dev_alloc<Top>(s, kArgmaxGroups));
+         (s->nonfinite = dev_alloc<uint32_t>(s, 1, true)) && (s->partial = dev_alloc<Top>(s, kArgmaxGroups)) &&
+         (s->params = dev_alloc<StepParams>(s, 1, true));
     if (!ok) {
         rmi_hip_qwen3_destroy(s);
         return nullptr;
@@ -767,12 +787,14 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
         RMI_HIP_CHECK(hipMalloc(reinterpret_cast<void **>(&d_dump), size_t(n_dump) * c.vocab * 4));
     }
     int rc = RMI_HIP_OK;
+    const StepParams start{0u, n_prompt};
     hipError_t e = hipMemcpyAsync(s->tok, prompt, size_t(n_prompt) * 4, hipMemcpyHostToDevice, st);
+    if (e == hipSuccess) e = hipMemcpyAsync(s->params, &start, sizeof start, hipMemcpyHostToDevice, st);
     if (e == hipSuccess) e = hipMemsetAsync(s->nonfinite, 0, 4, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     const auto t0 = std::chrono::steady_clock::now();
     for (uint32_t step = 0; e == hipSuccess && rc == RMI_HIP_OK && step < steps; step++) {
-        rc = enqueue_step(s, step, n_prompt, st);
+        rc = enqueue_step(s, st);
         for (uint32_t d = 0; rc == RMI_HIP_OK && d < n_dump; d++)
             if (dump_steps[d] == step)
                 e = hipMemcpyAsync(d_dump + size_t(d) * c.vocab, s->logits, size_t(c.vocab) * 4, hipMemcpyDeviceToDevice, st);
@@ -787,7 +809,7 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
         if (e == hipSuccess && n_dump) e = hipMemcpy(dump_logits, d_dump, size_t(n_dump) * c.vocab * 4, hipMemcpyDeviceToHost);
         if (e == hipSuccess) e = hipMemcpy(&nonfinite, s->nonfinite, 4, hipMemcpyDeviceToHost);
     }
-    if (d_dump) hipFree(d_dump);
+    if (d_dump) (void)hipFree(d_dump);
     if (rc != RMI_HIP_OK) return rc;
     if (e != hipSuccess) return rmi_fail(RMI_HIP_E_RUNTIME, "decode failed: %s", hipGetErrorString(e));
     if (nonfinite) return rmi_fail(RMI_HIP_E_RUNTIME, "non-finite logits in %u steps", nonfinite);
