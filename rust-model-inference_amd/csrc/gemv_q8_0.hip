@@ -55,8 +55,8 @@ struct OctetRegs {
 
 __device__ __forceinline__ void load_octet(OctetRegs &g, gptr_u4 sc_ptr, gptr_u4 q_ptr, uint32_t o) {
     g.sc = sc_ptr[o * 8];
-    g.qa = q_ptr[(2 * o) * 64];
-    g.qb = q_ptr[(2 * o + 1) * 64];
+    g.qa = __builtin_nontemporal_load(q_ptr + (2 * o) * 64);  // weights are read once: do not keep them in cache
+    g.qb = __builtin_nontemporal_load(q_ptr + (2 * o + 1) * 64);
 }
 
 template <int B>

@@ -115,7 +115,7 @@ struct SuperRegs {
 __device__ __forceinline__ void load_super(SuperRegs &g, gptr_u4 tile, uint32_t sb, uint32_t r, uint32_t lane) {
     gptr_u4 chunk = tile + size_t(sb) * (kQ4KSuperBytes / 16);
     g.hdr = chunk[r];
-    g.qv = chunk[8 + lane];
+    g.qv = __builtin_nontemporal_load(chunk + 8 + lane);  // weights are read once: do not keep them in cache
 }
 
 template <int B>
