@@ -39,6 +39,7 @@ extern "C" {
 
 #define RMI_HIP_DTYPE_Q8_0 8
 #define RMI_HIP_DTYPE_Q4_K 12
+#define RMI_HIP_DTYPE_Q6_K 14
 
 /* Activation rounding of quantize_q8_0_into: the reference picks it per host
  * architecture (src/ops/quant/q8_0.rs:3-24). */
@@ -61,6 +62,8 @@ int rmi_hip_device_info(char *name, size_t name_len, int *compute_units, size_t 
  * once; the host slice may be dropped afterwards.  NULL on failure. */
 rmi_hip_weight *rmi_hip_upload_q8_0(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
 rmi_hip_weight *rmi_hip_upload_q4_k(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
+/* Q6_KKernel::new (src/ops/kernel/q6_k.rs:15-18): rows of 210-byte super-blocks. */
+rmi_hip_weight *rmi_hip_upload_q6_k(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
 /* QTensorOwned::fuse_vstack (src/ops/kernel/qtensor_owned.rs:138-164) and
  * fuse_vstack_q8_0 / _q4_k (src/ops/quant/fuse.rs:25-64): rows of a then rows
  * of b.  NULL (the reference's None) when dtype or n_in differ. */
@@ -129,6 +132,29 @@ int rmi_hip_quantized_linear_forward(const rmi_hip_weight *w, const float *input
 int rmi_hip_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *q8k_qs, const int16_t *q8k_bsums, int32_t *isum,
                             int32_t *msum);
 
+/* ---- Q6_K, host slices ---------------------------------------------------*/
+
+/* Q6_KKernel::forward_prepared (src/ops/kernel/q6_k.rs:44-80): vec_dot_q6k_q8k
+ * (src/ops/quant/mod.rs:938-944, AVX2 kernel :964-1062) per row, Q8_K activation
+ * as three arrays. */
+int rmi_hip_q6_k_forward_prepared(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                                  const int16_t *q8k_bsums, float *output, uint32_t n_in, uint32_t n_out, uint32_t ith,
+                                  uint32_t nth);
+/* Same with f32 input (the `q8_k == None` branch, q6_k.rs:63-69): quantize_row_q8_k
+ * on the device; n_tokens rows, token-major out (Kernel::forward_batched,
+ * src/ops/kernel/trait_.rs:78-109). */
+int rmi_hip_q6_k_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens);
+/* Q6_KKernel::forward_prequantized = matmul_q6_k_scalar_range (q6_k.rs:83-119):
+ * dequantise-and-dot with the Q8_0 activation turned back into f32. */
+int rmi_hip_q6_k_forward_prequantized(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth);
+/* Exact integers of the Q6_K x Q8_K dot (parity entry point): lanes[n_out][n_in/256][8],
+ * the eight int32 the AVX2 kernel converts to f32 per super-block (quant/mod.rs:1053-1055);
+ * their sum is the scalar kernel's sum of aux32 (:676-688). */
+int rmi_hip_block_lanes_q6_k(const rmi_hip_weight *w, const int8_t *q8k_qs, const int16_t *q8k_bsums,
+                             int32_t *lanes);
+
 /* ---- device-resident entry points (activations stay in HBM) ---------------*/
 
 void *rmi_hip_malloc(size_t nbytes);
@@ -159,6 +185,11 @@ int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
  * integers, the f32 sums within rounding of the CPU kernels. */
 int rmi_hip_gemm_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
                               const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride, void *stream);
+/* y[t*y_stride + r] = vec_dot_q6k_q8k(row r, Q8_K token t) for rows [row_start,row_end), 1..n tokens
+ * (Q6_KKernel::forward_prepared, src/ops/kernel/q6_k.rs:44-80). */
+int rmi_hip_gemv_q6_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                              const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride,
+                              uint32_t row_start, uint32_t row_end, void *stream);
 int rmi_hip_quantize_row_q8_k_dev(const float *x, float *d, int8_t *qs, int16_t *bsums, uint32_t n_tokens,
                                   uint32_t n_in, void *stream);
 
@@ -172,6 +203,11 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
                                               float *const *y, uint32_t n_tokens);
 /* The same for Q4_K weights with Q8_K activations (three arrays per problem). */
 rmi_hip_gemv_group *rmi_hip_gemv_group_create_q4_k(uint32_t n_problems, const rmi_hip_weight *const *weights,
+                                                   const float *const *q8k_d, const int8_t *const *q8k_qs,
+                                                   const int16_t *const *q8k_bsums, float *const *y,
+                                                   uint32_t n_tokens);
+/* And for Q6_K weights (src/ops/kernel/q6_k.rs:44-80 per problem). */
+rmi_hip_gemv_group *rmi_hip_gemv_group_create_q6_k(uint32_t n_problems, const rmi_hip_weight *const *weights,
                                                    const float *const *q8k_d, const int8_t *const *q8k_qs,
                                                    const int16_t *const *q8k_bsums, float *const *y,
                                                    uint32_t n_tokens);

@@ -133,6 +133,35 @@ void rmi_ref_quantized_linear_forward(const uint8_t *weight,
                                       size_t in_features,
                                       size_t out_features);
 
+/* ---- rmi_q6_k.c: Q6_K x Q8_K ----
+ * Pinned by: the uniform-block value 256.0 (tests/quantized_inference.rs:252-263),
+ * the element layout cross-checked between dequantize_row_q6_k and the aux8
+ * unpack of the dot (two formulations inside the reference), brute-force
+ * integer sums, and the intrinsics twin below (same instructions as the
+ * reference's AVX2 kernel).  The exact f32 bits of the AVX2 kernel on random
+ * data have no golden vector in the reference: parity unpinned beyond that. */
+/* src/ops/quant/mod.rs:530-569 */
+void rmi_ref_dequantize_row_q6_k(const uint8_t *blocks, float *output, size_t n);
+/* src/ops/quant/mod.rs:640-692 (scalar) and :964-1062 (AVX2 order) */
+float rmi_ref_vec_dot_q6k_q8k(const uint8_t *q6k_row, size_t n_blocks, const float *d, const int8_t *qs,
+                              const int16_t *bsums, int variant);
+/* isum[b] = sum over the super-block of scale * q8 * (q6 - 32) */
+void rmi_ref_q6k_q8k_block_ints(const uint8_t *q6k_row, size_t n_blocks, const int8_t *qs, int32_t *isum);
+/* the eight int32 lanes the AVX2 kernel converts to f32, per super-block: lanes[b*8 + m] */
+void rmi_ref_q6k_q8k_lane_ints(const uint8_t *q6k_row, size_t n_blocks, const int8_t *qs, const int16_t *bsums,
+                               int32_t *lanes);
+/* src/ops/kernel/q6_k.rs:44-80 */
+void rmi_ref_q6k_forward_prepared(const uint8_t *weight, const float *d, const int8_t *qs, const int16_t *bsums,
+                                  float *output, size_t n_in, size_t n_out, size_t ith, size_t nth, int variant);
+/* src/ops/kernel/q6_k.rs:83-119 */
+void rmi_ref_q6k_forward_prequantized(const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, size_t n_in, size_t n_out, size_t ith, size_t nth);
+/* the reference's intrinsics, src/ops/quant/mod.rs:964-1062 */
+float rmi_ref_x86_vec_dot_q6k_q8k(const uint8_t *q6k_row, size_t n_blocks, const float *d, const int8_t *qs,
+                                  const int16_t *bsums);
+void rmi_ref_x86_q6k_forward_prepared(const uint8_t *weight, const float *d, const int8_t *qs, const int16_t *bsums,
+                                      float *output, size_t n_in, size_t n_out, size_t ith, size_t nth);
+
 /* ---- rmi_oracle_avx2.c: the same AVX2 kernels written with the same
  * intrinsics the reference uses; bit-identical to the RMI_REF_AVX2 variants
  * above on any AVX2+FMA host.  Used to cross-check the order emulation and

@@ -56,6 +56,14 @@ def _load():
         "rmi_ref_q4k_forward_prepared": (None, [_u8p, _f32p, _i8p, _i16p, _f32p, _sz, _sz, _sz, _sz, C.c_int]),
         "rmi_ref_q4k_forward_prequantized": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz, _sz]),
         "rmi_ref_quantized_linear_forward": (None, [_u8p, _f32p, _f32p, _sz, _sz]),
+        "rmi_ref_dequantize_row_q6_k": (None, [_u8p, _f32p, _sz]),
+        "rmi_ref_vec_dot_q6k_q8k": (C.c_float, [_u8p, _sz, _f32p, _i8p, _i16p, C.c_int]),
+        "rmi_ref_q6k_q8k_block_ints": (None, [_u8p, _sz, _i8p, _i32p]),
+        "rmi_ref_q6k_q8k_lane_ints": (None, [_u8p, _sz, _i8p, _i16p, _i32p]),
+        "rmi_ref_q6k_forward_prepared": (None, [_u8p, _f32p, _i8p, _i16p, _f32p, _sz, _sz, _sz, _sz, C.c_int]),
+        "rmi_ref_q6k_forward_prequantized": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz, _sz]),
+        "rmi_ref_x86_vec_dot_q6k_q8k": (C.c_float, [_u8p, _sz, _f32p, _i8p, _i16p]),
+        "rmi_ref_x86_q6k_forward_prepared": (None, [_u8p, _f32p, _i8p, _i16p, _f32p, _sz, _sz, _sz, _sz]),
         "rmi_ref_have_avx2": (C.c_int, []),
         "rmi_ref_x86_quantize_q8_0": (None, [_f32p, _sz, _u8p, _f32p]),
         "rmi_ref_x86_matmul_q8_0_range": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz]),
@@ -290,6 +298,73 @@ def quantized_linear_forward(w, x, in_features, out_features):
     w, x = _u8(w), _f32(x)
     out = np.zeros(out_features, np.float32)
     lib.rmi_ref_quantized_linear_forward(_p(w, _u8p), _p(x, _f32p), _p(out, _f32p), in_features, out_features)
+    return out
+
+
+# ---- Q6_K ----
+
+def dequantize_row_q6_k(blocks, n):
+    blocks = _u8(blocks)
+    out = np.zeros(n, np.float32)
+    lib.rmi_ref_dequantize_row_q6_k(_p(blocks, _u8p), _p(out, _f32p), n)
+    return out
+
+
+def _q8k_args(d, qs, bsums):
+    return _f32(d), np.ascontiguousarray(qs, np.int8), np.ascontiguousarray(bsums, np.int16)
+
+
+def vec_dot_q6k_q8k(row, d, qs, bsums, variant=AVX2):
+    row = _u8(row)
+    d, qs, bsums = _q8k_args(d, qs, bsums)
+    return np.float32(lib.rmi_ref_vec_dot_q6k_q8k(_p(row, _u8p), d.size, _p(d, _f32p), _p(qs, _i8p), _p(bsums, _i16p),
+                                                  variant))
+
+
+def q6k_q8k_block_ints(row, qs):
+    row = _u8(row)
+    qs = np.ascontiguousarray(qs, np.int8)
+    isum = np.zeros(qs.size // 256, np.int32)
+    lib.rmi_ref_q6k_q8k_block_ints(_p(row, _u8p), isum.size, _p(qs, _i8p), _p(isum, _i32p))
+    return isum
+
+
+def q6k_q8k_lane_ints(row, qs, bsums):
+    row = _u8(row)
+    qs = np.ascontiguousarray(qs, np.int8)
+    bsums = np.ascontiguousarray(bsums, np.int16)
+    lanes = np.zeros((qs.size // 256, 8), np.int32)
+    lib.rmi_ref_q6k_q8k_lane_ints(_p(row, _u8p), lanes.shape[0], _p(qs, _i8p), _p(bsums, _i16p), _p(lanes, _i32p))
+    return lanes
+
+
+def q6k_forward_prepared(w, d, qs, bsums, out, n_in, n_out, ith=0, nth=1, variant=AVX2):
+    w = _u8(w)
+    d, qs, bsums = _q8k_args(d, qs, bsums)
+    lib.rmi_ref_q6k_forward_prepared(_p(w, _u8p), _p(d, _f32p), _p(qs, _i8p), _p(bsums, _i16p), _p(out, _f32p), n_in,
+                                     n_out, ith, nth, variant)
+    return out
+
+
+def q6k_forward_prequantized(w, q8, sc, out, n_in, n_out, ith=0, nth=1):
+    w, q8, sc = _u8(w), _u8(q8), _f32(sc)
+    lib.rmi_ref_q6k_forward_prequantized(_p(w, _u8p), _p(q8, _u8p), _p(sc, _f32p), _p(out, _f32p), n_in, n_out, ith,
+                                         nth)
+    return out
+
+
+def x86_vec_dot_q6k_q8k(row, d, qs, bsums):
+    row = _u8(row)
+    d, qs, bsums = _q8k_args(d, qs, bsums)
+    return np.float32(lib.rmi_ref_x86_vec_dot_q6k_q8k(_p(row, _u8p), d.size, _p(d, _f32p), _p(qs, _i8p),
+                                                      _p(bsums, _i16p)))
+
+
+def x86_q6k_forward_prepared(w, d, qs, bsums, out, n_in, n_out, ith=0, nth=1):
+    w = _u8(w)
+    d, qs, bsums = _q8k_args(d, qs, bsums)
+    lib.rmi_ref_x86_q6k_forward_prepared(_p(w, _u8p), _p(d, _f32p), _p(qs, _i8p), _p(bsums, _i16p), _p(out, _f32p),
+                                         n_in, n_out, ith, nth)
     return out
 
 

@@ -363,6 +363,9 @@ void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g) {
 int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream) {
     RMI_REQUIRE_INIT();
     if (!g) return rmi_fail(RMI_HIP_E_INVALID, "null group");
+    if (g->dtype == RMI_HIP_DTYPE_Q6_K)
+        return rmi_launch_gemv_q6_k_group(static_cast<const RmiQ4kProblem *>(g->d_list), g->d_runs, g->n_runs,
+                                          g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
     if (g->dtype == RMI_HIP_DTYPE_Q4_K)
         return rmi_launch_gemv_q4_k_group(static_cast<const RmiQ4kProblem *>(g->d_list), g->d_runs, g->n_runs,
                                           g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));

@@ -61,6 +61,39 @@ __global__ __launch_bounds__(256) void repack_q4_k_kernel(const uint8_t *__restr
     }
 }
 
+// One workgroup per (tile, super-block) of the destination: 420 dwords.
+__global__ __launch_bounds__(256) void repack_q6_k_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                           uint32_t n_out, uint32_t n_sb) {
+    const uint32_t tile = blockIdx.x / n_sb;
+    const uint32_t sb = blockIdx.x % n_sb;
+    uint8_t *chunk = dst + (size_t(tile) * n_sb + sb) * kQ6KSuperBytes;
+    // the 210-byte source blocks are only 2-byte aligned: move 16-bit units
+    for (uint32_t idx = threadIdx.x; idx < 840; idx += 256) {
+        uint32_t r, src_half;  // destination 16-bit unit idx <- unit src_half of row r's block
+        if (idx < 64) {        // scales
+            r = idx >> 3;
+            src_half = 96 + (idx & 7);
+        } else if (idx < 72) {  // d
+            r = idx - 64;
+            src_half = 104;
+        } else if (idx < 584) {  // ql: (r, L, c) <- bytes 32c + 4L.. ; two units per dword
+            const uint32_t k = idx - 72;
+            r = k >> 6;
+            const uint32_t L = (k >> 3) & 7, c = (k >> 1) & 3, h = k & 1;
+            src_half = 16 * c + 2 * L + h;
+        } else {  // qh: (r, L, c) <- bytes 128 + 32c + 4L..
+            const uint32_t k = idx - 584;
+            r = k >> 5;
+            const uint32_t L = (k >> 2) & 7, c = (k >> 1) & 1, h = k & 1;
+            src_half = 64 + 16 * c + 2 * L + h;
+        }
+        const uint32_t row = tile * kTileRows + r;
+        uint16_t v = 0;
+        if (row < n_out) v = reinterpret_cast<const uint16_t *>(src + (size_t(row) * n_sb + sb) * 210)[src_half];
+        reinterpret_cast<uint16_t *>(chunk)[idx] = v;
+    }
+}
+
 // uint4 index, inside one tile, of piece p of (unit u, row r).
 __device__ __forceinline__ uint32_t piece_index(int dtype, uint32_t n_units, uint32_t u, uint32_t r, uint32_t p) {
     if (dtype == RMI_HIP_DTYPE_Q8_0) {
@@ -68,14 +101,23 @@ __device__ __forceinline__ uint32_t piece_index(int dtype, uint32_t n_units, uin
         const uint32_t q = 2 * u + ((p - 1) >> 3), L = (p - 1) & 7;
         return n_units * 8 + q * 64 + r * 8 + L;
     }
+    if (dtype == RMI_HIP_DTYPE_Q6_K) {  // 105 uint4 per unit; piece 0 scales, 1..8 ql, 9..12 qh (d is copied apart)
+        if (p == 0) return u * 105 + r;
+        if (p < 9) return u * 105 + 9 + r * 8 + (p - 1);
+        return u * 105 + 73 + r * 4 + (p - 9);
+    }
     if (p == 0) return u * 72 + r;
     return u * 72 + 8 + r * 8 + (p - 1);
+}
+
+__host__ __device__ __forceinline__ uint32_t pieces_of(int dtype) {
+    return dtype == RMI_HIP_DTYPE_Q8_0 ? 17 : (dtype == RMI_HIP_DTYPE_Q6_K ? 13 : 9);
 }
 
 __global__ __launch_bounds__(256) void copy_rows_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
                                                          int dtype, uint32_t n_rows, uint32_t n_units,
                                                          uint32_t tile_u4, uint32_t dst_row0) {
-    const uint32_t pieces = dtype == RMI_HIP_DTYPE_Q8_0 ? 17 : 9;
+    const uint32_t pieces = pieces_of(dtype);
     const uint64_t total = uint64_t(n_rows) * n_units * pieces;
     for (uint64_t i = blockIdx.x * uint64_t(blockDim.x) + threadIdx.x; i < total;
          i += uint64_t(gridDim.x) * blockDim.x) {
@@ -86,6 +128,11 @@ __global__ __launch_bounds__(256) void copy_rows_kernel(const uint4 *__restrict_
         const uint32_t drow = dst_row0 + row;
         const uint4 v = src[size_t(row >> 3) * tile_u4 + piece_index(dtype, n_units, u, row & 7, p)];
         dst[size_t(drow >> 3) * tile_u4 + piece_index(dtype, n_units, u, drow & 7, p)] = v;
+        if (dtype == RMI_HIP_DTYPE_Q6_K && p == 0) {  // the row's f16 d: 8 rows share one uint4
+            const uint16_t *s16 = reinterpret_cast<const uint16_t *>(src + size_t(row >> 3) * tile_u4 + u * 105 + 8);
+            uint16_t *d16 = reinterpret_cast<uint16_t *>(dst + size_t(drow >> 3) * tile_u4 + u * 105 + 8);
+            d16[drow & 7] = s16[row & 7];
+        }
     }
 }
 
@@ -108,11 +155,19 @@ int rmi_launch_repack_q4_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s)
     return RMI_HIP_OK;
 }
 
+int rmi_launch_repack_q6_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s) {
+    const uint32_t grid = w->n_tiles * w->n_units;
+    if (grid == 0) return RMI_HIP_OK;
+    hipLaunchKernelGGL(repack_q6_k_kernel, dim3(grid), dim3(256), 0, s, src, w->data, w->n_out, w->n_units);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
 int rmi_launch_copy_rows(const rmi_hip_weight *src, rmi_hip_weight *dst, uint32_t dst_row0, hipStream_t s) {
     if (src->n_out == 0 || src->n_units == 0) return RMI_HIP_OK;
     if (src->dtype != dst->dtype || src->n_units != dst->n_units || dst_row0 + src->n_out > dst->n_out)
         return rmi_fail(RMI_HIP_E_INVALID, "copy_rows: layouts differ");
-    const uint32_t pieces = src->dtype == RMI_HIP_DTYPE_Q8_0 ? 17 : 9;
+    const uint32_t pieces = pieces_of(src->dtype);
     const uint64_t total = uint64_t(src->n_out) * src->n_units * pieces;
     const uint32_t grid = uint32_t(total / 256 + 1 < 65535 ? total / 256 + 1 : 65535);
     hipLaunchKernelGGL(copy_rows_kernel, dim3(grid), dim3(256), 0, s, reinterpret_cast<const uint4 *>(src->data),

@@ -41,12 +41,24 @@ constexpr uint32_t kOctetBytes = 128 + 2048;  // per tile per octet
 // coalesced 1 KiB load.  144 bytes per super-block, as in the source format.
 constexpr uint32_t kQ4KSuperBytes = 8 * 16 + 1024;  // per tile per super-block
 
+// Q6_K weights in HBM.  Tiles of 8 rows; per tile and super-block:
+//
+//   [ scales : 8 rows x 16 int8 ]           128 B
+//   [ d      : 8 rows x f16 ]                16 B
+//   [ ql     : 8 rows x 8 L x 16 B ]       1024 B   bytes 4L.. of ql[0..32), [32..64), [64..96), [96..128)
+//   [ qh     : 8 rows x 8 L x 8 B ]         512 B   bytes 4L.. of qh[0..32), [32..64)
+//
+// Lane L of a row thus holds the quants 4L..4L+3 of each of the eight 32-element groups, which is
+// what lane L of the reference's 8-lane integer accumulator sums (quant/mod.rs:1010-1050).
+// 210 bytes per super-block, as in the source format.
+constexpr uint32_t kQ6KSuperBytes = 128 + 16 + 1024 + 512;  // per tile per super-block
+
 struct rmi_hip_weight {
     int dtype;
     uint32_t n_in;
     uint32_t n_out;
     uint32_t n_tiles;   // ceil(n_out / 8)
-    uint32_t n_units;   // Q8_0: octets per row; Q4_K: super-blocks per row
+    uint32_t n_units;   // Q8_0: octets per row; Q4_K, Q6_K: super-blocks per row
     size_t tile_bytes;  // bytes of one tile
     size_t nbytes;      // device allocation
     uint8_t *data;      // device pointer
@@ -89,6 +101,7 @@ int rmi_device_cus();
 // ------------------------------------------------- launchers (device ptrs)
 int rmi_launch_repack_q8_0(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
 int rmi_launch_repack_q4_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
+int rmi_launch_repack_q6_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
 int rmi_launch_copy_rows(const rmi_hip_weight *src, rmi_hip_weight *dst, uint32_t dst_row0, hipStream_t s);
 
 struct RmiGemvProblem {
@@ -153,10 +166,23 @@ int rmi_launch_q4_k_dequant_dot(const rmi_hip_weight *w, const float *x_f32, con
                                 const float *x_scales, float *y, uint32_t row_start, uint32_t row_end, int mode,
                                 hipStream_t s);
 
+// Q6_K x Q8_K: the same problem record (w = Q6_K tile stream)
+uint32_t rmi_q6k_tiles_per_wave(uint32_t n_sb, uint32_t launch_tiles, uint32_t n_tokens);
+int rmi_launch_gemv_q6_k_group(const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,
+                               uint32_t max_n_sb, uint32_t n_tokens, hipStream_t s);
+int rmi_launch_gemv_q6_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
+                         uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s);
+// lanes[(row*n_sb + sb)*8 + m]: the int32 each of the eight accumulator lanes converts to f32
+int rmi_launch_block_lanes_q6_k(const rmi_hip_weight *w, const int8_t *qs, const int16_t *bsums, int32_t *lanes,
+                                hipStream_t s);
+// x = q8 * scale rebuilt per element (Q6_KKernel::forward_prequantized)
+int rmi_launch_q6_k_dequant_dot(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                                uint32_t row_start, uint32_t row_end, hipStream_t s);
+
 // A fixed list of independent GEMVs (Q8_0 or Q4_K) launched as one kernel.
 struct rmi_hip_gemv_group {
     int dtype = 0;
-    void *d_list = nullptr;  // RmiGemvProblem[] or RmiQ4kProblem[]
+    void *d_list = nullptr;  // RmiGemvProblem[] (Q8_0) or RmiQ4kProblem[] (Q4_K, Q6_K)
     uint4 *d_runs = nullptr;
     uint32_t n_problems = 0;
     uint32_t n_runs = 0;

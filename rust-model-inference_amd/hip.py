@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "librmi_hip.so")
 
 DTYPE_Q8_0 = 8
 DTYPE_Q4_K = 12
+DTYPE_Q6_K = 14
 ROUND_HALF_AWAY = 0
 ROUND_TIES_EVEN = 1
 
@@ -53,6 +54,7 @@ SIGNATURES = {
     "rmi_hip_device_info": (C.c_int, [C.c_char_p, _sz, C.POINTER(C.c_int), C.POINTER(_sz)]),
     "rmi_hip_upload_q8_0": (_vp, [_u8p, _sz, _u32, _u32]),
     "rmi_hip_upload_q4_k": (_vp, [_u8p, _sz, _u32, _u32]),
+    "rmi_hip_upload_q6_k": (_vp, [_u8p, _sz, _u32, _u32]),
     "rmi_hip_fuse_vstack": (_vp, [_vp, _vp]),
     "rmi_hip_free_weight": (None, [_vp]),
     "rmi_hip_weight_n_in": (_u32, [_vp]),
@@ -72,6 +74,10 @@ SIGNATURES = {
     "rmi_hip_q4_k_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_quantized_linear_forward": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32]),
     "rmi_hip_block_ints_q4_k": (C.c_int, [_vp, _i8p, _i16p, _i32p, _i32p]),
+    "rmi_hip_q6_k_forward_prepared": (C.c_int, [_vp, _f32p, _i8p, _i16p, _f32p, _u32, _u32, _u32, _u32]),
+    "rmi_hip_q6_k_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32]),
+    "rmi_hip_q6_k_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
+    "rmi_hip_block_lanes_q6_k": (C.c_int, [_vp, _i8p, _i16p, _i32p]),
     "rmi_hip_malloc": (_vp, [_sz]),
     "rmi_hip_free": (None, [_vp]),
     "rmi_hip_memcpy_h2d": (C.c_int, [_vp, _vp, _sz]),
@@ -83,9 +89,12 @@ SIGNATURES = {
     "rmi_hip_gemm_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_gemm_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp]),
+    "rmi_hip_gemv_q6_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_quantize_row_q8_k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_group_create": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u32]),
     "rmi_hip_gemv_group_create_q4_k": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+                                             C.POINTER(_vp), _u32]),
+    "rmi_hip_gemv_group_create_q6_k": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                              C.POINTER(_vp), _u32]),
     "rmi_hip_expf_dev": (C.c_int, [_vp, _vp, _sz, _vp]),
     "rmi_hip_rms_norm_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, C.c_float, _vp, _vp, C.c_int, _vp]),

@@ -5,6 +5,7 @@ the Rust traits so that tests read like the reference's own:
   Kernel                 src/ops/kernel/trait_.rs:15-110
   Q8Kernel               src/ops/kernel/q8_0/mod.rs:21-56
   Q4_KKernel             src/ops/kernel/q4_k.rs:7-93
+  Q6_KKernel             src/ops/kernel/q6_k.rs:7-80
   QuantizedTensor        src/ops/kernel/quantized_tensor.rs:32-190  (from_bytes / into_kernel)
   QTensorOwned.fuse_vstack  src/ops/kernel/qtensor_owned.rs:138-164
   QuantizedLinear, Layer, ExecContext   src/core/model.rs:12-104, src/core/traits.rs:45-74
@@ -24,6 +25,7 @@ from .hip import C, _f32p, _i8p, _i16p, _i32p, _u8p, as_f32, as_u8, check, lib, 
 
 GGML_TYPE_Q8_0 = "Q8_0"
 GGML_TYPE_Q4_K = "Q4_K"
+GGML_TYPE_Q6_K = "Q6_K"
 
 
 @dataclass
@@ -218,6 +220,39 @@ class Q4_KKernel(Kernel):
         return isum, msum
 
 
+class Q6_KKernel(Kernel):
+    def __init__(self, data, n_in, n_out, _handle=None):
+        if _handle is None:
+            w = as_u8(data)
+            _handle = lib.rmi_hip_upload_q6_k(ptr(w, _u8p), w.size, n_in, n_out)
+        self.w = _DeviceWeight(_handle)
+
+    def forward_prequantized(self, input_q8, input_scales, output, n_in, n_out, ith, nth):
+        q8, sc = as_u8(input_q8), as_f32(input_scales)
+        check(lib.rmi_hip_q6_k_forward_prequantized(self.w.handle, ptr(q8, _u8p), ptr(sc, _f32p),
+                                                    ptr(_out(output, n_out), _f32p), n_in, n_out, ith, nth))
+
+    def forward_prepared(self, input_f32, input_q8, input_scales, q8_k, output, n_in, n_out, ith, nth):
+        if q8_k is None:  # q6_k.rs:63-69: the kernel quantizes input_f32[..n_in] itself
+            q8_k = quantize_row_q8_k(as_f32(input_f32)[:n_in])
+        d, qs, bs = _q8k_arrays(q8_k)
+        check(lib.rmi_hip_q6_k_forward_prepared(self.w.handle, ptr(d, _f32p), ptr(qs, _i8p), ptr(bs, _i16p),
+                                                ptr(_out(output, n_out), _f32p), n_in, n_out, ith, nth))
+
+    def forward_batched(self, input, output, n_in, n_out):
+        x = as_f32(input).reshape(-1)
+        n_tokens = x.size // n_in
+        check(lib.rmi_hip_q6_k_forward_batched(self.w.handle, ptr(x, _f32p),
+                                               ptr(_out(output, n_tokens * n_out), _f32p), n_in, n_out, n_tokens))
+
+    def block_lanes(self, q8_k):
+        """The eight int32 accumulator lanes per (row, super-block)."""
+        _, qs, bs = _q8k_arrays(q8_k)
+        lanes = np.zeros((self.w.n_out, self.w.n_in // 256, 8), np.int32)
+        check(lib.rmi_hip_block_lanes_q6_k(self.w.handle, ptr(qs, _i8p), ptr(bs, _i16p), ptr(lanes, _i32p)))
+        return lanes
+
+
 class QuantizedTensor:
     """`QuantizedTensor::from_bytes(..).into_kernel()`: the factory the `hip`
     back end hooks (quantized_tensor.rs:120-138, 167-190)."""
@@ -227,7 +262,7 @@ class QuantizedTensor:
 
     @classmethod
     def from_bytes(cls, ggml_type, data, n_in, n_out):
-        if ggml_type not in (GGML_TYPE_Q8_0, GGML_TYPE_Q4_K):
+        if ggml_type not in (GGML_TYPE_Q8_0, GGML_TYPE_Q4_K, GGML_TYPE_Q6_K):
             return None  # other dtypes stay on the reference's CPU kernels
         return cls(ggml_type, data, n_in, n_out)
 
@@ -240,6 +275,8 @@ class QuantizedTensor:
     def into_kernel(self):
         if self.ggml_type == GGML_TYPE_Q8_0:
             return Q8Kernel(self.data, self._n_in, self._n_out)
+        if self.ggml_type == GGML_TYPE_Q6_K:
+            return Q6_KKernel(self.data, self._n_in, self._n_out)
         return Q4_KKernel(self.data, self._n_in, self._n_out)
 
 

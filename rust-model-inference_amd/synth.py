@@ -4,12 +4,14 @@ configurations name (random Q8_0 / Q4_K weights, N(0,1) activations).
 Pure numpy; the same bytes feed the GPU path, the CPU checker and the CPU
 baseline.  Block layouts follow the reference's readers:
 Q8_0 = [f16 d][32 x int8] (src/ops/kernel/q8_0/scalar.rs:42-48),
-Q4_K = [f16 d][f16 dmin][12 B scales][128 B nibbles] (src/ops/quant/mod.rs:219-222).
+Q4_K = [f16 d][f16 dmin][12 B scales][128 B nibbles] (src/ops/quant/mod.rs:219-222),
+Q6_K = [128 B low nibbles][64 B high bit pairs][16 x int8 scales][f16 d] (src/ops/quant/mod.rs:530-541).
 """
 import numpy as np
 
 Q8_0_BLOCK = 34
 Q4_K_BLOCK = 144
+Q6_K_BLOCK = 210
 
 # Qwen3-0.6B projection set: (name, n_out, n_in) per layer, then lm_head.
 QWEN3_0_6B_LAYER = [
@@ -50,6 +52,16 @@ def q4_k_weight(seed, n_out, n_in, sigma=0.01):
     return w.reshape(-1)
 
 
+def q6_k_weight(seed, n_out, n_in, sigma=0.01):
+    """6-bit quants and int8 sub-block scales uniform, d f16(|N(0,sigma)|/32)."""
+    rng = np.random.default_rng(seed)
+    nb = n_in // 256
+    w = rng.integers(0, 256, (n_out, nb, Q6_K_BLOCK), dtype=np.uint8)
+    dd = (np.abs(rng.normal(0.0, sigma, (n_out, nb, 1))) / 32.0).astype(np.float16)
+    w[:, :, 208:210] = dd.view(np.uint8).reshape(n_out, nb, 2)
+    return w.reshape(-1)
+
+
 def activations(seed, n_tokens, n_in):
     rng = np.random.default_rng(seed)
     return rng.standard_normal((n_tokens, n_in), dtype=np.float32)
@@ -67,3 +79,7 @@ def q8_0_gemv_bytes(n_out, n_in, batch=1):
 
 def q4_k_gemv_bytes(n_out, n_in, batch=1):
     return n_out * (n_in // 256) * Q4_K_BLOCK + batch * (n_in // 256) * 292 + batch * 4 * n_out
+
+
+def q6_k_gemv_bytes(n_out, n_in, batch=1):
+    return n_out * (n_in // 256) * Q6_K_BLOCK + batch * (n_in // 256) * 292 + batch * 4 * n_out
