@@ -400,17 +400,33 @@ def run_gemm(args, pkg, ev):
 
 
 def run_q4k(args, pkg, ev):
-    """Q4_K x Q8_K decode GEMV at 1.7B-class FFN shapes (gate/up 6144x2048, down 2048x6144), 28 layers of
-    distinct weights (594 MB) so that every step streams from HBM; one grouped launch, or one per matrix with --mode per_matmul."""
+    return run_kquant(args, pkg, ev, "q4_k")
+
+
+def run_q6k(args, pkg, ev):
+    return run_kquant(args, pkg, ev, "q6_k")
+
+
+def run_kquant(args, pkg, ev, fmt):
+    """Q4_K / Q6_K x Q8_K decode GEMV at 1.7B-class FFN shapes (gate/up 6144x2048, down 2048x6144), 28 layers of
+    distinct weights (594 / 867 MB) so that every step streams from HBM; one grouped launch, or one per matrix with
+    --mode per_matmul."""
     H, synth, K = pkg.hip, pkg.synth, pkg.kernel
+    q6 = fmt == "q6_k"
+    name = "Q6_K" if q6 else "Q4_K"
+    make_weight = synth.q6_k_weight if q6 else synth.q4_k_weight
+    kernel_cls = K.Q6_KKernel if q6 else K.Q4_KKernel
+    group_create = H.lib.rmi_hip_gemv_group_create_q6_k if q6 else H.lib.rmi_hip_gemv_group_create_q4_k
+    gemv_dev = H.lib.rmi_hip_gemv_q6_k_q8k_dev if q6 else H.lib.rmi_hip_gemv_q4_k_q8k_dev
+    gemv_bytes = synth.q6_k_gemv_bytes if q6 else synth.q4_k_gemv_bytes
     dev_name, cus, hbm = H.device_info()
     batch = args.batch
     recs = []
     shapes = [(6144, 2048), (6144, 2048), (2048, 6144)] * 28
     for i, (n_out, n_in) in enumerate(shapes):
-        w = synth.q4_k_weight(synth.seed_for(3, i), n_out, n_in)
+        w = make_weight(synth.seed_for(3, i), n_out, n_in)
         x = synth.activations(synth.seed_for(3, 0x8000 + i), batch, n_in)
-        k = K.Q4_KKernel(w, n_in, n_out)
+        k = kernel_cls(w, n_in, n_out)
         d_x = H.DeviceBuffer.from_array(x)
         d_d, d_q, d_b = H.DeviceBuffer(batch * n_in // 256 * 4), H.DeviceBuffer(batch * n_in), H.DeviceBuffer(batch * n_in // 16 * 2)
         d_y = H.DeviceBuffer(batch * n_out * 4)
@@ -422,17 +438,16 @@ def run_q4k(args, pkg, ev):
 
     n = len(recs)
     arr = lambda vals: (C.c_void_p * n)(*vals)  # noqa: E731
-    group = H.lib.rmi_hip_gemv_group_create_q4_k(n, arr([r["k"].w.handle for r in recs]),
-                                                 arr([r["d_d"].ptr for r in recs]), arr([r["d_q"].ptr for r in recs]),
-                                                 arr([r["d_b"].ptr for r in recs]), arr([r["d_y"].ptr for r in recs]),
-                                                 batch)
+    group = group_create(n, arr([r["k"].w.handle for r in recs]), arr([r["d_d"].ptr for r in recs]),
+                         arr([r["d_q"].ptr for r in recs]), arr([r["d_b"].ptr for r in recs]),
+                         arr([r["d_y"].ptr for r in recs]), batch)
     if not group:
         raise RuntimeError(H.last_error())
 
     def step_per_matmul():
         for r in recs:
-            H.check(H.lib.rmi_hip_gemv_q4_k_q8k_dev(r["k"].w.handle, r["d_d"].ptr, r["d_q"].ptr, r["d_b"].ptr,
-                                                    r["d_y"].ptr, batch, r["n_out"], 0, r["n_out"], None))
+            H.check(gemv_dev(r["k"].w.handle, r["d_d"].ptr, r["d_q"].ptr, r["d_b"].ptr, r["d_y"].ptr, batch, r["n_out"], 0,
+                             r["n_out"], None))
 
     def step_grouped():
         H.check(H.lib.rmi_hip_gemv_group_run_dev(group, None))
@@ -442,20 +457,20 @@ def run_q4k(args, pkg, ev):
     launches = 1 if grouped else n
     copy_calibration(H, args)
     wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
-    alg = sum(synth.q4_k_gemv_bytes(r["n_out"], r["n_in"], batch) for r in recs)
+    alg = sum(gemv_bytes(r["n_out"], r["n_in"], batch) for r in recs)
     value = alg / wall / 1e9
     achieved = alg / (dev_ms * 1e-3) / 1e9
-    result = base_result(args, "Q4_K x Q8_K GEMV HBM GB/s, 1.7B-class FFN shapes, 1 GPU", "GB/s", round(value, 1), wall,
+    result = base_result(args, f"{name} x Q8_K GEMV HBM GB/s, 1.7B-class FFN shapes, 1 GPU", "GB/s", round(value, 1), wall,
                          "int8 dot4 -> f32", {
-        "workload": f"Q4_K GEMV, 28 layers x (gate 6144x2048, up 6144x2048, down 2048x6144), decode batch {batch}, "
+        "workload": f"{name} GEMV, 28 layers x (gate 6144x2048, up 6144x2048, down 2048x6144), decode batch {batch}, "
                     + ("one grouped launch" if grouped else "one launch per matrix"), "batch": batch,
         "launches_per_step": launches,
         "algorithmic_bytes_per_step": alg, "device": dev_name.strip(), "compute_units": cus})
-    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_k_kernel<{batch},{'true' if grouped else 'false'},{group_maxt(H, group) if grouped else '*'}>",
+    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_{fmt}_kernel<{batch},{'true' if grouped else 'false'},{group_maxt(H, group) if grouped else '*'}>",
                           "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(achieved / HBM_PEAK_GBS, 4),
                           "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
-                          "traffic": read_traffic("gemv_q4_k_grouped_1.7b_ffn") if grouped and batch == 1 else None}
+                          "traffic": read_traffic(f"gemv_{fmt}_grouped_1.7b_ffn") if grouped and batch == 1 else None}
     if not args.no_cpu_baseline and batch == 1:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
@@ -468,7 +483,7 @@ def run_q4k(args, pkg, ev):
             for it in range(6):
                 t0 = time.perf_counter()
                 for r, (d, q, b, out) in zip(recs, host):
-                    pool.matmul_q4k_q8k(r["w"], d, q, b, out, r["n_in"], r["n_out"])
+                    (pool.matmul_q6k_q8k if q6 else pool.matmul_q4k_q8k)(r["w"], d, q, b, out, r["n_in"], r["n_out"])
                 samples.append(time.perf_counter() - t0)
             pool.close()
             med = statistics.median(samples[1:])
@@ -478,7 +493,7 @@ def run_q4k(args, pkg, ev):
                                              != out.view(np.uint32))) for r, (_, _, _, out) in zip(recs, host))
             result["cpu_baseline"] = {"value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
                                       "sample": f"5 full steps (84 GEMVs, {alg / 1e6:.0f} MB), restated AVX2 "
-                                                f"vec_dot_q4k_q8k over {cores} threads, median",
+                                                f"vec_dot_{fmt.replace('_', '')}_q8k over {cores} threads, median",
                                       "gpu_outputs_differing_from_cpu": worst}
     return result
 
@@ -625,9 +640,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4k", "q4k_gemm", "decode"], default="projection_set",
+    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4k", "q6k", "q4k_gemm", "decode"], default="projection_set",
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
-                         "q4k: Q4_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); decode: end-to-end device-resident greedy decode "
+                         "q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); decode: end-to-end device-resident greedy decode "
                          "(one step = one 639-token-step generation)")
     ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill tokens M for --workload gemm")
@@ -647,7 +662,7 @@ def main():
     pkg = importlib.import_module("rust-model-inference_amd")
     pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
     ev = HipEvents()
-    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4k": run_q4k, "q4k_gemm": run_q4k_gemm,
+    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4k": run_q4k, "q6k": run_q6k, "q4k_gemm": run_q4k_gemm,
            "decode": run_decode}[args.workload]
     result = run(args, pkg, ev)
     if args.workload == "projection_set" and not args.no_decode and args.batch == 1:

@@ -278,3 +278,25 @@ void rmi_ref_x86_q6k_forward_prepared(const uint8_t *weight, const float *d, con
     for (size_t r = start; r < end; r++)
         output[r] = rmi_ref_x86_vec_dot_q6k_q8k(weight + r * nb * Q6K_BLOCK, nb, d, qs, bsums);
 }
+
+/* y = W x over the persistent pool: rows split as (ith, nth), the AVX2 kernel per row */
+typedef struct {
+    const uint8_t *weight;
+    const float *d;
+    const int8_t *qs;
+    const int16_t *bsums;
+    float *output;
+    size_t n_in, n_out;
+} q6k_job;
+
+static void q6k_slice(void *arg, int ith, int nth) {
+    const q6k_job *j = (const q6k_job *)arg;
+    rmi_ref_x86_q6k_forward_prepared(j->weight, j->d, j->qs, j->bsums, j->output, j->n_in, j->n_out, (size_t)ith,
+                                     (size_t)nth);
+}
+
+void rmi_ref_pool_matmul_q6k_q8k(rmi_ref_pool *pool, const uint8_t *weight, const float *d, const int8_t *qs,
+                                 const int16_t *bsums, float *output, size_t n_in, size_t n_out) {
+    q6k_job job = {weight, d, qs, bsums, output, n_in, n_out};
+    rmi_ref_pool_run(pool, q6k_slice, &job);
+}
