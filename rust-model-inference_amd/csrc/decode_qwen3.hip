@@ -42,9 +42,10 @@ __device__ __forceinline__ uint16_t f2h(float v) {
     return __builtin_bit_cast(uint16_t, _Float16(v));
 }
 
-// Where the session's kernels read the step from: with it in HBM every launch of a token-step has the same
-// arguments at every step (replaying the step as a HIP graph was measured: 676 vs 678 token-steps/s, no gain,
-// so the launches stay eager).  A null pointer means "use the value argument".
+// The step counter in HBM: the embedding kernel reads its token through it and the argmax kernel advances it,
+// so the next token never visits the host.  The kernels in between get the position as a launch argument:
+// reading it from HBM first would put one more memory round trip in front of their loads.  (Replaying a whole step as a HIP graph with the counter read everywhere was
+// measured: 676 vs 678 token-steps/s, no gain, so the launches stay eager.)
 struct StepParams {
     uint32_t step;      // position of the token being processed = row of the KV cache
     uint32_t n_prompt;  // steps below n_prompt - 1 read their token from the prompt
@@ -126,14 +127,8 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(const float *__r
                                                                 const float *__restrict__ sin_t, uint32_t pos,
                                                                 uint16_t *__restrict__ q16, uint16_t *__restrict__ k_row,
                                                                 uint16_t *__restrict__ v_row, uint32_t n_head,
-                                                                uint32_t n_head_kv, uint32_t hk, uint32_t hv, float eps,
-                                                                const StepParams *__restrict__ sp, uint32_t kv_stride) {
+                                                                uint32_t n_head_kv, uint32_t hk, uint32_t hv, float eps) {
     const uint32_t head = blockIdx.x, tid = threadIdx.x;
-    if (sp) {  // session: position and cache row follow the step counter (k_row, v_row = the layer's cache)
-        pos = sp->step;
-        k_row += size_t(pos) * kv_stride;
-        v_row += size_t(pos) * kv_stride;
-    }
     if (head >= n_head + n_head_kv) {  // v: rounding only
         const uint32_t kvh = head - n_head - n_head_kv;
         const float *src = qkv + size_t(n_head) * hk + size_t(n_head_kv) * hk + size_t(kvh) * hv;
@@ -186,13 +181,13 @@ __host__ __device__ inline size_t attn_lds_bytes(uint32_t n_keys, uint32_t hk, u
 __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
     uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, uint32_t hk, uint32_t hv,
-    int8_t *__restrict__ q8, float *__restrict__ scales, int rounding, const StepParams *__restrict__ sp) {
+    int8_t *__restrict__ q8, float *__restrict__ scales, int rounding) {
     extern __shared__ double lds_d[];
     __shared__ float red_f[kAttnThreads / 64];
     __shared__ uint64_t exp_tab[32];
     const uint32_t head = blockIdx.x, tid = threadIdx.x;
     const uint32_t kvh = head / (n_head / n_head_kv);
-    const uint32_t n_keys = (sp ? sp->step : step) + 1;
+    const uint32_t n_keys = step + 1;
     const uint32_t n_pad = (n_keys + kAttnPad - 1) / kAttnPad * kAttnPad;
     const uint32_t n_slices = kAttnThreads / hv ? kAttnThreads / hv : 1;
     double *wd = lds_d;                                          // [n_pad] softmax weights (f16 values), 0 beyond n_keys
@@ -300,13 +295,25 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
     for (uint32_t t = tid; t < n_pad; t += kAttnThreads) scores[t] = t < n_keys ? rmi_expf_tab(scores[t] - max_val, exp_tab) : 0.0f;
     __syncthreads();
     if (tid == 0) {  // the reference adds the weights one after the other in f32; the padding zeros change nothing
+        // one lane, one dependent chain of adds: the LDS reads run a batch of 32 values ahead of it
         float acc = 0.0f;
-        for (uint32_t t = 0; t < n_pad; t += 4) {
-            const float4 e = *reinterpret_cast<const float4 *>(scores + t);
-            acc += e.x;
-            acc += e.y;
-            acc += e.z;
-            acc += e.w;
+        float4 cur[8], nxt[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) cur[j] = reinterpret_cast<const float4 *>(scores)[j];
+        for (uint32_t t = 0; t < n_pad; t += 32) {  // n_pad is a multiple of 64
+            if (t + 32 < n_pad) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) nxt[j] = reinterpret_cast<const float4 *>(scores + t + 32)[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc += cur[j].x;
+                acc += cur[j].y;
+                acc += cur[j].z;
+                acc += cur[j].w;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) cur[j] = nxt[j];
         }
         red_f[0] = acc;
     }
@@ -530,13 +537,13 @@ int gemv(const rmi_hip_weight *w, const int8_t *q8, const float *scales, float *
     return rmi_launch_gemv_q8_0_single(p, 1, st);
 }
 
-// One decoder step: the token and the position come from the step counter in HBM, so every launch has the
-// same arguments at every step.  Leaves logits, argmax and the next token on the device and advances the counter.
-int enqueue_step(rmi_hip_qwen3 *s, hipStream_t st) {
+// One decoder step at position `step` (the host's copy of the counter in HBM, which the last kernel advances).
+// Leaves logits, argmax and the next token on the device.
+int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
     const rmi_hip_qwen3_config &c = s->cfg;
     const int rnd = c.rounding;
     StepParams *sp = static_cast<StepParams *>(s->params);
-    const size_t attn_lds = attn_lds_bytes(c.capacity, c.head_dim_k, c.head_dim_v);
+    const size_t attn_lds = attn_lds_bytes(step + 1, c.head_dim_k, c.head_dim_v);
     hipLaunchKernelGGL(embed_q8_0_kernel, dim3(1), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, sp, c.vocab,
                        s->x, c.n_embd);
     const float *pending = nullptr;  // matmul output still to be added to the residual stream
@@ -545,14 +552,14 @@ int enqueue_step(rmi_hip_qwen3 *s, hipStream_t st) {
                            c.eps, s->act_q8, s->act_scales, rnd);
         int rc = gemv(s->w_qkv[l], s->act_q8, s->act_scales, s->qkv, st);
         if (rc != RMI_HIP_OK) return rc;
-        const size_t layer_base = size_t(l) * c.capacity * s->kv_stride;
+        const size_t layer_base = size_t(l) * c.capacity * s->kv_stride, row = layer_base + size_t(step) * s->kv_stride;
         hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv), dim3(64), 0, st, s->qkv,
                            c.has_qk_norm ? s->q_norm[l] : nullptr, c.has_qk_norm ? s->k_norm[l] : nullptr, s->cos_t,
-                           s->sin_t, 0u, s->q16, s->k_cache + layer_base, s->v_cache + layer_base, c.n_head,
-                           c.n_head_kv, c.head_dim_k, c.head_dim_v, c.eps, sp, s->kv_stride);
+                           s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv,
+                           c.head_dim_k, c.head_dim_v, c.eps);
         hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(kAttnThreads), attn_lds, st, s->q16,
-                           s->k_cache + layer_base, s->v_cache + layer_base, 0u, s->kv_stride, c.n_head, c.n_head_kv,
-                           c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd, sp);
+                           s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv,
+                           c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
         rc = gemv(s->w_o[l], s->act_q8, s->act_scales, s->resid, st);
         if (rc != RMI_HIP_OK) return rc;
         hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, s->resid, s->ffn_norm[l], c.n_embd,
@@ -624,7 +631,7 @@ int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const fl
     if (n_head == 0 || n_head_kv == 0 || head_dim_k % 2) return rmi_fail(RMI_HIP_E_INVALID, "bad head shape");
     hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(n_head + 2 * n_head_kv), dim3(64), 0,
                        static_cast<hipStream_t>(stream), qkv, q_norm, k_norm, cos_row, sin_row, 0u, q16, k_row, v_row,
-                       n_head, n_head_kv, head_dim_k, head_dim_v, eps, static_cast<const StepParams *>(nullptr), 0u);
+                       n_head, n_head_kv, head_dim_k, head_dim_v, eps);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -642,7 +649,7 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     if (lds > 64 * 1024) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
     hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream), q16,
                        k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8, scales,
-                       rounding, static_cast<const StepParams *>(nullptr));
+                       rounding);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -794,7 +801,7 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     const auto t0 = std::chrono::steady_clock::now();
     for (uint32_t step = 0; e == hipSuccess && rc == RMI_HIP_OK && step < steps; step++) {
-        rc = enqueue_step(s, st);
+        rc = enqueue_step(s, step, st);
         for (uint32_t d = 0; rc == RMI_HIP_OK && d < n_dump; d++)
             if (dump_steps[d] == step)
                 e = hipMemcpyAsync(d_dump + size_t(d) * c.vocab, s->logits, size_t(c.vocab) * 4, hipMemcpyDeviceToDevice, st);

@@ -59,6 +59,49 @@ __device__ __forceinline__ void load_octet(OctetRegs &g, gptr_u4 sc_ptr, gptr_u4
     g.qb = __builtin_nontemporal_load(q_ptr + (2 * o + 1) * 64);
 }
 
+// Stages one token's activation in LDS: the int8 quants of n_oct octets, moved from source order to quad
+// order (dword l of block b -> [b/4][l][b%4]), then the f32 block scales; zeros beyond the nb source blocks.
+// The loads are 16 bytes wide, unconditional (clamped) and issued UNROLL at a time before the first LDS
+// write waits for them: a guarded load per dword costs one memory round trip per loop iteration.
+template <int UNROLL>
+__device__ __forceinline__ void stage_token(uint32_t *dq, const int8_t *x_q8, const float *x_scales, uint32_t n_oct,
+                                            uint32_t nb, uint32_t tid, uint32_t n_threads) {
+    gptr_u4 xq = as_global<gptr_u4>(x_q8);
+    gptr_f32 xs = as_global<gptr_f32>(x_scales);
+    const uint32_t n_u4 = n_oct * 16, src_u4 = nb * 2;
+    // the first two scales of this thread travel with the quants
+    const uint32_t s0 = tid, s1 = tid + n_threads;
+    const float sv0 = xs[s0 < nb ? s0 : nb - 1], sv1 = xs[s1 < nb ? s1 : nb - 1];
+    for (uint32_t base = tid; base < n_u4; base += n_threads * UNROLL) {
+        u32x4 v[UNROLL];
+#pragma unroll
+        for (int j = 0; j < UNROLL; j++) {
+            const uint32_t i = base + j * n_threads;
+            v[j] = xq[i < src_u4 ? i : src_u4 - 1];
+        }
+#pragma unroll
+        for (int j = 0; j < UNROLL; j++) {
+            const uint32_t i = base + j * n_threads;
+            if (i < n_u4) {
+                const uint32_t b = i >> 1;  // block; this uint4 holds its dwords l = 4*(i&1) .. +3
+                uint32_t *d = dq + (b >> 2) * 32 + (i & 1) * 16 + (b & 3);
+                const bool live = i < src_u4;
+                d[0] = live ? v[j].x : 0u;
+                d[4] = live ? v[j].y : 0u;
+                d[8] = live ? v[j].z : 0u;
+                d[12] = live ? v[j].w : 0u;
+            }
+        }
+    }
+    float *ds = reinterpret_cast<float *>(dq + n_oct * 64);
+    if (s0 < n_oct * 8) ds[s0] = s0 < nb ? sv0 : 0.0f;
+    if (s1 < n_oct * 8) ds[s1] = s1 < nb ? sv1 : 0.0f;
+    for (uint32_t i = tid + 2 * n_threads; i < n_oct * 8; i += n_threads) {
+        const float sv = xs[i < nb ? i : nb - 1];
+        ds[i] = i < nb ? sv : 0.0f;
+    }
+}
+
 template <int B>
 __device__ __forceinline__ void octet_fma(float (&acc)[B], const OctetRegs &g, const uint4 *lds, uint32_t tok_u4,
                                           uint32_t n_oct, uint32_t o, uint32_t L) {
@@ -124,17 +167,9 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
     {
         const uint32_t nb = p.n_in >> 5;
         uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
-        for (int t = 0; t < B; t++) {
-            gptr_u32 xq = as_global<gptr_u32>(p.x_q8 + size_t(t) * p.n_in);
-            gptr_f32 xs = as_global<gptr_f32>(p.x_scales + size_t(t) * nb);
-            uint32_t *dq = lds_dw + t * tok_u4 * 4;
-            for (uint32_t i = threadIdx.x; i < n_oct * 64; i += blockDim.x) {
-                const uint32_t b = i >> 3, l = i & 7;
-                dq[(b >> 2) * 32 + l * 4 + (b & 3)] = b < nb ? xq[i] : 0u;
-            }
-            float *ds = reinterpret_cast<float *>(dq + n_oct * 64);
-            for (uint32_t i = threadIdx.x; i < n_oct * 8; i += blockDim.x) ds[i] = i < nb ? xs[i] : 0.0f;
-        }
+        for (int t = 0; t < B; t++)
+            stage_token<4>(lds_dw + t * tok_u4 * 4, p.x_q8 + size_t(t) * p.n_in, p.x_scales + size_t(t) * nb, n_oct, nb,
+                           threadIdx.x, blockDim.x);
         __syncthreads();
     }
 
@@ -172,6 +207,54 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
             const float y = hsum8_lanes(acc[t]);
             if (L == 0 && row >= p.row_start && row < p.row_end) yp[size_t(t) * p.y_stride + row] = y;
         }
+    }
+}
+
+// Launches too small to fill the chip (one token, a matrix of at most a few thousand tiles) are bound by
+// latency, not bandwidth: one wave per tile, and all loads of the tile's NOCT octets go out at once, before
+// the activation is staged, so the wave sees one memory round trip instead of one per pipeline refill.
+// Same arithmetic and order as the streaming kernel above.
+template <int NOCT>
+__global__ __launch_bounds__(64) void gemv_q8_0_deep_kernel(RmiGemvProblem p) {
+    extern __shared__ uint4 lds[];
+    const uint32_t lane = threadIdx.x, r = lane >> 3, L = lane & 7;
+    const uint32_t k = blockIdx.x;
+    gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * NOCT * kOctetBytes);
+    OctetRegs g[NOCT];
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+    stage_token<(NOCT + 3) / 4>(reinterpret_cast<uint32_t *>(lds), p.x_q8, p.x_scales, NOCT, p.n_in >> 5, lane, 64);
+    __syncthreads();
+    float acc[1] = {0.0f};
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
+    const uint32_t row = (p.tile0 + k) * kTileRows + r;
+    const float y = hsum8_lanes(acc[0]);
+    if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
+}
+
+template <int NOCT>
+int launch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
+    hipLaunchKernelGGL((gemv_q8_0_deep_kernel<NOCT>), dim3(p.n_tiles), dim3(64), size_t(NOCT) * 288, s, p);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+constexpr uint32_t kDeepMaxOct = 12, kDeepMaxTiles = 4096;
+int dispatch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
+    switch (p.n_oct) {
+        case 1: return launch_gemv_deep<1>(p, s);
+        case 2: return launch_gemv_deep<2>(p, s);
+        case 3: return launch_gemv_deep<3>(p, s);
+        case 4: return launch_gemv_deep<4>(p, s);
+        case 5: return launch_gemv_deep<5>(p, s);
+        case 6: return launch_gemv_deep<6>(p, s);
+        case 7: return launch_gemv_deep<7>(p, s);
+        case 8: return launch_gemv_deep<8>(p, s);
+        case 9: return launch_gemv_deep<9>(p, s);
+        case 10: return launch_gemv_deep<10>(p, s);
+        case 11: return launch_gemv_deep<11>(p, s);
+        default: return launch_gemv_deep<12>(p, s);
     }
 }
 
@@ -322,6 +405,7 @@ int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s) {
 
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s) {
     if (p.n_tiles == 0 || p.n_oct == 0) return RMI_HIP_OK;
+    if (n_tokens == 1 && p.n_oct <= kDeepMaxOct && p.n_tiles <= kDeepMaxTiles) return dispatch_gemv_deep(p, s);
     const uint32_t tpw = rmi_gemv_tiles_per_wave(p.n_oct, p.n_tiles, n_tokens);
     const uint32_t wpg = rmi_gemv_waves_per_group(size_t(n_tokens) * p.n_oct * 288, size_t(tpw) * p.n_oct * kOctetBytes);
     return dispatch_gemv(n_tokens, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, wpg, tpw, p.n_oct, s);
