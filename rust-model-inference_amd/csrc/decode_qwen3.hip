@@ -75,29 +75,42 @@ __global__ __launch_bounds__(256) void embed_q8_0_kernel(const uint8_t *__restri
     }
 }
 
-// x += r (if r), then rms_norm(x, weight) quantized to Q8_0.  One workgroup of 256.
+// x += r (if r), then rms_norm(x, weight) quantized to Q8_0.  One workgroup of 256; R float4 per thread stay in
+// registers (n <= 1024 * R), and every load of the kernel goes out before the first wait, so the kernel sees
+// one memory round trip.  Sum of squares: per thread in ascending order, f64, then lanes and waves combined.
+template <int R>
 __global__ __launch_bounds__(256) void add_rmsnorm_quant_kernel(float *__restrict__ x, const float *__restrict__ r,
                                                                  const float *__restrict__ weight, uint32_t n, float eps,
                                                                  int8_t *__restrict__ q8, float *__restrict__ scales,
                                                                  int rounding) {
     __shared__ double red[4];
     const uint32_t tid = threadIdx.x;
+    float4 v[R], a[R], wv[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) {  // unconditional loads; a vector past the end re-reads the last one and is not used
+        const uint32_t i = tid * 4 + j * 1024, ic = i < n ? i : n - 4;
+        v[j] = *reinterpret_cast<const float4 *>(x + ic);
+        if (r) a[j] = *reinterpret_cast<const float4 *>(r + ic);
+        wv[j] = *reinterpret_cast<const float4 *>(weight + ic);
+    }
     double part = 0.0;
-    for (uint32_t i = tid * 4; i < n; i += 1024) {
-        float4 v = *reinterpret_cast<const float4 *>(x + i);
-        if (r) {
-            const float4 a = *reinterpret_cast<const float4 *>(r + i);
-            v.x += a.x;
-            v.y += a.y;
-            v.z += a.z;
-            v.w += a.w;
-            *reinterpret_cast<float4 *>(x + i) = v;
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        const uint32_t i = tid * 4 + j * 1024;
+        if (i < n) {
+            if (r) {
+                v[j].x += a[j].x;
+                v[j].y += a[j].y;
+                v[j].z += a[j].z;
+                v[j].w += a[j].w;
+                *reinterpret_cast<float4 *>(x + i) = v[j];
+            }
+            const float s0 = v[j].x * v[j].x, s1 = v[j].y * v[j].y, s2 = v[j].z * v[j].z, s3 = v[j].w * v[j].w;
+            part += double(s0);
+            part += double(s1);
+            part += double(s2);
+            part += double(s3);
         }
-        const float s0 = v.x * v.x, s1 = v.y * v.y, s2 = v.z * v.z, s3 = v.w * v.w;
-        part += double(s0);
-        part += double(s1);
-        part += double(s2);
-        part += double(s3);
     }
     part = wave_sum(part);
     if ((tid & 63) == 0) red[tid >> 6] = part;
@@ -105,18 +118,35 @@ __global__ __launch_bounds__(256) void add_rmsnorm_quant_kernel(float *__restric
     const double total = (red[0] + red[1]) + (red[2] + red[3]);
     const float mean_sq = float(total / double(n));
     const float scale = 1.0f / sqrtf(mean_sq + eps);
-    for (uint32_t i = tid * 4; i < n; i += 1024) {
-        const float4 v = *reinterpret_cast<const float4 *>(x + i);
-        const float4 wv = *reinterpret_cast<const float4 *>(weight + i);
-        float4 o;
-        o.x = (v.x * scale) * wv.x;
-        o.y = (v.y * scale) * wv.y;
-        o.z = (v.z * scale) * wv.z;
-        o.w = (v.w * scale) * wv.w;
-        float sc;
-        reinterpret_cast<uint32_t *>(q8)[i >> 2] = rmi_quantize_block8(o, rounding, &sc);
-        if ((tid & 7) == 0) scales[i >> 5] = sc;
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        const uint32_t i = tid * 4 + j * 1024;
+        if (i < n) {  // n is a multiple of 32: whole 8-lane groups
+            float4 o;
+            o.x = (v[j].x * scale) * wv[j].x;
+            o.y = (v[j].y * scale) * wv[j].y;
+            o.z = (v[j].z * scale) * wv[j].z;
+            o.w = (v[j].w * scale) * wv[j].w;
+            float sc;
+            reinterpret_cast<uint32_t *>(q8)[i >> 2] = rmi_quantize_block8(o, rounding, &sc);
+            if ((tid & 7) == 0) scales[i >> 5] = sc;
+        }
     }
+}
+
+constexpr uint32_t kNormMaxN = 1024 * 16;
+void launch_add_rmsnorm_quant(float *x, const float *r, const float *weight, uint32_t n, float eps, int8_t *q8,
+                              float *scales, int rounding, hipStream_t st) {
+    if (n <= 1024)
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<1>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+    else if (n <= 2048)
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<2>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+    else if (n <= 4096)
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<4>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+    else if (n <= 8192)
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<8>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+    else
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<16>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
 }
 
 // Per head of the stacked q|k|v vector: q/k RMS norm, NeoX rotation, f16 rounding; k and v go to the cache row.
@@ -132,6 +162,12 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(const float *__r
     if (head >= n_head + n_head_kv) {  // v: rounding only
         const uint32_t kvh = head - n_head - n_head_kv;
         const float *src = qkv + size_t(n_head) * hk + size_t(n_head_kv) * hk + size_t(kvh) * hv;
+        if (hv == 128) {
+            const float v0 = src[tid], v1 = src[tid + 64];
+            v_row[kvh * 128 + tid] = f2h(v0);
+            v_row[kvh * 128 + tid + 64] = f2h(v1);
+            return;
+        }
         for (uint32_t d = tid; d < hv; d += 64) v_row[kvh * hv + d] = f2h(src[d]);
         return;
     }
@@ -139,6 +175,28 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(const float *__r
     const uint32_t local = is_q ? head : head - n_head;
     const float *src = qkv + (is_q ? size_t(local) * hk : size_t(n_head) * hk + size_t(local) * hk);
     const float *nw = is_q ? q_norm : k_norm;
+    if (hk == 128) {  // lane i owns the pair (i, i + 64): every load goes out before the first wait
+        const float x0r = src[tid], x1r = src[tid + 64];
+        const float cos_a = cos_t[size_t(pos) * 64 + tid], sin_a = sin_t[size_t(pos) * 64 + tid];
+        float x0 = x0r, x1 = x1r;
+        if (nw) {
+            const float w0 = nw[tid], w1 = nw[tid + 64];
+            const float q0 = x0r * x0r, q1 = x1r * x1r;
+            double part = double(q0);
+            part += double(q1);
+            const double total = wave_sum(part);
+            const float mean_sq = float(total / 128.0);
+            const float sc = 1.0f / sqrtf(mean_sq + eps);
+            x0 = (x0r * sc) * w0;
+            x1 = (x1r * sc) * w1;
+        }
+        uint16_t *dst = is_q ? q16 + size_t(local) * 128 : k_row + size_t(local) * 128;
+        const float a = x1 * -sin_a;
+        const float b = x1 * cos_a;
+        dst[tid] = f2h(__builtin_fmaf(x0, cos_a, a));
+        dst[tid + 64] = f2h(__builtin_fmaf(x0, sin_a, b));
+        return;
+    }
     float scale = 1.0f;
     if (nw) {
         double part = 0.0;
@@ -548,8 +606,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                        s->x, c.n_embd);
     const float *pending = nullptr;  // matmul output still to be added to the residual stream
     for (uint32_t l = 0; l < c.n_layer; l++) {
-        hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, pending, s->attn_norm[l], c.n_embd,
-                           c.eps, s->act_q8, s->act_scales, rnd);
+        launch_add_rmsnorm_quant(s->x, pending, s->attn_norm[l], c.n_embd, c.eps, s->act_q8, s->act_scales, rnd, st);
         int rc = gemv(s->w_qkv[l], s->act_q8, s->act_scales, s->qkv, st);
         if (rc != RMI_HIP_OK) return rc;
         const size_t layer_base = size_t(l) * c.capacity * s->kv_stride, row = layer_base + size_t(step) * s->kv_stride;
@@ -562,8 +619,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                            c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
         rc = gemv(s->w_o[l], s->act_q8, s->act_scales, s->resid, st);
         if (rc != RMI_HIP_OK) return rc;
-        hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, s->resid, s->ffn_norm[l], c.n_embd,
-                           c.eps, s->act_q8, s->act_scales, rnd);
+        launch_add_rmsnorm_quant(s->x, s->resid, s->ffn_norm[l], c.n_embd, c.eps, s->act_q8, s->act_scales, rnd, st);
         rc = gemv(s->w_gu[l], s->act_q8, s->act_scales, s->gu, st);
         if (rc != RMI_HIP_OK) return rc;
         hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((c.n_ff + 1023) / 1024), dim3(256), 0, st, s->gu, c.n_ff,
@@ -572,8 +628,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
         if (rc != RMI_HIP_OK) return rc;
         pending = s->resid;
     }
-    hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, st, s->x, pending, s->output_norm, c.n_embd,
-                       c.eps, s->act_q8, s->act_scales, rnd);
+    launch_add_rmsnorm_quant(s->x, pending, s->output_norm, c.n_embd, c.eps, s->act_q8, s->act_scales, rnd, st);
     int rc = gemv(s->head, s->act_q8, s->act_scales, s->logits, st);
     if (rc != RMI_HIP_OK) return rc;
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxGroups), dim3(256), 0, st, s->logits, c.vocab,
@@ -604,9 +659,9 @@ int rmi_hip_rms_norm_quantize_q8_0_dev(float *x, const float *residual, const fl
     RMI_REQUIRE_INIT();
     if (n == 0) return RMI_HIP_OK;
     if (n % 32 != 0) return rmi_fail(RMI_HIP_E_INVALID, "n=%u is not a multiple of 32", n);
+    if (n > kNormMaxN) return rmi_fail(RMI_HIP_E_INVALID, "n=%u exceeds the %u elements the norm kernel holds", n, kNormMaxN);
     if (!x || !weight || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
-    hipLaunchKernelGGL(add_rmsnorm_quant_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), x, residual,
-                       weight, n, eps, q8, scales, rounding);
+    launch_add_rmsnorm_quant(x, residual, weight, n, eps, q8, scales, rounding, static_cast<hipStream_t>(stream));
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -679,6 +734,7 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
     if (c.n_embd == 0 || c.n_embd % 32 || c.n_ff == 0 || c.n_ff % 32 || c.n_layer == 0 || c.n_head == 0 ||
         c.n_head_kv == 0 || c.n_head % c.n_head_kv || c.head_dim_k == 0 || c.head_dim_k % 32 || c.head_dim_v == 0 ||
         c.head_dim_v % 32 || c.head_dim_k > 1024 || c.head_dim_v > 1024 || c.vocab == 0 || c.capacity == 0 ||
+        c.n_embd > kNormMaxN ||
         (c.rounding != RMI_HIP_ROUND_TIES_EVEN && c.rounding != RMI_HIP_ROUND_HALF_AWAY)) {
         rmi_set_error("unsupported model shape");
         return nullptr;
