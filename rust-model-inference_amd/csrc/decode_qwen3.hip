@@ -424,6 +424,211 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
     }
 }
 
+// ---- the same attention for head dimension 128 (keys and values), the Qwen3 shape.  Arithmetic as above;
+// what differs is the schedule.  The launch has 16 workgroups on a 256-CU chip, so its time is the length of one
+// thread's instruction stream plus memory round trips, not throughput: the query stays in registers as packed
+// f16 (product f16 x f16 is exact in f32, then an f64 add: the same value as the f64 fma above), every load of
+// the first round of keys and of the first 12 values per thread goes out before anything waits, values are read
+// 16 bytes (8 dimensions) at a time by 64 key slices, and the four slices of a wave combine in registers.
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ half8 as_half8(const uint4 &v) { return __builtin_bit_cast(half8, v); }
+__device__ __forceinline__ double quad_sum(double v) {  // (l0 + l1) + (l2 + l3) in every lane of the quad
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    v += __hiloint2double(__builtin_amdgcn_mov_dpp(hi, 0xB1, 0xf, 0xf, true), __builtin_amdgcn_mov_dpp(lo, 0xB1, 0xf, 0xf, true));
+    lo = __double2loint(v), hi = __double2hiint(v);
+    v += __hiloint2double(__builtin_amdgcn_mov_dpp(hi, 0x4E, 0xf, 0xf, true), __builtin_amdgcn_mov_dpp(lo, 0x4E, 0xf, 0xf, true));
+    return v;
+}
+__host__ __device__ inline size_t attn128_lds_bytes(uint32_t n_keys) {
+    const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
+    return n_pad * 12 + 16 * 128 * 8;
+}
+__global__ __launch_bounds__(kAttnThreads) void attention128_quant_kernel(
+    const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
+    uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, int8_t *__restrict__ q8,
+    float *__restrict__ scales, int rounding) {
+    extern __shared__ double lds_d[];
+    __shared__ float red_f[kAttnThreads / 64];
+    __shared__ uint64_t exp_tab[32];
+    // grid = (query heads per key/value head, key/value heads)
+    const uint32_t kvh = blockIdx.y, head = blockIdx.y * gridDim.x + blockIdx.x, tid = threadIdx.x;
+    const uint32_t n_keys = step + 1;
+    const uint32_t n_pad = (n_keys + kAttnPad - 1) / kAttnPad * kAttnPad;
+    double *wd = lds_d;                                        // [n_pad] softmax weights (f16 values), 0 beyond n_keys
+    double *part = wd + n_pad;                                 // [16 waves][128]
+    float *scores = reinterpret_cast<float *>(part + 16 * 128);  // [n_pad]
+    const uint32_t row_u4 = kv_stride >> 3;                    // uint4 per cache row
+    const uint64_t tab_entry = kRmiExp2fTab[tid & 31];         // first load out; stored to LDS after the scores
+
+    // scores: four lanes per key; lane4 takes the 16-byte pieces lane4, 4 + lane4, 8 + lane4, 12 + lane4 of the
+    // key's 256 bytes, so that the four lanes of a key read 64 consecutive bytes with each load (the memory
+    // pipeline handles a quad of lanes per step, and a quad that spans several cache lines takes several)
+    const uint32_t lane4 = tid & 3, key0 = tid >> 2;
+    const uint4 *qp = reinterpret_cast<const uint4 *>(q16 + size_t(head) * 128) + lane4;
+    const uint4 *kbase = reinterpret_cast<const uint4 *>(k_cache + size_t(kvh) * 128) + lane4;
+    uint4 qv[4], kk[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) qv[c] = qp[4 * c];
+    {
+        const uint4 *key = kbase + __umul24(key0 < n_keys ? key0 : n_keys - 1, row_u4);
+#pragma unroll
+        for (int c = 0; c < 4; c++) kk[c] = key[4 * c];
+    }
+    // values: lane = (8 dimensions dg, key slice sl): 16 consecutive lanes read the 256 bytes of one row
+    constexpr uint32_t kPre = 12;
+    const uint32_t dg = tid & 15, sl = tid >> 4;
+    const uint32_t chunk = (n_keys + 63) >> 6;
+    const uint32_t t_begin = sl * chunk, t_end = t_begin + chunk < n_keys ? t_begin + chunk : n_keys;
+    const uint4 *vbase = reinterpret_cast<const uint4 *>(v_cache + size_t(kvh) * 128 + dg * 8);
+    uint4 vp[kPre];
+#pragma unroll
+    for (uint32_t j = 0; j < kPre; j++) {  // j < chunk is uniform: no lane waits on a guarded load of its own
+        if (j < chunk) {
+            const uint32_t t = t_begin + j < n_keys ? t_begin + j : n_keys - 1;
+            vp[j] = vbase[__umul24(t, row_u4)];
+        }
+    }
+    const float kq_scale = 1.0f / sqrtf(128.0f);  // two f32 roundings, as the reference computes it
+    float my_max = -INFINITY;
+    for (uint32_t t0 = 0; t0 < n_keys; t0 += kAttnThreads / 4) {
+        const uint32_t t = t0 + key0, tn = t + kAttnThreads / 4;
+        uint4 kn[4];
+        if (t0 + kAttnThreads / 4 < n_keys) {  // the next round's keys are in flight while this one is summed
+            const uint4 *key = kbase + __umul24(tn < n_keys ? tn : n_keys - 1, row_u4);
+#pragma unroll
+            for (int c = 0; c < 4; c++) kn[c] = key[4 * c];
+        }
+        double sum = 0.0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const half8 kh = as_half8(kk[c]), qh = as_half8(qv[c]);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float prod = __builtin_fmaf(float(kh[j]), float(qh[j]), 0.0f);  // exact
+                sum += double(prod);
+            }
+        }
+        sum = quad_sum(sum);
+        if (t < n_keys) {
+            const float sc = float(sum) * kq_scale;
+            if (lane4 == 0) scores[t] = sc;
+            my_max = fmaxf(my_max, sc);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) kk[c] = kn[c];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) my_max = fmaxf(my_max, __shfl_xor(my_max, off, 64));
+    if ((tid & 63) == 0) red_f[tid >> 6] = my_max;
+    if (tid < 32) exp_tab[tid] = tab_entry;
+    __syncthreads();
+    float max_val = red_f[0];
+#pragma unroll
+    for (uint32_t i = 1; i < kAttnThreads / 64; i++) max_val = fmaxf(max_val, red_f[i]);
+    for (uint32_t t = tid; t < n_pad; t += kAttnThreads) scores[t] = t < n_keys ? rmi_expf_tab(scores[t] - max_val, exp_tab) : 0.0f;
+    __syncthreads();
+    if (tid == 0) {  // the reference adds the weights one after the other in f32; the padding zeros change nothing
+        // one lane, one dependent chain of adds; the LDS reads run 32 values ahead of it (two buffers, no copies)
+        float acc = 0.0f;
+        float4 a[8], b[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) a[j] = reinterpret_cast<const float4 *>(scores)[j];
+        for (uint32_t t = 0; t < n_pad; t += 64) {  // n_pad is a multiple of 64
+#pragma unroll
+            for (int j = 0; j < 8; j++) b[j] = reinterpret_cast<const float4 *>(scores + t + 32)[j];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc += a[j].x;
+                acc += a[j].y;
+                acc += a[j].z;
+                acc += a[j].w;
+            }
+            if (t + 64 < n_pad) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) a[j] = reinterpret_cast<const float4 *>(scores + t + 64)[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc += b[j].x;
+                acc += b[j].y;
+                acc += b[j].z;
+                acc += b[j].w;
+            }
+        }
+        red_f[0] = acc;
+    }
+    __syncthreads();
+    const float total = red_f[0];
+    for (uint32_t t = tid; t < n_pad; t += kAttnThreads) {
+        const float e = scores[t];
+        wd[t] = t < n_keys ? double(h2f(f2h(total > 0.0f ? e / total : e))) : 0.0;
+    }
+    __syncthreads();
+
+    double acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) acc[j] = 0.0;
+#pragma unroll
+    for (uint32_t j = 0; j < kPre; j++) {
+        if (t_begin + j < t_end) {
+            const double w = wd[t_begin + j];
+            const half8 vh = as_half8(vp[j]);
+#pragma unroll
+            for (int d = 0; d < 8; d++) acc[d] = __builtin_fma(double(float(vh[d])), w, acc[d]);
+        }
+    }
+    if (t_begin + kPre < t_end) {  // longer slices: batches of 8 keys, the next one in flight while one is added
+        uint4 cur[8], nxt[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; j++) {
+            const uint32_t t = t_begin + kPre + j;
+            cur[j] = vbase[__umul24(t < n_keys ? t : n_keys - 1, row_u4)];
+        }
+        for (uint32_t t0 = t_begin + kPre; t0 < t_end; t0 += 8) {
+#pragma unroll
+            for (uint32_t j = 0; j < 8; j++) {
+                const uint32_t t = t0 + 8 + j;
+                nxt[j] = vbase[__umul24(t < n_keys ? t : n_keys - 1, row_u4)];
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < 8; j++) {
+                if (t0 + j < t_end) {
+                    const double w = wd[t0 + j];
+                    const half8 vh = as_half8(cur[j]);
+#pragma unroll
+                    for (int d = 0; d < 8; d++) acc[d] = __builtin_fma(double(float(vh[d])), w, acc[d]);
+                }
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < 8; j++) cur[j] = nxt[j];
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < 8; d++) {  // the four slices of a wave: lanes 16 apart
+        acc[d] += __shfl_xor(acc[d], 16, 64);
+        acc[d] += __shfl_xor(acc[d], 32, 64);
+    }
+    if ((tid & 63) < 16) {
+        double *dst = part + (tid >> 6) * 128 + dg * 8;
+#pragma unroll
+        for (int d = 0; d < 8; d++) dst[d] = acc[d];
+    }
+    __syncthreads();
+    if (tid < 32) {  // four dimensions per lane: whole 8-lane groups for the quantizer
+        double o[4];
+#pragma unroll
+        for (int d = 0; d < 4; d++) o[d] = part[tid * 4 + d];
+        for (uint32_t w = 1; w < kAttnThreads / 64; w++) {
+#pragma unroll
+            for (int d = 0; d < 4; d++) o[d] += part[w * 128 + tid * 4 + d];
+        }
+        const float4 of = make_float4(float(o[0]), float(o[1]), float(o[2]), float(o[3]));
+        float sc;
+        reinterpret_cast<uint32_t *>(q8)[(size_t(head) * 128 >> 2) + tid] = rmi_quantize_block8(of, rounding, &sc);
+        if ((tid & 7) == 0) scales[(size_t(head) * 128 >> 5) + (tid >> 3)] = sc;
+    }
+}
+
 // gu = [W_gate x ; W_up x]: h = (W_up x) * silu(W_gate x), quantized to Q8_0
 __global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float *__restrict__ gu, uint32_t n_ff,
                                                              int8_t *__restrict__ q8, float *__restrict__ scales,
@@ -614,9 +819,14 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                            c.has_qk_norm ? s->q_norm[l] : nullptr, c.has_qk_norm ? s->k_norm[l] : nullptr, s->cos_t,
                            s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv,
                            c.head_dim_k, c.head_dim_v, c.eps);
-        hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(kAttnThreads), attn_lds, st, s->q16,
-                           s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv,
-                           c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
+        if (c.head_dim_k == 128 && c.head_dim_v == 128)
+            hipLaunchKernelGGL(attention128_quant_kernel, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kAttnThreads), attn128_lds_bytes(step + 1),
+                               st, s->q16, s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride,
+                               c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd);
+        else
+            hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(kAttnThreads), attn_lds, st, s->q16,
+                               s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head,
+                               c.n_head_kv, c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
         rc = gemv(s->w_o[l], s->act_q8, s->act_scales, s->resid, st);
         if (rc != RMI_HIP_OK) return rc;
         launch_add_rmsnorm_quant(s->x, s->resid, s->ffn_norm[l], c.n_embd, c.eps, s->act_q8, s->act_scales, rnd, st);
@@ -700,11 +910,16 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     if (n_keys == 0 || n_head == 0 || n_head_kv == 0 || n_head % n_head_kv || head_dim_k % 32 || head_dim_v % 32 ||
         head_dim_k == 0 || head_dim_v == 0 || head_dim_k > 1024 || head_dim_v > 1024 || kv_stride % 8)
         return rmi_fail(RMI_HIP_E_INVALID, "bad attention shape");
-    const size_t lds = attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
+    const bool d128 = head_dim_k == 128 && head_dim_v == 128;
+    const size_t lds = d128 ? attn128_lds_bytes(n_keys) : attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
     if (lds > 64 * 1024) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
-    hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream), q16,
-                       k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8, scales,
-                       rounding);
+    if (d128)
+        hipLaunchKernelGGL(attention128_quant_kernel, dim3(n_head / n_head_kv, n_head_kv), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream),
+                           q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding);
+    else
+        hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream),
+                           q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8,
+                           scales, rounding);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -740,7 +955,8 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
         return nullptr;
     }
     // attention keeps the scores of one head in LDS
-    if (attn_lds_bytes(c.capacity, c.head_dim_k, c.head_dim_v) > 64 * 1024) {
+    if ((c.head_dim_k == 128 && c.head_dim_v == 128 ? attn128_lds_bytes(c.capacity)
+                                                    : attn_lds_bytes(c.capacity, c.head_dim_k, c.head_dim_v)) > 64 * 1024) {
         rmi_set_error("capacity %u exceeds what the attention kernel holds in LDS", c.capacity);
         return nullptr;
     }
