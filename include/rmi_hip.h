@@ -256,6 +256,13 @@ typedef struct {
  * quantize_q8_0_into does (src/ops/quant/q8_0.rs); x keeps the sum.  n % 32 == 0. */
 int rmi_hip_rms_norm_quantize_q8_0_dev(float *x, const float *residual, const float *weight, uint32_t n, float eps,
                                        int8_t *q8, float *scales, int rounding, void *stream);
+/* The same three steps and the Q8_0 product that follows them in one launch: y = W . Q8_0(rms_norm(x_in +
+ * residual) * norm_weight), x_out = x_in + residual (src/models/qwen3.rs:719-774 and :1016-1019: norm,
+ * quantize_q8_0_into, then the q/k/v or the gate/up matmul).  One token; n_in a multiple of 256 up to 2048 and
+ * at most 32768 rows, else RMI_HIP_E_INVALID (use the separate calls).  x_out must not alias x_in. */
+int rmi_hip_rms_norm_gemv_q8_0_dev(const rmi_hip_weight *w, const float *x_in, const float *residual,
+                                   const float *norm_weight, float eps, int rounding, float *x_out, float *y,
+                                   void *stream);
 /* gate_up = [W_gate x ; W_up x] (2*n_ff): (W_up x) * silu(W_gate x), src/ops/activation/mod.rs:137-151
  * as called at src/models/qwen3.rs:1016-1027, quantized to Q8_0. */
 int rmi_hip_silu_mul_quantize_q8_0_dev(const float *gate_up, uint32_t n_ff, int8_t *q8, float *scales, int rounding,

@@ -24,6 +24,7 @@
 // bit-identical logits against the CPU path, not to a tolerance.
 #include <chrono>
 #include <cmath>
+#include <utility>
 #include <vector>
 
 #include "device_math.h"
@@ -726,7 +727,7 @@ struct rmi_hip_qwen3 {
     float *output_norm = nullptr;
     float *cos_t = nullptr, *sin_t = nullptr;
     uint16_t *k_cache = nullptr, *v_cache = nullptr, *q16 = nullptr;
-    float *x = nullptr, *resid = nullptr, *qkv = nullptr, *gu = nullptr, *logits = nullptr, *act_scales = nullptr;
+    float *x = nullptr, *x2 = nullptr, *resid = nullptr, *qkv = nullptr, *gu = nullptr, *logits = nullptr, *act_scales = nullptr;
     int8_t *act_q8 = nullptr;
     uint32_t *tok = nullptr, *step_argmax = nullptr, *nonfinite = nullptr;
     float *step_top2 = nullptr;
@@ -810,9 +811,19 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
     hipLaunchKernelGGL(embed_q8_0_kernel, dim3(1), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, sp, c.vocab,
                        s->x, c.n_embd);
     const float *pending = nullptr;  // matmul output still to be added to the residual stream
+    // the residual stream alternates between two buffers where the norm is folded into the next product
+    float *x = s->x, *x_other = s->x2;
+    auto norm_gemv = [&](const rmi_hip_weight *w, const float *resid, const float *norm_weight, float *y) -> int {
+        if (rmi_gemv_q8_0_norm_fusable(w)) {
+            int rc = rmi_launch_gemv_q8_0_norm(w, x, resid, norm_weight, x_other, c.eps, rnd, y, st);
+            std::swap(x, x_other);
+            return rc;
+        }
+        launch_add_rmsnorm_quant(x, resid, norm_weight, c.n_embd, c.eps, s->act_q8, s->act_scales, rnd, st);
+        return gemv(w, s->act_q8, s->act_scales, y, st);
+    };
     for (uint32_t l = 0; l < c.n_layer; l++) {
-        launch_add_rmsnorm_quant(s->x, pending, s->attn_norm[l], c.n_embd, c.eps, s->act_q8, s->act_scales, rnd, st);
-        int rc = gemv(s->w_qkv[l], s->act_q8, s->act_scales, s->qkv, st);
+        int rc = norm_gemv(s->w_qkv[l], pending, s->attn_norm[l], s->qkv);
         if (rc != RMI_HIP_OK) return rc;
         const size_t layer_base = size_t(l) * c.capacity * s->kv_stride, row = layer_base + size_t(step) * s->kv_stride;
         hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv), dim3(64), 0, st, s->qkv,
@@ -829,8 +840,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                                c.n_head_kv, c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
         rc = gemv(s->w_o[l], s->act_q8, s->act_scales, s->resid, st);
         if (rc != RMI_HIP_OK) return rc;
-        launch_add_rmsnorm_quant(s->x, s->resid, s->ffn_norm[l], c.n_embd, c.eps, s->act_q8, s->act_scales, rnd, st);
-        rc = gemv(s->w_gu[l], s->act_q8, s->act_scales, s->gu, st);
+        rc = norm_gemv(s->w_gu[l], s->resid, s->ffn_norm[l], s->gu);
         if (rc != RMI_HIP_OK) return rc;
         hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((c.n_ff + 1023) / 1024), dim3(256), 0, st, s->gu, c.n_ff,
                            s->act_q8, s->act_scales, rnd);
@@ -838,8 +848,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
         if (rc != RMI_HIP_OK) return rc;
         pending = s->resid;
     }
-    launch_add_rmsnorm_quant(s->x, pending, s->output_norm, c.n_embd, c.eps, s->act_q8, s->act_scales, rnd, st);
-    int rc = gemv(s->head, s->act_q8, s->act_scales, s->logits, st);
+    int rc = norm_gemv(s->head, pending, s->output_norm, s->logits);
     if (rc != RMI_HIP_OK) return rc;
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxGroups), dim3(256), 0, st, s->logits, c.vocab,
                        static_cast<Top *>(s->partial));
@@ -874,6 +883,16 @@ int rmi_hip_rms_norm_quantize_q8_0_dev(float *x, const float *residual, const fl
     launch_add_rmsnorm_quant(x, residual, weight, n, eps, q8, scales, rounding, static_cast<hipStream_t>(stream));
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
+}
+
+int rmi_hip_rms_norm_gemv_q8_0_dev(const rmi_hip_weight *w, const float *x_in, const float *residual,
+                                   const float *norm_weight, float eps, int rounding, float *x_out, float *y,
+                                   void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (!x_in || !norm_weight || !x_out || !y || x_in == x_out) return rmi_fail(RMI_HIP_E_INVALID, "null or aliased pointer");
+    return rmi_launch_gemv_q8_0_norm(w, x_in, residual, norm_weight, x_out, eps, rounding, y,
+                                     static_cast<hipStream_t>(stream));
 }
 
 int rmi_hip_silu_mul_quantize_q8_0_dev(const float *gate_up, uint32_t n_ff, int8_t *q8, float *scales, int rounding,
@@ -1028,7 +1047,7 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
     }
     const size_t cache = size_t(c.n_layer) * c.capacity * s->kv_stride;
     ok = ok && (s->k_cache = dev_alloc<uint16_t>(s, cache, true)) && (s->v_cache = dev_alloc<uint16_t>(s, cache, true)) &&
-         (s->q16 = dev_alloc<uint16_t>(s, s->n_q)) && (s->x = dev_alloc<float>(s, c.n_embd)) &&
+         (s->q16 = dev_alloc<uint16_t>(s, s->n_q)) && (s->x = dev_alloc<float>(s, c.n_embd)) && (s->x2 = dev_alloc<float>(s, c.n_embd)) &&
          (s->resid = dev_alloc<float>(s, c.n_embd)) && (s->qkv = dev_alloc<float>(s, size_t(s->n_q) + s->n_k + s->n_v)) &&
          (s->gu = dev_alloc<float>(s, size_t(2) * c.n_ff)) && (s->logits = dev_alloc<float>(s, c.vocab)) &&
          (s->act_q8 = dev_alloc<int8_t>(s, s->max_n_in)) && (s->act_scales = dev_alloc<float>(s, s->max_n_in / 32)) &&

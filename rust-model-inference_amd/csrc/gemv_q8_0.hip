@@ -233,6 +233,93 @@ __global__ __launch_bounds__(64) void gemv_q8_0_deep_kernel(RmiGemvProblem p) {
     if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
 }
 
+// The same kernel with the preceding "x += r; rms_norm(x, weight); quantize to Q8_0" folded into its prologue
+// (src/models/qwen3.rs:719-734 and :1016-1027 run those three steps before the q/k/v and the gate/up products):
+// every wave normalises and quantizes the whole activation itself, straight into the staged LDS layout, instead
+// of reading what one more dependent launch would have written.  n_in = NOCT * 256.  Workgroup 0 also stores the
+// updated residual stream to x_out, a buffer other than x_in (the other workgroups still read x_in).
+struct RmiNormArgs {
+    const float *x_in;    // residual stream
+    const float *resid;   // added to it first (may be null)
+    const float *weight;  // norm weight
+    float *x_out;         // x_in + resid
+    float eps;
+    int rounding;
+};
+
+template <int NOCT>
+__global__ __launch_bounds__(64) void gemv_q8_0_norm_deep_kernel(RmiGemvProblem p, RmiNormArgs na) {
+    extern __shared__ uint4 lds[];
+    const uint32_t lane = threadIdx.x, r = lane >> 3, L = lane & 7;
+    const uint32_t k = blockIdx.x;
+    const float4 *xin = reinterpret_cast<const float4 *>(na.x_in), *rin = reinterpret_cast<const float4 *>(na.resid),
+                 *win = reinterpret_cast<const float4 *>(na.weight);
+    float4 v[NOCT], a[NOCT], wv[NOCT];
+#pragma unroll
+    for (int j = 0; j < NOCT; j++) {  // lane owns the float4s lane, lane + 64, ...: element blocks stay in 8 lanes
+        v[j] = xin[lane + 64 * j];
+        if (na.resid) a[j] = rin[lane + 64 * j];
+        wv[j] = win[lane + 64 * j];
+    }
+    gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * NOCT * kOctetBytes);
+    OctetRegs g[NOCT];
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+
+    double part = 0.0;
+#pragma unroll
+    for (int j = 0; j < NOCT; j++) {
+        if (na.resid) {
+            v[j].x += a[j].x;
+            v[j].y += a[j].y;
+            v[j].z += a[j].z;
+            v[j].w += a[j].w;
+        }
+        const float s0 = v[j].x * v[j].x, s1 = v[j].y * v[j].y, s2 = v[j].z * v[j].z, s3 = v[j].w * v[j].w;
+        part += double(s0);
+        part += double(s1);
+        part += double(s2);
+        part += double(s3);
+    }
+    if (k == 0) {
+#pragma unroll
+        for (int j = 0; j < NOCT; j++) reinterpret_cast<float4 *>(na.x_out)[lane + 64 * j] = v[j];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+    const float mean_sq = float(part / double(NOCT * 256));
+    const float scale = 1.0f / sqrtf(mean_sq + na.eps);
+    uint32_t *dq = reinterpret_cast<uint32_t *>(lds);
+    float *ds = reinterpret_cast<float *>(dq + NOCT * 64);
+#pragma unroll
+    for (int j = 0; j < NOCT; j++) {
+        float4 o;
+        o.x = (v[j].x * scale) * wv[j].x;
+        o.y = (v[j].y * scale) * wv[j].y;
+        o.z = (v[j].z * scale) * wv[j].z;
+        o.w = (v[j].w * scale) * wv[j].w;
+        float sc;
+        const uint32_t q = rmi_quantize_block8(o, na.rounding, &sc);
+        const uint32_t b = (lane >> 3) + 8 * j;  // block of this float4; L = its dword inside the block
+        dq[(b >> 2) * 32 + L * 4 + (b & 3)] = q;
+        if (L == 0) ds[b] = sc;
+    }
+    __syncthreads();
+    float acc[1] = {0.0f};
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
+    const uint32_t row = (p.tile0 + k) * kTileRows + r;
+    const float y = hsum8_lanes(acc[0]);
+    if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
+}
+
+template <int NOCT>
+int launch_gemv_norm_deep(const RmiGemvProblem &p, const RmiNormArgs &na, hipStream_t s) {
+    hipLaunchKernelGGL((gemv_q8_0_norm_deep_kernel<NOCT>), dim3(p.n_tiles), dim3(64), size_t(NOCT) * 288, s, p, na);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
 template <int NOCT>
 int launch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
     hipLaunchKernelGGL((gemv_q8_0_deep_kernel<NOCT>), dim3(p.n_tiles), dim3(64), size_t(NOCT) * 288, s, p);
@@ -409,6 +496,36 @@ int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipS
     const uint32_t tpw = rmi_gemv_tiles_per_wave(p.n_oct, p.n_tiles, n_tokens);
     const uint32_t wpg = rmi_gemv_waves_per_group(size_t(n_tokens) * p.n_oct * 288, size_t(tpw) * p.n_oct * kOctetBytes);
     return dispatch_gemv(n_tokens, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, wpg, tpw, p.n_oct, s);
+}
+
+bool rmi_gemv_q8_0_norm_fusable(const rmi_hip_weight *w) {
+    return w->n_in % 256 == 0 && w->n_units >= 1 && w->n_units <= 8 && w->n_tiles >= 1 && w->n_tiles <= kDeepMaxTiles;
+}
+
+int rmi_launch_gemv_q8_0_norm(const rmi_hip_weight *w, const float *x_in, const float *resid, const float *norm_weight,
+                              float *x_out, float eps, int rounding, float *y, hipStream_t s) {
+    if (!rmi_gemv_q8_0_norm_fusable(w)) return rmi_fail(RMI_HIP_E_INVALID, "shape %u x %u is not fusable", w->n_out, w->n_in);
+    RmiGemvProblem p{};
+    p.w = w->data;
+    p.y = y;
+    p.n_in = w->n_in;
+    p.n_oct = w->n_units;
+    p.y_stride = w->n_out;
+    p.row_start = 0;
+    p.row_end = w->n_out;
+    p.tile0 = 0;
+    p.n_tiles = w->n_tiles;
+    const RmiNormArgs na{x_in, resid, norm_weight, x_out, eps, rounding};
+    switch (p.n_oct) {
+        case 1: return launch_gemv_norm_deep<1>(p, na, s);
+        case 2: return launch_gemv_norm_deep<2>(p, na, s);
+        case 3: return launch_gemv_norm_deep<3>(p, na, s);
+        case 4: return launch_gemv_norm_deep<4>(p, na, s);
+        case 5: return launch_gemv_norm_deep<5>(p, na, s);
+        case 6: return launch_gemv_norm_deep<6>(p, na, s);
+        case 7: return launch_gemv_norm_deep<7>(p, na, s);
+        default: return launch_gemv_norm_deep<8>(p, na, s);
+    }
 }
 
 int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,

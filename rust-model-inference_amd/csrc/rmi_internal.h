@@ -119,6 +119,11 @@ struct RmiGemvProblem {
     uint32_t reserved;
 };
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
+// y = W . Q8_0(rms_norm(x_in + resid) * norm_weight) in one launch, x_out = x_in + resid (x_out != x_in);
+// for one token and matrices the fused kernel covers (rmi_gemv_q8_0_norm_fusable)
+bool rmi_gemv_q8_0_norm_fusable(const rmi_hip_weight *w);
+int rmi_launch_gemv_q8_0_norm(const rmi_hip_weight *w, const float *x_in, const float *resid, const float *norm_weight,
+                              float *x_out, float eps, int rounding, float *y, hipStream_t s);
 // d_runs[w] = {problem index, first tile, tile count, 0}: the run of tiles wave w takes
 // the run table holds n_runs entries, a multiple of wpg (waves per workgroup); the wpg runs of one
 // workgroup belong to one problem (count 0 pads)

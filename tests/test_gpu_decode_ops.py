@@ -43,6 +43,39 @@ def test_rms_norm_quantize(hip, oracle, n):
             b.free()
 
 
+@pytest.mark.parametrize("n_in,n_out", [(1024, 4096), (1024, 6144), (256, 13), (2048, 1000)])
+def test_rms_norm_gemv_fused(hip, oracle, n_in, n_out):
+    """add + rms_norm + quantize folded into the Q8_0 product (src/models/qwen3.rs:719-774): the same bits
+    as the three restated steps followed by the restated AVX2 matmul."""
+    H, K = hip.hip, hip.kernel
+    rng = np.random.default_rng(n_in + n_out)
+    w = hip.synth.q8_0_weight(900 + n_out, n_out, n_in)
+    kernel = K.Q8Kernel(w, n_in, n_out)
+    for trial in range(12):
+        x = (rng.normal(0, 1, n_in) * rng.choice([1e-3, 1.0, 30.0])).astype(np.float32)
+        x[rng.integers(0, n_in, 3)] *= 50.0
+        r = rng.normal(0, 0.5, n_in).astype(np.float32) if trial % 2 else None
+        nw = (1.0 + 0.1 * rng.normal(0, 1, n_in)).astype(np.float32)
+        d_x, d_w = _dev(H, x), _dev(H, nw)
+        d_r = _dev(H, r) if r is not None else None
+        d_xo, d_y = H.DeviceBuffer(n_in * 4), H.DeviceBuffer(n_out * 4)
+        H.check(H.lib.rmi_hip_rms_norm_gemv_q8_0_dev(kernel.w.handle, d_x.ptr, d_r.ptr if d_r else None, d_w.ptr, 1e-6, A,
+                                                     d_xo.ptr, d_y.ptr, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        xs = x + r if r is not None else x
+        assert np.array_equal(d_xo.to_array(np.float32, (n_in,)).view(np.uint32), xs.view(np.uint32))
+        assert np.array_equal(d_x.to_array(np.float32, (n_in,)).view(np.uint32), x.view(np.uint32))  # input untouched
+        q_ref, s_ref = oracle.quantize_q8_0(oracle.rms_norm(xs, nw, 1e-6), A)
+        y_ref = oracle.matmul_q8_0_quantized(w, q_ref, s_ref, n_in, n_out, A)
+        assert np.array_equal(d_y.to_array(np.float32, (n_out,)).view(np.uint32), y_ref.view(np.uint32)), trial
+        for b in (d_x, d_w, d_xo, d_y) + ((d_r,) if d_r else ()):
+            b.free()
+    # shapes the fused kernel does not cover are refused, not mis-computed
+    big = K.Q8Kernel(hip.synth.q8_0_weight(1, 8, 4096), 4096, 8)
+    d = H.DeviceBuffer(4096 * 4)
+    assert H.lib.rmi_hip_rms_norm_gemv_q8_0_dev(big.w.handle, d.ptr, None, d.ptr, 1e-6, A, d_y.ptr, d_y.ptr, None) != 0
+
+
 def test_silu_mul_quantize(hip, oracle):
     H = hip.hip
     rng = np.random.default_rng(3)
