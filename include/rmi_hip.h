@@ -263,6 +263,12 @@ int rmi_hip_rms_norm_quantize_q8_0_dev(float *x, const float *residual, const fl
 int rmi_hip_rms_norm_gemv_q8_0_dev(const rmi_hip_weight *w, const float *x_in, const float *residual,
                                    const float *norm_weight, float eps, int rounding, float *x_out, float *y,
                                    void *stream);
+/* The FFN's first half in one launch (src/models/qwen3.rs:1016-1027): norm as above, the gate and up products
+ * of the stacked weight [W_gate ; W_up] (rmi_hip_fuse_vstack), then h = up * silu(gate) quantized to Q8_0
+ * (h_q8[n_ff], h_scales[n_ff/32]).  n_in a multiple of 256 up to 2048, n_ff a multiple of 32. */
+int rmi_hip_rms_norm_ffn_gate_up_q8_0_dev(const rmi_hip_weight *w_gate_up, const float *x_in, const float *residual,
+                                          const float *norm_weight, float eps, int rounding, float *x_out,
+                                          int8_t *h_q8, float *h_scales, void *stream);
 /* gate_up = [W_gate x ; W_up x] (2*n_ff): (W_up x) * silu(W_gate x), src/ops/activation/mod.rs:137-151
  * as called at src/models/qwen3.rs:1016-1027, quantized to Q8_0. */
 int rmi_hip_silu_mul_quantize_q8_0_dev(const float *gate_up, uint32_t n_ff, int8_t *q8, float *scales, int rounding,

@@ -840,10 +840,16 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                                c.n_head_kv, c.head_dim_k, c.head_dim_v, s->act_q8, s->act_scales, rnd);
         rc = gemv(s->w_o[l], s->act_q8, s->act_scales, s->resid, st);
         if (rc != RMI_HIP_OK) return rc;
-        rc = norm_gemv(s->w_gu[l], s->resid, s->ffn_norm[l], s->gu);
+        if (rmi_gemv_q8_0_norm_silu_fusable(s->w_gu[l])) {  // norm, gate/up products and SiLU*up in one launch
+            rc = rmi_launch_gemv_q8_0_norm_silu(s->w_gu[l], x, s->resid, s->ffn_norm[l], x_other, c.eps, rnd, s->act_q8,
+                                                s->act_scales, st);
+            std::swap(x, x_other);
+        } else {
+            rc = norm_gemv(s->w_gu[l], s->resid, s->ffn_norm[l], s->gu);
+            hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((c.n_ff + 1023) / 1024), dim3(256), 0, st, s->gu, c.n_ff,
+                               s->act_q8, s->act_scales, rnd);
+        }
         if (rc != RMI_HIP_OK) return rc;
-        hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((c.n_ff + 1023) / 1024), dim3(256), 0, st, s->gu, c.n_ff,
-                           s->act_q8, s->act_scales, rnd);
         rc = gemv(s->w_down[l], s->act_q8, s->act_scales, s->resid, st);
         if (rc != RMI_HIP_OK) return rc;
         pending = s->resid;
@@ -893,6 +899,17 @@ int rmi_hip_rms_norm_gemv_q8_0_dev(const rmi_hip_weight *w, const float *x_in, c
     if (!x_in || !norm_weight || !x_out || !y || x_in == x_out) return rmi_fail(RMI_HIP_E_INVALID, "null or aliased pointer");
     return rmi_launch_gemv_q8_0_norm(w, x_in, residual, norm_weight, x_out, eps, rounding, y,
                                      static_cast<hipStream_t>(stream));
+}
+
+int rmi_hip_rms_norm_ffn_gate_up_q8_0_dev(const rmi_hip_weight *w_gate_up, const float *x_in, const float *residual,
+                                          const float *norm_weight, float eps, int rounding, float *x_out,
+                                          int8_t *h_q8, float *h_scales, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w_gate_up || w_gate_up->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (!x_in || !norm_weight || !x_out || !h_q8 || !h_scales || x_in == x_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "null or aliased pointer");
+    return rmi_launch_gemv_q8_0_norm_silu(w_gate_up, x_in, residual, norm_weight, x_out, eps, rounding, h_q8, h_scales,
+                                          static_cast<hipStream_t>(stream));
 }
 
 int rmi_hip_silu_mul_quantize_q8_0_dev(const float *gate_up, uint32_t n_ff, int8_t *q8, float *scales, int rounding,

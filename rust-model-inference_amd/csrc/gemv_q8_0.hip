@@ -6,6 +6,7 @@
 // taking fma(f32(wd)*xs[b], float(sum_{k=4L..4L+3} w*x), acc_L) block after
 // block, then hsum_ps (src/ops/dot.rs:447-456).  Eight GPU lanes hold the eight
 // accumulators of one row, so results match that kernel bit for bit.
+#include "device_math.h"
 #include "device_quant.h"
 #include "rmi_internal.h"
 
@@ -320,6 +321,98 @@ int launch_gemv_norm_deep(const RmiGemvProblem &p, const RmiNormArgs &na, hipStr
     return RMI_HIP_OK;
 }
 
+// The gate and up products of one FFN with both neighbours folded in: the norm in front (as above, here shared
+// by the workgroup) and `h = up * silu(gate)` quantized to Q8_0 behind (src/models/qwen3.rs:1016-1027,
+// src/ops/activation/mod.rs:137-151).  The weight is the gate matrix stacked on the up matrix (n_ff rows each).
+// A workgroup of eight waves takes 32 consecutive gate rows (waves 0-3, a tile each) and the same 32 up rows
+// (waves 4-7): one Q8_0 block of h, which leaves as 32 int8 and its scale.  n_in = NOCT * 256 <= 2048.
+template <int NOCT>
+__global__ __launch_bounds__(512) void gemv_q8_0_norm_silu_kernel(const uint8_t *__restrict__ w, uint32_t up_tile0,
+                                                                   RmiNormArgs na, int8_t *__restrict__ h_q8,
+                                                                   float *__restrict__ h_scales) {
+    extern __shared__ uint4 lds[];
+    __shared__ double red[8];
+    __shared__ float gu[64];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane >> 3, L = lane & 7;
+    const uint32_t tile_idx = (wave < 4 ? 0u : up_tile0) + blockIdx.x * 4 + (wave & 3);
+    constexpr uint32_t kVec = NOCT * 64;  // float4s of the activation
+    const bool owner = tid < kVec;        // whole waves: kVec is a multiple of 64
+    float4 v, a, wv;
+    if (owner) {
+        v = reinterpret_cast<const float4 *>(na.x_in)[tid];
+        if (na.resid) a = reinterpret_cast<const float4 *>(na.resid)[tid];
+        wv = reinterpret_cast<const float4 *>(na.weight)[tid];
+    }
+    gptr_u4 tile = as_global<gptr_u4>(w + size_t(tile_idx) * NOCT * kOctetBytes);
+    OctetRegs g[NOCT];
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+
+    if (owner) {
+        if (na.resid) {
+            v.x += a.x;
+            v.y += a.y;
+            v.z += a.z;
+            v.w += a.w;
+        }
+        if (blockIdx.x == 0) reinterpret_cast<float4 *>(na.x_out)[tid] = v;
+        const float s0 = v.x * v.x, s1 = v.y * v.y, s2 = v.z * v.z, s3 = v.w * v.w;
+        double part = double(s0);
+        part += double(s1);
+        part += double(s2);
+        part += double(s3);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        if (lane == 0) red[wave] = part;
+    }
+    __syncthreads();
+    uint32_t *dq = reinterpret_cast<uint32_t *>(lds);
+    if (owner) {
+        double total = red[0];
+#pragma unroll
+        for (uint32_t i = 1; i < kVec / 64; i++) total += red[i];
+        const float mean_sq = float(total / double(NOCT * 256));
+        const float scale = 1.0f / sqrtf(mean_sq + na.eps);
+        float4 o;
+        o.x = (v.x * scale) * wv.x;
+        o.y = (v.y * scale) * wv.y;
+        o.z = (v.z * scale) * wv.z;
+        o.w = (v.w * scale) * wv.w;
+        float sc;
+        const uint32_t q = rmi_quantize_block8(o, na.rounding, &sc);
+        const uint32_t b = tid >> 3;  // block of this float4; L = its dword inside the block
+        dq[(b >> 2) * 32 + L * 4 + (b & 3)] = q;
+        if (L == 0) reinterpret_cast<float *>(dq + NOCT * 64)[b] = sc;
+    }
+    __syncthreads();
+    float acc[1] = {0.0f};
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
+    const float y = hsum8_lanes(acc[0]);
+    if (L == 0) gu[wave * 8 + r] = y;  // [0,32): gate rows of this block, [32,64): up rows
+    __syncthreads();
+    if (tid < 8) {
+        const float4 gt = reinterpret_cast<const float4 *>(gu)[tid], up = reinterpret_cast<const float4 *>(gu + 32)[tid];
+        float4 h;
+        h.x = up.x * (gt.x / (1.0f + rmi_expf(-gt.x)));
+        h.y = up.y * (gt.y / (1.0f + rmi_expf(-gt.y)));
+        h.z = up.z * (gt.z / (1.0f + rmi_expf(-gt.z)));
+        h.w = up.w * (gt.w / (1.0f + rmi_expf(-gt.w)));
+        float sc;
+        reinterpret_cast<uint32_t *>(h_q8)[blockIdx.x * 8 + tid] = rmi_quantize_block8(h, na.rounding, &sc);
+        if (tid == 0) h_scales[blockIdx.x] = sc;
+    }
+}
+
+template <int NOCT>
+int launch_gemv_norm_silu(const rmi_hip_weight *w, const RmiNormArgs &na, int8_t *h_q8, float *h_scales, hipStream_t s) {
+    const uint32_t n_ff = w->n_out / 2;
+    hipLaunchKernelGGL((gemv_q8_0_norm_silu_kernel<NOCT>), dim3(n_ff / 32), dim3(512), size_t(NOCT) * 288, s, w->data,
+                       n_ff / 8, na, h_q8, h_scales);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
 template <int NOCT>
 int launch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
     hipLaunchKernelGGL((gemv_q8_0_deep_kernel<NOCT>), dim3(p.n_tiles), dim3(64), size_t(NOCT) * 288, s, p);
@@ -525,6 +618,29 @@ int rmi_launch_gemv_q8_0_norm(const rmi_hip_weight *w, const float *x_in, const 
         case 6: return launch_gemv_norm_deep<6>(p, na, s);
         case 7: return launch_gemv_norm_deep<7>(p, na, s);
         default: return launch_gemv_norm_deep<8>(p, na, s);
+    }
+}
+
+bool rmi_gemv_q8_0_norm_silu_fusable(const rmi_hip_weight *w) {
+    return w->n_in % 256 == 0 && w->n_units >= 1 && w->n_units <= 8 && w->n_out >= 64 && w->n_out % 64 == 0 &&
+           w->n_out / 64 <= 65535;
+}
+
+int rmi_launch_gemv_q8_0_norm_silu(const rmi_hip_weight *w_gate_up, const float *x_in, const float *resid,
+                                   const float *norm_weight, float *x_out, float eps, int rounding, int8_t *h_q8,
+                                   float *h_scales, hipStream_t s) {
+    if (!rmi_gemv_q8_0_norm_silu_fusable(w_gate_up))
+        return rmi_fail(RMI_HIP_E_INVALID, "shape %u x %u is not fusable", w_gate_up->n_out, w_gate_up->n_in);
+    const RmiNormArgs na{x_in, resid, norm_weight, x_out, eps, rounding};
+    switch (w_gate_up->n_units) {
+        case 1: return launch_gemv_norm_silu<1>(w_gate_up, na, h_q8, h_scales, s);
+        case 2: return launch_gemv_norm_silu<2>(w_gate_up, na, h_q8, h_scales, s);
+        case 3: return launch_gemv_norm_silu<3>(w_gate_up, na, h_q8, h_scales, s);
+        case 4: return launch_gemv_norm_silu<4>(w_gate_up, na, h_q8, h_scales, s);
+        case 5: return launch_gemv_norm_silu<5>(w_gate_up, na, h_q8, h_scales, s);
+        case 6: return launch_gemv_norm_silu<6>(w_gate_up, na, h_q8, h_scales, s);
+        case 7: return launch_gemv_norm_silu<7>(w_gate_up, na, h_q8, h_scales, s);
+        default: return launch_gemv_norm_silu<8>(w_gate_up, na, h_q8, h_scales, s);
     }
 }
 

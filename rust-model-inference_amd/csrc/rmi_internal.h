@@ -122,6 +122,12 @@ int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipS
 // y = W . Q8_0(rms_norm(x_in + resid) * norm_weight) in one launch, x_out = x_in + resid (x_out != x_in);
 // for one token and matrices the fused kernel covers (rmi_gemv_q8_0_norm_fusable)
 bool rmi_gemv_q8_0_norm_fusable(const rmi_hip_weight *w);
+// h = up * silu(gate) of [gate; up] = W . Q8_0(rms_norm(x_in + resid) * norm_weight), quantized to Q8_0, in one
+// launch; W holds the gate rows, then as many up rows (n_out = 2 * n_ff, n_ff a multiple of 32)
+bool rmi_gemv_q8_0_norm_silu_fusable(const rmi_hip_weight *w);
+int rmi_launch_gemv_q8_0_norm_silu(const rmi_hip_weight *w_gate_up, const float *x_in, const float *resid,
+                                   const float *norm_weight, float *x_out, float eps, int rounding, int8_t *h_q8,
+                                   float *h_scales, hipStream_t s);
 int rmi_launch_gemv_q8_0_norm(const rmi_hip_weight *w, const float *x_in, const float *resid, const float *norm_weight,
                               float *x_out, float eps, int rounding, float *y, hipStream_t s);
 // d_runs[w] = {problem index, first tile, tile count, 0}: the run of tiles wave w takes

@@ -76,6 +76,37 @@ def test_rms_norm_gemv_fused(hip, oracle, n_in, n_out):
     assert H.lib.rmi_hip_rms_norm_gemv_q8_0_dev(big.w.handle, d.ptr, None, d.ptr, 1e-6, A, d_y.ptr, d_y.ptr, None) != 0
 
 
+@pytest.mark.parametrize("n_in,n_ff", [(1024, 3072), (2048, 6144), (256, 32), (512, 96)])
+def test_rms_norm_ffn_gate_up_fused(hip, oracle, n_in, n_ff):
+    """norm + gate/up products + SiLU*up + quantizer in one launch (src/models/qwen3.rs:1016-1027): the same
+    bits as the restated steps one after the other."""
+    H, K = hip.hip, hip.kernel
+    rng = np.random.default_rng(n_in + n_ff)
+    wg = hip.synth.q8_0_weight(910 + n_ff, n_ff, n_in, scale_sigma=0.05)
+    wu = hip.synth.q8_0_weight(911 + n_ff, n_ff, n_in, scale_sigma=0.05)
+    fused = K.fuse_vstack(K.Q8Kernel(wg, n_in, n_ff), K.Q8Kernel(wu, n_in, n_ff))
+    for trial in range(10):
+        x = (rng.normal(0, 1, n_in) * rng.choice([0.1, 1.0, 30.0])).astype(np.float32)
+        r = rng.normal(0, 0.5, n_in).astype(np.float32) if trial % 2 else None
+        nw = (1.0 + 0.1 * rng.normal(0, 1, n_in)).astype(np.float32)
+        d_x, d_w = _dev(H, x), _dev(H, nw)
+        d_r = _dev(H, r) if r is not None else None
+        d_xo, d_q, d_s = H.DeviceBuffer(n_in * 4), H.DeviceBuffer(n_ff), H.DeviceBuffer(n_ff // 32 * 4)
+        H.check(H.lib.rmi_hip_rms_norm_ffn_gate_up_q8_0_dev(fused.w.handle, d_x.ptr, d_r.ptr if d_r else None, d_w.ptr,
+                                                            1e-6, A, d_xo.ptr, d_q.ptr, d_s.ptr, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        xs = x + r if r is not None else x
+        assert np.array_equal(d_xo.to_array(np.float32, (n_in,)).view(np.uint32), xs.view(np.uint32))
+        q_in, s_in = oracle.quantize_q8_0(oracle.rms_norm(xs, nw, 1e-6), A)
+        g = oracle.matmul_q8_0_quantized(wg, q_in, s_in, n_in, n_ff, A)
+        u = oracle.matmul_q8_0_quantized(wu, q_in, s_in, n_in, n_ff, A)
+        q_ref, s_ref = _quant(oracle, oracle.silu_mul(g, u))
+        assert np.array_equal(d_q.to_array(np.int8, (n_ff,)), q_ref), trial
+        assert np.array_equal(d_s.to_array(np.float32, (n_ff // 32,)).view(np.uint32), s_ref.view(np.uint32)), trial
+        for b in (d_x, d_w, d_xo, d_q, d_s) + ((d_r,) if d_r else ()):
+            b.free()
+
+
 def test_silu_mul_quantize(hip, oracle):
     H = hip.hip
     rng = np.random.default_rng(3)
