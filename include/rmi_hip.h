@@ -263,6 +263,14 @@ int rmi_hip_rms_norm_quantize_q8_0_dev(float *x, const float *residual, const fl
 int rmi_hip_rms_norm_gemv_q8_0_dev(const rmi_hip_weight *w, const float *x_in, const float *residual,
                                    const float *norm_weight, float eps, int rounding, float *x_out, float *y,
                                    void *stream);
+/* The attention block's first half in one launch (src/models/qwen3.rs:719-874), head dimension 128: norm as
+ * above, the q, k and v products of the stacked weight [W_q ; W_k ; W_v], then what
+ * rmi_hip_qk_norm_rope_f16_dev does to the three vectors.  n_in a multiple of 256 up to 1024. */
+int rmi_hip_rms_norm_qkv_rope_q8_0_dev(const rmi_hip_weight *w_qkv, const float *x_in, const float *residual,
+                                       const float *norm_weight, float eps, int rounding, float *x_out,
+                                       const float *q_norm, const float *k_norm, const float *cos_row,
+                                       const float *sin_row, uint16_t *q16, uint16_t *k_row, uint16_t *v_row,
+                                       uint32_t n_head, uint32_t n_head_kv, void *stream);
 /* The FFN's first half in one launch (src/models/qwen3.rs:1016-1027): norm as above, the gate and up products
  * of the stacked weight [W_gate ; W_up] (rmi_hip_fuse_vstack), then h = up * silu(gate) quantized to Q8_0
  * (h_q8[n_ff], h_scales[n_ff/32]).  n_in a multiple of 256 up to 2048, n_ff a multiple of 32. */

@@ -36,12 +36,7 @@ namespace {
 __device__ __forceinline__ float h2f(uint32_t bits16) {
     return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
 }
-// f32 -> f16 of a value that has already been rounded to f32.  The empty asm keeps the compiler from folding
-// a preceding fma into v_fma_mixlo_f16, which rounds the exact result once; the reference rounds twice.
-__device__ __forceinline__ uint16_t f2h(float v) {
-    asm volatile("" : "+v"(v));
-    return __builtin_bit_cast(uint16_t, _Float16(v));
-}
+__device__ __forceinline__ uint16_t f2h(float v) { return rmi_f2h(v); }
 
 // The step counter in HBM: the embedding kernel reads its token through it and the argmax kernel advances it,
 // so the next token never visits the host.  The kernels in between get the position as a launch argument:
@@ -823,13 +818,24 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
         return gemv(w, s->act_q8, s->act_scales, y, st);
     };
     for (uint32_t l = 0; l < c.n_layer; l++) {
-        int rc = norm_gemv(s->w_qkv[l], pending, s->attn_norm[l], s->qkv);
-        if (rc != RMI_HIP_OK) return rc;
+        int rc;
         const size_t layer_base = size_t(l) * c.capacity * s->kv_stride, row = layer_base + size_t(step) * s->kv_stride;
-        hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv), dim3(64), 0, st, s->qkv,
-                           c.has_qk_norm ? s->q_norm[l] : nullptr, c.has_qk_norm ? s->k_norm[l] : nullptr, s->cos_t,
-                           s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv,
-                           c.head_dim_k, c.head_dim_v, c.eps);
+        const float *qn = c.has_qk_norm ? s->q_norm[l] : nullptr, *kn = c.has_qk_norm ? s->k_norm[l] : nullptr;
+        if (rmi_gemv_q8_0_norm_rope_fusable(s->w_qkv[l], c.n_head, c.n_head_kv, c.head_dim_k, c.head_dim_v)) {
+            // norm, q/k/v products, head norms, rotation and the cache row in one launch
+            const size_t half = c.head_dim_k / 2;
+            rc = rmi_launch_gemv_q8_0_norm_rope(s->w_qkv[l], x, pending, s->attn_norm[l], x_other, c.eps, rnd, qn, kn,
+                                                s->cos_t + size_t(step) * half, s->sin_t + size_t(step) * half, s->q16,
+                                                s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv, st);
+            std::swap(x, x_other);
+            if (rc != RMI_HIP_OK) return rc;
+        } else {
+            rc = norm_gemv(s->w_qkv[l], pending, s->attn_norm[l], s->qkv);
+            if (rc != RMI_HIP_OK) return rc;
+            hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv), dim3(64), 0, st, s->qkv, qn, kn,
+                               s->cos_t, s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head,
+                               c.n_head_kv, c.head_dim_k, c.head_dim_v, c.eps);
+        }
         if (c.head_dim_k == 128 && c.head_dim_v == 128)
             hipLaunchKernelGGL(attention128_quant_kernel, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kAttnThreads), attn128_lds_bytes(step + 1),
                                st, s->q16, s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride,
@@ -899,6 +905,21 @@ int rmi_hip_rms_norm_gemv_q8_0_dev(const rmi_hip_weight *w, const float *x_in, c
     if (!x_in || !norm_weight || !x_out || !y || x_in == x_out) return rmi_fail(RMI_HIP_E_INVALID, "null or aliased pointer");
     return rmi_launch_gemv_q8_0_norm(w, x_in, residual, norm_weight, x_out, eps, rounding, y,
                                      static_cast<hipStream_t>(stream));
+}
+
+int rmi_hip_rms_norm_qkv_rope_q8_0_dev(const rmi_hip_weight *w_qkv, const float *x_in, const float *residual,
+                                       const float *norm_weight, float eps, int rounding, float *x_out,
+                                       const float *q_norm, const float *k_norm, const float *cos_row,
+                                       const float *sin_row, uint16_t *q16, uint16_t *k_row, uint16_t *v_row,
+                                       uint32_t n_head, uint32_t n_head_kv, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w_qkv || w_qkv->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (!x_in || !norm_weight || !x_out || !cos_row || !sin_row || !q16 || !k_row || !v_row || x_in == x_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "null or aliased pointer");
+    if (n_head == 0 || n_head_kv == 0) return rmi_fail(RMI_HIP_E_INVALID, "bad head shape");
+    return rmi_launch_gemv_q8_0_norm_rope(w_qkv, x_in, residual, norm_weight, x_out, eps, rounding, q_norm, k_norm,
+                                          cos_row, sin_row, q16, k_row, v_row, n_head, n_head_kv,
+                                          static_cast<hipStream_t>(stream));
 }
 
 int rmi_hip_rms_norm_ffn_gate_up_q8_0_dev(const rmi_hip_weight *w_gate_up, const float *x_in, const float *residual,

@@ -54,3 +54,10 @@ __device__ __forceinline__ float rmi_expf_tab(float x, const uint64_t *tab) {
 }
 
 __device__ __forceinline__ float rmi_expf(float x) { return rmi_expf_tab(x, kRmiExp2fTab); }
+
+// f32 -> f16 of a value that has already been rounded to f32.  The empty asm keeps the compiler from folding
+// a preceding fma into v_fma_mixlo_f16, which rounds the exact result once; the reference rounds twice.
+__device__ __forceinline__ uint16_t rmi_f2h(float v) {
+    asm volatile("" : "+v"(v));
+    return __builtin_bit_cast(uint16_t, _Float16(v));
+}

@@ -413,6 +413,130 @@ int launch_gemv_norm_silu(const rmi_hip_weight *w, const RmiNormArgs &na, int8_t
     return RMI_HIP_OK;
 }
 
+// The q, k and v products of one attention block with both neighbours folded in, for head dimension 128: the
+// norm in front (shared by the workgroup, as above) and, behind, what src/models/qwen3.rs:776-874 does to the
+// three vectors: per-head RMS norm of q and k (when the model has those weights), NeoX rotation, rounding to
+// f16, k and v into their cache row.  The weight is q stacked on k stacked on v.  A workgroup of 16 waves takes
+// one head (16 tiles); its first wave finishes the head.  n_in = NOCT * 256 <= 1024.
+struct RmiRopeArgs {
+    const float *q_norm, *k_norm;     // [128] each, or null
+    const float *cos_row, *sin_row;   // [64] each: the angles of this position
+    uint16_t *q16, *k_row, *v_row;    // f16 outputs: [n_head][128], [n_head_kv][128], [n_head_kv][128]
+    uint32_t n_head, n_head_kv;
+    float eps;
+};
+
+template <int NOCT>
+__global__ __launch_bounds__(1024) void gemv_q8_0_norm_rope_kernel(const uint8_t *__restrict__ w, RmiNormArgs na,
+                                                                    RmiRopeArgs ra) {
+    extern __shared__ uint4 lds[];
+    __shared__ double red[16];
+    __shared__ float yl[128];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane >> 3, L = lane & 7;
+    const uint32_t head = blockIdx.x;
+    constexpr uint32_t kVec = NOCT * 64;
+    const bool owner = tid < kVec;
+    float4 v, a, wv;
+    if (owner) {
+        v = reinterpret_cast<const float4 *>(na.x_in)[tid];
+        if (na.resid) a = reinterpret_cast<const float4 *>(na.resid)[tid];
+        wv = reinterpret_cast<const float4 *>(na.weight)[tid];
+    }
+    gptr_u4 tile = as_global<gptr_u4>(w + size_t(head * 16 + wave) * NOCT * kOctetBytes);
+    OctetRegs g[NOCT];
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+    // what the first wave needs at the end: out now, used after the products
+    const bool is_q = head < ra.n_head, is_v = head >= ra.n_head + ra.n_head_kv;
+    const float *nw = is_q ? ra.q_norm : ra.k_norm;
+    float cos_a = 0.0f, sin_a = 0.0f, w0 = 1.0f, w1 = 1.0f;
+    if (wave == 0 && !is_v) {
+        cos_a = ra.cos_row[lane];
+        sin_a = ra.sin_row[lane];
+        if (nw) {
+            w0 = nw[lane];
+            w1 = nw[lane + 64];
+        }
+    }
+
+    if (owner) {
+        if (na.resid) {
+            v.x += a.x;
+            v.y += a.y;
+            v.z += a.z;
+            v.w += a.w;
+        }
+        if (head == 0) reinterpret_cast<float4 *>(na.x_out)[tid] = v;
+        const float s0 = v.x * v.x, s1 = v.y * v.y, s2 = v.z * v.z, s3 = v.w * v.w;
+        double part = double(s0);
+        part += double(s1);
+        part += double(s2);
+        part += double(s3);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        if (lane == 0) red[wave] = part;
+    }
+    __syncthreads();
+    uint32_t *dq = reinterpret_cast<uint32_t *>(lds);
+    if (owner) {
+        double total = red[0];
+#pragma unroll
+        for (uint32_t i = 1; i < kVec / 64; i++) total += red[i];
+        const float mean_sq = float(total / double(NOCT * 256));
+        const float scale = 1.0f / sqrtf(mean_sq + na.eps);
+        float4 o;
+        o.x = (v.x * scale) * wv.x;
+        o.y = (v.y * scale) * wv.y;
+        o.z = (v.z * scale) * wv.z;
+        o.w = (v.w * scale) * wv.w;
+        float sc;
+        const uint32_t q = rmi_quantize_block8(o, na.rounding, &sc);
+        const uint32_t b = tid >> 3;
+        dq[(b >> 2) * 32 + L * 4 + (b & 3)] = q;
+        if (L == 0) reinterpret_cast<float *>(dq + NOCT * 64)[b] = sc;
+    }
+    __syncthreads();
+    float acc[1] = {0.0f};
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
+    const float y = hsum8_lanes(acc[0]);
+    if (L == 0) yl[wave * 8 + r] = y;
+    __syncthreads();
+    if (wave != 0) return;
+    const float x0r = yl[lane], x1r = yl[lane + 64];
+    if (is_v) {
+        uint16_t *dst = ra.v_row + size_t(head - ra.n_head - ra.n_head_kv) * 128;
+        dst[lane] = rmi_f2h(x0r);
+        dst[lane + 64] = rmi_f2h(x1r);
+        return;
+    }
+    float x0 = x0r, x1 = x1r;
+    if (nw) {
+        const float q0 = x0r * x0r, q1 = x1r * x1r;
+        double part = double(q0);
+        part += double(q1);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        const float mean_sq = float(part / 128.0);
+        const float sc = 1.0f / sqrtf(mean_sq + ra.eps);
+        x0 = (x0r * sc) * w0;
+        x1 = (x1r * sc) * w1;
+    }
+    uint16_t *dst = is_q ? ra.q16 + size_t(head) * 128 : ra.k_row + size_t(head - ra.n_head) * 128;
+    const float ta = x1 * -sin_a;
+    const float tb = x1 * cos_a;
+    dst[lane] = rmi_f2h(__builtin_fmaf(x0, cos_a, ta));
+    dst[lane + 64] = rmi_f2h(__builtin_fmaf(x0, sin_a, tb));
+}
+
+template <int NOCT>
+int launch_gemv_norm_rope(const rmi_hip_weight *w, const RmiNormArgs &na, const RmiRopeArgs &ra, hipStream_t s) {
+    hipLaunchKernelGGL((gemv_q8_0_norm_rope_kernel<NOCT>), dim3(ra.n_head + 2 * ra.n_head_kv), dim3(1024),
+                       size_t(NOCT) * 288, s, w->data, na, ra);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
 template <int NOCT>
 int launch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
     hipLaunchKernelGGL((gemv_q8_0_deep_kernel<NOCT>), dim3(p.n_tiles), dim3(64), size_t(NOCT) * 288, s, p);
@@ -641,6 +765,28 @@ int rmi_launch_gemv_q8_0_norm_silu(const rmi_hip_weight *w_gate_up, const float 
         case 6: return launch_gemv_norm_silu<6>(w_gate_up, na, h_q8, h_scales, s);
         case 7: return launch_gemv_norm_silu<7>(w_gate_up, na, h_q8, h_scales, s);
         default: return launch_gemv_norm_silu<8>(w_gate_up, na, h_q8, h_scales, s);
+    }
+}
+
+bool rmi_gemv_q8_0_norm_rope_fusable(const rmi_hip_weight *w, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim_k,
+                                     uint32_t head_dim_v) {
+    return head_dim_k == 128 && head_dim_v == 128 && w->n_in % 256 == 0 && w->n_units >= 1 && w->n_units <= 4 &&
+           w->n_out == (n_head + 2 * n_head_kv) * 128;
+}
+
+int rmi_launch_gemv_q8_0_norm_rope(const rmi_hip_weight *w_qkv, const float *x_in, const float *resid,
+                                   const float *norm_weight, float *x_out, float eps, int rounding, const float *q_norm,
+                                   const float *k_norm, const float *cos_row, const float *sin_row, uint16_t *q16,
+                                   uint16_t *k_row, uint16_t *v_row, uint32_t n_head, uint32_t n_head_kv, hipStream_t s) {
+    if (!rmi_gemv_q8_0_norm_rope_fusable(w_qkv, n_head, n_head_kv, 128, 128))
+        return rmi_fail(RMI_HIP_E_INVALID, "shape %u x %u is not fusable", w_qkv->n_out, w_qkv->n_in);
+    const RmiNormArgs na{x_in, resid, norm_weight, x_out, eps, rounding};
+    const RmiRopeArgs ra{q_norm, k_norm, cos_row, sin_row, q16, k_row, v_row, n_head, n_head_kv, eps};
+    switch (w_qkv->n_units) {
+        case 1: return launch_gemv_norm_rope<1>(w_qkv, na, ra, s);
+        case 2: return launch_gemv_norm_rope<2>(w_qkv, na, ra, s);
+        case 3: return launch_gemv_norm_rope<3>(w_qkv, na, ra, s);
+        default: return launch_gemv_norm_rope<4>(w_qkv, na, ra, s);
     }
 }
 

@@ -128,6 +128,14 @@ bool rmi_gemv_q8_0_norm_silu_fusable(const rmi_hip_weight *w);
 int rmi_launch_gemv_q8_0_norm_silu(const rmi_hip_weight *w_gate_up, const float *x_in, const float *resid,
                                    const float *norm_weight, float *x_out, float eps, int rounding, int8_t *h_q8,
                                    float *h_scales, hipStream_t s);
+// q|k|v = W . Q8_0(rms_norm(x_in + resid) * norm_weight) with the per-head q/k norm, the NeoX rotation and the
+// f16 rounding behind it, in one launch; head dimension 128, W = q rows, k rows, v rows
+bool rmi_gemv_q8_0_norm_rope_fusable(const rmi_hip_weight *w, uint32_t n_head, uint32_t n_head_kv, uint32_t head_dim_k,
+                                     uint32_t head_dim_v);
+int rmi_launch_gemv_q8_0_norm_rope(const rmi_hip_weight *w_qkv, const float *x_in, const float *resid,
+                                   const float *norm_weight, float *x_out, float eps, int rounding, const float *q_norm,
+                                   const float *k_norm, const float *cos_row, const float *sin_row, uint16_t *q16,
+                                   uint16_t *k_row, uint16_t *v_row, uint32_t n_head, uint32_t n_head_kv, hipStream_t s);
 int rmi_launch_gemv_q8_0_norm(const rmi_hip_weight *w, const float *x_in, const float *resid, const float *norm_weight,
                               float *x_out, float eps, int rounding, float *y, hipStream_t s);
 // d_runs[w] = {problem index, first tile, tile count, 0}: the run of tiles wave w takes

@@ -99,6 +99,8 @@ SIGNATURES = {
     "rmi_hip_expf_dev": (C.c_int, [_vp, _vp, _sz, _vp]),
     "rmi_hip_rms_norm_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, C.c_float, _vp, _vp, C.c_int, _vp]),
     "rmi_hip_rms_norm_gemv_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, C.c_int, _vp, _vp, _vp]),
+    "rmi_hip_rms_norm_qkv_rope_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, C.c_int, _vp, _vp, _vp, _vp, _vp, _vp,
+                                                     _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_rms_norm_ffn_gate_up_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, C.c_int, _vp, _vp, _vp, _vp]),
     "rmi_hip_silu_mul_quantize_q8_0_dev": (C.c_int, [_vp, _u32, _vp, _vp, C.c_int, _vp]),
     "rmi_hip_qk_norm_rope_f16_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32,

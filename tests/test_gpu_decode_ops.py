@@ -159,6 +159,58 @@ def test_qk_norm_rope_f16(hip, oracle, hk):
             b.free()
 
 
+@pytest.mark.parametrize("n_in,n_head,n_kv", [(1024, 16, 8), (512, 4, 4), (256, 3, 1)])
+def test_rms_norm_qkv_rope_fused(hip, oracle, n_in, n_head, n_kv):
+    """norm + q/k/v products + head norms + rotation + f16 rounding in one launch (src/models/qwen3.rs:719-874):
+    the same bits as the restated steps one after the other."""
+    H, K = hip.hip, hip.kernel
+    rng = np.random.default_rng(n_in + n_head)
+    hk = 128
+    n_q, n_k = n_head * hk, n_kv * hk
+    wq = hip.synth.q8_0_weight(920, n_q, n_in, scale_sigma=0.05)
+    wk = hip.synth.q8_0_weight(921, n_k, n_in, scale_sigma=0.05)
+    wv = hip.synth.q8_0_weight(922, n_k, n_in, scale_sigma=0.05)
+    fused = K.fuse_vstack(K.fuse_vstack(K.Q8Kernel(wq, n_in, n_q), K.Q8Kernel(wk, n_in, n_k)), K.Q8Kernel(wv, n_in, n_k))
+    for trial in range(10):
+        pos = int(rng.integers(0, 4000))
+        x = (rng.normal(0, 1, n_in) * rng.choice([0.1, 1.0, 30.0])).astype(np.float32)
+        r = rng.normal(0, 0.5, n_in).astype(np.float32) if trial % 2 else None
+        nw = (1.0 + 0.1 * rng.normal(0, 1, n_in)).astype(np.float32)
+        qn = (1.0 + 0.2 * rng.normal(0, 1, hk)).astype(np.float32)
+        kn = (1.0 + 0.2 * rng.normal(0, 1, hk)).astype(np.float32)
+        with_norm = trial % 3 != 0
+        c, s = oracle.rope_angles(pos, hk, 1e6)
+        d = [_dev(H, a) for a in (x, nw, qn, kn, c, s)]
+        d_r = _dev(H, r) if r is not None else None
+        d_xo, d_q16, d_k, d_v = H.DeviceBuffer(n_in * 4), H.DeviceBuffer(n_q * 2), H.DeviceBuffer(n_k * 2), H.DeviceBuffer(n_k * 2)
+        H.check(H.lib.rmi_hip_rms_norm_qkv_rope_q8_0_dev(fused.w.handle, d[0].ptr, d_r.ptr if d_r else None, d[1].ptr, 1e-6,
+                                                         A, d_xo.ptr, d[2].ptr if with_norm else None,
+                                                         d[3].ptr if with_norm else None, d[4].ptr, d[5].ptr, d_q16.ptr,
+                                                         d_k.ptr, d_v.ptr, n_head, n_kv, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        xs = x + r if r is not None else x
+        assert np.array_equal(d_xo.to_array(np.float32, (n_in,)).view(np.uint32), xs.view(np.uint32))
+        q_in, s_in = oracle.quantize_q8_0(oracle.rms_norm(xs, nw, 1e-6), A)
+        qv = oracle.matmul_q8_0_quantized(wq, q_in, s_in, n_in, n_q, A)
+        kv = oracle.matmul_q8_0_quantized(wk, q_in, s_in, n_in, n_k, A)
+        vv = oracle.matmul_q8_0_quantized(wv, q_in, s_in, n_in, n_k, A)
+
+        def ref_heads(vec, n, w):
+            out = []
+            for h in range(n):
+                hx = vec[h * hk:(h + 1) * hk]
+                if with_norm:
+                    hx = oracle.rms_norm(hx, w, 1e-6)
+                out.append(oracle.rope_neox(hx, pos, 1e6))
+            return np.concatenate(out).astype(np.float16).view(np.uint16)
+
+        assert np.array_equal(d_q16.to_array(np.uint16, (n_q,)), ref_heads(qv, n_head, qn)), trial
+        assert np.array_equal(d_k.to_array(np.uint16, (n_k,)), ref_heads(kv, n_kv, kn)), trial
+        assert np.array_equal(d_v.to_array(np.uint16, (n_k,)), vv.astype(np.float16).view(np.uint16)), trial
+        for b in d + [d_xo, d_q16, d_k, d_v] + ([d_r] if d_r else []):
+            b.free()
+
+
 @pytest.mark.parametrize("hk,n_head,n_kv", [(128, 16, 8), (64, 8, 4)])
 def test_attention_f16_quantize(hip, oracle, hk, n_head, n_kv):
     H = hip.hip
