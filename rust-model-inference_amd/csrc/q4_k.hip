@@ -7,6 +7,7 @@
 // then acc_T = fma(d*q8d, float(sumi_T), acc_T)) and four min accumulators
 // (acc_m[t] = fma(-dmin*q8d, float(mn[2t]*s[2t] + mn[2t+1]*s[2t+1]), acc_m[t]));
 // result hsum(acc) + ((m0+m2)+(m1+m3)).  Eight GPU lanes per row hold them.
+#include "device_stage_q8k.h"
 #include "rmi_internal.h"
 
 namespace {
@@ -175,24 +176,10 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_kernel(RmiQ4kProblem single, c
     }
     const uint32_t n_sb = p.n_sb, n_in = n_sb * 256;
     uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
-    for (int t = 0; t < B; t++) {
-        uint32_t *dst = lds_dw + size_t(t) * n_sb * kSbDwords;
-        gptr_u32 xq = as_global<gptr_u32>(p.q8qs + size_t(t) * n_in);
-        for (uint32_t i = threadIdx.x; i < n_sb * 64; i += blockDim.x) {
-            // source dword i of the row: super-block sb, element offset 4*(i%64) = 64g + 32*hi + 4T'
-            const uint32_t sb = i >> 6, e = i & 63;
-            const uint32_t g = e >> 4, hi = (e >> 3) & 1, tq = e & 7;
-            dst[sb * kSbDwords + tq * 8 + g * 2 + hi] = xq[i];
-        }
-        gptr_i16 bs = as_global<gptr_i16>(p.q8bs + size_t(t) * (n_in / 16));
-        for (uint32_t i = threadIdx.x; i < n_sb * 8; i += blockDim.x) {
-            const uint32_t sb = i >> 3, j = i & 7;
-            const int16_t s = int16_t(bs[sb * 16 + 2 * j] + bs[sb * 16 + 2 * j + 1]);
-            dst[sb * kSbDwords + 64 + j] = uint32_t(int32_t(s));
-        }
-        gptr_f32 dptr = as_global<gptr_f32>(p.q8d + size_t(t) * n_sb);
-        for (uint32_t i = threadIdx.x; i < n_sb; i += blockDim.x) dst[i * kSbDwords + 72] = __float_as_uint(dptr[i]);
-    }
+    for (int t = 0; t < B; t++)
+        rmi_stage_q8k_token<true, 2>(lds_dw + size_t(t) * n_sb * kSbDwords, p.q8qs + size_t(t) * n_in,
+                                     p.q8bs + size_t(t) * (n_in / 16), p.q8d + size_t(t) * n_sb, n_sb, threadIdx.x,
+                                     blockDim.x);
     __syncthreads();
 
     for (; k < k_end; k++) {

@@ -8,6 +8,7 @@
 //   - 32 * (bsums[2m]*scale[2m] + bsums[2m+1]*scale[2m+1]),
 // then acc_m = fma(d*q8d, float(that), acc_m); result hsum(acc).  Eight GPU lanes
 // per row hold the eight accumulators.
+#include "device_stage_q8k.h"
 #include "rmi_internal.h"
 
 namespace {
@@ -133,19 +134,10 @@ __global__ __launch_bounds__(MAXT) void gemv_q6_k_kernel(RmiQ4kProblem single, c
     }
     const uint32_t n_sb = p.n_sb, n_in = n_sb * 256;
     uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
-    for (int t = 0; t < B; t++) {
-        uint32_t *dst = lds_dw + size_t(t) * n_sb * kSbDwords;
-        gptr_u32 xq = as_global<gptr_u32>(p.q8qs + size_t(t) * n_in);
-        for (uint32_t i = threadIdx.x; i < n_sb * 64; i += blockDim.x) {
-            // source dword i of the row: super-block sb, elements 4*(i%64).. = 32g + 4m'
-            const uint32_t sb = i >> 6, e = i & 63;
-            dst[sb * kSbDwords + (e & 7) * 8 + (e >> 3)] = xq[i];
-        }
-        gptr_u32 bs = as_global<gptr_u32>(reinterpret_cast<const uint32_t *>(p.q8bs) + size_t(t) * (n_in / 32));
-        for (uint32_t i = threadIdx.x; i < n_sb * 8; i += blockDim.x) dst[(i >> 3) * kSbDwords + 64 + (i & 7)] = bs[i];
-        gptr_f32 dptr = as_global<gptr_f32>(p.q8d + size_t(t) * n_sb);
-        for (uint32_t i = threadIdx.x; i < n_sb; i += blockDim.x) dst[i * kSbDwords + 72] = __float_as_uint(dptr[i]);
-    }
+    for (int t = 0; t < B; t++)
+        rmi_stage_q8k_token<false, 2>(lds_dw + size_t(t) * n_sb * kSbDwords, p.q8qs + size_t(t) * n_in,
+                                      p.q8bs + size_t(t) * (n_in / 16), p.q8d + size_t(t) * n_sb, n_sb, threadIdx.x,
+                                      blockDim.x);
     __syncthreads();
 
     for (; k < k_end; k++) {
