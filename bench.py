@@ -601,15 +601,15 @@ def run_decode(args, pkg, ev):
                          round(token_steps / wall, 1), wall, "int8 dot4 -> f32 (F16 KV cache)", {
         "workload": "device-resident greedy decode of a synthetic Q8_0 GGUF (Qwen3-0.6B architecture, 28 layers, "
                     "vocab 151936), 639 token-steps per generation; one bench step = one generation",
-        "token_steps_per_generation": token_steps, "launches_per_token_step": 1 + 9 * 28 + 4,
+        "token_steps_per_generation": token_steps, "launches_per_token_step": 1 + 5 * 28 + 4,
         "device": dev_name.strip(), "compute_units": cus})
     result["ms_per_token_step"] = round(per_token * 1e3, 4)
     achieved = alg / per_token / 1e9
-    result["roofline"] = {"bound": "hbm", "kernel": "gemv_q8_0_kernel<1,false,*> (113 GEMV launches per token-step)",
+    result["roofline"] = {"bound": "hbm", "kernel": "Q8_0 GEMV kernels (4 per layer + lm_head = 113 launches per token-step)",
                           "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(achieved / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_token_step": alg,
                           "traffic": None,
-                          "note": "a token-step is 257 dependent launches of 3-6 us each; weights are read once per "
+                          "note": "a token-step is 145 dependent launches of 4-13 us each; weights are read once per "
                                   "step, so the step is launch-latency-bound, not HBM-bound"}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))

@@ -424,8 +424,11 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
 // what differs is the schedule.  The launch has 16 workgroups on a 256-CU chip, so its time is the length of one
 // thread's instruction stream plus memory round trips, not throughput: the query stays in registers as packed
 // f16 (product f16 x f16 is exact in f32, then an f64 add: the same value as the f64 fma above), every load of
-// the first round of keys and of the first 12 values per thread goes out before anything waits, values are read
-// 16 bytes (8 dimensions) at a time by 64 key slices, and the four slices of a wave combine in registers.
+// the first round of keys and of the first values of each thread goes out before anything waits, values are read
+// 16 bytes (8 dimensions) at a time by 32 key slices, and the four slices of a wave combine in registers.  Eight
+// waves, two per SIMD: with sixteen the kernel took a third longer (the waves of a SIMD run one after another
+// through such dependent code, so more of them only repeat the per-thread set-up), with four it lost on long contexts.
+constexpr uint32_t kA128Threads = 512;
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 __device__ __forceinline__ half8 as_half8(const uint4 &v) { return __builtin_bit_cast(half8, v); }
 __device__ __forceinline__ double quad_sum(double v) {  // (l0 + l1) + (l2 + l3) in every lane of the quad
@@ -437,22 +440,22 @@ __device__ __forceinline__ double quad_sum(double v) {  // (l0 + l1) + (l2 + l3)
 }
 __host__ __device__ inline size_t attn128_lds_bytes(uint32_t n_keys) {
     const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
-    return n_pad * 12 + 16 * 128 * 8;
+    return n_pad * 12 + (kA128Threads / 64) * 128 * 8;
 }
-__global__ __launch_bounds__(kAttnThreads) void attention128_quant_kernel(
+__global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
     uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, int8_t *__restrict__ q8,
     float *__restrict__ scales, int rounding) {
     extern __shared__ double lds_d[];
-    __shared__ float red_f[kAttnThreads / 64];
+    __shared__ float red_f[kA128Threads / 64];
     __shared__ uint64_t exp_tab[32];
     // grid = (query heads per key/value head, key/value heads)
     const uint32_t kvh = blockIdx.y, head = blockIdx.y * gridDim.x + blockIdx.x, tid = threadIdx.x;
     const uint32_t n_keys = step + 1;
     const uint32_t n_pad = (n_keys + kAttnPad - 1) / kAttnPad * kAttnPad;
     double *wd = lds_d;                                        // [n_pad] softmax weights (f16 values), 0 beyond n_keys
-    double *part = wd + n_pad;                                 // [16 waves][128]
-    float *scores = reinterpret_cast<float *>(part + 16 * 128);  // [n_pad]
+    double *part = wd + n_pad;                                 // [waves][128]
+    float *scores = reinterpret_cast<float *>(part + (kA128Threads / 64) * 128);  // [n_pad]
     const uint32_t row_u4 = kv_stride >> 3;                    // uint4 per cache row
     const uint64_t tab_entry = kRmiExp2fTab[tid & 31];         // first load out; stored to LDS after the scores
 
@@ -471,9 +474,9 @@ __global__ __launch_bounds__(kAttnThreads) void attention128_quant_kernel(
         for (int c = 0; c < 4; c++) kk[c] = key[4 * c];
     }
     // values: lane = (8 dimensions dg, key slice sl): 16 consecutive lanes read the 256 bytes of one row
-    constexpr uint32_t kPre = 12;
+    constexpr uint32_t kPre = kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40);
     const uint32_t dg = tid & 15, sl = tid >> 4;
-    const uint32_t chunk = (n_keys + 63) >> 6;
+    const uint32_t chunk = (n_keys + kA128Threads / 16 - 1) / (kA128Threads / 16);
     const uint32_t t_begin = sl * chunk, t_end = t_begin + chunk < n_keys ? t_begin + chunk : n_keys;
     const uint4 *vbase = reinterpret_cast<const uint4 *>(v_cache + size_t(kvh) * 128 + dg * 8);
     uint4 vp[kPre];
@@ -486,10 +489,10 @@ __global__ __launch_bounds__(kAttnThreads) void attention128_quant_kernel(
     }
     const float kq_scale = 1.0f / sqrtf(128.0f);  // two f32 roundings, as the reference computes it
     float my_max = -INFINITY;
-    for (uint32_t t0 = 0; t0 < n_keys; t0 += kAttnThreads / 4) {
-        const uint32_t t = t0 + key0, tn = t + kAttnThreads / 4;
+    for (uint32_t t0 = 0; t0 < n_keys; t0 += kA128Threads / 4) {
+        const uint32_t t = t0 + key0, tn = t + kA128Threads / 4;
         uint4 kn[4];
-        if (t0 + kAttnThreads / 4 < n_keys) {  // the next round's keys are in flight while this one is summed
+        if (t0 + kA128Threads / 4 < n_keys) {  // the next round's keys are in flight while this one is summed
             const uint4 *key = kbase + __umul24(tn < n_keys ? tn : n_keys - 1, row_u4);
 #pragma unroll
             for (int c = 0; c < 4; c++) kn[c] = key[4 * c];
@@ -520,8 +523,8 @@ __global__ __launch_bounds__(kAttnThreads) void attention128_quant_kernel(
     __syncthreads();
     float max_val = red_f[0];
 #pragma unroll
-    for (uint32_t i = 1; i < kAttnThreads / 64; i++) max_val = fmaxf(max_val, red_f[i]);
-    for (uint32_t t = tid; t < n_pad; t += kAttnThreads) scores[t] = t < n_keys ? rmi_expf_tab(scores[t] - max_val, exp_tab) : 0.0f;
+    for (uint32_t i = 1; i < kA128Threads / 64; i++) max_val = fmaxf(max_val, red_f[i]);
+    for (uint32_t t = tid; t < n_pad; t += kA128Threads) scores[t] = t < n_keys ? rmi_expf_tab(scores[t] - max_val, exp_tab) : 0.0f;
     __syncthreads();
     if (tid == 0) {  // the reference adds the weights one after the other in f32; the padding zeros change nothing
         // one lane, one dependent chain of adds; the LDS reads run 32 values ahead of it (two buffers, no copies)
@@ -555,7 +558,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention128_quant_kernel(
     }
     __syncthreads();
     const float total = red_f[0];
-    for (uint32_t t = tid; t < n_pad; t += kAttnThreads) {
+    for (uint32_t t = tid; t < n_pad; t += kA128Threads) {
         const float e = scores[t];
         wd[t] = t < n_keys ? double(h2f(f2h(total > 0.0f ? e / total : e))) : 0.0;
     }
@@ -614,7 +617,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention128_quant_kernel(
         double o[4];
 #pragma unroll
         for (int d = 0; d < 4; d++) o[d] = part[tid * 4 + d];
-        for (uint32_t w = 1; w < kAttnThreads / 64; w++) {
+        for (uint32_t w = 1; w < kA128Threads / 64; w++) {
 #pragma unroll
             for (int d = 0; d < 4; d++) o[d] += part[w * 128 + tid * 4 + d];
         }
@@ -837,7 +840,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                                c.n_head_kv, c.head_dim_k, c.head_dim_v, c.eps);
         }
         if (c.head_dim_k == 128 && c.head_dim_v == 128)
-            hipLaunchKernelGGL(attention128_quant_kernel, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kAttnThreads), attn128_lds_bytes(step + 1),
+            hipLaunchKernelGGL(attention128_quant_kernel, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kA128Threads), attn128_lds_bytes(step + 1),
                                st, s->q16, s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride,
                                c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd);
         else
@@ -971,7 +974,7 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     const size_t lds = d128 ? attn128_lds_bytes(n_keys) : attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
     if (lds > 64 * 1024) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
     if (d128)
-        hipLaunchKernelGGL(attention128_quant_kernel, dim3(n_head / n_head_kv, n_head_kv), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream),
+        hipLaunchKernelGGL(attention128_quant_kernel, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
                            q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding);
     else
         hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream),
