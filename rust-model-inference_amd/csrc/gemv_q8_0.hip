@@ -416,8 +416,8 @@ int launch_gemv_norm_silu(const rmi_hip_weight *w, const RmiNormArgs &na, int8_t
 // The q, k and v products of one attention block with both neighbours folded in, for head dimension 128: the
 // norm in front (shared by the workgroup, as above) and, behind, what src/models/qwen3.rs:776-874 does to the
 // three vectors: per-head RMS norm of q and k (when the model has those weights), NeoX rotation, rounding to
-// f16, k and v into their cache row.  The weight is q stacked on k stacked on v.  A workgroup of 16 waves takes
-// one head (16 tiles); its first wave finishes the head.  n_in = NOCT * 256 <= 1024.
+// f16, k and v into their cache row.  The weight is q stacked on k stacked on v.  A workgroup of 8 waves takes
+// one head (16 tiles, two per wave); its first wave finishes the head.  n_in = NOCT * 256 <= 1024.
 struct RmiRopeArgs {
     const float *q_norm, *k_norm;     // [128] each, or null
     const float *cos_row, *sin_row;   // [64] each: the angles of this position
@@ -427,10 +427,10 @@ struct RmiRopeArgs {
 };
 
 template <int NOCT>
-__global__ __launch_bounds__(1024) void gemv_q8_0_norm_rope_kernel(const uint8_t *__restrict__ w, RmiNormArgs na,
+__global__ __launch_bounds__(512) void gemv_q8_0_norm_rope_kernel(const uint8_t *__restrict__ w, RmiNormArgs na,
                                                                     RmiRopeArgs ra) {
     extern __shared__ uint4 lds[];
-    __shared__ double red[16];
+    __shared__ double red[8];
     __shared__ float yl[128];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane >> 3, L = lane & 7;
     const uint32_t head = blockIdx.x;
@@ -442,10 +442,14 @@ __global__ __launch_bounds__(1024) void gemv_q8_0_norm_rope_kernel(const uint8_t
         if (na.resid) a = reinterpret_cast<const float4 *>(na.resid)[tid];
         wv = reinterpret_cast<const float4 *>(na.weight)[tid];
     }
-    gptr_u4 tile = as_global<gptr_u4>(w + size_t(head * 16 + wave) * NOCT * kOctetBytes);
-    OctetRegs g[NOCT];
+    // two tiles per wave: eight waves finish sooner than sixteen with a tile each
+    gptr_u4 tile = as_global<gptr_u4>(w + size_t(head * 16 + wave * 2) * NOCT * kOctetBytes);
+    gptr_u4 tile2 = tile + NOCT * (kOctetBytes / 16);
+    OctetRegs g[NOCT], g2[NOCT];
 #pragma unroll
     for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) load_octet(g2[o], tile2 + r, tile2 + NOCT * 8 + lane, o);
     // what the first wave needs at the end: out now, used after the products
     const bool is_q = head < ra.n_head, is_v = head >= ra.n_head + ra.n_head_kv;
     const float *nw = is_q ? ra.q_norm : ra.k_norm;
@@ -496,11 +500,16 @@ __global__ __launch_bounds__(1024) void gemv_q8_0_norm_rope_kernel(const uint8_t
         if (L == 0) reinterpret_cast<float *>(dq + NOCT * 64)[b] = sc;
     }
     __syncthreads();
-    float acc[1] = {0.0f};
+    float acc[1] = {0.0f}, acc2[1] = {0.0f};
 #pragma unroll
     for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
-    const float y = hsum8_lanes(acc[0]);
-    if (L == 0) yl[wave * 8 + r] = y;
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc2, g2[o], lds, NOCT * 18, NOCT, o, L);
+    const float y = hsum8_lanes(acc[0]), y2 = hsum8_lanes(acc2[0]);
+    if (L == 0) {
+        yl[wave * 16 + r] = y;
+        yl[wave * 16 + 8 + r] = y2;
+    }
     __syncthreads();
     if (wave != 0) return;
     const float x0r = yl[lane], x1r = yl[lane + 64];
@@ -531,7 +540,7 @@ __global__ __launch_bounds__(1024) void gemv_q8_0_norm_rope_kernel(const uint8_t
 
 template <int NOCT>
 int launch_gemv_norm_rope(const rmi_hip_weight *w, const RmiNormArgs &na, const RmiRopeArgs &ra, hipStream_t s) {
-    hipLaunchKernelGGL((gemv_q8_0_norm_rope_kernel<NOCT>), dim3(ra.n_head + 2 * ra.n_head_kv), dim3(1024),
+    hipLaunchKernelGGL((gemv_q8_0_norm_rope_kernel<NOCT>), dim3(ra.n_head + 2 * ra.n_head_kv), dim3(512),
                        size_t(NOCT) * 288, s, w->data, na, ra);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
