@@ -6,6 +6,7 @@
 //   Kernel            src/ops/kernel/trait_.rs:15-110
 //   Q8Kernel          src/ops/kernel/q8_0/mod.rs:21-56
 //   Q4_KKernel        src/ops/kernel/q4_k.rs:7-93
+//   Q6_KKernel        src/ops/kernel/q6_k.rs:7-80
 //   BlockQ8K          src/ops/quant/mod.rs:35-40
 //   fuse_vstack       src/ops/kernel/qtensor_owned.rs:138-164
 //   Layer, ExecContext, QuantizedLinear   src/core/traits.rs:45-74, src/core/model.rs:12-104
@@ -160,6 +161,41 @@ class Q4_KKernel : public Kernel {
             for (int k = 0; k < 16; k++) bs[i * 16 + k] = (*q8_k)[i].bsums[k];
         }
         check(rmi_hip_q4_k_forward_prepared(w_->get(), d.data(), qs.data(), bs.data(), output, uint32_t(n_in),
+                                            uint32_t(n_out), uint32_t(ith), uint32_t(nth)));
+    }
+    const std::shared_ptr<DeviceWeight> &weight() const { return w_; }
+
+  private:
+    std::shared_ptr<DeviceWeight> w_;
+};
+
+class Q6_KKernel : public Kernel {
+  public:
+    Q6_KKernel(const uint8_t *data, size_t nbytes, size_t n_in, size_t n_out)
+        : w_(std::make_shared<DeviceWeight>(rmi_hip_upload_q6_k(data, nbytes, uint32_t(n_in), uint32_t(n_out)))) {}
+    explicit Q6_KKernel(std::shared_ptr<DeviceWeight> w) : w_(std::move(w)) {}
+
+    void forward_prequantized(const uint8_t *input_q8, const float *input_scales, float *output, size_t n_in,
+                              size_t n_out, size_t ith, size_t nth) const override {
+        check(rmi_hip_q6_k_forward_prequantized(w_->get(), input_q8, input_scales, output, uint32_t(n_in),
+                                                uint32_t(n_out), uint32_t(ith), uint32_t(nth)));
+    }
+    void forward_prepared(const float *input_f32, const uint8_t *, const float *, const std::vector<BlockQ8K> *q8_k,
+                          float *output, size_t n_in, size_t n_out, size_t ith, size_t nth) const override {
+        std::vector<BlockQ8K> owned;
+        if (!q8_k) {  // q6_k.rs:63-69
+            owned = quantize_row_q8_k(input_f32, n_in);
+            q8_k = &owned;
+        }
+        std::vector<float> d(q8_k->size());
+        std::vector<int8_t> qs(q8_k->size() * 256);
+        std::vector<int16_t> bs(q8_k->size() * 16);
+        for (size_t i = 0; i < q8_k->size(); i++) {
+            d[i] = (*q8_k)[i].d;
+            for (int k = 0; k < 256; k++) qs[i * 256 + k] = (*q8_k)[i].qs[k];
+            for (int k = 0; k < 16; k++) bs[i * 16 + k] = (*q8_k)[i].bsums[k];
+        }
+        check(rmi_hip_q6_k_forward_prepared(w_->get(), d.data(), qs.data(), bs.data(), output, uint32_t(n_in),
                                             uint32_t(n_out), uint32_t(ith), uint32_t(nth)));
     }
     const std::shared_ptr<DeviceWeight> &weight() const { return w_; }

@@ -10,7 +10,7 @@
 //! Hook points in the crate:
 //!   * `QuantizedTensor::into_kernel` (src/ops/kernel/quantized_tensor.rs:167-190):
 //!     when `ops::hip_enabled()` return `Box::new(HipKernel::upload(..))` for
-//!     `Q8_0` / `Q4_K` instead of `Q8Kernel` / `Q4_KKernel`;
+//!     `Q8_0` / `Q4_K` / `Q6_K` instead of `Q8Kernel` / `Q4_KKernel` / `Q6_KKernel`;
 //!   * `ops::enable_gpu` / the lazy context of src/ops/float.rs:44-58: call
 //!     `hip::init(0)`; on `Err` print and stay on the CPU kernels, as today;
 //!   * `matmul_q8_0_quantized_range` (src/ops/kernel/q8_0/dispatch.rs:36-52) is NOT
@@ -33,6 +33,7 @@ extern "C" {
     fn rmi_hip_last_error() -> *const c_char;
     fn rmi_hip_upload_q8_0(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
     fn rmi_hip_upload_q4_k(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
+    fn rmi_hip_upload_q6_k(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
     fn rmi_hip_fuse_vstack(a: *const RmiHipWeight, b: *const RmiHipWeight) -> *mut RmiHipWeight;
     fn rmi_hip_free_weight(w: *mut RmiHipWeight);
     fn rmi_hip_q8_0_forward_prequantized(
@@ -54,6 +55,17 @@ extern "C" {
         w: *const RmiHipWeight, input_q8: *const u8, input_scales: *const f32, output: *mut f32,
         n_in: u32, n_out: u32, ith: u32, nth: u32,
     ) -> c_int;
+    fn rmi_hip_q6_k_forward_prepared(
+        w: *const RmiHipWeight, d: *const f32, qs: *const i8, bsums: *const i16, output: *mut f32,
+        n_in: u32, n_out: u32, ith: u32, nth: u32,
+    ) -> c_int;
+    fn rmi_hip_q6_k_forward_batched(
+        w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
+    ) -> c_int;
+    fn rmi_hip_q6_k_forward_prequantized(
+        w: *const RmiHipWeight, input_q8: *const u8, input_scales: *const f32, output: *mut f32,
+        n_in: u32, n_out: u32, ith: u32, nth: u32,
+    ) -> c_int;
     fn rmi_hip_quantized_linear_forward(
         w: *const RmiHipWeight, input: *const f32, output: *mut f32, in_features: u32, out_features: u32,
     ) -> c_int;
@@ -71,7 +83,7 @@ pub fn init(device: i32) -> Result<(), String> {
 }
 
 #[derive(Clone, Copy, PartialEq)]
-enum Dtype { Q8_0, Q4K }
+enum Dtype { Q8_0, Q4K, Q6K }
 
 /// A weight resident in HBM.  `Kernel: Send + Sync`: the library gives every
 /// calling thread its own stream and staging, so `&self` calls may overlap.
@@ -90,6 +102,10 @@ impl HipKernel {
     pub fn upload_q4_k(weight: &[u8], n_in: usize, n_out: usize) -> Result<Self, String> {
         let h = unsafe { rmi_hip_upload_q4_k(weight.as_ptr(), weight.len(), n_in as u32, n_out as u32) };
         if h.is_null() { Err(last_error()) } else { Ok(Self { handle: h, dtype: Dtype::Q4K }) }
+    }
+    pub fn upload_q6_k(weight: &[u8], n_in: usize, n_out: usize) -> Result<Self, String> {
+        let h = unsafe { rmi_hip_upload_q6_k(weight.as_ptr(), weight.len(), n_in as u32, n_out as u32) };
+        if h.is_null() { Err(last_error()) } else { Ok(Self { handle: h, dtype: Dtype::Q6K }) }
     }
     /// `QTensorOwned::fuse_vstack` (src/ops/kernel/qtensor_owned.rs:138-164)
     pub fn fuse_vstack(a: &Self, b: &Self) -> Option<Self> {
@@ -119,6 +135,9 @@ impl Kernel for HipKernel {
                 Dtype::Q4K => rmi_hip_q4_k_forward_prequantized(
                     self.handle, input_q8.as_ptr(), input_scales.as_ptr(), output.as_mut_ptr(),
                     n_in as u32, n_out as u32, ith as u32, nth as u32),
+                Dtype::Q6K => rmi_hip_q6_k_forward_prequantized(
+                    self.handle, input_q8.as_ptr(), input_scales.as_ptr(), output.as_mut_ptr(),
+                    n_in as u32, n_out as u32, ith as u32, nth as u32),
             }
         };
         expect_ok(rc);
@@ -135,14 +154,15 @@ impl Kernel for HipKernel {
         let owned;
         let blocks: &[BlockQ8K] = match q8_k {
             Some(b) => b,
-            None => { owned = crate::ops::quant::quantize_row_q8_k(&input_f32[..n_in]); &owned } // q4_k.rs:77-84
+            None => { owned = crate::ops::quant::quantize_row_q8_k(&input_f32[..n_in]); &owned } // q4_k.rs:77-84, q6_k.rs:63-69
         };
         let d: Vec<f32> = blocks.iter().map(|b| b.d).collect();
         let qs: Vec<i8> = blocks.iter().flat_map(|b| b.qs.iter().copied()).collect();
         let bs: Vec<i16> = blocks.iter().flat_map(|b| b.bsums.iter().copied()).collect();
+        let prepared = if self.dtype == Dtype::Q6K { rmi_hip_q6_k_forward_prepared } else { rmi_hip_q4_k_forward_prepared };
         expect_ok(unsafe {
-            rmi_hip_q4_k_forward_prepared(self.handle, d.as_ptr(), qs.as_ptr(), bs.as_ptr(), output.as_mut_ptr(),
-                                          n_in as u32, n_out as u32, ith as u32, nth as u32)
+            prepared(self.handle, d.as_ptr(), qs.as_ptr(), bs.as_ptr(), output.as_mut_ptr(),
+                     n_in as u32, n_out as u32, ith as u32, nth as u32)
         });
     }
 
@@ -157,6 +177,8 @@ impl Kernel for HipKernel {
                 Dtype::Q8_0 => rmi_hip_q8_0_forward_batched(self.handle, input.as_ptr(), output.as_mut_ptr(),
                                                             n_in as u32, n_out as u32, n_tokens, ROUND_TIES_EVEN),
                 Dtype::Q4K => rmi_hip_q4_k_forward_batched(self.handle, input.as_ptr(), output.as_mut_ptr(),
+                                                           n_in as u32, n_out as u32, n_tokens),
+                Dtype::Q6K => rmi_hip_q6_k_forward_batched(self.handle, input.as_ptr(), output.as_mut_ptr(),
                                                            n_in as u32, n_out as u32, n_tokens),
             }
         });

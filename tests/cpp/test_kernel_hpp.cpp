@@ -1,7 +1,7 @@
 // Exercises include/rmi_hip_kernel.hpp (the C++ mirror of the reference's Kernel /
 // Layer interface) on a GPU.  The cases are the reference's own unit tests:
 // src/ops/kernel/q8_0/mod.rs:74-156 (closed forms, thread partition),
-// tests/quantized_inference.rs:233-249 (Q4_K uniform block), plus eight
+// tests/quantized_inference.rs:233-263 (Q4_K and Q6_K uniform blocks), plus eight
 // std::threads calling one kernel at once, as pool.compute does.
 #include <cmath>
 #include <cstdio>
@@ -115,6 +115,21 @@ int main() {
         layer.forward(x.data(), &out, ctx);
         EXPECT(out == 256.0f && layer.input_dim() == 256 && layer.output_dim() == 1);
         // integer path with the kernel quantizing the f32 input itself
+        k.forward_prepared(x.data(), nullptr, nullptr, nullptr, &out, 256, 1, 0, 1);
+        EXPECT(std::fabs(out - 256.0f) < 1e-3f);
+    }
+    {  // tests/quantized_inference.rs:252-263: Q6_K uniform block, ql 0x11, qh 0xaa, scales 1, d 1.0
+        std::vector<uint8_t> w(210, 0x11);
+        std::memset(&w[128], 0xaa, 64);
+        std::memset(&w[192], 1, 16);
+        w[208] = uint8_t(one & 0xff);
+        w[209] = uint8_t(one >> 8);
+        rmi::Q6_KKernel k(w.data(), w.size(), 256, 1);
+        std::vector<uint8_t> xq(256, 1);
+        std::vector<float> xs(8, 1.0f), x(256, 1.0f);
+        float out = 0;
+        k.forward_prequantized(xq.data(), xs.data(), &out, 256, 1, 0, 1);
+        EXPECT(out == 256.0f);
         k.forward_prepared(x.data(), nullptr, nullptr, nullptr, &out, 256, 1, 0, 1);
         EXPECT(std::fabs(out - 256.0f) < 1e-3f);
     }
