@@ -37,6 +37,7 @@ extern "C" {
 #define RMI_HIP_E_NOT_INIT (-3)  /* rmi_hip_init has not succeeded           */
 #define RMI_HIP_E_NO_DEVICE (-4) /* no gfx950 device visible                 */
 
+#define RMI_HIP_DTYPE_Q4_0 2
 #define RMI_HIP_DTYPE_Q8_0 8
 #define RMI_HIP_DTYPE_Q4_K 12
 #define RMI_HIP_DTYPE_Q6_K 14
@@ -62,6 +63,8 @@ int rmi_hip_device_info(char *name, size_t name_len, int *compute_units, size_t 
  * once; the host slice may be dropped afterwards.  NULL on failure. */
 rmi_hip_weight *rmi_hip_upload_q8_0(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
 rmi_hip_weight *rmi_hip_upload_q4_k(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
+/* Q4_0Kernel::new (src/ops/kernel/q4_0/mod.rs:26-28): rows of 18-byte blocks. */
+rmi_hip_weight *rmi_hip_upload_q4_0(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
 /* Q6_KKernel::new (src/ops/kernel/q6_k.rs:15-18): rows of 210-byte super-blocks. */
 rmi_hip_weight *rmi_hip_upload_q6_k(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out);
 /* QTensorOwned::fuse_vstack (src/ops/kernel/qtensor_owned.rs:138-164) and
@@ -132,6 +135,21 @@ int rmi_hip_quantized_linear_forward(const rmi_hip_weight *w, const float *input
 int rmi_hip_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *q8k_qs, const int16_t *q8k_bsums, int32_t *isum,
                             int32_t *msum);
 
+/* ---- Q4_0, host slices ---------------------------------------------------*/
+
+/* Q4_0Kernel::forward_prequantized (src/ops/kernel/q4_0/mod.rs:33-84): rows
+ * [ith*ceil(n_out/nth), ...) of the full output; the scalar kernel's arithmetic
+ * (q4_0/scalar.rs:13-52), which the AVX2 one (q4_0/avx2.rs:24-105) equals bit for bit. */
+int rmi_hip_q4_0_forward_prequantized(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth);
+/* Kernel::forward / forward_batched on a Q4_0 kernel (src/ops/kernel/trait_.rs:59-109): quantize_q8_0_into on
+ * the device, then the product; n_tokens rows, token-major out. */
+int rmi_hip_q4_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens, int rounding);
+/* Exact per-block integers (parity entry point): dots[n_out][n_in/32] = sum of (nibble - 8) * q8
+ * (q4_0/scalar.rs:40-47). */
+int rmi_hip_block_dots_q4_0(const rmi_hip_weight *w, const uint8_t *input_q8, int32_t *dots);
+
 /* ---- Q6_K, host slices ---------------------------------------------------*/
 
 /* Q6_KKernel::forward_prepared (src/ops/kernel/q6_k.rs:44-80): vec_dot_q6k_q8k
@@ -185,6 +203,9 @@ int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
  * integers, the f32 sums within rounding of the CPU kernels. */
 int rmi_hip_gemm_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
                               const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride, void *stream);
+/* Q4_0 weights, Q8_0 activations on the device (src/ops/kernel/q4_0/scalar.rs:13-52); x_q8 16-byte aligned. */
+int rmi_hip_gemv_q4_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, void *stream);
 /* y[t*y_stride + r] = vec_dot_q6k_q8k(row r, Q8_K token t) for rows [row_start,row_end), 1..n tokens
  * (Q6_KKernel::forward_prepared, src/ops/kernel/q6_k.rs:44-80). */
 int rmi_hip_gemv_q6_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,

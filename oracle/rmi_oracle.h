@@ -133,6 +133,18 @@ void rmi_ref_quantized_linear_forward(const uint8_t *weight,
                                       size_t in_features,
                                       size_t out_features);
 
+/* ---- rmi_q4_0.c: Q4_0 x Q8_0 ----
+ * Pinned by the closed forms of the reference's own tests (src/ops/kernel/q4_0/avx2.rs:243-330: all-zero,
+ * all-max and all-min inputs against nibbles 0 and 15), integer dots by brute force, f64 dequantised dots, and
+ * the intrinsics twin, which the reference requires to equal the scalar kernel bit for bit. */
+/* src/ops/kernel/q4_0/scalar.rs:13-52 */
+void rmi_ref_matmul_q4_0_scalar_range(const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, size_t n_in, size_t n_out, size_t ith, size_t nth);
+void rmi_ref_block_dots_q4_0(const uint8_t *weight, const uint8_t *input_q8, int32_t *dots, size_t n_in, size_t n_out);
+/* src/ops/kernel/q4_0/avx2.rs:24-105, output pre-sliced (index 0 = row_start) */
+void rmi_ref_x86_matmul_q4_0_range(const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
+                                   float *output, size_t n_in, size_t row_start, size_t row_end);
+
 /* ---- rmi_q6_k.c: Q6_K x Q8_K ----
  * Pinned by: the uniform-block value 256.0 (tests/quantized_inference.rs:252-263),
  * the element layout cross-checked between dequantize_row_q6_k and the aux8

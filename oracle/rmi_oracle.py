@@ -56,6 +56,9 @@ def _load():
         "rmi_ref_q4k_forward_prepared": (None, [_u8p, _f32p, _i8p, _i16p, _f32p, _sz, _sz, _sz, _sz, C.c_int]),
         "rmi_ref_q4k_forward_prequantized": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz, _sz]),
         "rmi_ref_quantized_linear_forward": (None, [_u8p, _f32p, _f32p, _sz, _sz]),
+        "rmi_ref_matmul_q4_0_scalar_range": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz, _sz]),
+        "rmi_ref_block_dots_q4_0": (None, [_u8p, _u8p, _i32p, _sz, _sz]),
+        "rmi_ref_x86_matmul_q4_0_range": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz]),
         "rmi_ref_dequantize_row_q6_k": (None, [_u8p, _f32p, _sz]),
         "rmi_ref_vec_dot_q6k_q8k": (C.c_float, [_u8p, _sz, _f32p, _i8p, _i16p, C.c_int]),
         "rmi_ref_q6k_q8k_block_ints": (None, [_u8p, _sz, _i8p, _i32p]),
@@ -299,6 +302,28 @@ def quantized_linear_forward(w, x, in_features, out_features):
     w, x = _u8(w), _f32(x)
     out = np.zeros(out_features, np.float32)
     lib.rmi_ref_quantized_linear_forward(_p(w, _u8p), _p(x, _f32p), _p(out, _f32p), in_features, out_features)
+    return out
+
+
+# ---- Q4_0 ----
+
+def matmul_q4_0_scalar_range(w, q8, sc, out, n_in, n_out, ith=0, nth=1):
+    w, q8, sc = _u8(w), _u8(q8), _f32(sc)
+    lib.rmi_ref_matmul_q4_0_scalar_range(_p(w, _u8p), _p(q8, _u8p), _p(sc, _f32p), _p(out, _f32p), n_in, n_out, ith, nth)
+    return out
+
+
+def block_dots_q4_0(w, q8, n_in, n_out):
+    w, q8 = _u8(w), _u8(q8)
+    dots = np.zeros((n_out, n_in // 32), np.int32)
+    lib.rmi_ref_block_dots_q4_0(_p(w, _u8p), _p(q8, _u8p), _p(dots, _i32p), n_in, n_out)
+    return dots
+
+
+def x86_matmul_q4_0_range(w, q8, sc, n_in, row_start, row_end):
+    w, q8, sc = _u8(w), _u8(q8), _f32(sc)
+    out = np.zeros(max(row_end - row_start, 0), np.float32)
+    lib.rmi_ref_x86_matmul_q4_0_range(_p(w, _u8p), _p(q8, _u8p), _p(sc, _f32p), _p(out, _f32p), n_in, row_start, row_end)
     return out
 
 

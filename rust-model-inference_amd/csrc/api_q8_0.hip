@@ -36,7 +36,7 @@ RmiGemvProblem make_problem(const rmi_hip_weight *w, const int8_t *x_q8, const f
 
 // tokens per GEMV launch so that the LDS staging fits
 uint32_t gemv_chunk(const rmi_hip_weight *w) {
-    const size_t per_token = size_t(w->n_units) * 288;
+    const size_t per_token = size_t(w->n_units) * (w->dtype == RMI_HIP_DTYPE_Q4_0 ? 320 : 288);
     uint32_t c = per_token ? uint32_t((64 * 1024) / per_token) : 8;
     return c > 8 ? 8 : c;
 }
@@ -51,7 +51,7 @@ int gemv_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scal
         const uint32_t nt = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
         RmiGemvProblem p = make_problem(w, x_q8 + size_t(t0) * w->n_in, x_scales + size_t(t0) * nb,
                                         y + size_t(t0) * y_stride, y_stride, row_start, row_end);
-        int rc = rmi_launch_gemv_q8_0_single(p, nt, s);
+        int rc = w->dtype == RMI_HIP_DTYPE_Q4_0 ? rmi_launch_gemv_q4_0(p, nt, s) : rmi_launch_gemv_q8_0_single(p, nt, s);
         if (rc != RMI_HIP_OK) return rc;
     }
     return RMI_HIP_OK;
@@ -371,6 +371,81 @@ int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream) {
                                           g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
     return rmi_launch_gemv_q8_0_group(static_cast<const RmiGemvProblem *>(g->d_list), g->d_runs, g->n_runs,
                                       g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
+}
+
+// ---- Q4_0 weights (Q8_0 activations): the same staging and row partition as the Q8_0 calls
+
+int rmi_hip_q4_0_forward_prequantized(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
+                                      float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_0 weight handle");
+    if (w->n_in != n_in || w->n_out != n_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "weight is %u x %u, call says %u x %u", w->n_out, w->n_in, n_out, n_in);
+    if (nth == 0) nth = 1;
+    if (n_out == 0) return RMI_HIP_OK;
+    const uint32_t per_thread = (n_out + nth - 1) / nth;  // q4_0/mod.rs:46-51
+    const uint64_t s64 = uint64_t(ith) * per_thread;
+    if (s64 >= n_out) return RMI_HIP_OK;
+    const uint32_t start = uint32_t(s64), end = start + per_thread < n_out ? start + per_thread : n_out;
+    if (!output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    return host_gemv_range(w, input_q8, input_scales, output + start, 1, end - start, start, end);
+}
+
+int rmi_hip_q4_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens, int rounding) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_0 weight handle");
+    if (w->n_in != n_in || w->n_out != n_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "weight is %u x %u, call says %u x %u", w->n_out, w->n_in, n_out, n_in);
+    if (n_tokens == 0 || n_out == 0) return RMI_HIP_OK;
+    if (!input || !output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const size_t n_x = size_t(n_tokens) * n_in;
+    float *pin = static_cast<float *>(rmi_pin_buf(c, 2, n_x * 4));
+    float *d_x = static_cast<float *>(rmi_dev_buf(c, 2, n_x * 4));
+    int8_t *d_q8 = static_cast<int8_t *>(rmi_dev_buf(c, 0, n_x));
+    float *d_sc = static_cast<float *>(rmi_dev_buf(c, 3, n_x / 32 * 4));
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(n_tokens) * n_out * 4));
+    if (!pin || !d_x || !d_q8 || !d_sc || !d_y) return RMI_HIP_E_RUNTIME;
+    memcpy(pin, input, n_x * 4);
+    RMI_HIP_CHECK(hipMemcpyAsync(d_x, pin, n_x * 4, hipMemcpyHostToDevice, c->stream));
+    int rc = rmi_launch_quantize_q8_0(d_x, d_q8, d_sc, n_tokens, n_in, rounding, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    rc = gemv_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, output, d_y, size_t(n_tokens) * n_out * 4, 1);
+}
+
+int rmi_hip_block_dots_q4_0(const rmi_hip_weight *w, const uint8_t *input_q8, int32_t *dots) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_0 weight handle");
+    const size_t n = size_t(w->n_out) * (w->n_in / 32);
+    if (n == 0) return RMI_HIP_OK;
+    if (!input_q8 || !dots) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    uint8_t *pin = static_cast<uint8_t *>(rmi_pin_buf(c, 0, w->n_in));
+    int8_t *d_q8 = static_cast<int8_t *>(rmi_dev_buf(c, 0, w->n_in));
+    int32_t *d_out = static_cast<int32_t *>(rmi_dev_buf(c, 1, n * 4));
+    if (!pin || !d_q8 || !d_out) return RMI_HIP_E_RUNTIME;
+    memcpy(pin, input_q8, w->n_in);
+    RMI_HIP_CHECK(hipMemcpyAsync(d_q8, pin, w->n_in, hipMemcpyHostToDevice, c->stream));
+    int rc = rmi_launch_block_dots_q4_0(w, d_q8, d_out, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, dots, d_out, n * 4, 1);
+}
+
+int rmi_hip_gemv_q4_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_0 weight handle");
+    if (row_start >= row_end || n_tokens == 0) return RMI_HIP_OK;
+    if (row_end > w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) exceed n_out=%u", row_start, row_end, w->n_out);
+    if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
+    if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (reinterpret_cast<uintptr_t>(x_q8) % 16) return rmi_fail(RMI_HIP_E_INVALID, "x_q8 must be 16-byte aligned");
+    return gemv_tokens(w, x_q8, x_scales, y, n_tokens, y_stride, row_start, row_end, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -41,6 +41,14 @@ constexpr uint32_t kOctetBytes = 128 + 2048;  // per tile per octet
 // coalesced 1 KiB load.  144 bytes per super-block, as in the source format.
 constexpr uint32_t kQ4KSuperBytes = 8 * 16 + 1024;  // per tile per super-block
 
+// Q4_0 weights in HBM.  Tiles of 8 rows, blocks in octets of 8; per tile and octet:
+//
+//   [ scales : 8 rows x 8 f16 ]            128 B
+//   [ quants : 8 rows x 8 L x 16 B ]      1024 B   lane L of row r = the 16 nibble bytes of block 8o + L
+//
+// 18 bytes per block, as in the source format; rows beyond n_out and blocks beyond n_in/32 are zero.
+constexpr uint32_t kQ40OctetBytes = 128 + 1024;  // per tile per octet
+
 // Q6_K weights in HBM.  Tiles of 8 rows; per tile and super-block:
 //
 //   [ scales : 8 rows x 16 int8 ]           128 B
@@ -58,7 +66,7 @@ struct rmi_hip_weight {
     uint32_t n_in;
     uint32_t n_out;
     uint32_t n_tiles;   // ceil(n_out / 8)
-    uint32_t n_units;   // Q8_0: octets per row; Q4_K, Q6_K: super-blocks per row
+    uint32_t n_units;   // Q8_0, Q4_0: octets per row; Q4_K, Q6_K: super-blocks per row
     size_t tile_bytes;  // bytes of one tile
     size_t nbytes;      // device allocation
     uint8_t *data;      // device pointer
@@ -102,6 +110,7 @@ int rmi_device_cus();
 int rmi_launch_repack_q8_0(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
 int rmi_launch_repack_q4_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
 int rmi_launch_repack_q6_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
+int rmi_launch_repack_q4_0(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
 int rmi_launch_copy_rows(const rmi_hip_weight *src, rmi_hip_weight *dst, uint32_t dst_row0, hipStream_t s);
 
 struct RmiGemvProblem {
@@ -119,6 +128,9 @@ struct RmiGemvProblem {
     uint32_t reserved;
 };
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
+// the same problem record with w = a Q4_0 tile stream (Q8_0 activation)
+int rmi_launch_gemv_q4_0(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
+int rmi_launch_block_dots_q4_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s);
 // y = W . Q8_0(rms_norm(x_in + resid) * norm_weight) in one launch, x_out = x_in + resid (x_out != x_in);
 // for one token and matrices the fused kernel covers (rmi_gemv_q8_0_norm_fusable)
 bool rmi_gemv_q8_0_norm_fusable(const rmi_hip_weight *w);

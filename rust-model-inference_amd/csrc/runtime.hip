@@ -195,9 +195,9 @@ static rmi_hip_weight *alloc_weight(int dtype, uint32_t n_in, uint32_t n_out) {
     w->n_in = n_in;
     w->n_out = n_out;
     w->n_tiles = (n_out + kTileRows - 1) / kTileRows;
-    if (dtype == RMI_HIP_DTYPE_Q8_0) {
+    if (dtype == RMI_HIP_DTYPE_Q8_0 || dtype == RMI_HIP_DTYPE_Q4_0) {
         w->n_units = (n_in / 32 + 7) / 8;
-        w->tile_bytes = size_t(w->n_units) * kOctetBytes;
+        w->tile_bytes = size_t(w->n_units) * (dtype == RMI_HIP_DTYPE_Q8_0 ? kOctetBytes : kQ40OctetBytes);
     } else {
         w->n_units = n_in / 256;
         w->tile_bytes = size_t(w->n_units) * (dtype == RMI_HIP_DTYPE_Q6_K ? kQ6KSuperBytes : kQ4KSuperBytes);
@@ -218,8 +218,11 @@ static rmi_hip_weight *upload(int dtype, const uint8_t *blocks, size_t nbytes, u
         rmi_set_error("rmi_hip_init has not succeeded");
         return nullptr;
     }
-    const uint32_t block_elems = dtype == RMI_HIP_DTYPE_Q8_0 ? 32 : 256;
-    const size_t block_bytes = dtype == RMI_HIP_DTYPE_Q8_0 ? 34 : (dtype == RMI_HIP_DTYPE_Q6_K ? 210 : 144);
+    const uint32_t block_elems = dtype == RMI_HIP_DTYPE_Q8_0 || dtype == RMI_HIP_DTYPE_Q4_0 ? 32 : 256;
+    const size_t block_bytes = dtype == RMI_HIP_DTYPE_Q8_0   ? 34
+                               : dtype == RMI_HIP_DTYPE_Q4_0 ? 18
+                               : dtype == RMI_HIP_DTYPE_Q6_K ? 210
+                                                             : 144;
     if (n_in == 0 || n_in % block_elems != 0) {
         rmi_set_error("n_in=%u is not a positive multiple of %u", n_in, block_elems);
         return nullptr;
@@ -240,6 +243,7 @@ static rmi_hip_weight *upload(int dtype, const uint8_t *blocks, size_t nbytes, u
     int rc = RMI_HIP_OK;
     if (e == hipSuccess)
         rc = dtype == RMI_HIP_DTYPE_Q8_0   ? rmi_launch_repack_q8_0(staging, w, c->stream)
+             : dtype == RMI_HIP_DTYPE_Q4_0 ? rmi_launch_repack_q4_0(staging, w, c->stream)
              : dtype == RMI_HIP_DTYPE_Q6_K ? rmi_launch_repack_q6_k(staging, w, c->stream)
                                            : rmi_launch_repack_q4_k(staging, w, c->stream);
     if (e == hipSuccess && rc == RMI_HIP_OK) e = hipStreamSynchronize(c->stream);
@@ -258,6 +262,10 @@ rmi_hip_weight *rmi_hip_upload_q8_0(const uint8_t *blocks, size_t nbytes, uint32
 
 rmi_hip_weight *rmi_hip_upload_q4_k(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {
     return upload(RMI_HIP_DTYPE_Q4_K, blocks, nbytes, n_in, n_out);
+}
+
+rmi_hip_weight *rmi_hip_upload_q4_0(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {
+    return upload(RMI_HIP_DTYPE_Q4_0, blocks, nbytes, n_in, n_out);
 }
 
 rmi_hip_weight *rmi_hip_upload_q6_k(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {

@@ -11,6 +11,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "librmi_hip.so")
 
+DTYPE_Q4_0 = 2
 DTYPE_Q8_0 = 8
 DTYPE_Q4_K = 12
 DTYPE_Q6_K = 14
@@ -54,6 +55,7 @@ SIGNATURES = {
     "rmi_hip_device_info": (C.c_int, [C.c_char_p, _sz, C.POINTER(C.c_int), C.POINTER(_sz)]),
     "rmi_hip_upload_q8_0": (_vp, [_u8p, _sz, _u32, _u32]),
     "rmi_hip_upload_q4_k": (_vp, [_u8p, _sz, _u32, _u32]),
+    "rmi_hip_upload_q4_0": (_vp, [_u8p, _sz, _u32, _u32]),
     "rmi_hip_upload_q6_k": (_vp, [_u8p, _sz, _u32, _u32]),
     "rmi_hip_fuse_vstack": (_vp, [_vp, _vp]),
     "rmi_hip_free_weight": (None, [_vp]),
@@ -74,6 +76,9 @@ SIGNATURES = {
     "rmi_hip_q4_k_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_quantized_linear_forward": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32]),
     "rmi_hip_block_ints_q4_k": (C.c_int, [_vp, _i8p, _i16p, _i32p, _i32p]),
+    "rmi_hip_q4_0_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
+    "rmi_hip_q4_0_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32, C.c_int]),
+    "rmi_hip_block_dots_q4_0": (C.c_int, [_vp, _u8p, _i32p]),
     "rmi_hip_q6_k_forward_prepared": (C.c_int, [_vp, _f32p, _i8p, _i16p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_q6_k_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32]),
     "rmi_hip_q6_k_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
@@ -89,6 +94,7 @@ SIGNATURES = {
     "rmi_hip_gemm_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_gemm_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp]),
+    "rmi_hip_gemv_q4_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_gemv_q6_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_quantize_row_q8_k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_group_create": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u32]),

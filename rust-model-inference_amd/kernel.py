@@ -4,6 +4,7 @@ the Rust traits so that tests read like the reference's own:
 
   Kernel                 src/ops/kernel/trait_.rs:15-110
   Q8Kernel               src/ops/kernel/q8_0/mod.rs:21-56
+  Q4_0Kernel             src/ops/kernel/q4_0/mod.rs:18-123
   Q4_KKernel             src/ops/kernel/q4_k.rs:7-93
   Q6_KKernel             src/ops/kernel/q6_k.rs:7-80
   QuantizedTensor        src/ops/kernel/quantized_tensor.rs:32-190  (from_bytes / into_kernel)
@@ -24,6 +25,7 @@ from . import hip
 from .hip import C, _f32p, _i8p, _i16p, _i32p, _u8p, as_f32, as_u8, check, lib, ptr
 
 GGML_TYPE_Q8_0 = "Q8_0"
+GGML_TYPE_Q4_0 = "Q4_0"
 GGML_TYPE_Q4_K = "Q4_K"
 GGML_TYPE_Q6_K = "Q6_K"
 
@@ -186,6 +188,35 @@ class Q8Kernel(Kernel):
         return dots
 
 
+class Q4_0Kernel(Kernel):
+    def __init__(self, data, n_in, n_out, _handle=None):
+        if _handle is None:
+            w = as_u8(data)
+            _handle = lib.rmi_hip_upload_q4_0(ptr(w, _u8p), w.size, n_in, n_out)
+        self.w = _DeviceWeight(_handle)
+
+    def forward_prequantized(self, input_q8, input_scales, output, n_in, n_out, ith, nth):
+        q8, sc = as_u8(input_q8), as_f32(input_scales)
+        check(lib.rmi_hip_q4_0_forward_prequantized(self.w.handle, ptr(q8, _u8p), ptr(sc, _f32p),
+                                                    ptr(_out(output, n_out), _f32p), n_in, n_out, ith, nth))
+
+    def forward(self, input, output, n_in, n_out, rounding=hip.ROUND_TIES_EVEN):
+        self.forward_batched(as_f32(input)[:n_in], output, n_in, n_out, rounding)
+
+    def forward_batched(self, input, output, n_in, n_out, rounding=hip.ROUND_TIES_EVEN):
+        x = as_f32(input).reshape(-1)
+        n_tokens = x.size // n_in
+        check(lib.rmi_hip_q4_0_forward_batched(self.w.handle, ptr(x, _f32p),
+                                               ptr(_out(output, n_tokens * n_out), _f32p), n_in, n_out, n_tokens,
+                                               rounding))
+
+    def block_dots(self, input_q8):
+        q8 = as_u8(input_q8)
+        dots = np.zeros((self.w.n_out, self.w.n_in // 32), np.int32)
+        check(lib.rmi_hip_block_dots_q4_0(self.w.handle, ptr(q8, _u8p), ptr(dots, _i32p)))
+        return dots
+
+
 class Q4_KKernel(Kernel):
     def __init__(self, data, n_in, n_out, _handle=None):
         if _handle is None:
@@ -262,7 +293,7 @@ class QuantizedTensor:
 
     @classmethod
     def from_bytes(cls, ggml_type, data, n_in, n_out):
-        if ggml_type not in (GGML_TYPE_Q8_0, GGML_TYPE_Q4_K, GGML_TYPE_Q6_K):
+        if ggml_type not in (GGML_TYPE_Q8_0, GGML_TYPE_Q4_0, GGML_TYPE_Q4_K, GGML_TYPE_Q6_K):
             return None  # other dtypes stay on the reference's CPU kernels
         return cls(ggml_type, data, n_in, n_out)
 
@@ -277,6 +308,8 @@ class QuantizedTensor:
             return Q8Kernel(self.data, self._n_in, self._n_out)
         if self.ggml_type == GGML_TYPE_Q6_K:
             return Q6_KKernel(self.data, self._n_in, self._n_out)
+        if self.ggml_type == GGML_TYPE_Q4_0:
+            return Q4_0Kernel(self.data, self._n_in, self._n_out)
         return Q4_KKernel(self.data, self._n_in, self._n_out)
 
 

@@ -10,6 +10,7 @@ Q6_K = [128 B low nibbles][64 B high bit pairs][16 x int8 scales][f16 d] (src/op
 import numpy as np
 
 Q8_0_BLOCK = 34
+Q4_0_BLOCK = 18
 Q4_K_BLOCK = 144
 Q6_K_BLOCK = 210
 
@@ -39,6 +40,17 @@ def q8_0_weight(seed, n_out, n_in, scale_sigma=0.02):
     d = (np.abs(rng.normal(0.0, scale_sigma, (n_out, nb))) / 127.0).astype(np.float16)
     w[:, :, 0:2] = d.view(np.uint8).reshape(n_out, nb, 2)
     w[:, :, 2:] = rng.integers(-127, 128, (n_out, nb, 32), dtype=np.int8).view(np.uint8)
+    return w.reshape(-1)
+
+
+def q4_0_weight(seed, n_out, n_in, scale_sigma=0.02):
+    """Nibbles uniform in [0,15] (values -8..7); per-block scale f16(|N(0,sigma)|/8)
+    (block layout: src/ops/kernel/q4_0/scalar.rs:24-47)."""
+    rng = np.random.default_rng(seed)
+    nb = n_in // 32
+    w = rng.integers(0, 256, (n_out, nb, Q4_0_BLOCK), dtype=np.uint8)
+    d = (np.abs(rng.normal(0.0, scale_sigma, (n_out, nb))) / 8.0).astype(np.float16)
+    w[:, :, 0:2] = d.view(np.uint8).reshape(n_out, nb, 2)
     return w.reshape(-1)
 
 
@@ -83,3 +95,7 @@ def q4_k_gemv_bytes(n_out, n_in, batch=1):
 
 def q6_k_gemv_bytes(n_out, n_in, batch=1):
     return n_out * (n_in // 256) * Q6_K_BLOCK + batch * (n_in // 256) * 292 + batch * 4 * n_out
+
+
+def q4_0_gemv_bytes(n_out, n_in, batch=1):
+    return n_out * (n_in // 32) * Q4_0_BLOCK + batch * (n_in + 4 * (n_in // 32)) + batch * 4 * n_out
