@@ -498,6 +498,70 @@ def run_kquant(args, pkg, ev, fmt):
     return result
 
 
+def run_q4_0(args, pkg, ev):
+    """Q4_0 x Q8_0 decode GEMV, one large matrix per launch so that the launch streams from HBM: eight distinct
+    151936 x 1024 matrices (the lm_head shape, 87.5 MB each as Q4_0) taken in turn."""
+    H, synth, K = pkg.hip, pkg.synth, pkg.kernel
+    dev_name, cus, hbm = H.device_info()
+    batch, n_out, n_in, n_mats = args.batch, 151936, 1024, 8
+    base = synth.q4_0_weight(synth.seed_for(5, 0), n_out, n_in)
+    recs = []
+    for i in range(n_mats):
+        w = np.roll(base, 18 * 1024 * i)  # distinct bytes per matrix, one generator pass
+        x = synth.activations(synth.seed_for(5, 0x8000 + i), batch, n_in)
+        k = K.Q4_0Kernel(w, n_in, n_out)
+        d_x = H.DeviceBuffer.from_array(x)
+        d_q, d_s, d_y = H.DeviceBuffer(batch * n_in), H.DeviceBuffer(batch * n_in // 32 * 4), H.DeviceBuffer(batch * n_out * 4)
+        H.check(H.lib.rmi_hip_quantize_q8_0_dev(d_x.ptr, d_q.ptr, d_s.ptr, batch, n_in, H.ROUND_TIES_EVEN, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        d_x.free()
+        recs.append(dict(w=w if not args.no_cpu_baseline else None, k=k, d_q=d_q, d_s=d_s, d_y=d_y))
+
+    def step():
+        for r in recs:
+            H.check(H.lib.rmi_hip_gemv_q4_0_dev(r["k"].w.handle, r["d_q"].ptr, r["d_s"].ptr, r["d_y"].ptr, batch, n_out, 0,
+                                                n_out, None))
+
+    copy_calibration(H, args)
+    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
+    alg = n_mats * synth.q4_0_gemv_bytes(n_out, n_in, batch)
+    achieved = alg / (dev_ms * 1e-3) / 1e9
+    result = base_result(args, "Q4_0 x Q8_0 GEMV HBM GB/s, lm_head shape, 1 GPU", "GB/s", round(alg / wall / 1e9, 1), wall,
+                         "int8 dot4 -> f32", {
+        "workload": f"Q4_0 GEMV, {n_mats} distinct matrices {n_out} x {n_in}, decode batch {batch}, one launch per matrix",
+        "batch": batch, "launches_per_step": n_mats, "algorithmic_bytes_per_step": alg, "device": dev_name.strip(),
+        "compute_units": cus})
+    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_0_kernel<{batch},*>", "achieved": round(achieved, 1),
+                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                          "avg_launch_us": round(dev_ms * 1e3 / n_mats, 3),
+                          "traffic": read_traffic("gemv_q4_0_lm_head") if batch == 1 else None}
+    if not args.no_cpu_baseline and batch == 1:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import rmi_oracle as oracle
+        if oracle.have_avx2():
+            cores = min(16, physical_cores())
+            pool = oracle.Pool(cores)
+            host = [(r["d_q"].to_array(np.uint8, (n_in,)), r["d_s"].to_array(np.float32, (n_in // 32,)),
+                     np.zeros(n_out, np.float32)) for r in recs]
+            samples = []
+            for it in range(6):
+                t0 = time.perf_counter()
+                for r, (q, sc, out) in zip(recs, host):
+                    pool.matmul_q4_0(r["w"], q, sc, out, n_in, n_out)
+                samples.append(time.perf_counter() - t0)
+            pool.close()
+            med = statistics.median(samples[1:])
+            step()
+            H.check(H.lib.rmi_hip_synchronize())
+            worst = max(int(np.count_nonzero(r["d_y"].to_array(np.float32, (n_out,)).view(np.uint32) != out.view(np.uint32)))
+                        for r, (_, _, out) in zip(recs, host))
+            result["cpu_baseline"] = {"value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                                      "sample": f"5 full steps ({n_mats} GEMVs, {alg / 1e6:.0f} MB), restated AVX2 "
+                                                f"matmul_q4_0_vs_q8_0 over {cores} threads, median",
+                                      "gpu_outputs_differing_from_cpu": worst}
+    return result
+
+
 def run_q4k_gemm(args, pkg, ev):
     """Q4_K prefill: X[M x 2048] through gate and up (6144 x 2048 each) and X[M x 6144] through down (2048 x 6144),
     Q8_K activations already quantized in HBM; one step = the three products."""
@@ -640,9 +704,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4k", "q6k", "q4k_gemm", "decode"], default="projection_set",
+    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "decode"], default="projection_set",
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
-                         "q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); decode: end-to-end device-resident greedy decode "
+                         "q4_0: Q4_0 x Q8_0 decode GEMV; q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); decode: end-to-end device-resident greedy decode "
                          "(one step = one 639-token-step generation)")
     ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill tokens M for --workload gemm")
@@ -662,7 +726,7 @@ def main():
     pkg = importlib.import_module("rust-model-inference_amd")
     pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
     ev = HipEvents()
-    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4k": run_q4k, "q6k": run_q6k, "q4k_gemm": run_q4k_gemm,
+    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4_0": run_q4_0, "q4k": run_q4k, "q6k": run_q6k, "q4k_gemm": run_q4k_gemm,
            "decode": run_decode}[args.workload]
     result = run(args, pkg, ev)
     if args.workload == "projection_set" and not args.no_decode and args.batch == 1:

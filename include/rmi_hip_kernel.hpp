@@ -5,6 +5,7 @@
 //
 //   Kernel            src/ops/kernel/trait_.rs:15-110
 //   Q8Kernel          src/ops/kernel/q8_0/mod.rs:21-56
+//   Q4_0Kernel        src/ops/kernel/q4_0/mod.rs:18-123
 //   Q4_KKernel        src/ops/kernel/q4_k.rs:7-93
 //   Q6_KKernel        src/ops/kernel/q6_k.rs:7-80
 //   BlockQ8K          src/ops/quant/mod.rs:35-40
@@ -127,6 +128,23 @@ class Q8Kernel : public Kernel {
                          size_t n_out) const override {
         check(rmi_hip_q8_0_forward_batched(w_->get(), input, output, uint32_t(n_in), uint32_t(n_out),
                                            uint32_t(n_tokens), RMI_HIP_ROUND_TIES_EVEN));
+    }
+    const std::shared_ptr<DeviceWeight> &weight() const { return w_; }
+
+  private:
+    std::shared_ptr<DeviceWeight> w_;
+};
+
+class Q4_0Kernel : public Kernel {
+  public:
+    Q4_0Kernel(const uint8_t *data, size_t nbytes, size_t n_in, size_t n_out)
+        : w_(std::make_shared<DeviceWeight>(rmi_hip_upload_q4_0(data, nbytes, uint32_t(n_in), uint32_t(n_out)))) {}
+    explicit Q4_0Kernel(std::shared_ptr<DeviceWeight> w) : w_(std::move(w)) {}
+
+    void forward_prequantized(const uint8_t *input_q8, const float *input_scales, float *output, size_t n_in,
+                              size_t n_out, size_t ith, size_t nth) const override {
+        check(rmi_hip_q4_0_forward_prequantized(w_->get(), input_q8, input_scales, output, uint32_t(n_in),
+                                                uint32_t(n_out), uint32_t(ith), uint32_t(nth)));
     }
     const std::shared_ptr<DeviceWeight> &weight() const { return w_; }
 

@@ -210,6 +210,8 @@ void rmi_ref_pool_matmul_q4k_q8k(rmi_ref_pool *pool, const uint8_t *weight,
                                  size_t n_in, size_t n_out);
 
 /* generic job on the pool: fn(arg, ith, nth) on every thread, then a barrier */
+void rmi_ref_pool_matmul_q4_0(rmi_ref_pool *pool, const uint8_t *weight, const uint8_t *input_q8,
+                              const float *input_scales, float *output, size_t n_in, size_t n_out);
 void rmi_ref_pool_matmul_q6k_q8k(rmi_ref_pool *pool, const uint8_t *weight, const float *d, const int8_t *qs,
                                  const int16_t *bsums, float *output, size_t n_in, size_t n_out);
 void rmi_ref_pool_run(rmi_ref_pool *pool, void (*fn)(void *arg, int ith, int nth), void *arg);

@@ -77,6 +77,7 @@ def _load():
         "rmi_ref_pool_threads": (C.c_int, [C.c_void_p]),
         "rmi_ref_pool_matmul_q8_0": (None, [C.c_void_p, _u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz]),
         "rmi_ref_pool_matmul_q4k_q8k": (None, [C.c_void_p, _u8p, _f32p, _i8p, _i16p, _f32p, _sz, _sz]),
+        "rmi_ref_pool_matmul_q4_0": (None, [C.c_void_p, _u8p, _u8p, _f32p, _f32p, _sz, _sz]),
         "rmi_ref_pool_matmul_q6k_q8k": (None, [C.c_void_p, _u8p, _f32p, _i8p, _i16p, _f32p, _sz, _sz]),
     }
     for name, (res, args) in sig.items():
@@ -445,6 +446,10 @@ class Pool:
     def matmul_q4k_q8k(self, w, d, qs, bsums, out, n_in, n_out):
         lib.rmi_ref_pool_matmul_q4k_q8k(self._h, _p(w, _u8p), _p(d, _f32p), _p(qs, _i8p), _p(bsums, _i16p),
                                         _p(out, _f32p), n_in, n_out)
+        return out
+
+    def matmul_q4_0(self, w, q8, sc, out, n_in, n_out):
+        lib.rmi_ref_pool_matmul_q4_0(self._h, _p(w, _u8p), _p(q8, _u8p), _p(sc, _f32p), _p(out, _f32p), n_in, n_out)
         return out
 
     def matmul_q6k_q8k(self, w, d, qs, bsums, out, n_in, n_out):

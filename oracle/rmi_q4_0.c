@@ -99,3 +99,24 @@ void rmi_ref_x86_matmul_q4_0_range(const uint8_t *weight, const uint8_t *input_q
         output[i] = acc;
     }
 }
+
+/* y = W x over the persistent pool: rows split as (ith, nth) (q4_0/mod.rs:46-51), the AVX2 kernel per slice */
+typedef struct {
+    const uint8_t *weight, *q8;
+    const float *scales;
+    float *output;
+    size_t n_in, n_out;
+} q40_job;
+
+static void q40_slice(void *arg, int ith, int nth) {
+    const q40_job *j = (const q40_job *)arg;
+    size_t per = (j->n_out + (size_t)nth - 1) / (size_t)nth, start = (size_t)ith * per;
+    size_t end = start + per < j->n_out ? start + per : j->n_out;
+    if (start < end) rmi_ref_x86_matmul_q4_0_range(j->weight, j->q8, j->scales, j->output + start, j->n_in, start, end);
+}
+
+void rmi_ref_pool_matmul_q4_0(rmi_ref_pool *pool, const uint8_t *weight, const uint8_t *input_q8,
+                              const float *input_scales, float *output, size_t n_in, size_t n_out) {
+    q40_job job = {weight, input_q8, input_scales, output, n_in, n_out};
+    rmi_ref_pool_run(pool, q40_slice, &job);
+}

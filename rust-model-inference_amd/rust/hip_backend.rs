@@ -33,6 +33,7 @@ extern "C" {
     fn rmi_hip_last_error() -> *const c_char;
     fn rmi_hip_upload_q8_0(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
     fn rmi_hip_upload_q4_k(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
+    fn rmi_hip_upload_q4_0(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
     fn rmi_hip_upload_q6_k(blocks: *const u8, nbytes: usize, n_in: u32, n_out: u32) -> *mut RmiHipWeight;
     fn rmi_hip_fuse_vstack(a: *const RmiHipWeight, b: *const RmiHipWeight) -> *mut RmiHipWeight;
     fn rmi_hip_free_weight(w: *mut RmiHipWeight);
@@ -54,6 +55,14 @@ extern "C" {
     fn rmi_hip_q4_k_forward_prequantized(
         w: *const RmiHipWeight, input_q8: *const u8, input_scales: *const f32, output: *mut f32,
         n_in: u32, n_out: u32, ith: u32, nth: u32,
+    ) -> c_int;
+    fn rmi_hip_q4_0_forward_prequantized(
+        w: *const RmiHipWeight, input_q8: *const u8, input_scales: *const f32, output: *mut f32,
+        n_in: u32, n_out: u32, ith: u32, nth: u32,
+    ) -> c_int;
+    fn rmi_hip_q4_0_forward_batched(
+        w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
+        rounding: c_int,
     ) -> c_int;
     fn rmi_hip_q6_k_forward_prepared(
         w: *const RmiHipWeight, d: *const f32, qs: *const i8, bsums: *const i16, output: *mut f32,
@@ -83,7 +92,7 @@ pub fn init(device: i32) -> Result<(), String> {
 }
 
 #[derive(Clone, Copy, PartialEq)]
-enum Dtype { Q8_0, Q4K, Q6K }
+enum Dtype { Q8_0, Q4_0, Q4K, Q6K }
 
 /// A weight resident in HBM.  `Kernel: Send + Sync`: the library gives every
 /// calling thread its own stream and staging, so `&self` calls may overlap.
@@ -102,6 +111,10 @@ impl HipKernel {
     pub fn upload_q4_k(weight: &[u8], n_in: usize, n_out: usize) -> Result<Self, String> {
         let h = unsafe { rmi_hip_upload_q4_k(weight.as_ptr(), weight.len(), n_in as u32, n_out as u32) };
         if h.is_null() { Err(last_error()) } else { Ok(Self { handle: h, dtype: Dtype::Q4K }) }
+    }
+    pub fn upload_q4_0(weight: &[u8], n_in: usize, n_out: usize) -> Result<Self, String> {
+        let h = unsafe { rmi_hip_upload_q4_0(weight.as_ptr(), weight.len(), n_in as u32, n_out as u32) };
+        if h.is_null() { Err(last_error()) } else { Ok(Self { handle: h, dtype: Dtype::Q4_0 }) }
     }
     pub fn upload_q6_k(weight: &[u8], n_in: usize, n_out: usize) -> Result<Self, String> {
         let h = unsafe { rmi_hip_upload_q6_k(weight.as_ptr(), weight.len(), n_in as u32, n_out as u32) };
@@ -132,6 +145,9 @@ impl Kernel for HipKernel {
                 Dtype::Q8_0 => rmi_hip_q8_0_forward_prequantized(
                     self.handle, input_q8.as_ptr(), input_scales.as_ptr(), output.as_mut_ptr(),
                     n_in as u32, n_out as u32, ith as u32, nth as u32),
+                Dtype::Q4_0 => rmi_hip_q4_0_forward_prequantized(
+                    self.handle, input_q8.as_ptr(), input_scales.as_ptr(), output.as_mut_ptr(),
+                    n_in as u32, n_out as u32, ith as u32, nth as u32),
                 Dtype::Q4K => rmi_hip_q4_k_forward_prequantized(
                     self.handle, input_q8.as_ptr(), input_scales.as_ptr(), output.as_mut_ptr(),
                     n_in as u32, n_out as u32, ith as u32, nth as u32),
@@ -147,7 +163,7 @@ impl Kernel for HipKernel {
         &self, input_f32: &[f32], input_q8: &[u8], input_scales: &[f32], q8_k: Option<&[BlockQ8K]>,
         output: &mut [f32], n_in: usize, n_out: usize, ith: usize, nth: usize,
     ) {
-        if self.dtype == Dtype::Q8_0 {
+        if self.dtype == Dtype::Q8_0 || self.dtype == Dtype::Q4_0 {
             return self.forward_prequantized(input_q8, input_scales, output, n_in, n_out, ith, nth);
         }
         // BlockQ8K has no repr(C) (src/ops/quant/mod.rs:35-40): pass three arrays.
@@ -175,6 +191,8 @@ impl Kernel for HipKernel {
         expect_ok(unsafe {
             match self.dtype {
                 Dtype::Q8_0 => rmi_hip_q8_0_forward_batched(self.handle, input.as_ptr(), output.as_mut_ptr(),
+                                                            n_in as u32, n_out as u32, n_tokens, ROUND_TIES_EVEN),
+                Dtype::Q4_0 => rmi_hip_q4_0_forward_batched(self.handle, input.as_ptr(), output.as_mut_ptr(),
                                                             n_in as u32, n_out as u32, n_tokens, ROUND_TIES_EVEN),
                 Dtype::Q4K => rmi_hip_q4_k_forward_batched(self.handle, input.as_ptr(), output.as_mut_ptr(),
                                                            n_in as u32, n_out as u32, n_tokens),
