@@ -77,6 +77,8 @@ uint32_t rmi_hip_weight_n_out(const rmi_hip_weight *w);
 int rmi_hip_weight_dtype(const rmi_hip_weight *w);
 /* bytes this weight occupies in HBM after repacking */
 size_t rmi_hip_weight_device_bytes(const rmi_hip_weight *w);
+/* device address of that repacked tile stream (read-only for callers; valid until rmi_hip_free_weight) */
+const void *rmi_hip_weight_device_data(const rmi_hip_weight *w);
 
 /* ---- Q8_0, host slices ---------------------------------------------------*/
 
@@ -325,6 +327,55 @@ void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s);
 int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_prompt, uint32_t max_new,
                            uint32_t *generated, uint32_t *step_argmax, float *step_top2, const uint32_t *dump_steps,
                            uint32_t n_dump, float *dump_logits, double *seconds);
+
+/* ------------------------------------------------------------------ GGUF file -> HBM
+ * The reference maps the file and hands slices of the mapping to its layers (GGUFLoader::from_file,
+ * src/core/loader.rs:211-320; TensorSource::tensor_data, :363-372).  Here the same mapping feeds the uploads:
+ * tensor bytes go from the page cache through two pinned staging chunks to the device, where the repack kernel
+ * writes the tile stream; no whole-tensor copy on the host, no intermediate device copy of a whole tensor.
+ * Parsing accepts what from_mmap accepts (versions 2 and 3, every metadata and tensor type it knows) and
+ * rejects what it rejects (truncation, unknown tags, nested arrays, a tensor past the end of the file), with
+ * the reference's message in rmi_hip_last_error().  open/close and the metadata and tensor queries need no
+ * device and no rmi_hip_init. */
+typedef struct rmi_hip_gguf rmi_hip_gguf;
+rmi_hip_gguf *rmi_hip_gguf_open(const char *path); /* NULL on error */
+void rmi_hip_gguf_close(rmi_hip_gguf *g);          /* weights and sessions made from it stay valid */
+uint32_t rmi_hip_gguf_version(const rmi_hip_gguf *g);
+uint64_t rmi_hip_gguf_alignment(const rmi_hip_gguf *g);   /* general.alignment, default 32 */
+uint64_t rmi_hip_gguf_data_offset(const rmi_hip_gguf *g); /* GGUFLoader::data_offset */
+uint64_t rmi_hip_gguf_n_tensors(const rmi_hip_gguf *g);
+uint64_t rmi_hip_gguf_n_kv(const rmi_hip_gguf *g);
+const char *rmi_hip_gguf_kv_key(const rmi_hip_gguf *g, uint64_t index); /* NULL past the end */
+/* Metadata (GGUFLoader::metadata + the MetaValue conversions, src/core/tensor.rs:146-187).  meta_type gives the
+ * value tag (0 u8 .. 12 f64, 8 string, 9 array) or -1 when the key is absent; the getters return 1 and store
+ * the value, or 0 when the key is absent or the conversion is one the reference refuses (to_u64: every
+ * integer and float type, `as u64` semantics; to_f64: f32, f64 and the 32/64-bit integers). */
+int rmi_hip_gguf_meta_type(const rmi_hip_gguf *g, const char *key);
+int rmi_hip_gguf_meta_u64(const rmi_hip_gguf *g, const char *key, uint64_t *out);
+int rmi_hip_gguf_meta_f64(const rmi_hip_gguf *g, const char *key, double *out);
+int rmi_hip_gguf_meta_bool(const rmi_hip_gguf *g, const char *key, int *out);
+/* to_string_val: length of the string or -1; up to cap - 1 bytes and a terminator are stored in buf */
+int64_t rmi_hip_gguf_meta_str(const rmi_hip_gguf *g, const char *key, char *buf, size_t cap);
+/* to_arr: element count (and element tag) or -1; element `index` of a numeric array through to_u64 */
+int64_t rmi_hip_gguf_meta_array_len(const rmi_hip_gguf *g, const char *key, int *elem_type);
+int rmi_hip_gguf_meta_array_u64(const rmi_hip_gguf *g, const char *key, uint64_t index, uint64_t *out);
+/* Tensors (GGUFLoader::tensor_info / tensor_data).  find: index or -1.  dims are [columns, rows, ..]. */
+int64_t rmi_hip_gguf_find_tensor(const rmi_hip_gguf *g, const char *name);
+int rmi_hip_gguf_tensor_info(const rmi_hip_gguf *g, uint64_t index, const char **name, uint32_t *n_dims,
+                             uint64_t *dims, uint32_t dims_cap, int *ggml_type, uint64_t *offset, uint64_t *nbytes);
+const uint8_t *rmi_hip_gguf_tensor_data(const rmi_hip_gguf *g, uint64_t index); /* into the mapping */
+/* A 2-D Q8_0, Q4_0, Q4K or Q6K tensor as a device weight (the same result as rmi_hip_upload_* on its bytes). */
+rmi_hip_weight *rmi_hip_gguf_upload(const rmi_hip_gguf *g, const char *name);
+/* Up to 16 tensors of one type and column count as one weight, rows one below the other ([q ; k ; v],
+ * [gate ; up]): what rmi_hip_fuse_vstack gives, written in place. */
+rmi_hip_weight *rmi_hip_gguf_upload_stack(const rmi_hip_gguf *g, const char *const *names, int n_names);
+/* Qwen3Config::from_source (src/models/qwen3.rs:46-94, keys of src/core/loader.rs:379-461, has_qk_norm of
+ * :556) for the architectures that use rope_neox; capacity is checked against context_length as
+ * checked_session_capacity does (src/models/qwen3.rs:108-121). */
+int rmi_hip_gguf_qwen3_config(const rmi_hip_gguf *g, uint32_t capacity, int rounding, rmi_hip_qwen3_config *out);
+/* Qwen3Model::from_source + Qwen3Session::new over the file (tensor names, shapes and types of
+ * src/models/qwen3.rs:262-349; "Missing tensor: .." / "Invalid tensor ..: .." as checked_tensor, :1350-1380). */
+rmi_hip_qwen3 *rmi_hip_qwen3_create_from_gguf(const rmi_hip_gguf *g, uint32_t capacity, int rounding);
 
 #ifdef __cplusplus
 }

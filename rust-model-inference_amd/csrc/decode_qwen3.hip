@@ -760,27 +760,7 @@ float *upload_f32(rmi_hip_qwen3 *s, const float *host, size_t n) {
 }
 
 rmi_hip_weight *upload_stack(const uint8_t *const *parts, const uint32_t *rows, int n_parts, uint32_t n_in) {
-    rmi_hip_weight *acc = nullptr;
-    for (int i = 0; i < n_parts; i++) {
-        rmi_hip_weight *w = rmi_hip_upload_q8_0(parts[i], size_t(rows[i]) * (n_in / 32) * 34, n_in, rows[i]);
-        if (!w) {
-            if (acc) rmi_hip_free_weight(acc);
-            return nullptr;
-        }
-        if (!acc) {
-            acc = w;
-            continue;
-        }
-        rmi_hip_weight *f = rmi_hip_fuse_vstack(acc, w);
-        rmi_hip_free_weight(acc);
-        rmi_hip_free_weight(w);
-        if (!f) {
-            rmi_set_error("stacking projection weights failed");
-            return nullptr;
-        }
-        acc = f;
-    }
-    return acc;
+    return rmi_upload_stack(RMI_HIP_DTYPE_Q8_0, parts, rows, n_parts, n_in);
 }
 
 int gemv(const rmi_hip_weight *w, const int8_t *q8, const float *scales, float *y, hipStream_t st) {

@@ -162,10 +162,10 @@ __global__ __launch_bounds__(256) void block_dots_q4_0_kernel(const uint8_t *__r
 }
 
 // ---- upload-time repack: one workgroup per (tile, octet) of the destination, 576 16-bit units (the 18-byte
-// source blocks are only 2-byte aligned)
+// source blocks are only 2-byte aligned); `src` holds the rows from tile `tile0` on
 __global__ __launch_bounds__(256) void repack_q4_0_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
-                                                           uint32_t n_out, uint32_t nb, uint32_t n_oct) {
-    const uint32_t tile = blockIdx.x / n_oct, o = blockIdx.x % n_oct;
+                                                           uint32_t n_out, uint32_t nb, uint32_t n_oct, uint32_t tile0) {
+    const uint32_t tile = tile0 + blockIdx.x / n_oct, o = blockIdx.x % n_oct;
     uint16_t *chunk = reinterpret_cast<uint16_t *>(dst + (size_t(tile) * n_oct + o) * kQ40OctetBytes);
     for (uint32_t idx = threadIdx.x; idx < 576; idx += 256) {
         uint32_t r, blk, half;  // destination unit idx <- unit `half` of block `blk` of row r
@@ -181,7 +181,8 @@ __global__ __launch_bounds__(256) void repack_q4_0_kernel(const uint8_t *__restr
         }
         const uint32_t row = tile * kTileRows + r;
         uint16_t v = 0;
-        if (row < n_out && blk < nb) v = reinterpret_cast<const uint16_t *>(src + (size_t(row) * nb + blk) * 18)[half];
+        if (row < n_out && blk < nb)
+            v = reinterpret_cast<const uint16_t *>(src + (size_t(row - tile0 * kTileRows) * nb + blk) * 18)[half];
         chunk[idx] = v;
     }
 }
@@ -231,10 +232,11 @@ int rmi_launch_block_dots_q4_0(const rmi_hip_weight *w, const int8_t *x_q8, int3
     return RMI_HIP_OK;
 }
 
-int rmi_launch_repack_q4_0(const uint8_t *src, rmi_hip_weight *w, hipStream_t s) {
-    const uint32_t grid = w->n_tiles * w->n_units;
+int rmi_launch_repack_q4_0(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0, uint32_t n_tiles, hipStream_t s) {
+    const uint32_t grid = n_tiles * w->n_units;
     if (grid == 0) return RMI_HIP_OK;
-    hipLaunchKernelGGL(repack_q4_0_kernel, dim3(grid), dim3(256), 0, s, src, w->data, w->n_out, w->n_in / 32, w->n_units);
+    hipLaunchKernelGGL(repack_q4_0_kernel, dim3(grid), dim3(256), 0, s, src, w->data, w->n_out, w->n_in / 32, w->n_units,
+                       tile0);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }

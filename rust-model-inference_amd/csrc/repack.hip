@@ -1,15 +1,18 @@
 // Upload-time repacking of GGUF block rows into the HBM tile streams described
-// in rmi_internal.h, and the row copier behind fuse_vstack.
+// in rmi_internal.h, and the row copier behind fuse_vstack.  A weight arrives in
+// chunks of whole tiles: `src` holds the rows from tile `tile0` on, the grid
+// covers the tiles of the chunk.
 #include "rmi_internal.h"
 
 namespace {
 
 // One workgroup per (tile, octet) of the destination.
 __global__ __launch_bounds__(256) void repack_q8_0_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
-                                                           uint32_t n_out, uint32_t nb, uint32_t n_oct) {
-    const uint32_t tile = blockIdx.x / n_oct;
+                                                           uint32_t n_out, uint32_t nb, uint32_t n_oct, uint32_t tile0) {
+    const uint32_t tile = tile0 + blockIdx.x / n_oct;
     const uint32_t o = blockIdx.x % n_oct;
     const uint32_t tid = threadIdx.x;
+    const uint32_t row0 = tile0 * kTileRows;
     uint8_t *tile_base = dst + size_t(tile) * n_oct * kOctetBytes;
     const size_t row_stride = size_t(nb) * 34;
 
@@ -18,7 +21,7 @@ __global__ __launch_bounds__(256) void repack_q8_0_kernel(const uint8_t *__restr
         const uint32_t row = tile * kTileRows + r, blk = o * 8 + jj;
         uint16_t d = 0;
         if (row < n_out && blk < nb) {
-            const uint8_t *p = src + row * row_stride + size_t(blk) * 34;
+            const uint8_t *p = src + (row - row0) * row_stride + size_t(blk) * 34;
             d = uint16_t(p[0]) | (uint16_t(p[1]) << 8);
         }
         reinterpret_cast<uint16_t *>(tile_base + size_t(o) * 128 + r * 16)[jj] = d;
@@ -30,7 +33,7 @@ __global__ __launch_bounds__(256) void repack_q8_0_kernel(const uint8_t *__restr
         const uint32_t row = tile * kTileRows + r, q = 2 * o + ql, blk = q * 4 + j;
         uint32_t v = 0;
         if (row < n_out && blk < nb) {
-            const uint8_t *p = src + row * row_stride + size_t(blk) * 34 + 2 + 4 * L;
+            const uint8_t *p = src + (row - row0) * row_stride + size_t(blk) * 34 + 2 + 4 * L;
             v = uint32_t(p[0]) | (uint32_t(p[1]) << 8) | (uint32_t(p[2]) << 16) | (uint32_t(p[3]) << 24);
         }
         reinterpret_cast<uint32_t *>(quants + size_t(q) * 1024 + (r * 8 + L) * 16)[j] = v;
@@ -39,8 +42,8 @@ __global__ __launch_bounds__(256) void repack_q8_0_kernel(const uint8_t *__restr
 
 // One workgroup per (tile, super-block) of the destination: 288 dwords.
 __global__ __launch_bounds__(256) void repack_q4_k_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
-                                                           uint32_t n_out, uint32_t n_sb) {
-    const uint32_t tile = blockIdx.x / n_sb;
+                                                           uint32_t n_out, uint32_t n_sb, uint32_t tile0) {
+    const uint32_t tile = tile0 + blockIdx.x / n_sb;
     const uint32_t sb = blockIdx.x % n_sb;
     uint32_t *chunk = reinterpret_cast<uint32_t *>(dst + (size_t(tile) * n_sb + sb) * kQ4KSuperBytes);
     for (uint32_t idx = threadIdx.x; idx < 288; idx += 256) {
@@ -56,15 +59,16 @@ __global__ __launch_bounds__(256) void repack_q4_k_kernel(const uint8_t *__restr
         }
         const uint32_t row = tile * kTileRows + r;
         uint32_t v = 0;
-        if (row < n_out) v = reinterpret_cast<const uint32_t *>(src + (size_t(row) * n_sb + sb) * 144)[src_dword];
+        if (row < n_out)
+            v = reinterpret_cast<const uint32_t *>(src + (size_t(row - tile0 * kTileRows) * n_sb + sb) * 144)[src_dword];
         chunk[idx] = v;
     }
 }
 
 // One workgroup per (tile, super-block) of the destination: 420 dwords.
 __global__ __launch_bounds__(256) void repack_q6_k_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
-                                                           uint32_t n_out, uint32_t n_sb) {
-    const uint32_t tile = blockIdx.x / n_sb;
+                                                           uint32_t n_out, uint32_t n_sb, uint32_t tile0) {
+    const uint32_t tile = tile0 + blockIdx.x / n_sb;
     const uint32_t sb = blockIdx.x % n_sb;
     uint8_t *chunk = dst + (size_t(tile) * n_sb + sb) * kQ6KSuperBytes;
     // the 210-byte source blocks are only 2-byte aligned: move 16-bit units
@@ -89,7 +93,8 @@ __global__ __launch_bounds__(256) void repack_q6_k_kernel(const uint8_t *__restr
         }
         const uint32_t row = tile * kTileRows + r;
         uint16_t v = 0;
-        if (row < n_out) v = reinterpret_cast<const uint16_t *>(src + (size_t(row) * n_sb + sb) * 210)[src_half];
+        if (row < n_out)
+            v = reinterpret_cast<const uint16_t *>(src + (size_t(row - tile0 * kTileRows) * n_sb + sb) * 210)[src_half];
         reinterpret_cast<uint16_t *>(chunk)[idx] = v;
     }
 }
@@ -138,27 +143,27 @@ __global__ __launch_bounds__(256) void copy_rows_kernel(const uint4 *__restrict_
 
 }  // namespace
 
-int rmi_launch_repack_q8_0(const uint8_t *src, rmi_hip_weight *w, hipStream_t s) {
-    const uint32_t grid = w->n_tiles * w->n_units;
+int rmi_launch_repack_q8_0(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0, uint32_t n_tiles, hipStream_t s) {
+    const uint32_t grid = n_tiles * w->n_units;
     if (grid == 0) return RMI_HIP_OK;
     hipLaunchKernelGGL(repack_q8_0_kernel, dim3(grid), dim3(256), 0, s, src, w->data, w->n_out, w->n_in / 32,
-                       w->n_units);
+                       w->n_units, tile0);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
 
-int rmi_launch_repack_q4_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s) {
-    const uint32_t grid = w->n_tiles * w->n_units;
+int rmi_launch_repack_q4_k(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0, uint32_t n_tiles, hipStream_t s) {
+    const uint32_t grid = n_tiles * w->n_units;
     if (grid == 0) return RMI_HIP_OK;
-    hipLaunchKernelGGL(repack_q4_k_kernel, dim3(grid), dim3(256), 0, s, src, w->data, w->n_out, w->n_units);
+    hipLaunchKernelGGL(repack_q4_k_kernel, dim3(grid), dim3(256), 0, s, src, w->data, w->n_out, w->n_units, tile0);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
 
-int rmi_launch_repack_q6_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s) {
-    const uint32_t grid = w->n_tiles * w->n_units;
+int rmi_launch_repack_q6_k(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0, uint32_t n_tiles, hipStream_t s) {
+    const uint32_t grid = n_tiles * w->n_units;
     if (grid == 0) return RMI_HIP_OK;
-    hipLaunchKernelGGL(repack_q6_k_kernel, dim3(grid), dim3(256), 0, s, src, w->data, w->n_out, w->n_units);
+    hipLaunchKernelGGL(repack_q6_k_kernel, dim3(grid), dim3(256), 0, s, src, w->data, w->n_out, w->n_units, tile0);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }

@@ -95,6 +95,11 @@ bool rmi_ready();
 // buffers that grow on demand, so concurrent Kernel calls never share state.
 struct RmiThreadCtx {
     hipStream_t stream = nullptr;
+    // weight upload: two pinned and two device staging chunks taken in turn, an event per pair
+    void *up_pin[2] = {nullptr, nullptr};
+    void *up_dev[2] = {nullptr, nullptr};
+    hipEvent_t up_done[2] = {nullptr, nullptr};
+    size_t up_cap = 0;
     void *dev[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     size_t dev_cap[6] = {0, 0, 0, 0, 0, 0};
     void *pin[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -107,10 +112,17 @@ void *rmi_pin_buf(RmiThreadCtx *c, int slot, size_t nbytes);
 int rmi_device_cus();
 
 // ------------------------------------------------- launchers (device ptrs)
-int rmi_launch_repack_q8_0(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
-int rmi_launch_repack_q4_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
-int rmi_launch_repack_q6_k(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
-int rmi_launch_repack_q4_0(const uint8_t *src, rmi_hip_weight *w, hipStream_t s);
+// repack tiles [tile0, tile0 + n_tiles) of w; src = the source rows from row tile0 * 8 on (device memory)
+int rmi_launch_repack_q8_0(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0, uint32_t n_tiles, hipStream_t s);
+int rmi_launch_repack_q4_k(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0, uint32_t n_tiles, hipStream_t s);
+int rmi_launch_repack_q6_k(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0, uint32_t n_tiles, hipStream_t s);
+int rmi_launch_repack_q4_0(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0, uint32_t n_tiles, hipStream_t s);
+// Host rows -> the tile stream of w from row0 (a multiple of 8) on, chunk by chunk through the thread's staging
+// pair; enqueues on c->stream and returns without waiting for the last chunk.
+int rmi_upload_rows(RmiThreadCtx *c, rmi_hip_weight *w, uint32_t row0, const uint8_t *blocks, uint32_t n_rows);
+// One weight whose rows are the parts one below the other ([a ; b ; c]); synchronises.  NULL + error text on failure.
+rmi_hip_weight *rmi_upload_stack(int dtype, const uint8_t *const *parts, const uint32_t *rows, int n_parts,
+                                 uint32_t n_in);
 int rmi_launch_copy_rows(const rmi_hip_weight *src, rmi_hip_weight *dst, uint32_t dst_row0, hipStream_t s);
 
 struct RmiGemvProblem {

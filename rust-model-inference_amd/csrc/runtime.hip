@@ -1,5 +1,6 @@
 // Context, error reporting, per-thread staging, weight upload / fusion.
 #include <mutex>
+#include <thread>
 #include <vector>
 
 #include "rmi_internal.h"
@@ -132,6 +133,14 @@ void rmi_hip_shutdown(void) {
             c->pin[i] = nullptr;
             c->dev_cap[i] = c->pin_cap[i] = 0;
         }
+        for (int i = 0; i < 2; i++) {
+            if (c->up_pin[i]) hipHostFree(c->up_pin[i]);
+            if (c->up_dev[i]) hipFree(c->up_dev[i]);
+            if (c->up_done[i]) hipEventDestroy(c->up_done[i]);
+            c->up_pin[i] = c->up_dev[i] = nullptr;
+            c->up_done[i] = nullptr;
+        }
+        c->up_cap = 0;
         if (c->stream) hipStreamDestroy(c->stream);
         c->stream = nullptr;
     }
@@ -213,47 +222,174 @@ static rmi_hip_weight *alloc_weight(int dtype, uint32_t n_in, uint32_t n_out) {
     return w;
 }
 
-static rmi_hip_weight *upload(int dtype, const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {
+}  // extern "C"
+
+static size_t row_bytes_of(int dtype, uint32_t n_in) {
+    switch (dtype) {
+        case RMI_HIP_DTYPE_Q8_0: return size_t(n_in / 32) * 34;
+        case RMI_HIP_DTYPE_Q4_0: return size_t(n_in / 32) * 18;
+        case RMI_HIP_DTYPE_Q6_K: return size_t(n_in / 256) * 210;
+        default: return size_t(n_in / 256) * 144;
+    }
+}
+
+static bool dtype_known(int dtype) {
+    return dtype == RMI_HIP_DTYPE_Q8_0 || dtype == RMI_HIP_DTYPE_Q4_0 || dtype == RMI_HIP_DTYPE_Q4_K ||
+           dtype == RMI_HIP_DTYPE_Q6_K;
+}
+
+// The staging pair of this thread: pinned host chunks the host fills while the previous chunk's copy and repack
+// are still running, device chunks the repack kernel reads.  Grows when one 8-row tile is larger than a chunk.
+static constexpr size_t kUploadChunkBytes = size_t(16) << 20;
+
+static int upload_staging(RmiThreadCtx *c, size_t tile_src_bytes) {
+    const size_t want = tile_src_bytes > kUploadChunkBytes ? tile_src_bytes : kUploadChunkBytes;
+    if (c->up_cap >= want) return RMI_HIP_OK;
+    RMI_HIP_CHECK(hipStreamSynchronize(c->stream));
+    for (int i = 0; i < 2; i++) {
+        if (c->up_pin[i]) hipHostFree(c->up_pin[i]);
+        if (c->up_dev[i]) hipFree(c->up_dev[i]);
+        c->up_pin[i] = c->up_dev[i] = nullptr;
+    }
+    c->up_cap = 0;
+    for (int i = 0; i < 2; i++) {
+        RMI_HIP_CHECK(hipHostMalloc(&c->up_pin[i], want, hipHostMallocDefault));
+        RMI_HIP_CHECK(hipMalloc(&c->up_dev[i], want));
+        if (!c->up_done[i]) RMI_HIP_CHECK(hipEventCreateWithFlags(&c->up_done[i], hipEventDisableTiming));
+    }
+    c->up_cap = want;
+    return RMI_HIP_OK;
+}
+
+// host memcpy over a few threads: one core moves 5-10 GB/s (less while it also takes the page faults of a
+// freshly mapped file), the link to the GPU several times that
+static void copy_to_pinned(uint8_t *dst, const uint8_t *src, size_t n) {
+    const size_t kPerThread = size_t(2) << 20;
+    size_t n_thr = n / kPerThread;
+    if (n_thr > 4) n_thr = 4;
+    if (n_thr < 2) {
+        memcpy(dst, src, n);
+        return;
+    }
+    const size_t piece = ((n + n_thr - 1) / n_thr + 4095) & ~size_t(4095);
+    std::vector<std::thread> pool;
+    for (size_t t = 1; t < n_thr; t++) {
+        const size_t off = t * piece;
+        if (off >= n) break;
+        const size_t len = n - off < piece ? n - off : piece;
+        pool.emplace_back([=] { memcpy(dst + off, src + off, len); });
+    }
+    memcpy(dst, src, piece < n ? piece : n);
+    for (std::thread &th : pool) th.join();
+}
+
+int rmi_upload_rows(RmiThreadCtx *c, rmi_hip_weight *w, uint32_t row0, const uint8_t *blocks, uint32_t n_rows) {
+    if (row0 % kTileRows != 0 || row0 + n_rows > w->n_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "upload of rows %u..%u into a weight of %u rows", row0, row0 + n_rows, w->n_out);
+    if ((row0 + n_rows) % kTileRows != 0 && row0 + n_rows != w->n_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "a row range that ends inside a tile must end the weight");
+    const size_t row_bytes = row_bytes_of(w->dtype, w->n_in);
+    if (n_rows == 0 || row_bytes == 0) return RMI_HIP_OK;
+    int rc = upload_staging(c, row_bytes * kTileRows);
+    if (rc != RMI_HIP_OK) return rc;
+    uint32_t rows_per_chunk = uint32_t(c->up_cap / (row_bytes * kTileRows)) * kTileRows;
+    uint32_t i = 0;
+    for (uint64_t done = 0; done < n_rows; done += rows_per_chunk, i++) {
+        const int slot = int(i & 1);
+        const uint32_t rows = n_rows - done < rows_per_chunk ? uint32_t(n_rows - done) : rows_per_chunk;
+        const size_t nbytes = size_t(rows) * row_bytes;
+        // the copy and the repack that last used this pair are done (at once for an event never recorded)
+        RMI_HIP_CHECK(hipEventSynchronize(c->up_done[slot]));
+        copy_to_pinned(static_cast<uint8_t *>(c->up_pin[slot]), blocks + size_t(done) * row_bytes, nbytes);
+        RMI_HIP_CHECK(hipMemcpyAsync(c->up_dev[slot], c->up_pin[slot], nbytes, hipMemcpyHostToDevice, c->stream));
+        const uint8_t *src = static_cast<const uint8_t *>(c->up_dev[slot]);
+        const uint32_t tile0 = uint32_t((row0 + done) / kTileRows), n_tiles = (rows + kTileRows - 1) / kTileRows;
+        rc = w->dtype == RMI_HIP_DTYPE_Q8_0   ? rmi_launch_repack_q8_0(src, w, tile0, n_tiles, c->stream)
+             : w->dtype == RMI_HIP_DTYPE_Q4_0 ? rmi_launch_repack_q4_0(src, w, tile0, n_tiles, c->stream)
+             : w->dtype == RMI_HIP_DTYPE_Q6_K ? rmi_launch_repack_q6_k(src, w, tile0, n_tiles, c->stream)
+                                              : rmi_launch_repack_q4_k(src, w, tile0, n_tiles, c->stream);
+        if (rc != RMI_HIP_OK) return rc;
+        RMI_HIP_CHECK(hipEventRecord(c->up_done[slot], c->stream));
+    }
+    return RMI_HIP_OK;
+}
+
+rmi_hip_weight *rmi_upload_stack(int dtype, const uint8_t *const *parts, const uint32_t *rows, int n_parts,
+                                 uint32_t n_in) {
     if (!rmi_ready()) {
         rmi_set_error("rmi_hip_init has not succeeded");
         return nullptr;
     }
     const uint32_t block_elems = dtype == RMI_HIP_DTYPE_Q8_0 || dtype == RMI_HIP_DTYPE_Q4_0 ? 32 : 256;
-    const size_t block_bytes = dtype == RMI_HIP_DTYPE_Q8_0   ? 34
-                               : dtype == RMI_HIP_DTYPE_Q4_0 ? 18
-                               : dtype == RMI_HIP_DTYPE_Q6_K ? 210
-                                                             : 144;
+    if (!dtype_known(dtype) || n_parts < 1) {
+        rmi_set_error("unknown weight type %d or no parts", dtype);
+        return nullptr;
+    }
     if (n_in == 0 || n_in % block_elems != 0) {
         rmi_set_error("n_in=%u is not a positive multiple of %u", n_in, block_elems);
         return nullptr;
     }
-    const size_t want = size_t(n_out) * (n_in / block_elems) * block_bytes;
-    if (nbytes < want || (!blocks && want)) {
-        rmi_set_error("weight slice holds %zu bytes, %u x %u needs %zu", nbytes, n_out, n_in, want);
+    uint64_t total = 0;
+    bool aligned = true;  // every part but the last ends on a tile boundary
+    for (int i = 0; i < n_parts; i++) {
+        if (!parts[i] && rows[i]) {
+            rmi_set_error("null weight slice");
+            return nullptr;
+        }
+        if (i + 1 < n_parts && rows[i] % kTileRows != 0) aligned = false;
+        total += rows[i];
+    }
+    if (total > 0xffffffffull) {
+        rmi_set_error("stacked weight has %llu rows", (unsigned long long)total);
         return nullptr;
     }
     RmiThreadCtx *c = rmi_thread_ctx();
     if (!c) return nullptr;
-    rmi_hip_weight *w = alloc_weight(dtype, n_in, n_out);
+    if (!aligned) {  // a part that starts inside a tile goes through the row copier
+        rmi_hip_weight *acc = nullptr;
+        for (int i = 0; i < n_parts; i++) {
+            rmi_hip_weight *w = rmi_upload_stack(dtype, parts + i, rows + i, 1, n_in);
+            rmi_hip_weight *f = w && acc ? rmi_hip_fuse_vstack(acc, w) : w;
+            if (acc) {
+                rmi_hip_free_weight(acc);
+                if (w) rmi_hip_free_weight(w);
+            }
+            if (!f) return nullptr;
+            acc = f;
+        }
+        return acc;
+    }
+    rmi_hip_weight *w = alloc_weight(dtype, n_in, uint32_t(total));
     if (!w) return nullptr;
-    if (want == 0) return w;
-    uint8_t *staging = nullptr;
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&staging), want);
-    if (e == hipSuccess) e = hipMemcpyAsync(staging, blocks, want, hipMemcpyHostToDevice, c->stream);
     int rc = RMI_HIP_OK;
-    if (e == hipSuccess)
-        rc = dtype == RMI_HIP_DTYPE_Q8_0   ? rmi_launch_repack_q8_0(staging, w, c->stream)
-             : dtype == RMI_HIP_DTYPE_Q4_0 ? rmi_launch_repack_q4_0(staging, w, c->stream)
-             : dtype == RMI_HIP_DTYPE_Q6_K ? rmi_launch_repack_q6_k(staging, w, c->stream)
-                                           : rmi_launch_repack_q4_k(staging, w, c->stream);
-    if (e == hipSuccess && rc == RMI_HIP_OK) e = hipStreamSynchronize(c->stream);
-    if (staging) hipFree(staging);
-    if (e != hipSuccess || rc != RMI_HIP_OK) {
-        if (e != hipSuccess) rmi_set_error("weight upload failed: %s", hipGetErrorString(e));
+    uint32_t row0 = 0;
+    for (int i = 0; i < n_parts && rc == RMI_HIP_OK; row0 += rows[i], i++)
+        rc = rmi_upload_rows(c, w, row0, parts[i], rows[i]);
+    if (rc == RMI_HIP_OK) {
+        hipError_t e = hipStreamSynchronize(c->stream);
+        if (e != hipSuccess) rc = rmi_fail(RMI_HIP_E_RUNTIME, "weight upload failed: %s", hipGetErrorString(e));
+    }
+    if (rc != RMI_HIP_OK) {
         rmi_hip_free_weight(w);
         return nullptr;
     }
     return w;
+}
+
+extern "C" {
+
+static rmi_hip_weight *upload(int dtype, const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {
+    const uint32_t block_elems = dtype == RMI_HIP_DTYPE_Q8_0 || dtype == RMI_HIP_DTYPE_Q4_0 ? 32 : 256;
+    if (n_in == 0 || n_in % block_elems != 0) {
+        rmi_set_error("n_in=%u is not a positive multiple of %u", n_in, block_elems);
+        return nullptr;
+    }
+    const size_t want = size_t(n_out) * row_bytes_of(dtype, n_in);
+    if (nbytes < want || (!blocks && want)) {
+        rmi_set_error("weight slice holds %zu bytes, %u x %u needs %zu", nbytes, n_out, n_in, want);
+        return nullptr;
+    }
+    return rmi_upload_stack(dtype, &blocks, &n_out, 1, n_in);
 }
 
 rmi_hip_weight *rmi_hip_upload_q8_0(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {
@@ -313,5 +449,6 @@ uint32_t rmi_hip_weight_n_in(const rmi_hip_weight *w) { return w ? w->n_in : 0; 
 uint32_t rmi_hip_weight_n_out(const rmi_hip_weight *w) { return w ? w->n_out : 0; }
 int rmi_hip_weight_dtype(const rmi_hip_weight *w) { return w ? w->dtype : 0; }
 size_t rmi_hip_weight_device_bytes(const rmi_hip_weight *w) { return w ? w->nbytes : 0; }
+const void *rmi_hip_weight_device_data(const rmi_hip_weight *w) { return w ? w->data : nullptr; }
 
 }  // extern "C"

@@ -60,6 +60,18 @@ class Qwen3Session:
         if not self._h:
             raise hip.RmiHipError(-1, hip.last_error())
 
+    @classmethod
+    def from_gguf(cls, loader, capacity, rounding=hip.ROUND_TIES_EVEN):
+        """Qwen3Model::from_source + Qwen3Session::new over an open ``loader.GGUFLoader``: tensor bytes go from
+        the file's mapping to HBM inside the library (src/models/qwen3.rs:262-349)."""
+        self = cls.__new__(cls)
+        self._h = None
+        self.config = loader.qwen3_config(capacity, rounding)
+        self._h = hip.lib.rmi_hip_qwen3_create_from_gguf(loader._h, int(capacity), rounding)
+        if not self._h:
+            raise hip.RmiHipError(-1, hip.last_error())
+        return self
+
     def generate(self, prompt, max_new, dump_steps=()):
         prompt = np.ascontiguousarray(prompt, np.uint32)
         steps = prompt.size + max_new - 1

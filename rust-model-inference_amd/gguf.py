@@ -11,8 +11,9 @@ import struct
 
 import numpy as np
 
-GGML_F32, GGML_F16, GGML_Q8_0, GGML_Q4_K = 0, 1, 8, 12
-_TYPE_TRAITS = {GGML_F32: (1, 4), GGML_F16: (1, 2), GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144)}
+GGML_F32, GGML_F16, GGML_Q4_0, GGML_Q8_0, GGML_Q4_K, GGML_Q6_K = 0, 1, 2, 8, 12, 14
+_TYPE_TRAITS = {GGML_F32: (1, 4), GGML_F16: (1, 2), GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144),
+                GGML_Q6_K: (256, 210)}
 # metadata value type tags (src/core/loader.rs MetaValueType)
 _U32, _I32, _F32, _BOOL, _STR, _ARR, _U64, _F64 = 4, 5, 6, 7, 8, 9, 10, 12
 ALIGNMENT = 32

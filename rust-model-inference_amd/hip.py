@@ -25,6 +25,7 @@ _i32p = C.POINTER(C.c_int32)
 _f32p = C.POINTER(C.c_float)
 _vp = C.c_void_p
 _u32 = C.c_uint32
+_u64 = C.c_uint64
 _sz = C.c_size_t
 
 _u32p = C.POINTER(C.c_uint32)
@@ -63,6 +64,7 @@ SIGNATURES = {
     "rmi_hip_weight_n_out": (_u32, [_vp]),
     "rmi_hip_weight_dtype": (C.c_int, [_vp]),
     "rmi_hip_weight_device_bytes": (_sz, [_vp]),
+    "rmi_hip_weight_device_data": (_vp, [_vp]),
     "rmi_hip_q8_0_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_matmul_q8_0_quantized_range": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32]),
     "rmi_hip_matmul_q8_0_quantized_batch": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32]),
@@ -117,6 +119,29 @@ SIGNATURES = {
     "rmi_hip_qwen3_destroy": (None, [_vp]),
     "rmi_hip_qwen3_generate": (C.c_int, [_vp, _u32p, _u32, _u32, _u32p, _u32p, _f32p, _u32p, _u32, _f32p,
                                          C.POINTER(C.c_double)]),
+    "rmi_hip_gguf_open": (_vp, [C.c_char_p]),
+    "rmi_hip_gguf_close": (None, [_vp]),
+    "rmi_hip_gguf_version": (_u32, [_vp]),
+    "rmi_hip_gguf_alignment": (_u64, [_vp]),
+    "rmi_hip_gguf_data_offset": (_u64, [_vp]),
+    "rmi_hip_gguf_n_tensors": (_u64, [_vp]),
+    "rmi_hip_gguf_n_kv": (_u64, [_vp]),
+    "rmi_hip_gguf_kv_key": (C.c_char_p, [_vp, _u64]),
+    "rmi_hip_gguf_meta_type": (C.c_int, [_vp, C.c_char_p]),
+    "rmi_hip_gguf_meta_u64": (C.c_int, [_vp, C.c_char_p, C.POINTER(_u64)]),
+    "rmi_hip_gguf_meta_f64": (C.c_int, [_vp, C.c_char_p, C.POINTER(C.c_double)]),
+    "rmi_hip_gguf_meta_bool": (C.c_int, [_vp, C.c_char_p, C.POINTER(C.c_int)]),
+    "rmi_hip_gguf_meta_str": (C.c_int64, [_vp, C.c_char_p, C.c_char_p, _sz]),
+    "rmi_hip_gguf_meta_array_len": (C.c_int64, [_vp, C.c_char_p, C.POINTER(C.c_int)]),
+    "rmi_hip_gguf_meta_array_u64": (C.c_int, [_vp, C.c_char_p, _u64, C.POINTER(_u64)]),
+    "rmi_hip_gguf_find_tensor": (C.c_int64, [_vp, C.c_char_p]),
+    "rmi_hip_gguf_tensor_info": (C.c_int, [_vp, _u64, C.POINTER(C.c_char_p), C.POINTER(_u32), C.POINTER(_u64), _u32,
+                                           C.POINTER(C.c_int), C.POINTER(_u64), C.POINTER(_u64)]),
+    "rmi_hip_gguf_tensor_data": (_vp, [_vp, _u64]),
+    "rmi_hip_gguf_upload": (_vp, [_vp, C.c_char_p]),
+    "rmi_hip_gguf_upload_stack": (_vp, [_vp, C.POINTER(C.c_char_p), C.c_int]),
+    "rmi_hip_gguf_qwen3_config": (C.c_int, [_vp, _u32, C.c_int, C.POINTER(Qwen3Config)]),
+    "rmi_hip_qwen3_create_from_gguf": (_vp, [_vp, _u32, C.c_int]),
     "rmi_hip_gemv_group_shape": (C.c_int, [_vp, C.POINTER(_u32), C.POINTER(_u32)]),
     "rmi_hip_gemv_group_destroy": (None, [_vp]),
     "rmi_hip_gemv_group_run_dev": (C.c_int, [_vp, _vp]),

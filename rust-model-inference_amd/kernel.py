@@ -352,14 +352,26 @@ class Layer:
 class QuantizedLinear(Layer):
     """src/core/model.rs:12-104: always reads its weight as Q4_K, ignores bias."""
 
-    def __init__(self, weight, bias, in_features, out_features, name):
-        self.kernel = Q4_KKernel(weight, in_features, out_features)
+    def __init__(self, weight, bias, in_features, out_features, name, _kernel=None):
+        self.kernel = _kernel if _kernel is not None else Q4_KKernel(weight, in_features, out_features)
         self.bias = bias
         self.in_features, self.out_features, self.layer_name = in_features, out_features, name
 
     @classmethod
     def from_weight_slice(cls, weight, bias, in_features, out_features, name):
         return cls(weight, bias, in_features, out_features, name)
+
+    @classmethod
+    def from_source(cls, source, weight_name, bias_name, in_features, out_features, name):
+        """src/core/model.rs:38-55 over a `loader.GGUFLoader`: None when the weight is not in the file.  The
+        bytes go from the file's mapping to HBM inside the library."""
+        info = source.tensor_info(weight_name)
+        if info is None:
+            return None
+        bias = source.tensor_data(bias_name) if bias_name else None
+        if info.ggml_type == GGML_TYPE_Q4_K and info.dims == (in_features, out_features):
+            return cls(None, bias, in_features, out_features, name, _kernel=source.kernel(weight_name))
+        return cls(source.tensor_data(weight_name), bias, in_features, out_features, name)
 
     def forward_dequant(self, input, output, scratch=None):
         x = as_f32(input)
