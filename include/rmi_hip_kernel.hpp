@@ -271,11 +271,89 @@ class QuantizedLinear : public Layer {
     std::string name_;
 };
 
+// GGUFLoader (src/core/loader.rs:187-372) over the library's parser: the TensorSource a model is built from,
+// plus the uploads that take a tensor from the file's mapping to HBM.
+class GGUFLoader {
+  public:
+    struct TensorInfo {  // src/core/tensor.rs:189-195
+        std::string name;
+        std::vector<uint64_t> dims;  // [columns, rows, ..]
+        int ggml_type;
+        uint64_t offset, nbytes;
+    };
+    // GGUFLoader::from_file; the message of a file the reference rejects is the reference's
+    static GGUFLoader from_file(const std::string &path) {
+        rmi_hip_gguf *g = rmi_hip_gguf_open(path.c_str());
+        if (!g) throw HipError(RMI_HIP_E_INVALID, rmi_hip_last_error());
+        return GGUFLoader(g);
+    }
+    GGUFLoader(GGUFLoader &&o) noexcept : g_(o.g_) { o.g_ = nullptr; }
+    GGUFLoader(const GGUFLoader &) = delete;
+    GGUFLoader &operator=(const GGUFLoader &) = delete;
+    ~GGUFLoader() { rmi_hip_gguf_close(g_); }
+
+    uint32_t version() const { return rmi_hip_gguf_version(g_); }
+    uint64_t alignment() const { return rmi_hip_gguf_alignment(g_); }
+    size_t data_offset() const { return size_t(rmi_hip_gguf_data_offset(g_)); }
+    size_t n_tensors() const { return size_t(rmi_hip_gguf_n_tensors(g_)); }
+    size_t n_kv() const { return size_t(rmi_hip_gguf_n_kv(g_)); }
+    // metadata(key).and_then(MetaValue::to_u64) and its siblings: false where the reference gives None
+    bool to_u64(const std::string &key, uint64_t *out) const { return rmi_hip_gguf_meta_u64(g_, key.c_str(), out) != 0; }
+    bool to_f64(const std::string &key, double *out) const { return rmi_hip_gguf_meta_f64(g_, key.c_str(), out) != 0; }
+    bool to_string_val(const std::string &key, std::string *out) const {
+        const int64_t n = rmi_hip_gguf_meta_str(g_, key.c_str(), nullptr, 0);
+        if (n < 0) return false;
+        out->assign(size_t(n) + 1, '\0');
+        rmi_hip_gguf_meta_str(g_, key.c_str(), &(*out)[0], size_t(n) + 1);
+        out->resize(size_t(n));
+        return true;
+    }
+    bool tensor_info(const std::string &name, TensorInfo *out) const {
+        const int64_t i = rmi_hip_gguf_find_tensor(g_, name.c_str());
+        if (i < 0) return false;
+        const char *nm;
+        uint32_t nd;
+        uint64_t dims[8];
+        check(rmi_hip_gguf_tensor_info(g_, uint64_t(i), &nm, &nd, dims, 8, &out->ggml_type, &out->offset, &out->nbytes));
+        out->name = nm;
+        out->dims.assign(dims, dims + nd);
+        return true;
+    }
+    // tensor_slice: the bytes in the mapping, valid while the loader lives; {nullptr, 0} for an unknown name
+    std::pair<const uint8_t *, size_t> tensor_slice(const std::string &name) const {
+        TensorInfo t;
+        if (!tensor_info(name, &t)) return {nullptr, 0};
+        return {rmi_hip_gguf_tensor_data(g_, uint64_t(rmi_hip_gguf_find_tensor(g_, name.c_str()))), size_t(t.nbytes)};
+    }
+    // one matrix, or several of one type and width stacked row-wise ([q ; k ; v]), as a weight in HBM
+    std::shared_ptr<DeviceWeight> upload_stack(const std::vector<std::string> &names) const {
+        std::vector<const char *> p;
+        for (const std::string &n : names) p.push_back(n.c_str());
+        return std::make_shared<DeviceWeight>(rmi_hip_gguf_upload_stack(g_, p.data(), int(p.size())));
+    }
+    std::shared_ptr<DeviceWeight> upload(const std::string &name) const { return upload_stack({name}); }
+    rmi_hip_qwen3_config qwen3_config(uint32_t capacity, int rounding = RMI_HIP_ROUND_TIES_EVEN) const {
+        rmi_hip_qwen3_config c;
+        check(rmi_hip_gguf_qwen3_config(g_, capacity, rounding, &c));
+        return c;
+    }
+    rmi_hip_gguf *get() const { return g_; }
+
+  private:
+    explicit GGUFLoader(rmi_hip_gguf *g) : g_(g) {}
+    rmi_hip_gguf *g_;
+};
+
 // Qwen3Session (src/models/qwen3.rs:581-1158) with the whole token step on the device.
 class Qwen3Session {
   public:
     Qwen3Session(const rmi_hip_qwen3_config &cfg, const rmi_hip_qwen3_weights &weights)
         : cfg_(cfg), h_(rmi_hip_qwen3_create(&cfg, &weights)) {
+        if (!h_) throw HipError(RMI_HIP_E_RUNTIME, rmi_hip_last_error());
+    }
+    // Qwen3Model::from_source + Qwen3Session::new over an open file: tensor bytes go from its mapping to HBM
+    Qwen3Session(const GGUFLoader &source, uint32_t capacity, int rounding = RMI_HIP_ROUND_TIES_EVEN)
+        : cfg_(source.qwen3_config(capacity, rounding)), h_(rmi_hip_qwen3_create_from_gguf(source.get(), capacity, rounding)) {
         if (!h_) throw HipError(RMI_HIP_E_RUNTIME, rmi_hip_last_error());
     }
     ~Qwen3Session() { rmi_hip_qwen3_destroy(h_); }

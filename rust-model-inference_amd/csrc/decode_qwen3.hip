@@ -760,7 +760,8 @@ float *upload_f32(rmi_hip_qwen3 *s, const float *host, size_t n) {
 }
 
 rmi_hip_weight *upload_stack(const uint8_t *const *parts, const uint32_t *rows, int n_parts, uint32_t n_in) {
-    return rmi_upload_stack(RMI_HIP_DTYPE_Q8_0, parts, rows, n_parts, n_in);
+    // the session's constructor waits once, after the last weight
+    return rmi_upload_stack(RMI_HIP_DTYPE_Q8_0, parts, rows, n_parts, n_in, false);
 }
 
 int gemv(const rmi_hip_weight *w, const int8_t *q8, const float *scales, float *y, hipStream_t st) {
@@ -1077,6 +1078,10 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
          (s->step_top2 = dev_alloc<float>(s, size_t(2) * c.capacity, true)) &&
          (s->nonfinite = dev_alloc<uint32_t>(s, 1, true)) && (s->partial = dev_alloc<Top>(s, kArgmaxGroups)) &&
          (s->params = dev_alloc<StepParams>(s, 1, true));
+    if (ok && hipStreamSynchronize(rmi_thread_ctx()->stream) != hipSuccess) {  // the uploads enqueued above
+        rmi_set_error("weight upload failed");
+        ok = false;
+    }
     if (!ok) {
         rmi_hip_qwen3_destroy(s);
         return nullptr;

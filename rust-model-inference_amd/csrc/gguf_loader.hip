@@ -554,7 +554,7 @@ rmi_hip_weight *rmi_hip_gguf_upload_stack(const rmi_hip_gguf *g, const char *con
         parts[i] = g->bytes(*t);
         rows[i] = uint32_t(t->dims[1]);
     }
-    return rmi_upload_stack(dtype, parts, rows, n_names, uint32_t(n_in));
+    return rmi_upload_stack(dtype, parts, rows, n_names, uint32_t(n_in), true);
 }
 
 rmi_hip_weight *rmi_hip_gguf_upload(const rmi_hip_gguf *g, const char *name) {

@@ -120,9 +120,12 @@ int rmi_launch_repack_q4_0(const uint8_t *src, rmi_hip_weight *w, uint32_t tile0
 // Host rows -> the tile stream of w from row0 (a multiple of 8) on, chunk by chunk through the thread's staging
 // pair; enqueues on c->stream and returns without waiting for the last chunk.
 int rmi_upload_rows(RmiThreadCtx *c, rmi_hip_weight *w, uint32_t row0, const uint8_t *blocks, uint32_t n_rows);
-// One weight whose rows are the parts one below the other ([a ; b ; c]); synchronises.  NULL + error text on failure.
+// One weight whose rows are the parts one below the other ([a ; b ; c]).  NULL + error text on failure.  With
+// wait = false the last chunks may still be in flight on the calling thread's stream when it returns (the
+// source bytes are already in the staging pair): the caller synchronises that stream before any other
+// stream reads the weight.
 rmi_hip_weight *rmi_upload_stack(int dtype, const uint8_t *const *parts, const uint32_t *rows, int n_parts,
-                                 uint32_t n_in);
+                                 uint32_t n_in, bool wait);
 int rmi_launch_copy_rows(const rmi_hip_weight *src, rmi_hip_weight *dst, uint32_t dst_row0, hipStream_t s);
 
 struct RmiGemvProblem {

@@ -315,7 +315,7 @@ int rmi_upload_rows(RmiThreadCtx *c, rmi_hip_weight *w, uint32_t row0, const uin
 }
 
 rmi_hip_weight *rmi_upload_stack(int dtype, const uint8_t *const *parts, const uint32_t *rows, int n_parts,
-                                 uint32_t n_in) {
+                                 uint32_t n_in, bool wait) {
     if (!rmi_ready()) {
         rmi_set_error("rmi_hip_init has not succeeded");
         return nullptr;
@@ -348,7 +348,7 @@ rmi_hip_weight *rmi_upload_stack(int dtype, const uint8_t *const *parts, const u
     if (!aligned) {  // a part that starts inside a tile goes through the row copier
         rmi_hip_weight *acc = nullptr;
         for (int i = 0; i < n_parts; i++) {
-            rmi_hip_weight *w = rmi_upload_stack(dtype, parts + i, rows + i, 1, n_in);
+            rmi_hip_weight *w = rmi_upload_stack(dtype, parts + i, rows + i, 1, n_in, true);
             rmi_hip_weight *f = w && acc ? rmi_hip_fuse_vstack(acc, w) : w;
             if (acc) {
                 rmi_hip_free_weight(acc);
@@ -365,7 +365,7 @@ rmi_hip_weight *rmi_upload_stack(int dtype, const uint8_t *const *parts, const u
     uint32_t row0 = 0;
     for (int i = 0; i < n_parts && rc == RMI_HIP_OK; row0 += rows[i], i++)
         rc = rmi_upload_rows(c, w, row0, parts[i], rows[i]);
-    if (rc == RMI_HIP_OK) {
+    if (rc == RMI_HIP_OK && wait) {
         hipError_t e = hipStreamSynchronize(c->stream);
         if (e != hipSuccess) rc = rmi_fail(RMI_HIP_E_RUNTIME, "weight upload failed: %s", hipGetErrorString(e));
     }
@@ -389,7 +389,7 @@ static rmi_hip_weight *upload(int dtype, const uint8_t *blocks, size_t nbytes, u
         rmi_set_error("weight slice holds %zu bytes, %u x %u needs %zu", nbytes, n_out, n_in, want);
         return nullptr;
     }
-    return rmi_upload_stack(dtype, &blocks, &n_out, 1, n_in);
+    return rmi_upload_stack(dtype, &blocks, &n_out, 1, n_in, true);
 }
 
 rmi_hip_weight *rmi_hip_upload_q8_0(const uint8_t *blocks, size_t nbytes, uint32_t n_in, uint32_t n_out) {

@@ -262,6 +262,67 @@ extern "C" {
                               dump_logits: *mut f32, seconds: *mut f64) -> c_int;
 }
 
+extern "C" {
+    fn rmi_hip_gguf_open(path: *const std::os::raw::c_char) -> *mut c_void;
+    fn rmi_hip_gguf_close(g: *mut c_void);
+    fn rmi_hip_gguf_meta_u64(g: *const c_void, key: *const std::os::raw::c_char, out: *mut u64) -> c_int;
+    fn rmi_hip_gguf_meta_f64(g: *const c_void, key: *const std::os::raw::c_char, out: *mut f64) -> c_int;
+    fn rmi_hip_gguf_upload_stack(g: *const c_void, names: *const *const std::os::raw::c_char, n: c_int)
+                                 -> *mut RmiHipWeight;
+    fn rmi_hip_weight_dtype(w: *const RmiHipWeight) -> c_int;
+    fn rmi_hip_qwen3_create_from_gguf(g: *const c_void, capacity: u32, rounding: c_int) -> *mut c_void;
+}
+
+/// The file as the library maps and parses it (`GGUFLoader::from_file`, src/core/loader.rs:211-320, with the
+/// reference's error messages).  A crate that keeps its own `GGUFLoader` for tokenizer metadata opens this one
+/// next to it for the weights: tensor bytes then go from the page cache to HBM without passing through a slice.
+pub struct HipGguf { handle: *mut c_void }
+unsafe impl Send for HipGguf {}
+
+impl HipGguf {
+    pub fn from_file(path: &str) -> Result<Self, String> {
+        let c = std::ffi::CString::new(path).map_err(|e| e.to_string())?;
+        let handle = unsafe { rmi_hip_gguf_open(c.as_ptr()) };
+        if handle.is_null() { Err(last_error()) } else { Ok(Self { handle }) }
+    }
+    /// `metadata(key).and_then(MetaValue::to_u64)`
+    pub fn to_u64(&self, key: &str) -> Option<u64> {
+        let c = std::ffi::CString::new(key).ok()?;
+        let mut v = 0u64;
+        if unsafe { rmi_hip_gguf_meta_u64(self.handle, c.as_ptr(), &mut v) } != 0 { Some(v) } else { None }
+    }
+    /// `metadata(key).and_then(MetaValue::to_f64)`
+    pub fn to_f64(&self, key: &str) -> Option<f64> {
+        let c = std::ffi::CString::new(key).ok()?;
+        let mut v = 0f64;
+        if unsafe { rmi_hip_gguf_meta_f64(self.handle, c.as_ptr(), &mut v) } != 0 { Some(v) } else { None }
+    }
+    /// One matrix of the file, or several stacked row-wise (`[q ; k ; v]`, `[gate ; up]`), as a kernel in HBM.
+    pub fn kernel(&self, names: &[&str]) -> Result<HipKernel, String> {
+        let owned: Vec<std::ffi::CString> =
+            names.iter().map(|n| std::ffi::CString::new(*n).map_err(|e| e.to_string())).collect::<Result<_, _>>()?;
+        let ptrs: Vec<*const std::os::raw::c_char> = owned.iter().map(|c| c.as_ptr()).collect();
+        let h = unsafe { rmi_hip_gguf_upload_stack(self.handle, ptrs.as_ptr(), ptrs.len() as c_int) };
+        if h.is_null() { return Err(last_error()); }
+        let dtype = match unsafe { rmi_hip_weight_dtype(h) } {
+            2 => Dtype::Q4_0,
+            8 => Dtype::Q8_0,
+            12 => Dtype::Q4K,
+            _ => Dtype::Q6K,
+        };
+        Ok(HipKernel { handle: h, dtype })
+    }
+    /// `Qwen3Model::from_source` + `Qwen3Session::new` (src/models/qwen3.rs:262-349) on the device.
+    pub fn qwen3_session(&self, capacity: usize) -> Result<HipQwen3Session, String> {
+        let handle = unsafe { rmi_hip_qwen3_create_from_gguf(self.handle, capacity as u32, 1) };
+        if handle.is_null() { Err(last_error()) } else { Ok(HipQwen3Session { handle }) }
+    }
+}
+
+impl Drop for HipGguf {
+    fn drop(&mut self) { unsafe { rmi_hip_gguf_close(self.handle) } }
+}
+
 /// Owns the HBM copy of a model and its KV cache.  Built from the tensors `Qwen3Model::from_gguf`
 /// (src/models/qwen3.rs:263-420) borrows from the mmap; the slices may be dropped after `new`.
 pub struct HipQwen3Session { handle: *mut c_void }

@@ -2,10 +2,15 @@
 // Layer interface) on a GPU.  The cases are the reference's own unit tests:
 // src/ops/kernel/q8_0/mod.rs:74-156 (closed forms, thread partition),
 // tests/quantized_inference.rs:233-263 (Q4_K and Q6_K uniform blocks), plus eight
-// std::threads calling one kernel at once, as pool.compute does.
+// std::threads calling one kernel at once, as pool.compute does, and a GGUF file written here and
+// read through GGUFLoader (src/core/loader.rs:846-889 in miniature).
+#include <unistd.h>
+
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <string>
 #include <thread>
 #include <vector>
 
@@ -191,6 +196,73 @@ int main() {
             threw = e.code == RMI_HIP_E_INVALID;
         }
         EXPECT(threw);
+    }
+    {
+        // GGUFLoader over a file written here: one u32 key, one 32 x 4 Q8_0 tensor of ones (the closed form above),
+        // read back through the mapping and uploaded from it
+        std::string b = "GGUF";
+        auto put = [&b](const void *p, size_t n) { b.append(static_cast<const char *>(p), n); };
+        auto put_str = [&](const std::string &t) {
+            const uint64_t n = t.size();
+            put(&n, 8);
+            b += t;
+        };
+        const uint32_t version = 3, u32_tag = 4, n_dims = 2, ctx = 4096;
+        const uint64_t n_tensors = 1, n_kv = 1, dims[2] = {32, 4}, offset = 0;
+        const int32_t q8_0 = 8;
+        put(&version, 4), put(&n_tensors, 8), put(&n_kv, 8);
+        put_str("qwen3.context_length"), put(&u32_tag, 4), put(&ctx, 4);
+        put_str("blk.0.attn_q.weight"), put(&n_dims, 4), put(dims, 16), put(&q8_0, 4), put(&offset, 8);
+        b.resize((b.size() + 31) / 32 * 32, '\0');
+        for (int r = 0; r < 4; r++) {
+            auto row = q8_0_uniform_row(1, one);
+            b.append(reinterpret_cast<const char *>(row.data()), row.size());
+        }
+        char path[] = "/tmp/rmi_hip_cpp_XXXXXX";
+        const int fd = mkstemp(path);
+        EXPECT(fd >= 0 && write(fd, b.data(), b.size()) == ssize_t(b.size()));
+        close(fd);
+        {
+            rmi::GGUFLoader g = rmi::GGUFLoader::from_file(path);
+            uint64_t v = 0;
+            double f = 0;
+            std::string sv;
+            EXPECT(g.version() == 3 && g.alignment() == 32 && g.n_tensors() == 1 && g.n_kv() == 1);
+            EXPECT(g.to_u64("qwen3.context_length", &v) && v == 4096 && g.to_f64("qwen3.context_length", &f) && f == 4096.0);
+            EXPECT(!g.to_u64("absent", &v) && !g.to_string_val("qwen3.context_length", &sv));
+            rmi::GGUFLoader::TensorInfo t;
+            EXPECT(g.tensor_info("blk.0.attn_q.weight", &t) && t.dims == std::vector<uint64_t>({32, 4}) &&
+                   t.ggml_type == 8 && t.nbytes == 136);
+            auto slice = g.tensor_slice("blk.0.attn_q.weight");
+            EXPECT(slice.second == 136 && slice.first[2] == 1 && g.tensor_slice("absent").first == nullptr);
+            rmi::Q8Kernel k(g.upload("blk.0.attn_q.weight"));
+            float out[4] = {0, 0, 0, 0};
+            k.forward_prequantized(ones_q.data(), &one_s, out, 32, 4, 0, 1);
+            EXPECT(out[0] == 32 && out[1] == 32 && out[2] == 32 && out[3] == 32);
+            rmi::Q8Kernel k2(g.upload_stack({"blk.0.attn_q.weight", "blk.0.attn_q.weight"}));
+            float out8[8] = {0};
+            k2.forward_prequantized(ones_q.data(), &one_s, out8, 32, 8, 0, 1);
+            EXPECT(out8[0] == 32 && out8[7] == 32);
+            bool threw = false;
+            try {
+                g.upload("absent");
+            } catch (const rmi::HipError &e) {
+                threw = std::strstr(e.what(), "Missing tensor: absent") != nullptr;
+            }
+            EXPECT(threw);
+        }
+        b[3] = 'L';
+        FILE *fp = std::fopen(path, "wb");
+        std::fwrite(b.data(), 1, b.size(), fp);
+        std::fclose(fp);
+        bool threw = false;
+        try {
+            rmi::GGUFLoader::from_file(path);
+        } catch (const rmi::HipError &e) {
+            threw = std::strstr(e.what(), "Invalid GGUF magic") != nullptr;
+        }
+        EXPECT(threw);
+        std::remove(path);
     }
     std::printf(failures ? "%d FAILED\n" : "all C++ interface checks passed\n", failures);
     return failures ? 1 : 0;
