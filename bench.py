@@ -499,15 +499,16 @@ def run_kquant(args, pkg, ev, fmt):
 
 
 def run_q4_0(args, pkg, ev):
-    """Q4_0 x Q8_0 decode GEMV, one large matrix per launch so that the launch streams from HBM: eight distinct
-    151936 x 1024 matrices (the lm_head shape, 87.5 MB each as Q4_0) taken in turn."""
+    """Q4_0 x Q8_0 decode GEMV at the 1.7B-class FFN shapes of the Q4_K / Q6_K workloads (gate/up 6144x2048, down
+    2048x6144), 28 layers of distinct weights (595 MB) so that every step streams from HBM; one grouped launch, or
+    one per matrix with --mode per_matmul."""
     H, synth, K = pkg.hip, pkg.synth, pkg.kernel
     dev_name, cus, hbm = H.device_info()
-    batch, n_out, n_in, n_mats = args.batch, 151936, 1024, 8
-    base = synth.q4_0_weight(synth.seed_for(5, 0), n_out, n_in)
+    batch = args.batch
     recs = []
-    for i in range(n_mats):
-        w = np.roll(base, 18 * 1024 * i)  # distinct bytes per matrix, one generator pass
+    shapes = [(6144, 2048), (6144, 2048), (2048, 6144)] * 28
+    for i, (n_out, n_in) in enumerate(shapes):
+        w = synth.q4_0_weight(synth.seed_for(5, i), n_out, n_in)
         x = synth.activations(synth.seed_for(5, 0x8000 + i), batch, n_in)
         k = K.Q4_0Kernel(w, n_in, n_out)
         d_x = H.DeviceBuffer.from_array(x)
@@ -515,48 +516,62 @@ def run_q4_0(args, pkg, ev):
         H.check(H.lib.rmi_hip_quantize_q8_0_dev(d_x.ptr, d_q.ptr, d_s.ptr, batch, n_in, H.ROUND_TIES_EVEN, None))
         H.check(H.lib.rmi_hip_synchronize())
         d_x.free()
-        recs.append(dict(w=w if not args.no_cpu_baseline else None, k=k, d_q=d_q, d_s=d_s, d_y=d_y))
+        recs.append(dict(w=w if not args.no_cpu_baseline else None, k=k, d_q=d_q, d_s=d_s, d_y=d_y, n_out=n_out, n_in=n_in))
 
-    def step():
+    n = len(recs)
+    arr = lambda vals: (C.c_void_p * n)(*vals)  # noqa: E731
+    group = H.lib.rmi_hip_gemv_group_create(n, arr([r["k"].w.handle for r in recs]), arr([r["d_q"].ptr for r in recs]),
+                                            arr([r["d_s"].ptr for r in recs]), arr([r["d_y"].ptr for r in recs]), batch)
+    if not group:
+        raise RuntimeError(H.last_error())
+
+    def step_per_matmul():
         for r in recs:
-            H.check(H.lib.rmi_hip_gemv_q4_0_dev(r["k"].w.handle, r["d_q"].ptr, r["d_s"].ptr, r["d_y"].ptr, batch, n_out, 0,
-                                                n_out, None))
+            H.check(H.lib.rmi_hip_gemv_q4_0_dev(r["k"].w.handle, r["d_q"].ptr, r["d_s"].ptr, r["d_y"].ptr, batch, r["n_out"],
+                                                0, r["n_out"], None))
 
+    def step_grouped():
+        H.check(H.lib.rmi_hip_gemv_group_run_dev(group, None))
+
+    grouped = args.mode != "per_matmul"
+    step = step_grouped if grouped else step_per_matmul
+    launches = 1 if grouped else n
     copy_calibration(H, args)
     wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
-    alg = n_mats * synth.q4_0_gemv_bytes(n_out, n_in, batch)
+    alg = sum(synth.q4_0_gemv_bytes(r["n_out"], r["n_in"], batch) for r in recs)
     achieved = alg / (dev_ms * 1e-3) / 1e9
-    result = base_result(args, "Q4_0 x Q8_0 GEMV HBM GB/s, lm_head shape, 1 GPU", "GB/s", round(alg / wall / 1e9, 1), wall,
-                         "int8 dot4 -> f32", {
-        "workload": f"Q4_0 GEMV, {n_mats} distinct matrices {n_out} x {n_in}, decode batch {batch}, one launch per matrix",
-        "batch": batch, "launches_per_step": n_mats, "algorithmic_bytes_per_step": alg, "device": dev_name.strip(),
+    result = base_result(args, "Q4_0 x Q8_0 GEMV HBM GB/s, 1.7B-class FFN shapes, 1 GPU", "GB/s", round(alg / wall / 1e9, 1),
+                         wall, "int8 dot4 -> f32", {
+        "workload": f"Q4_0 GEMV, 28 layers x (gate 6144x2048, up 6144x2048, down 2048x6144), decode batch {batch}, "
+                    + ("one grouped launch" if grouped else "one launch per matrix"), "batch": batch,
+        "launches_per_step": launches, "algorithmic_bytes_per_step": alg, "device": dev_name.strip(),
         "compute_units": cus})
-    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_0_kernel<{batch},*>", "achieved": round(achieved, 1),
-                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                          "avg_launch_us": round(dev_ms * 1e3 / n_mats, 3),
-                          "traffic": read_traffic("gemv_q4_0_lm_head") if batch == 1 else None}
+    result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_0_kernel<{batch},{'true' if grouped else 'false'},{group_maxt(H, group) if grouped else '*'}>",
+                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
+                          "traffic": read_traffic("gemv_q4_0_grouped_1.7b_ffn") if grouped and batch == 1 else None}
     if not args.no_cpu_baseline and batch == 1:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
         if oracle.have_avx2():
             cores = min(16, physical_cores())
             pool = oracle.Pool(cores)
-            host = [(r["d_q"].to_array(np.uint8, (n_in,)), r["d_s"].to_array(np.float32, (n_in // 32,)),
-                     np.zeros(n_out, np.float32)) for r in recs]
+            host = [(r["d_q"].to_array(np.uint8, (r["n_in"],)), r["d_s"].to_array(np.float32, (r["n_in"] // 32,)),
+                     np.zeros(r["n_out"], np.float32)) for r in recs]
             samples = []
             for it in range(6):
                 t0 = time.perf_counter()
                 for r, (q, sc, out) in zip(recs, host):
-                    pool.matmul_q4_0(r["w"], q, sc, out, n_in, n_out)
+                    pool.matmul_q4_0(r["w"], q, sc, out, r["n_in"], r["n_out"])
                 samples.append(time.perf_counter() - t0)
             pool.close()
             med = statistics.median(samples[1:])
             step()
             H.check(H.lib.rmi_hip_synchronize())
-            worst = max(int(np.count_nonzero(r["d_y"].to_array(np.float32, (n_out,)).view(np.uint32) != out.view(np.uint32)))
-                        for r, (_, _, out) in zip(recs, host))
+            worst = max(int(np.count_nonzero(r["d_y"].to_array(np.float32, (r["n_out"],)).view(np.uint32)
+                                             != out.view(np.uint32))) for r, (_, _, out) in zip(recs, host))
             result["cpu_baseline"] = {"value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
-                                      "sample": f"5 full steps ({n_mats} GEMVs, {alg / 1e6:.0f} MB), restated AVX2 "
+                                      "sample": f"5 full steps (84 GEMVs, {alg / 1e6:.0f} MB), restated AVX2 "
                                                 f"matmul_q4_0_vs_q8_0 over {cores} threads, median",
                                       "gpu_outputs_differing_from_cpu": worst}
     return result

@@ -219,7 +219,9 @@ int rmi_hip_quantize_row_q8_k_dev(const float *x, float *d, int8_t *qs, int16_t 
 /* A fixed list of independent Q8_0 GEMVs (a token-step's projection set, or
  * the q/k/v and gate/up pairs that share an input) run as ONE launch.  The
  * reference issues them one after another inside one pool.compute closure
- * (src/models/qwen3.rs:738-774, 991-1019). */
+ * (src/models/qwen3.rs:738-774, 991-1019).  The weights are all Q8_0 or all
+ * Q4_0 (src/ops/kernel/q4_0/mod.rs:33-84 per problem); both take Q8_0
+ * activations. */
 typedef struct rmi_hip_gemv_group rmi_hip_gemv_group;
 rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip_weight *const *weights,
                                               const int8_t *const *x_q8, const float *const *x_scales,

@@ -296,13 +296,16 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
     if (!rmi_thread_ctx()) return nullptr;
     std::vector<RmiGemvProblem> list(n_problems);
     rmi_hip_gemv_group *g = new rmi_hip_gemv_group();
-    g->dtype = RMI_HIP_DTYPE_Q8_0;
+    // Q8_0 weights, or Q4_0 weights (the same Q8_0 activations); one type per group
+    g->dtype = weights[0] && weights[0]->dtype == RMI_HIP_DTYPE_Q4_0 ? RMI_HIP_DTYPE_Q4_0 : RMI_HIP_DTYPE_Q8_0;
+    const size_t oct_bytes = g->dtype == RMI_HIP_DTYPE_Q4_0 ? kQ40OctetBytes : kOctetBytes;
+    const size_t lds_per_oct = g->dtype == RMI_HIP_DTYPE_Q4_0 ? 320 : 288;  // staged activation, per token and octet
     g->n_problems = n_problems;
     g->n_tokens = n_tokens;
     uint64_t total_tiles = 0;
     for (uint32_t i = 0; i < n_problems; i++) {
         const rmi_hip_weight *w = weights[i];
-        if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0 || !x_q8[i] || !x_scales[i] || !y[i]) {
+        if (!w || w->dtype != g->dtype || !x_q8[i] || !x_scales[i] || !y[i]) {
             rmi_set_error("gemv group problem %u: bad weight handle or null pointer", i);
             delete g;
             return nullptr;
@@ -311,7 +314,7 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
         total_tiles += list[i].n_tiles;
         if (w->n_units > g->max_units) g->max_units = w->n_units;
     }
-    if (total_tiles > 0x7fffffffull || size_t(n_tokens) * g->max_units * 288 > 64 * 1024) {
+    if (total_tiles > 0x7fffffffull || size_t(n_tokens) * g->max_units * lds_per_oct > 64 * 1024) {
         rmi_set_error("gemv group too large (%llu tiles, %u tokens x %u octets)", (unsigned long long)total_tiles,
                       n_tokens, g->max_units);
         delete g;
@@ -319,8 +322,8 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
     }
     // one run of consecutive tiles per wave, never across two matrices; the waves of a workgroup share a matrix
     g->wpg = rmi_gemv_waves_per_group(
-        size_t(n_tokens) * g->max_units * 288,
-        size_t(rmi_gemv_tiles_per_wave(g->max_units, uint32_t(total_tiles), n_tokens)) * g->max_units * kOctetBytes);
+        size_t(n_tokens) * g->max_units * lds_per_oct,
+        size_t(rmi_gemv_tiles_per_wave(g->max_units, uint32_t(total_tiles), n_tokens)) * g->max_units * oct_bytes);
     std::vector<uint4> runs;
     for (uint32_t i = 0; i < n_problems; i++) {
         if (list[i].n_oct == 0) continue;
@@ -368,6 +371,9 @@ int rmi_hip_gemv_group_run_dev(const rmi_hip_gemv_group *g, void *stream) {
                                           g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
     if (g->dtype == RMI_HIP_DTYPE_Q4_K)
         return rmi_launch_gemv_q4_k_group(static_cast<const RmiQ4kProblem *>(g->d_list), g->d_runs, g->n_runs,
+                                          g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
+    if (g->dtype == RMI_HIP_DTYPE_Q4_0)
+        return rmi_launch_gemv_q4_0_group(static_cast<const RmiGemvProblem *>(g->d_list), g->d_runs, g->n_runs,
                                           g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));
     return rmi_launch_gemv_q8_0_group(static_cast<const RmiGemvProblem *>(g->d_list), g->d_runs, g->n_runs,
                                       g->wpg, g->max_units, g->n_tokens, static_cast<hipStream_t>(stream));

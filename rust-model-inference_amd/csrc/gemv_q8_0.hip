@@ -10,6 +10,8 @@
 #include "device_quant.h"
 #include "rmi_internal.h"
 
+#include "device_run_ring.h"
+
 namespace {
 
 __device__ __forceinline__ float h2f(uint32_t bits16) {
@@ -140,8 +142,10 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
                                                         const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
     extern __shared__ uint4 lds[];
     const uint32_t lane = threadIdx.x & 63, r = lane >> 3, L = lane & 7;
-    // run of this wave; the waves of a workgroup always work on the same matrix and share its activation
-    const uint32_t w_idx = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    // run of this wave; the waves of a workgroup always work on the same matrix and share its activation.
+    // The index is the same for all lanes, and said so: the problem's fields, the octet counter and the
+    // addresses of the walk then live in scalar registers.
+    const uint32_t w_idx = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
 
     RmiGemvProblem p;
     uint32_t k, k_end;
@@ -158,13 +162,35 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
 
     const uint32_t n_oct = p.n_oct;
     const uint32_t tok_u4 = n_oct * 18;  // per token: 16 uint4 of quants + 2 of scales per octet
-    // The weight loads of the first tile go out before the activation is staged: the two round trips overlap.
-    OctetRegs ra, rb, rc, rd;
-    if (k < k_end) {
-        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * n_oct * kOctetBytes);
-        load_octet(ra, tile + r, tile + n_oct * 8 + lane, 0);
-        if (n_oct > 1) load_octet(rb, tile + r, tile + n_oct * 8 + lane, 1);
+    // Units of the run (device_run_ring.h): one octet of one tile.  A tile holds its n_oct scale pieces (128
+    // bytes each) before its n_oct quant pieces (2048 bytes each), so the two addresses of a unit move apart
+    // within a tile and jump at its end.  The first four units' loads go out before the activation is staged.
+    const uint32_t n_units = (k_end - k) * n_oct;
+    struct Cursor {
+        gptr_u4 sc_unit, q_unit;  // the same for all lanes
+        uint32_t o, n_oct, r, lane;
+        __device__ __forceinline__ void load(OctetRegs &g) const {
+            g.sc = sc_unit[r];
+            g.qa = __builtin_nontemporal_load(q_unit + lane);  // weights are read once: do not keep them in cache
+            g.qb = __builtin_nontemporal_load(q_unit + 64 + lane);
+        }
+        __device__ __forceinline__ void step() {
+            sc_unit += 8;
+            q_unit += 128;
+            if (++o == n_oct) {  // over this tile's quants / the next tile's scales
+                o = 0;
+                sc_unit += size_t(n_oct) * 128;
+                q_unit += size_t(n_oct) * 8;
+            }
+        }
+    } cur;
+    {
+        // a wave without tiles (padding of the last workgroup) prefetches from the matrix's first tile: in bounds, unused
+        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + (n_units ? k : 0)) * n_oct * kOctetBytes);
+        cur = Cursor{tile, tile + n_oct * 8, 0, n_oct, r, lane};
     }
+    RmiRing<OctetRegs> ring;
+    rmi_ring_fill(ring, n_units, cur);
     {
         const uint32_t nb = p.n_in >> 5;
         uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
@@ -174,41 +200,28 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
         __syncthreads();
     }
 
-    for (bool first = true; k < k_end; k++, first = false) {
-        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * n_oct * kOctetBytes);
-        gptr_u4 sc_ptr = tile + r;
-        gptr_u4 q_ptr = tile + n_oct * 8 + lane;
-
-        float acc[B];
+    float acc[B];
 #pragma unroll
-        for (int t = 0; t < B; t++) acc[t] = 0.0f;
-
-        // Software pipeline over the octets of the tile: while one pair of octets is
-        // multiplied, the loads of the next pair are in flight.  The accumulation
-        // order over blocks stays strictly ascending.
-        if (!first) {
-            load_octet(ra, sc_ptr, q_ptr, 0);
-            if (n_oct > 1) load_octet(rb, sc_ptr, q_ptr, 1);
-        }
-        for (uint32_t o = 0; o < n_oct; o += 4) {
-            if (o + 2 < n_oct) load_octet(rc, sc_ptr, q_ptr, o + 2);
-            if (o + 3 < n_oct) load_octet(rd, sc_ptr, q_ptr, o + 3);
-            octet_fma<B>(acc, ra, lds, tok_u4, n_oct, o, L);
-            if (o + 1 < n_oct) octet_fma<B>(acc, rb, lds, tok_u4, n_oct, o + 1, L);
-            if (o + 4 < n_oct) load_octet(ra, sc_ptr, q_ptr, o + 4);
-            if (o + 5 < n_oct) load_octet(rb, sc_ptr, q_ptr, o + 5);
-            if (o + 2 < n_oct) octet_fma<B>(acc, rc, lds, tok_u4, n_oct, o + 2, L);
-            if (o + 3 < n_oct) octet_fma<B>(acc, rd, lds, tok_u4, n_oct, o + 3, L);
-        }
-
-        const uint32_t row = (p.tile0 + k) * kTileRows + r;
-        gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    for (int t = 0; t < B; t++) acc[t] = 0.0f;
+    RmiRunResults<B> out{};
+    uint32_t o = 0;
+    gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    auto consume = [&](const OctetRegs &g) {
+        octet_fma<B>(acc, g, lds, tok_u4, n_oct, o, L);
+        if (++o == n_oct) {
+            float y[B];
 #pragma unroll
-        for (int t = 0; t < B; t++) {
-            const float y = hsum8_lanes(acc[t]);
-            if (L == 0 && row >= p.row_start && row < p.row_end) yp[size_t(t) * p.y_stride + row] = y;
+            for (int t = 0; t < B; t++) {
+                y[t] = hsum8_lanes(acc[t]);  // the same in the row's eight lanes
+                acc[t] = 0.0f;
+            }
+            o = 0;
+            out.keep(y, L);
+            if (out.group_full()) out.flush(yp, p.y_stride, p.tile0 + k, r, L, p.row_start, p.row_end);
         }
-    }
+    };
+    rmi_ring_walk(ring, n_units, cur, consume);
+    if (out.pending()) out.flush(yp, p.y_stride, p.tile0 + k, r, L, p.row_start, p.row_end);
 }
 
 // Launches too small to fill the chip (one token, a matrix of at most a few thousand tiles) are bound by
@@ -683,12 +696,13 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4 *__restrict__ src
 
 }  // namespace
 
-// Tiles a wave takes in one run: about 16 tile-octets (34 KiB of weights) at one
-// token and 8 per token of a batch, so that staging the activation (n_in bytes per token) stays
-// small against the weights read; fewer when the launch would otherwise have too
-// few waves to fill the chip.
+// Tiles a wave takes in one run: about 16 tile-octets (34 KiB of weights), whatever the batch, so that
+// staging the activation stays small against the weights read while the launch keeps many more runs than the
+// chip holds waves; fewer when the launch would otherwise have too few waves to fill the chip.  (Measured on
+// the Qwen3-0.6B set: 8..32 octets within 2 % of each other at one token, 16 best at 4 and 8 tokens.)
 uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles, uint32_t n_tokens) {
-    const uint32_t target = n_tokens > 1 ? 8 * n_tokens : 16;  // measured best: 16 at one token, 8 per token above
+    (void)n_tokens;
+    const uint32_t target = 16;
     uint32_t tpw = n_oct >= target ? 1 : target / (n_oct ? n_oct : 1);
     const uint32_t fill = uint32_t(rmi_device_cus()) * 8;
     while (tpw > 1 && launch_tiles / tpw < fill) tpw >>= 1;

@@ -7,6 +7,8 @@
 // chain per row: lane 0 of the row takes the products of lanes 0, 1, .. 7 in turn through lane shifts.
 #include "rmi_internal.h"
 
+#include "device_run_ring.h"
+
 namespace {
 
 __device__ __forceinline__ float h2f(uint32_t bits16) {
@@ -34,12 +36,6 @@ struct OctetRegs {
     uint32_t d;  // f16 scale of block 8o + L of the row
     u32x4 q;     // its 16 nibble bytes
 };
-
-__device__ __forceinline__ void load_octet(OctetRegs &g, gptr_u4 tile, uint32_t o, uint32_t lane) {
-    gptr_u4 chunk = tile + size_t(o) * (kQ40OctetBytes / 16);
-    g.d = ((gptr_u16)chunk)[lane];
-    g.q = __builtin_nontemporal_load(chunk + 8 + lane);  // weights are read once: do not keep them in cache
-}
 
 // LDS per token: n_oct * 8 blocks x 32 int8 in source order, then per block {f32 scale, int32 8 * sum of its q8}
 template <int B>
@@ -81,20 +77,44 @@ __device__ __forceinline__ void octet_fma(float (&acc)[B], const OctetRegs &g, c
     }
 }
 
-// Same launch shapes as the Q8_0 GEMV (gemv_q8_0.hip): a wave owns a run of consecutive 8-row tiles; up to
-// eight waves of a workgroup share one staged activation.
-template <int B, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemv_q4_0_kernel(RmiGemvProblem p, uint32_t tiles_per_wave) {
+// Same launch shapes as the Q8_0 GEMV (gemv_q8_0.hip): a wave owns a run of consecutive 8-row tiles and walks
+// it four octets deep (device_run_ring.h); up to eight waves of a workgroup share one staged activation.  GROUPED = false: one matrix (`single`), run w starts
+// at tile w * tiles_per_wave.  GROUPED = true: runs[w] = {problem index, first tile, tile count, -}.
+template <int B, bool GROUPED, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_q4_0_kernel(RmiGemvProblem single, const RmiGemvProblem *__restrict__ list,
+                                                        const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
     extern __shared__ uint4 lds[];
     const uint32_t lane = threadIdx.x & 63, r = lane >> 3, L = lane & 7;
-    const uint32_t w_idx = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    uint32_t k = w_idx * tiles_per_wave < p.n_tiles ? w_idx * tiles_per_wave : p.n_tiles;
-    const uint32_t k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
+    // wave-uniform, and said so: the problem's fields and the octet counter live in scalar registers
+    const uint32_t w_idx = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    RmiGemvProblem p;
+    uint32_t k, k_end;
+    if (GROUPED) {
+        const uint4 run = runs[w_idx];
+        p = list[run.x];
+        k = run.y;
+        k_end = run.y + run.z;
+    } else {
+        p = single;
+        k = w_idx * tiles_per_wave < p.n_tiles ? w_idx * tiles_per_wave : p.n_tiles;
+        k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
+    }
     const uint32_t n_oct = p.n_oct, nb = p.n_in >> 5;
     const uint32_t tok_u4 = n_oct * 20;  // per token: 16 uint4 of quants + 4 of {scale, 8 * sum} per octet
-    const size_t tile_u4 = size_t(n_oct) * (kQ40OctetBytes / 16);
-    OctetRegs ra, rb;
-    if (k < k_end) load_octet(ra, as_global<gptr_u4>(p.w) + size_t(p.tile0 + k) * tile_u4, 0, lane);
+    // units of the run (device_run_ring.h): one octet of one tile, 1152 bytes, tile after tile
+    const uint32_t n_units = (k_end - k) * n_oct;
+    struct Cursor {
+        gptr_u4 unit;  // the same for all lanes
+        uint32_t lane;
+        __device__ __forceinline__ void load(OctetRegs &g) const {
+            g.d = ((gptr_u16)unit)[lane];
+            g.q = __builtin_nontemporal_load(unit + 8 + lane);  // weights are read once: do not keep them in cache
+        }
+        __device__ __forceinline__ void step() { unit += kQ40OctetBytes / 16; }
+        // a wave without tiles (padding of the last workgroup) prefetches from the matrix's first tile: in bounds, unused
+    } cur{as_global<gptr_u4>(p.w) + size_t(p.tile0 + (n_units ? k : 0)) * n_oct * (kQ40OctetBytes / 16), lane};
+    RmiRing<OctetRegs> ring;
+    rmi_ring_fill(ring, n_units, cur);
     for (int t = 0; t < B; t++) {  // a thread stages whole blocks: two 16-byte loads, the sum, the scale
         uint4 *dst = lds + t * tok_u4;
         gptr_u4 xq = as_global<gptr_u4>(p.x_q8 + size_t(t) * p.n_in);
@@ -123,24 +143,28 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_0_kernel(RmiGemvProblem p, uint3
     }
     __syncthreads();
 
-    for (bool first = true; k < k_end; k++, first = false) {
-        gptr_u4 tile = as_global<gptr_u4>(p.w) + size_t(p.tile0 + k) * tile_u4;
-        float acc[B];
+    float acc[B];
 #pragma unroll
-        for (int t = 0; t < B; t++) acc[t] = 0.0f;
-        if (!first) load_octet(ra, tile, 0, lane);
-        for (uint32_t o = 0; o < n_oct; o += 2) {  // the next octet's loads are in flight while one is multiplied
-            if (o + 1 < n_oct) load_octet(rb, tile, o + 1, lane);
-            octet_fma<B>(acc, ra, lds, tok_u4, n_oct, o, L, nb);
-            if (o + 2 < n_oct) load_octet(ra, tile, o + 2, lane);
-            if (o + 1 < n_oct) octet_fma<B>(acc, rb, lds, tok_u4, n_oct, o + 1, L, nb);
+    for (int t = 0; t < B; t++) acc[t] = 0.0f;
+    RmiRunResults<B> out{};
+    uint32_t o = 0;
+    gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    auto consume = [&](const OctetRegs &g) {
+        octet_fma<B>(acc, g, lds, tok_u4, n_oct, o, L, nb);
+        if (++o == n_oct) {
+            float y[B];
+#pragma unroll
+            for (int t = 0; t < B; t++) {
+                y[t] = __shfl(acc[t], int(lane & ~7u), 64);  // the row's chain ends in its lane 0
+                acc[t] = 0.0f;
+            }
+            o = 0;
+            out.keep(y, L);
+            if (out.group_full()) out.flush(yp, p.y_stride, p.tile0 + k, r, L, p.row_start, p.row_end);
         }
-        const uint32_t row = (p.tile0 + k) * kTileRows + r;
-        gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
-#pragma unroll
-        for (int t = 0; t < B; t++)
-            if (L == 0 && row >= p.row_start && row < p.row_end) yp[size_t(t) * p.y_stride + row] = acc[t];
-    }
+    };
+    rmi_ring_walk(ring, n_units, cur, consume);
+    if (out.pending()) out.flush(yp, p.y_stride, p.tile0 + k, r, L, p.row_start, p.row_end);
 }
 
 // ---- per-block integer dots from the repacked stream
@@ -188,18 +212,40 @@ __global__ __launch_bounds__(256) void repack_q4_0_kernel(const uint8_t *__restr
 }
 
 template <int B>
-int launch_q4_0(const RmiGemvProblem &p, uint32_t n_waves, uint32_t wpg, uint32_t tpw, hipStream_t s) {
-    const size_t lds_bytes = size_t(B) * p.n_oct * 320;
+int launch_q4_0(const RmiGemvProblem *single, const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_waves,
+                uint32_t wpg, uint32_t tpw, uint32_t max_n_oct, hipStream_t s) {
+    const size_t lds_bytes = size_t(B) * max_n_oct * 320;
     if (lds_bytes > 64 * 1024)
         return rmi_fail(RMI_HIP_E_INVALID, "activation of %d tokens x %u elements does not fit the LDS staging", B,
-                        p.n_oct * 256);
+                        max_n_oct * 256);
+    if (n_waves == 0) return RMI_HIP_OK;
     const dim3 grid((n_waves + wpg - 1) / wpg), block(64 * wpg);
-    if (wpg == 1)
-        hipLaunchKernelGGL((gemv_q4_0_kernel<B, 64>), grid, block, lds_bytes, s, p, tpw);
+    if (single && wpg == 1)
+        hipLaunchKernelGGL((gemv_q4_0_kernel<B, false, 64>), grid, block, lds_bytes, s, *single, nullptr, nullptr, tpw);
+    else if (single)
+        hipLaunchKernelGGL((gemv_q4_0_kernel<B, false, 512>), grid, block, lds_bytes, s, *single, nullptr, nullptr, tpw);
+    else if (wpg == 1)
+        hipLaunchKernelGGL((gemv_q4_0_kernel<B, true, 64>), grid, block, lds_bytes, s, RmiGemvProblem{}, d_list, d_runs, tpw);
     else
-        hipLaunchKernelGGL((gemv_q4_0_kernel<B, 512>), grid, block, lds_bytes, s, p, tpw);
+        hipLaunchKernelGGL((gemv_q4_0_kernel<B, true, 512>), grid, block, lds_bytes, s, RmiGemvProblem{}, d_list, d_runs,
+                           tpw);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
+}
+
+int dispatch_q4_0(uint32_t n_tokens, const RmiGemvProblem *single, const RmiGemvProblem *d_list, const uint4 *d_runs,
+                  uint32_t n_waves, uint32_t wpg, uint32_t tpw, uint32_t max_n_oct, hipStream_t s) {
+    switch (n_tokens) {
+        case 1: return launch_q4_0<1>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_oct, s);
+        case 2: return launch_q4_0<2>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_oct, s);
+        case 3: return launch_q4_0<3>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_oct, s);
+        case 4: return launch_q4_0<4>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_oct, s);
+        case 5: return launch_q4_0<5>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_oct, s);
+        case 6: return launch_q4_0<6>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_oct, s);
+        case 7: return launch_q4_0<7>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_oct, s);
+        case 8: return launch_q4_0<8>(single, d_list, d_runs, n_waves, wpg, tpw, max_n_oct, s);
+        default: return rmi_fail(RMI_HIP_E_INVALID, "gemv takes 1..8 tokens per launch, got %u", n_tokens);
+    }
 }
 
 }  // namespace
@@ -208,18 +254,12 @@ int rmi_launch_gemv_q4_0(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t
     if (p.n_tiles == 0 || p.n_oct == 0) return RMI_HIP_OK;
     const uint32_t tpw = rmi_gemv_tiles_per_wave(p.n_oct, p.n_tiles, n_tokens);
     const uint32_t wpg = rmi_gemv_waves_per_group(size_t(n_tokens) * p.n_oct * 320, size_t(tpw) * p.n_oct * kQ40OctetBytes);
-    const uint32_t n_waves = (p.n_tiles + tpw - 1) / tpw;
-    switch (n_tokens) {
-        case 1: return launch_q4_0<1>(p, n_waves, wpg, tpw, s);
-        case 2: return launch_q4_0<2>(p, n_waves, wpg, tpw, s);
-        case 3: return launch_q4_0<3>(p, n_waves, wpg, tpw, s);
-        case 4: return launch_q4_0<4>(p, n_waves, wpg, tpw, s);
-        case 5: return launch_q4_0<5>(p, n_waves, wpg, tpw, s);
-        case 6: return launch_q4_0<6>(p, n_waves, wpg, tpw, s);
-        case 7: return launch_q4_0<7>(p, n_waves, wpg, tpw, s);
-        case 8: return launch_q4_0<8>(p, n_waves, wpg, tpw, s);
-        default: return rmi_fail(RMI_HIP_E_INVALID, "gemv takes 1..8 tokens per launch, got %u", n_tokens);
-    }
+    return dispatch_q4_0(n_tokens, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, wpg, tpw, p.n_oct, s);
+}
+
+int rmi_launch_gemv_q4_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,
+                               uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s) {
+    return dispatch_q4_0(n_tokens, nullptr, d_list, d_runs, n_runs, wpg, 0, max_n_oct, s);
 }
 
 int rmi_launch_block_dots_q4_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s) {

@@ -7,8 +7,10 @@
 // then acc_T = fma(d*q8d, float(sumi_T), acc_T)) and four min accumulators
 // (acc_m[t] = fma(-dmin*q8d, float(mn[2t]*s[2t] + mn[2t+1]*s[2t+1]), acc_m[t]));
 // result hsum(acc) + ((m0+m2)+(m1+m3)).  Eight GPU lanes per row hold them.
-#include "device_stage_q8k.h"
 #include "rmi_internal.h"
+
+#include "device_run_ring.h"
+#include "device_stage_q8k.h"
 
 namespace {
 
@@ -113,19 +115,15 @@ struct SuperRegs {
     u32x4 qv;   // dwords 32g+4T (g = 0..3) of the row's nibble bytes
 };
 
-__device__ __forceinline__ void load_super(SuperRegs &g, gptr_u4 tile, uint32_t sb, uint32_t r, uint32_t lane) {
-    gptr_u4 chunk = tile + size_t(sb) * (kQ4KSuperBytes / 16);
-    g.hdr = chunk[r];
-    g.qv = __builtin_nontemporal_load(chunk + 8 + lane);  // weights are read once: do not keep them in cache
-}
-
 template <int B>
 __device__ __forceinline__ void super_fma(float (&acc)[B], float (&acc_m)[B], const SuperRegs &g,
                                           const uint32_t *lds_dw, uint32_t n_sb, uint32_t sb, uint32_t T) {
     const float wd = h2f(g.hdr.x & 0xffffu), wdmin = h2f(g.hdr.x >> 16);
     const uint4 sm = unpack_scales(g.hdr.y, g.hdr.z, g.hdr.w);
     const uint32_t qd[4] = {g.qv.x, g.qv.y, g.qv.z, g.qv.w};
-    const int mn0 = int(byte_of(sm.z, sm.w, (2 * T) & 7)), mn1 = int(byte_of(sm.z, sm.w, (2 * T + 1) & 7));
+    // mins 2T and 2T+1 (mod 8) are neighbours in one dword of the unpacked eight
+    const uint32_t mn_dw = (T & 2) ? sm.w : sm.z;
+    const int mn0 = int(__builtin_amdgcn_ubfe(mn_dw, 16 * (T & 1), 8)), mn1 = int(__builtin_amdgcn_ubfe(mn_dw, 16 * (T & 1) + 8, 8));
 #pragma unroll
     for (int t = 0; t < B; t++) {
         const uint32_t *xs = lds_dw + (size_t(t) * n_sb + sb) * kSbDwords;
@@ -161,7 +159,9 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_kernel(RmiQ4kProblem single, c
                                                         const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
     extern __shared__ uint4 lds[];
     const uint32_t lane = threadIdx.x & 63, r = lane >> 3, T = lane & 7;
-    const uint32_t w_idx = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    // the same for all lanes of the wave: said so, the problem's fields, the super-block counter and the
+    // staged activation's offsets live in scalar registers and the tile-end test is a scalar branch
+    const uint32_t w_idx = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     RmiQ4kProblem p;
     uint32_t k, k_end;
     if (GROUPED) {
@@ -175,6 +175,21 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_kernel(RmiQ4kProblem single, c
         k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
     }
     const uint32_t n_sb = p.n_sb, n_in = n_sb * 256;
+    // units of the run (device_run_ring.h): one super-block of one tile, 1152 bytes, tile after tile
+    const uint32_t n_units = (k_end - k) * n_sb;
+    // a wave without tiles (padding of the last workgroup) prefetches from the matrix's first tile: in bounds, unused
+    gptr_u4 base = as_global<gptr_u4>(p.w + size_t(p.tile0 + (n_units ? k : 0)) * n_sb * kQ4KSuperBytes);
+    struct Cursor {
+        gptr_u4 unit;  // the same for all lanes
+        uint32_t r, lane;
+        __device__ __forceinline__ void load(SuperRegs &g) const {
+            g.hdr = unit[r];
+            g.qv = __builtin_nontemporal_load(unit + 8 + lane);  // weights are read once: not kept in cache
+        }
+        __device__ __forceinline__ void step() { unit += kQ4KSuperBytes / 16; }
+    } cur{base, r, lane};
+    RmiRing<SuperRegs> ring;
+    rmi_ring_fill(ring, n_units, cur);
     uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
     for (int t = 0; t < B; t++)
         rmi_stage_q8k_token<true, 2>(lds_dw + size_t(t) * n_sb * kSbDwords, p.q8qs + size_t(t) * n_in,
@@ -182,36 +197,32 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_kernel(RmiQ4kProblem single, c
                                      blockDim.x);
     __syncthreads();
 
-    for (; k < k_end; k++) {
-        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * n_sb * kQ4KSuperBytes);
-        float acc[B], acc_m[B];
+    float acc[B], acc_m[B];
 #pragma unroll
-        for (int t = 0; t < B; t++) acc[t] = acc_m[t] = 0.0f;
-        // software pipeline over super-blocks, two pairs deep; ascending order is kept
-        SuperRegs ra, rb, rc, rd;
-        load_super(ra, tile, 0, r, lane);
-        if (n_sb > 1) load_super(rb, tile, 1, r, lane);
-        for (uint32_t sb = 0; sb < n_sb; sb += 4) {
-            if (sb + 2 < n_sb) load_super(rc, tile, sb + 2, r, lane);
-            if (sb + 3 < n_sb) load_super(rd, tile, sb + 3, r, lane);
-            super_fma<B>(acc, acc_m, ra, lds_dw, n_sb, sb, T);
-            if (sb + 1 < n_sb) super_fma<B>(acc, acc_m, rb, lds_dw, n_sb, sb + 1, T);
-            if (sb + 4 < n_sb) load_super(ra, tile, sb + 4, r, lane);
-            if (sb + 5 < n_sb) load_super(rb, tile, sb + 5, r, lane);
-            if (sb + 2 < n_sb) super_fma<B>(acc, acc_m, rc, lds_dw, n_sb, sb + 2, T);
-            if (sb + 3 < n_sb) super_fma<B>(acc, acc_m, rd, lds_dw, n_sb, sb + 3, T);
-        }
-        const uint32_t row = (p.tile0 + k) * kTileRows + r;
-        gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    for (int t = 0; t < B; t++) acc[t] = acc_m[t] = 0.0f;
+    RmiRunResults<B> out{};
+    uint32_t sb = 0;
+    gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    auto consume = [&](const SuperRegs &g) {
+        super_fma<B>(acc, acc_m, g, lds_dw, n_sb, sb, T);
+        if (++sb == n_sb) {
+            float y[B];
 #pragma unroll
-        for (int t = 0; t < B; t++) {
-            const float main_val = hsum8_lanes(acc[t]);
-            float m = acc_m[t];  // lanes T<4 hold acc_m[T]
-            m = m + __shfl_xor(m, 2, 64);
-            m = m + __shfl_xor(m, 1, 64);
-            if (T == 0 && row >= p.row_start && row < p.row_end) yp[size_t(t) * p.y_stride + row] = main_val + m;
+            for (int t = 0; t < B; t++) {
+                const float main_val = hsum8_lanes(acc[t]);
+                float m = acc_m[t];  // lanes T and T + 4 hold the same acc_m
+                m = m + __shfl_xor(m, 2, 64);
+                m = m + __shfl_xor(m, 1, 64);
+                y[t] = main_val + m;  // the same in the row's eight lanes
+                acc[t] = acc_m[t] = 0.0f;
+            }
+            sb = 0;
+            out.keep(y, T);
+            if (out.group_full()) out.flush(yp, p.y_stride, p.tile0 + k, r, T, p.row_start, p.row_end);
         }
-    }
+    };
+    rmi_ring_walk(ring, n_units, cur, consume);
+    if (out.pending()) out.flush(yp, p.y_stride, p.tile0 + k, r, T, p.row_start, p.row_end);
 }
 
 // ---- exact integers per (row, super-block), read back from the repacked stream

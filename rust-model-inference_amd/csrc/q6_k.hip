@@ -8,8 +8,10 @@
 //   - 32 * (bsums[2m]*scale[2m] + bsums[2m+1]*scale[2m+1]),
 // then acc_m = fma(d*q8d, float(that), acc_m); result hsum(acc).  Eight GPU lanes
 // per row hold the eight accumulators.
-#include "device_stage_q8k.h"
 #include "rmi_internal.h"
+
+#include "device_run_ring.h"
+#include "device_stage_q8k.h"
 
 namespace {
 
@@ -56,14 +58,6 @@ struct SuperRegs {
     u32x4 ql;    // low nibbles: bytes 4m.. of ql[0..32), [32..64), [64..96), [96..128)
     u32x2 qh;    // high bit pairs: bytes 4m.. of qh[0..32), [32..64)
 };
-
-__device__ __forceinline__ void load_super(SuperRegs &g, gptr_u4 tile, uint32_t sb, uint32_t r, uint32_t lane) {
-    gptr_u4 chunk = tile + size_t(sb) * (kQ6KSuperBytes / 16);
-    g.sc = chunk[r];
-    g.d = ((gptr_u16)(chunk + 8))[r];
-    g.ql = __builtin_nontemporal_load(chunk + 9 + lane);  // weights are read once: do not keep them in cache
-    g.qh = __builtin_nontemporal_load((gptr_u2)(chunk + 73) + lane);
-}
 
 // the eight groups' unsigned 6-bit quants (4 per dword) of one lane
 __device__ __forceinline__ void unpack_q6(const SuperRegs &g, uint32_t (&q)[8]) {
@@ -113,13 +107,15 @@ __device__ __forceinline__ void super_fma(float (&acc)[B], const SuperRegs &g, c
 }
 
 // Same launch shapes as the Q4_K GEMV (q4_k.hip): a wave owns a short run of consecutive
-// 8-row tiles of one matrix; up to eight waves of a workgroup share one staged activation.
+// 8-row tiles of one matrix and walks it four super-blocks deep (device_run_ring.h); up to eight waves of a
+// workgroup share one staged activation.
 template <int B, bool GROUPED, int MAXT>
 __global__ __launch_bounds__(MAXT) void gemv_q6_k_kernel(RmiQ4kProblem single, const RmiQ4kProblem *__restrict__ list,
                                                         const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
     extern __shared__ uint4 lds[];
     const uint32_t lane = threadIdx.x & 63, r = lane >> 3, m = lane & 7;
-    const uint32_t w_idx = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    // wave-uniform, and said so: the problem's fields and the super-block counter live in scalar registers
+    const uint32_t w_idx = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     RmiQ4kProblem p;
     uint32_t k, k_end;
     if (GROUPED) {
@@ -133,6 +129,23 @@ __global__ __launch_bounds__(MAXT) void gemv_q6_k_kernel(RmiQ4kProblem single, c
         k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
     }
     const uint32_t n_sb = p.n_sb, n_in = n_sb * 256;
+    // units of the run (device_run_ring.h): one super-block of one tile, 1680 bytes, tile after tile
+    const uint32_t n_units = (k_end - k) * n_sb;
+    // a wave without tiles (padding of the last workgroup) prefetches from the matrix's first tile: in bounds, unused
+    gptr_u4 base = as_global<gptr_u4>(p.w + size_t(p.tile0 + (n_units ? k : 0)) * n_sb * kQ6KSuperBytes);
+    struct Cursor {
+        gptr_u4 unit;  // the same for all lanes
+        uint32_t r, lane;
+        __device__ __forceinline__ void load(SuperRegs &g) const {
+            g.sc = unit[r];
+            g.d = ((gptr_u16)(unit + 8))[r];
+            g.ql = __builtin_nontemporal_load(unit + 9 + lane);  // weights are read once: not kept in cache
+            g.qh = __builtin_nontemporal_load((gptr_u2)(unit + 73) + lane);
+        }
+        __device__ __forceinline__ void step() { unit += kQ6KSuperBytes / 16; }
+    } cur{base, r, lane};
+    RmiRing<SuperRegs> ring;
+    rmi_ring_fill(ring, n_units, cur);
     uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
     for (int t = 0; t < B; t++)
         rmi_stage_q8k_token<false, 2>(lds_dw + size_t(t) * n_sb * kSbDwords, p.q8qs + size_t(t) * n_in,
@@ -140,33 +153,28 @@ __global__ __launch_bounds__(MAXT) void gemv_q6_k_kernel(RmiQ4kProblem single, c
                                       blockDim.x);
     __syncthreads();
 
-    for (; k < k_end; k++) {
-        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * n_sb * kQ6KSuperBytes);
-        float acc[B];
+    float acc[B];
 #pragma unroll
-        for (int t = 0; t < B; t++) acc[t] = 0.0f;
-        // software pipeline over super-blocks, two pairs deep; ascending order is kept
-        SuperRegs ra, rb, rc, rd;
-        load_super(ra, tile, 0, r, lane);
-        if (n_sb > 1) load_super(rb, tile, 1, r, lane);
-        for (uint32_t sb = 0; sb < n_sb; sb += 4) {
-            if (sb + 2 < n_sb) load_super(rc, tile, sb + 2, r, lane);
-            if (sb + 3 < n_sb) load_super(rd, tile, sb + 3, r, lane);
-            super_fma<B>(acc, ra, lds_dw, n_sb, sb, m);
-            if (sb + 1 < n_sb) super_fma<B>(acc, rb, lds_dw, n_sb, sb + 1, m);
-            if (sb + 4 < n_sb) load_super(ra, tile, sb + 4, r, lane);
-            if (sb + 5 < n_sb) load_super(rb, tile, sb + 5, r, lane);
-            if (sb + 2 < n_sb) super_fma<B>(acc, rc, lds_dw, n_sb, sb + 2, m);
-            if (sb + 3 < n_sb) super_fma<B>(acc, rd, lds_dw, n_sb, sb + 3, m);
-        }
-        const uint32_t row = (p.tile0 + k) * kTileRows + r;
-        gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    for (int t = 0; t < B; t++) acc[t] = 0.0f;
+    RmiRunResults<B> out{};
+    uint32_t sb = 0;
+    gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    auto consume = [&](const SuperRegs &g) {
+        super_fma<B>(acc, g, lds_dw, n_sb, sb, m);
+        if (++sb == n_sb) {
+            float y[B];
 #pragma unroll
-        for (int t = 0; t < B; t++) {
-            const float v = hsum8_lanes(acc[t]);
-            if (m == 0 && row >= p.row_start && row < p.row_end) yp[size_t(t) * p.y_stride + row] = v;
+            for (int t = 0; t < B; t++) {
+                y[t] = hsum8_lanes(acc[t]);  // the same in the row's eight lanes
+                acc[t] = 0.0f;
+            }
+            sb = 0;
+            out.keep(y, m);
+            if (out.group_full()) out.flush(yp, p.y_stride, p.tile0 + k, r, m, p.row_start, p.row_end);
         }
-    }
+    };
+    rmi_ring_walk(ring, n_units, cur, consume);
+    if (out.pending()) out.flush(yp, p.y_stride, p.tile0 + k, r, m, p.row_start, p.row_end);
 }
 
 // ---- the eight exact lane integers per (row, super-block), read back from the repacked stream

@@ -145,6 +145,8 @@ struct RmiGemvProblem {
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
 // the same problem record with w = a Q4_0 tile stream (Q8_0 activation)
 int rmi_launch_gemv_q4_0(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
+int rmi_launch_gemv_q4_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,
+                               uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s);
 int rmi_launch_block_dots_q4_0(const rmi_hip_weight *w, const int8_t *x_q8, int32_t *dots, hipStream_t s);
 // y = W . Q8_0(rms_norm(x_in + resid) * norm_weight) in one launch, x_out = x_in + resid (x_out != x_in);
 // for one token and matrices the fused kernel covers (rmi_gemv_q8_0_norm_fusable)

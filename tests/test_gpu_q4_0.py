@@ -121,3 +121,38 @@ def test_q4_0_fusion_and_errors(hip, oracle):
                                                         H.ptr(out, H._f32p), n_in, 1000, 0, 1))
     k2 = K.QuantizedTensor.from_bytes(K.GGML_TYPE_Q4_0, a, n_in, 1000).into_kernel()
     assert isinstance(k2, K.Q4_0Kernel) and k2.w.dtype == H.DTYPE_Q4_0
+
+
+def test_q4_0_grouped_launch_equals_the_scalar_kernel(hip, oracle):
+    """One launch over a list of independent Q4_0 GEMVs of different shapes (a ragged row count, a partly filled
+    octet, a wide head); mixing weight types in one group is refused."""
+    H, K = hip.hip, hip.kernel
+    shapes = [(2048, 1024), (1024, 1024), (1024, 2048), (3072, 1024), (1024, 3072), (4099, 1024), (13, 96), (520, 288)]
+    for n_tokens in (1, 3, 8):
+        kernels, xq, xs, ys, refs = [], [], [], [], []
+        for i, (n_out, n_in) in enumerate(shapes):
+            w = hip.synth.q4_0_weight(1300 + i, n_out, n_in)
+            x = hip.synth.activations(1400 + i, n_tokens, n_in)
+            qs = [oracle.quantize_q8_0(x[t], A) for t in range(n_tokens)]
+            q8, sc = np.stack([q for q, _ in qs]), np.stack([s for _, s in qs])
+            kernels.append(K.Q4_0Kernel(w, n_in, n_out))
+            xq.append(H.DeviceBuffer.from_array(q8))
+            xs.append(H.DeviceBuffer.from_array(sc))
+            ys.append(H.DeviceBuffer(n_tokens * n_out * 4))
+            refs.append(np.stack([_ref(oracle, w, q8[t], sc[t], n_in, n_out) for t in range(n_tokens)]))
+        n = len(shapes)
+        arr = lambda vals: (H.C.c_void_p * n)(*vals)  # noqa: E731
+        g = H.lib.rmi_hip_gemv_group_create(n, arr([k.w.handle for k in kernels]), arr([b.ptr for b in xq]),
+                                            arr([b.ptr for b in xs]), arr([b.ptr for b in ys]), n_tokens)
+        assert g, H.last_error()
+        H.check(H.lib.rmi_hip_gemv_group_run_dev(g, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        for i, (n_out, _) in enumerate(shapes):
+            got = ys[i].to_array(np.float32, (n_tokens, n_out))
+            assert np.array_equal(bits(got), bits(refs[i])), (n_tokens, i)
+        H.lib.rmi_hip_gemv_group_destroy(g)
+    q8k = K.Q8Kernel(hip.synth.q8_0_weight(5, 64, 1024), 1024, 64)
+    two = lambda a, b: (H.C.c_void_p * 2)(a, b)  # noqa: E731
+    g = H.lib.rmi_hip_gemv_group_create(2, two(kernels[0].w.handle, q8k.w.handle), two(xq[0].ptr, xq[0].ptr),
+                                        two(xs[0].ptr, xs[0].ptr), two(ys[0].ptr, ys[0].ptr), 1)
+    assert not g and "bad weight handle" in H.last_error()
