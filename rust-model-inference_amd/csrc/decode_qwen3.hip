@@ -491,8 +491,11 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     float my_max = -INFINITY;
     for (uint32_t t0 = 0; t0 < n_keys; t0 += kA128Threads / 4) {
         const uint32_t t = t0 + key0, tn = t + kA128Threads / 4;
+        // The next round's keys are in flight while this one is summed.  The loads are unconditional (after the
+        // last round they read the last key again): behind a branch they could not be counted on, and the wait
+        // for this round's keys would have to drain them, too.
         uint4 kn[4];
-        if (t0 + kA128Threads / 4 < n_keys) {  // the next round's keys are in flight while this one is summed
+        {
             const uint4 *key = kbase + __umul24(tn < n_keys ? tn : n_keys - 1, row_u4);
 #pragma unroll
             for (int c = 0; c < 4; c++) kn[c] = key[4 * c];
