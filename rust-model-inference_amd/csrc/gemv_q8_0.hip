@@ -128,10 +128,10 @@ __device__ __forceinline__ void octet_fma(float (&acc)[B], const OctetRegs &g, c
     }
 }
 
-// One wave per workgroup; a wave owns a short run of consecutive 8-row tiles
-// of ONE matrix (about 16 KiB of weights).  A launch has far more waves than
-// fit on the chip at once: the dispatcher hands out runs as waves retire, which
-// balances the load and keeps the waves in flight reading one compact window of
+// A wave owns a short run of consecutive 8-row tiles of ONE matrix (about 34 KiB of
+// weights) and walks it four octets deep (device_run_ring.h).  A launch has far more
+// waves than fit on the chip at once: the dispatcher hands out runs as waves retire,
+// which balances the load and keeps the waves in flight reading one compact window of
 // HBM.  The activation of the matrix sits in LDS, permuted to quad order.
 // GROUPED = false: one matrix (`single`), run w starts at tile w * tiles_per_wave.
 // GROUPED = true: runs[w] = {problem index, first tile, tile count, -}.

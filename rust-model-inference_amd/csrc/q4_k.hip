@@ -149,8 +149,8 @@ __device__ __forceinline__ void super_fma(float (&acc)[B], float (&acc_m)[B], co
     }
 }
 
-// One wave per workgroup; a wave owns a short run of consecutive 8-row tiles of one
-// matrix, and a launch has far more waves than fit on the chip (see gemv_q8_0.hip).
+// A wave owns a short run of consecutive 8-row tiles of one matrix and walks it four super-blocks deep
+// (device_run_ring.h); a launch has far more waves than fit on the chip (see gemv_q8_0.hip).
 // GROUPED = false: one matrix (`single`), run w starts at tile w * tiles_per_wave.
 // GROUPED = true: runs[w] = {problem index, first tile, tile count, -}.
 // MAXT = 64: one wave per workgroup; 512: up to eight waves sharing one staged activation
