@@ -577,6 +577,60 @@ def run_q4_0(args, pkg, ev):
     return result
 
 
+def run_qlinear(args, pkg, ev):
+    """QuantizedLinear::forward (src/core/model.rs:65-91): f32 activation, Q4_K weight dequantised on the fly, one
+    strictly sequential f32 sum per output row.  One step = the three FFN products of a 1.7B-class layer (gate, up
+    6144x2048, down 2048x6144).  The bound is neither HBM nor the matrix cores but the add chain: n_in dependent f32
+    adds per row, about 8.4 clocks each on one lane; rows run side by side."""
+    H, synth, K = pkg.hip, pkg.synth, pkg.kernel
+    dev_name, cus, hbm = H.device_info()
+    recs = []
+    for i, (n_out, n_in) in enumerate([(6144, 2048), (6144, 2048), (2048, 6144)]):
+        w = synth.q4_k_weight(synth.seed_for(3, i), n_out, n_in)
+        x = synth.activations(synth.seed_for(3, 0x8000 + i), 1, n_in).reshape(-1)
+        k = K.Q4_KKernel(w, n_in, n_out)
+        recs.append(dict(w=w, x=x, k=k, d_x=H.DeviceBuffer.from_array(x), d_y=H.DeviceBuffer(n_out * 4), n_out=n_out,
+                         n_in=n_in))
+
+    def step():
+        for r in recs:
+            H.check(H.lib.rmi_hip_quantized_linear_forward_dev(r["k"].w.handle, r["d_x"].ptr, r["d_y"].ptr, None))
+
+    copy_calibration(H, args)
+    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
+    alg = sum(r["n_out"] * (r["n_in"] // 256) * 144 + 4 * r["n_in"] + 4 * r["n_out"] for r in recs)
+    achieved = alg / (dev_ms * 1e-3) / 1e9
+    chain_us = sum(r["n_in"] * 8.4 / 2.0e3 for r in recs)  # at 2.0 GHz under load
+    result = base_result(args, "QuantizedLinear::forward (Q4_K dequantise-and-dot) GB/s, 1.7B-class FFN shapes, 1 GPU", "GB/s",
+                         round(alg / wall / 1e9, 1), wall, "f32 (sequential sum per row)", {
+        "workload": "QuantizedLinear::forward, gate and up (6144x2048) and down (2048x6144), f32 activation, 3 launches per step",
+        "launches_per_step": 3, "algorithmic_bytes_per_step": alg, "device": dev_name.strip(), "compute_units": cus})
+    result["roofline"] = {"bound": "hbm", "kernel": "q4_k_dequant_dot_split_kernel", "achieved": round(achieved, 1),
+                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                          "avg_launch_us": round(dev_ms * 1e3 / 3, 3), "traffic": None,
+                          "limit": "one dependent f32 add per element and row (the reference's summation order): "
+                                   f"{chain_us:.1f} us per step at 8.4 clocks an add and 2.0 GHz, whatever the bandwidth",
+                          "add_chain_us_per_step": round(chain_us, 1)}
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import rmi_oracle as oracle
+        samples, worst = [], 0
+        step()
+        H.check(H.lib.rmi_hip_synchronize())
+        for it in range(2):
+            t0 = time.perf_counter()
+            refs = [oracle.quantized_linear_forward(r["w"], r["x"], r["n_in"], r["n_out"]) for r in recs]
+            samples.append(time.perf_counter() - t0)
+        for r, ref in zip(recs, refs):
+            worst = max(worst, int(np.count_nonzero(r["d_y"].to_array(np.float32, (r["n_out"],)).view(np.uint32)
+                                                    != ref.view(np.uint32))))
+        result["cpu_baseline"] = {"value": round(alg / min(samples) / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                                  "sample": "2 full steps of the restated forward_dequant (dequantise the weight, then "
+                                            "the sequential dot per row), one thread as the reference runs it, best",
+                                  "gpu_outputs_differing_from_cpu": worst}
+    return result
+
+
 def run_q4k_gemm(args, pkg, ev):
     """Q4_K prefill: X[M x 2048] through gate and up (6144 x 2048 each) and X[M x 6144] through down (2048 x 6144),
     Q8_K activations already quantized in HBM; one step = the three products."""
@@ -719,9 +773,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "decode"], default="projection_set",
+    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "qlinear", "decode"], default="projection_set",
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
-                         "q4_0: Q4_0 x Q8_0 decode GEMV; q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); decode: end-to-end device-resident greedy decode "
+                         "q4_0: Q4_0 x Q8_0 decode GEMV; q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); qlinear: QuantizedLinear::forward (Q4_K dequantise-and-dot, f32 activation); decode: end-to-end device-resident greedy decode "
                          "(one step = one 639-token-step generation)")
     ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill tokens M for --workload gemm")
@@ -741,7 +795,7 @@ def main():
     pkg = importlib.import_module("rust-model-inference_amd")
     pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
     ev = HipEvents()
-    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4_0": run_q4_0, "q4k": run_q4k, "q6k": run_q6k, "q4k_gemm": run_q4k_gemm,
+    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4_0": run_q4_0, "q4k": run_q4k, "q6k": run_q6k, "q4k_gemm": run_q4k_gemm, "qlinear": run_qlinear,
            "decode": run_decode}[args.workload]
     result = run(args, pkg, ev)
     if args.workload == "projection_set" and not args.no_decode and args.batch == 1:

@@ -132,6 +132,8 @@ int rmi_hip_q4_k_forward_prequantized(const rmi_hip_weight *w, const uint8_t *in
  * input, Q4_K weight dequantised in registers, no scratch needed. */
 int rmi_hip_quantized_linear_forward(const rmi_hip_weight *w, const float *input, float *output, uint32_t in_features,
                                      uint32_t out_features);
+/* The same on device pointers (x f32[in_features], y f32[out_features]); does not synchronise. */
+int rmi_hip_quantized_linear_forward_dev(const rmi_hip_weight *w, const float *x, float *y, void *stream);
 /* Exact integers of the Q4_K x Q8_K dot per super-block (parity entry point):
  * isum/msum[n_out][n_in/256] as in vec_dot_q4k_q8k_scalar, quant/mod.rs:260-284. */
 int rmi_hip_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *q8k_qs, const int16_t *q8k_bsums, int32_t *isum,

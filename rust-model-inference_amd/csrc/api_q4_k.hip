@@ -161,6 +161,14 @@ int rmi_hip_quantized_linear_forward(const rmi_hip_weight *w, const float *input
     return fetch(c, output, d_y, size_t(out_features) * 4, 1);
 }
 
+int rmi_hip_quantized_linear_forward_dev(const rmi_hip_weight *w, const float *x, float *y, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_K) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_K weight handle");
+    if (w->n_out == 0) return RMI_HIP_OK;
+    if (!x || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    return rmi_launch_q4_k_dequant_dot(w, x, nullptr, nullptr, y, 0, w->n_out, 1, static_cast<hipStream_t>(stream));
+}
+
 int rmi_hip_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *q8k_qs, const int16_t *q8k_bsums, int32_t *isum,
                             int32_t *msum) {
     RMI_REQUIRE_INIT();

@@ -77,6 +77,7 @@ SIGNATURES = {
     "rmi_hip_quantize_row_q8_k": (C.c_int, [_f32p, _u32, _f32p, _i8p, _i16p]),
     "rmi_hip_q4_k_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_quantized_linear_forward": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32]),
+    "rmi_hip_quantized_linear_forward_dev": (C.c_int, [_vp, _vp, _vp, _vp]),
     "rmi_hip_block_ints_q4_k": (C.c_int, [_vp, _i8p, _i16p, _i32p, _i32p]),
     "rmi_hip_q4_0_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_q4_0_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32, C.c_int]),

@@ -219,7 +219,9 @@ def test_q4_k_kernel_multiplies_uniform_block(hip):
     assert list(out) == [256.0]
 
 
-@pytest.mark.parametrize("n_out,n_in", [(6144, 2048), (2048, 6144), (5, 256), (77, 768)])
+# the last two: an activation that needs more than 64 KiB of LDS beside the products, and one beyond the
+# workgroup's LDS altogether (the one-lane-per-row kernel takes it)
+@pytest.mark.parametrize("n_out,n_in", [(6144, 2048), (2048, 6144), (5, 256), (77, 768), (41, 12288), (19, 36864)])
 def test_dequant_dot_paths_bit_exact(hip, oracle, n_out, n_in):
     K = hip.kernel
     w = hip.synth.q4_k_weight(80 + n_out, n_out, n_in)
