@@ -273,13 +273,17 @@ static void copy_to_pinned(uint8_t *dst, const uint8_t *src, size_t n) {
     }
     const size_t piece = ((n + n_thr - 1) / n_thr + 4095) & ~size_t(4095);
     std::vector<std::thread> pool;
-    for (size_t t = 1; t < n_thr; t++) {
-        const size_t off = t * piece;
-        if (off >= n) break;
-        const size_t len = n - off < piece ? n - off : piece;
-        pool.emplace_back([=] { memcpy(dst + off, src + off, len); });
+    size_t handed = piece < n ? piece : n;  // bytes [0, handed) are this thread's or a helper's
+    try {
+        for (size_t t = 1; t < n_thr && handed < n; t++) {
+            const size_t off = handed, len = n - off < piece ? n - off : piece;
+            pool.emplace_back([=] { memcpy(dst + off, src + off, len); });
+            handed = off + len;
+        }
+    } catch (...) {  // no more threads to be had: this one copies the rest
     }
     memcpy(dst, src, piece < n ? piece : n);
+    if (handed < n) memcpy(dst + handed, src + handed, n - handed);
     for (std::thread &th : pool) th.join();
 }
 
