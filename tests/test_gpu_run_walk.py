@@ -137,3 +137,46 @@ def test_row_ranges_and_batches_over_long_runs(hip, oracle, fmt):
     _run(hip, oracle, fmt, 131, n_out, n_units, 1, r0=13, r1=n_out - 5)
     _run(hip, oracle, fmt, 132, n_out, n_units, 2, r0=8 * 1000 + 7, r1=8 * 1000 + 9)
     _run(hip, oracle, fmt, 133, n_out, n_units, 1, r0=40000, r1=40000)  # empty range: nothing is written
+
+
+def _group_create(H, fmt, kernels, acts, ys, n_tokens):
+    n = len(kernels)
+    arr = lambda vals: (H.C.c_void_p * n)(*vals)  # noqa: E731
+    handles = arr([k.w.handle for k in kernels])
+    outs = arr([y.ptr for y in ys])
+    if fmt in ("q8_0", "q4_0"):
+        return H.lib.rmi_hip_gemv_group_create(n, handles, arr([a[0].ptr for a in acts]), arr([a[1].ptr for a in acts]), outs,
+                                               n_tokens)
+    create = H.lib.rmi_hip_gemv_group_create_q4_k if fmt == "q4_k" else H.lib.rmi_hip_gemv_group_create_q6_k
+    return create(n, handles, arr([a[0].ptr for a in acts]), arr([a[1].ptr for a in acts]), arr([a[2].ptr for a in acts]),
+                  outs, n_tokens)
+
+
+@pytest.mark.parametrize("fmt", list(FORMATS))
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_grouped_launches(hip, oracle, fmt, seed):
+    """One launch over a random list of matrices of unlike widths and heights (so the runs of one workgroup's
+    waves, their lengths and the padding runs differ from launch to launch), 1 / 2 / 5 / 8 tokens."""
+    H, F = hip.hip, FORMATS[fmt]
+    rng = np.random.default_rng(1000 * seed + len(fmt))
+    for n_tokens in (1, 2, 5, 8):
+        shapes = [(int(rng.integers(1, 700)), int(rng.integers(1, 14))) for _ in range(int(rng.integers(3, 12)))]
+        shapes.append((int(rng.integers(30000, 50000)), int(rng.integers(1, 4))))  # one tall matrix: runs of many tiles
+        kernels, acts, ys, refs = [], [], [], []
+        for i, (n_out, n_units) in enumerate(shapes):
+            n_in = n_units * F.unit
+            w, kernel_cls = F.weight(hip, 7000 + 100 * seed + i, n_out, n_in)
+            kernels.append(kernel_cls(w, n_in, n_out))
+            x = hip.synth.activations(8000 + 100 * seed + i, n_tokens, n_in)
+            per_token = [F.quantize(oracle, x[t]) for t in range(n_tokens)]
+            acts.append([H.DeviceBuffer.from_array(np.stack([a[j] for a in per_token])) for j in range(len(per_token[0]))])
+            ys.append(H.DeviceBuffer.from_array(np.full((n_tokens, n_out), np.float32(3.5))))
+            refs.append(np.stack([F.ref(oracle, w, per_token[t], n_in, n_out) for t in range(n_tokens)]))
+        g = _group_create(H, fmt, kernels, acts, ys, n_tokens)
+        assert g, H.last_error()
+        H.check(H.lib.rmi_hip_gemv_group_run_dev(g, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        for i, (n_out, n_units) in enumerate(shapes):
+            got = ys[i].to_array(np.float32, (n_tokens, n_out))
+            assert np.array_equal(bits(got), bits(refs[i])), (fmt, seed, n_tokens, i, n_out, n_units)
+        H.lib.rmi_hip_gemv_group_destroy(g)
