@@ -771,8 +771,10 @@ def run_decode(args, pkg, ev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default 50; 500 for the q4_0 / q4k / q6k GEMV workloads, whose compute-heavy kernels "
+                         "read 10-15 %% slower until the clocks have settled, a few hundred launches in)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before (default 10; 100 for q4_0 / q4k / q6k)")
     ap.add_argument("--workload", choices=["projection_set", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "qlinear", "decode"], default="projection_set",
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
                          "q4_0: Q4_0 x Q8_0 decode GEMV; q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); qlinear: QuantizedLinear::forward (Q4_K dequantise-and-dot, f32 activation); decode: end-to-end device-resident greedy decode "
@@ -788,6 +790,11 @@ def main():
     ap.add_argument("--no-decode", action="store_true",
                     help="projection_set only: skip the end-to-end decode figure that is attached to the JSON line")
     args = ap.parse_args()
+    long_run = args.workload in ("q4_0", "q4k", "q6k")
+    if args.steps is None:
+        args.steps = 500 if long_run else 50
+    if args.warmup is None:
+        args.warmup = 100 if long_run else 10
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across GPUs", file=sys.stderr)
         sys.exit(2)

@@ -26,7 +26,7 @@ __device__ __forceinline__ float hsum8_lanes(float a) {
     return a;
 }
 
-// signed 4 x int8 dot (v_dot4c_i32_i8 into a cleared register)
+// signed 4 x int8 dot from zero (the build turns v_dot4c off, so this is one v_dot4_i32_i8 with a literal 0)
 __device__ __forceinline__ int dot4_i8(int a, int b) {
     return __builtin_amdgcn_sdot4(a, b, 0, false);
 }
