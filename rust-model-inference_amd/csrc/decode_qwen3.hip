@@ -31,11 +31,10 @@
 #include "device_quant.h"
 #include "rmi_internal.h"
 
+#include "device_common.h"
+
 namespace {
 
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
-}
 __device__ __forceinline__ uint16_t f2h(float v) { return rmi_f2h(v); }
 
 // The step counter in HBM: the embedding kernel reads its token through it and the argmax kernel advances it,

@@ -18,18 +18,15 @@
 // piece (the four dwords of lane T) is widened and scattered into natural element order by the LDS store.
 #include "rmi_internal.h"
 
+#include "device_common.h"
+
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v32f __attribute__((ext_vector_type(32)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kRow = 272;  // bytes between LDS rows of 256 quants: 16-byte reads of 8 lanes hit 8 bank groups
-
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
-}
 
 // the kmask unpack of quant/mod.rs:237-258: .x,.y = 8 scales, .z,.w = 8 mins, one byte each
 __device__ __forceinline__ uint4 unpack_scales(uint32_t u0, uint32_t u1, uint32_t u2) {

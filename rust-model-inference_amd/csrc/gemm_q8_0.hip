@@ -30,19 +30,15 @@
 // the multiply loop alone, with operands held in registers).
 #include "rmi_internal.h"
 
+#include "device_common.h"
+
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v32f __attribute__((ext_vector_type(32)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kRowStride = 144;  // bytes between rows of the LDS tiles
-
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
-}
 
 // NTW x TTW 32x32 sub-tiles per wave, WN x WT waves per workgroup
 template <int NTW, int TTW, int WN, int WT>

@@ -10,43 +10,16 @@
 #include "device_quant.h"
 #include "rmi_internal.h"
 
+#include "device_common.h"
+
 #include "device_run_ring.h"
 
 namespace {
-
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
-}
-
-// lane L of 8: ((l0+l4)+(l1+l5)) + ((l2+l6)+(l3+l7)), valid in lane 0 of the group
-__device__ __forceinline__ float hsum8_lanes(float a) {
-    a = a + __shfl_xor(a, 4, 64);
-    a = a + __shfl_xor(a, 1, 64);
-    a = a + __shfl_xor(a, 2, 64);
-    return a;
-}
-
-// signed 4 x int8 dot from zero (the build turns v_dot4c off, so this is one v_dot4_i32_i8 with a literal 0)
-__device__ __forceinline__ int dot4_i8(int a, int b) {
-    return __builtin_amdgcn_sdot4(a, b, 0, false);
-}
 
 __device__ __forceinline__ void block_fma(float &acc, uint32_t w_bits, float xs, int wq, int xq) {
     const float s = h2f(w_bits) * xs;  // one rounding, as _mm_mul_ps(cvtph, set1(bd))
     const int p = dot4_i8(wq, xq);
     acc = __builtin_fmaf(s, float(p), acc);
-}
-
-// Pointers that arrive inside a struct are generic; these casts tell the
-// compiler they are HBM addresses so that it emits global_load / global_store.
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef const u32x4 __attribute__((address_space(1))) *gptr_u4;
-typedef const uint32_t __attribute__((address_space(1))) *gptr_u32;
-typedef const float __attribute__((address_space(1))) *gptr_f32;
-typedef float __attribute__((address_space(1))) *gptr_f32_w;
-template <typename T, typename U>
-__device__ __forceinline__ T as_global(U *p) {
-    return (T)(uintptr_t)p;
 }
 
 // The three 16-byte loads one lane issues for one octet of its row.

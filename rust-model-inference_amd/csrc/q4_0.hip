@@ -7,23 +7,11 @@
 // chain per row: lane 0 of the row takes the products of lanes 0, 1, .. 7 in turn through lane shifts.
 #include "rmi_internal.h"
 
+#include "device_common.h"
+
 #include "device_run_ring.h"
 
 namespace {
-
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
-}
-
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef const u32x4 __attribute__((address_space(1))) *gptr_u4;
-typedef const uint16_t __attribute__((address_space(1))) *gptr_u16;
-typedef const float __attribute__((address_space(1))) *gptr_f32;
-typedef float __attribute__((address_space(1))) *gptr_f32_w;
-template <typename T, typename U>
-__device__ __forceinline__ T as_global(U *p) {
-    return (T)(uintptr_t)p;
-}
 
 // value of lane (l + K) of the same 16-lane row (only lanes 0 and 8 of a row use it, K <= 7)
 template <int K>

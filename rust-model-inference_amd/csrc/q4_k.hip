@@ -9,25 +9,12 @@
 // result hsum(acc) + ((m0+m2)+(m1+m3)).  Eight GPU lanes per row hold them.
 #include "rmi_internal.h"
 
+#include "device_common.h"
+
 #include "device_run_ring.h"
 #include "device_stage_q8k.h"
 
 namespace {
-
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
-}
-
-__device__ __forceinline__ float hsum8_lanes(float a) {
-    a = a + __shfl_xor(a, 4, 64);
-    a = a + __shfl_xor(a, 1, 64);
-    a = a + __shfl_xor(a, 2, 64);
-    return a;
-}
-
-__device__ __forceinline__ int dot4_i8(int a, int b) {  // signed 4 x int8 dot
-    return __builtin_amdgcn_sdot4(a, b, 0, false);
-}
 
 // the kmask unpack of quant/mod.rs:237-258: sm.x,.y = 8 scales, sm.z,.w = 8 mins
 __device__ __forceinline__ uint4 unpack_scales(uint32_t u0, uint32_t u1, uint32_t u2) {
@@ -98,17 +85,6 @@ __global__ __launch_bounds__(64) void quantize_q8_k_kernel(const float *__restri
 // 8 dwords of pair sums s_j = bsums[2j]+bsums[2j+1] (i16 wrap, as _mm_hadd_epi16),
 // 1 dword d (+3 pad) = 76 dwords.
 constexpr uint32_t kSbDwords = 76;
-
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef const u32x4 __attribute__((address_space(1))) *gptr_u4;
-typedef const uint32_t __attribute__((address_space(1))) *gptr_u32;
-typedef const int16_t __attribute__((address_space(1))) *gptr_i16;
-typedef const float __attribute__((address_space(1))) *gptr_f32;
-typedef float __attribute__((address_space(1))) *gptr_f32_w;
-template <typename T, typename U>
-__device__ __forceinline__ T as_global(U *p) {
-    return (T)(uintptr_t)p;
-}
 
 struct SuperRegs {
     u32x4 hdr;  // f16 d, f16 dmin, 12 packed scale bytes of the row

@@ -10,25 +10,12 @@
 // per row hold the eight accumulators.
 #include "rmi_internal.h"
 
+#include "device_common.h"
+
 #include "device_run_ring.h"
 #include "device_stage_q8k.h"
 
 namespace {
-
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
-}
-
-__device__ __forceinline__ float hsum8_lanes(float a) {
-    a = a + __shfl_xor(a, 4, 64);
-    a = a + __shfl_xor(a, 1, 64);
-    a = a + __shfl_xor(a, 2, 64);
-    return a;
-}
-
-__device__ __forceinline__ int dot4_i8(int a, int b) {  // signed 4 x int8 dot
-    return __builtin_amdgcn_sdot4(a, b, 0, false);
-}
 
 __device__ __forceinline__ int sbfe(uint32_t v, uint32_t off, uint32_t width) {
     return __builtin_amdgcn_sbfe(int(v), off, width);
@@ -38,19 +25,6 @@ __device__ __forceinline__ int sbfe(uint32_t v, uint32_t off, uint32_t width) {
 // elements 32g+4m..), 8 dwords of bsums (dword m = bsums[2m] | bsums[2m+1] << 16),
 // 1 dword d (+3 pad) = 76 dwords.
 constexpr uint32_t kSbDwords = 76;
-
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-typedef const u32x4 __attribute__((address_space(1))) *gptr_u4;
-typedef const u32x2 __attribute__((address_space(1))) *gptr_u2;
-typedef const uint16_t __attribute__((address_space(1))) *gptr_u16;
-typedef const uint32_t __attribute__((address_space(1))) *gptr_u32;
-typedef const float __attribute__((address_space(1))) *gptr_f32;
-typedef float __attribute__((address_space(1))) *gptr_f32_w;
-template <typename T, typename U>
-__device__ __forceinline__ T as_global(U *p) {
-    return (T)(uintptr_t)p;
-}
 
 struct SuperRegs {
     u32x4 sc;    // the row's 16 int8 scales
