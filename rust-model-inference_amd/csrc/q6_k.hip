@@ -223,6 +223,101 @@ __global__ __launch_bounds__(64) void q6_k_dequant_dot_kernel(const uint8_t *__r
     y[row] = sum;
 }
 
+// The same sum for 16 rows per workgroup with the work split by kind, as for Q4_K (q4_k.hip): the sum of a row
+// is one chain of f32 adds in element order, about eight clocks an add on one lane; what feeds it has no order.
+// Two producer waves turn one super-block of the 16 rows into products in LDS (a lane takes piece m of a row:
+// 32 elements) while a third wave, one lane per row, adds the previous super-block's products in order, its
+// LDS reads 32 values ahead; one barrier per super-block.  The activation is rebuilt as q8 * scale once, in LDS.
+constexpr uint32_t kDdRows = 16, kDdProducers = kDdRows * 8, kDdThreads = kDdProducers + 64;
+__global__ __launch_bounds__(kDdThreads) void q6_k_dequant_dot_split_kernel(
+    const uint8_t *__restrict__ w, const int8_t *__restrict__ x_q8, const float *__restrict__ x_scales,
+    float *__restrict__ y, uint32_t n_sb, uint32_t n_tiles, uint32_t row_start, uint32_t row_end) {
+    extern __shared__ float4 dd_lds[];
+    float4 *prod = dd_lds;                                             // [2][64 float4 per row][16 rows]
+    float *xs = reinterpret_cast<float *>(dd_lds + 2 * 64 * kDdRows);  // [n_in]
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t row0 = (row_start / kDdRows + blockIdx.x) * kDdRows;  // first row of this workgroup
+    const uint32_t n_in = n_sb * 256;
+    for (uint32_t k = tid; k < n_in; k += kDdThreads) xs[k] = float(int(x_q8[k])) * x_scales[k >> 5];
+    __syncthreads();
+
+    // producer lane: row pr of the 16, piece m of its super-block
+    const uint32_t pid = tid % kDdProducers, pr = pid % kDdRows, m = pid / kDdRows;
+    const bool producer = tid < kDdProducers;
+    uint32_t ptile = (row0 + pr) >> 3;
+    if (ptile >= n_tiles) ptile = n_tiles - 1;  // rows past the padded stream: in bounds, never stored
+    const uint8_t *ptile_base = w + size_t(ptile) * n_sb * kQ6KSuperBytes;
+    const uint32_t r8 = (row0 + pr) & 7;
+    auto produce = [&](uint32_t sb) {
+        const uint8_t *chunk = ptile_base + size_t(sb) * kQ6KSuperBytes;
+        const int8_t *sc = reinterpret_cast<const int8_t *>(chunk + r8 * 16);
+        const float d = h2f(reinterpret_cast<const uint16_t *>(chunk + 128)[r8]);
+        const uint4 qlv = reinterpret_cast<const uint4 *>(chunk + 144)[r8 * 8 + m];
+        const uint2 qhv = reinterpret_cast<const uint2 *>(chunk + 144 + 1024)[r8 * 8 + m];
+        SuperRegs g;
+        g.ql.x = qlv.x, g.ql.y = qlv.y, g.ql.z = qlv.z, g.ql.w = qlv.w;
+        g.qh.x = qhv.x, g.qh.y = qhv.y;
+        uint32_t q[8];
+        unpack_q6(g, q);
+        float4 *dst = prod + size_t(sb & 1) * 64 * kDdRows + pr;
+        const float4 *xsb = reinterpret_cast<const float4 *>(xs + sb * 256);
+#pragma unroll
+        for (int gg = 0; gg < 8; gg++) {
+            const float dsc = d * float(int(sc[2 * gg + (m >> 2)]));
+            const uint32_t k4 = 8 * gg + m;  // elements 4 k4 .. 4 k4 + 3 of the super-block
+            const float4 xv = xsb[k4];
+            const float xe[4] = {xv.x, xv.y, xv.z, xv.w};
+            float pe[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int qv = int((q[gg] >> (8 * i)) & 0xffu) - 32;
+                const float wv = dsc * float(qv);
+                pe[i] = wv * xe[i];
+            }
+            dst[size_t(k4) * kDdRows] = make_float4(pe[0], pe[1], pe[2], pe[3]);
+        }
+    };
+    if (producer) produce(0);
+    __syncthreads();
+    float sum = 0.0f;
+    for (uint32_t sb = 0; sb < n_sb; sb++) {
+        if (producer) {
+            if (sb + 1 < n_sb) produce(sb + 1);
+        } else if (lane < kDdRows) {
+            const float4 *src = prod + size_t(sb & 1) * 64 * kDdRows + lane;
+            float4 a[8], b[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) a[j] = src[size_t(j) * kDdRows];
+#pragma unroll
+            for (int blk = 0; blk < 4; blk++) {  // 16 float4 per round, the reads 8 float4 ahead of the adds
+#pragma unroll
+                for (int j = 0; j < 8; j++) b[j] = src[size_t(16 * blk + 8 + j) * kDdRows];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    sum = sum + a[j].x;
+                    sum = sum + a[j].y;
+                    sum = sum + a[j].z;
+                    sum = sum + a[j].w;
+                }
+                if (blk < 3) {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) a[j] = src[size_t(16 * blk + 16 + j) * kDdRows];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    sum = sum + b[j].x;
+                    sum = sum + b[j].y;
+                    sum = sum + b[j].z;
+                    sum = sum + b[j].w;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    const uint32_t row = row0 + lane;
+    if (!producer && lane < kDdRows && row >= row_start && row < row_end) y[row] = sum;
+}
+
 template <int B>
 int launch_gemv_q6k(const RmiQ4kProblem *single, const RmiQ4kProblem *d_list, const uint4 *d_runs, uint32_t n_waves,
                     uint32_t wpg, uint32_t tiles_per_wave, uint32_t max_n_sb, hipStream_t s) {
@@ -315,6 +410,20 @@ int rmi_launch_block_lanes_q6_k(const rmi_hip_weight *w, const int8_t *qs, const
 int rmi_launch_q6_k_dequant_dot(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                                 uint32_t row_start, uint32_t row_end, hipStream_t s) {
     if (row_start >= row_end) return RMI_HIP_OK;
+    const size_t lds_bytes = size_t(2) * 64 * kDdRows * 16 + size_t(w->n_in) * 4;
+    if (lds_bytes <= 160 * 1024 && w->n_units > 0) {
+        static const bool raised = [] {  // more than 64 KiB of dynamic LDS has to be asked for once
+            return hipFuncSetAttribute(reinterpret_cast<const void *>(q6_k_dequant_dot_split_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
+        }();
+        if (raised || lds_bytes <= 64 * 1024) {
+            const uint32_t grid = (row_end - 1) / kDdRows - row_start / kDdRows + 1;
+            hipLaunchKernelGGL(q6_k_dequant_dot_split_kernel, dim3(grid), dim3(kDdThreads), lds_bytes, s, w->data, x_q8,
+                               x_scales, y, w->n_units, w->n_tiles, row_start, row_end);
+            RMI_HIP_CHECK(hipGetLastError());
+            return RMI_HIP_OK;
+        }
+    }
     const uint32_t grid = (row_end - row_start + 63) / 64;
     hipLaunchKernelGGL(q6_k_dequant_dot_kernel, dim3(grid), dim3(64), 0, s, w->data, x_q8, x_scales, y, w->n_units,
                        row_start, row_end);

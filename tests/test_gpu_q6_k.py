@@ -198,7 +198,9 @@ def test_q6k_grouped_launch_bit_exact(hip, oracle):
     assert "bad weight handle" in H.last_error()
 
 
-@pytest.mark.parametrize("n_out,n_in", [(1024, 2048), (5, 256), (77, 768)])
+# the last two: an activation that needs more than 64 KiB of LDS beside the products, and one beyond the
+# workgroup's LDS altogether (the one-lane-per-row kernel takes it)
+@pytest.mark.parametrize("n_out,n_in", [(1024, 2048), (2048, 6144), (5, 256), (77, 768), (41, 12288), (19, 36864)])
 def test_q6k_dequant_dot_path_bit_exact(hip, oracle, n_out, n_in):
     """Q6_KKernel::forward_prequantized = matmul_q6_k_scalar_range (q6_k.rs:83-119), (ith, nth) slices."""
     K = hip.kernel
