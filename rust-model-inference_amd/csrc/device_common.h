@@ -27,6 +27,20 @@ __device__ __forceinline__ float h2f(uint32_t bits16) {
     return float(__builtin_bit_cast(_Float16, uint16_t(bits16)));
 }
 
+// f32(h) * x with one rounding, h an f16 sitting in either half of a 32-bit register.  MIX: written as
+// fma(h, x, -0.0), which is the product in every case (signed zeros included), with the -0.0 opaque to the
+// compiler, so that it becomes one v_fma_mix_f32 that reads the f16 half in place; otherwise a conversion and a
+// multiply.  The mixed form saves the shift, mask and conversion where they are not shared by several tokens.
+template <bool MIX>
+__device__ __forceinline__ float h2f_times(uint32_t bits16, float x) {
+    if (MIX) {
+        float neg_zero = -0.0f;
+        asm("" : "+v"(neg_zero));  // opaque, or the fma is folded back into a multiply
+        return __builtin_fmaf(h2f(bits16), x, neg_zero);
+    }
+    return h2f(bits16) * x;
+}
+
 // signed 4 x int8 dot from zero (the build turns v_dot4c off, so this is one v_dot4_i32_i8 with a literal 0)
 __device__ __forceinline__ int dot4_i8(int a, int b) {
     return __builtin_amdgcn_sdot4(a, b, 0, false);

@@ -49,7 +49,7 @@ __device__ __forceinline__ void octet_fma(float (&acc)[B], const OctetRegs &g, c
         dot = __builtin_amdgcn_sdot4(int(hi[2]), int(xb.z), dot, false);
         dot = __builtin_amdgcn_sdot4(int(hi[3]), int(xb.w), dot, false);
         dot -= int(meta.y);  // sum (nibble - 8) * q8 = sum nibble * q8 - 8 * sum q8
-        float p = float(dot) * wd;
+        float p = B == 1 ? h2f_times<true>(g.d, float(dot)) : float(dot) * wd;
         p = p * __uint_as_float(meta.x);
         p = live ? p : -0.0f;  // a block past the end of the row adds nothing, not even a sign
         float a = acc[t];

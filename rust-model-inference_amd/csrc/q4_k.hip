@@ -116,8 +116,8 @@ __device__ __forceinline__ void super_fma(float (&acc)[B], float (&acc_m)[B], co
             sumi += __mul24(int(byte_of(sm.x, sm.y, 2 * gg)), dl) + __mul24(int(byte_of(sm.x, sm.y, 2 * gg + 1)), dh);
         }
         const float d8 = __uint_as_float(xs[72]);
-        const float dd = wd * d8;
-        const float dm = (-wdmin) * d8;
+        const float dd = B == 1 ? h2f_times<true>(g.hdr.x & 0xffffu, d8) : wd * d8;
+        const float dm = B == 1 ? -h2f_times<true>(g.hdr.x >> 16, d8) : (-wdmin) * d8;
         acc[t] = __builtin_fmaf(dd, float(sumi), acc[t]);
         const int s0 = int(xs[64 + ((2 * T) & 7)]), s1 = int(xs[64 + ((2 * T + 1) & 7)]);
         const int prod = __mul24(mn0, s0) + __mul24(mn1, s1);  // 6-bit min x 16-bit pair sum

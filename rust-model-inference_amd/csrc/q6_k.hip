@@ -75,7 +75,7 @@ __device__ __forceinline__ void super_fma(float (&acc)[B], const SuperRegs &g, c
         const uint32_t bs = xs[64 + m];
         const int off = __mul24(sbfe(bs, 0, 16), so0) + __mul24(int(bs) >> 16, so1);
         sumi -= int(uint32_t(off) << 5);
-        const float dd = wd * __uint_as_float(xs[72]);
+        const float dd = B == 1 ? h2f_times<true>(g.d, __uint_as_float(xs[72])) : wd * __uint_as_float(xs[72]);
         acc[t] = __builtin_fmaf(dd, float(sumi), acc[t]);
     }
 }
