@@ -381,15 +381,18 @@ __global__ __launch_bounds__(512) void gemv_q8_0_norm_silu_kernel(const uint8_t 
     const float y = hsum8_lanes(acc[0]);
     if (L == 0) gu[wave * 8 + r] = y;  // [0,32): gate rows of this block, [32,64): up rows
     __syncthreads();
-    if (tid < 8) {
-        const float4 gt = reinterpret_cast<const float4 *>(gu)[tid], up = reinterpret_cast<const float4 *>(gu + 32)[tid];
+    if (tid < 64) {  // the first wave: one of the 32 values per lane (one exp each), then four per lane for the quantizer
+        const uint32_t i = tid & 31;
+        const float gt = gu[i], up = gu[32 + i];
+        const float hv = up * (gt / (1.0f + rmi_expf(-gt)));
         float4 h;
-        h.x = up.x * (gt.x / (1.0f + rmi_expf(-gt.x)));
-        h.y = up.y * (gt.y / (1.0f + rmi_expf(-gt.y)));
-        h.z = up.z * (gt.z / (1.0f + rmi_expf(-gt.z)));
-        h.w = up.w * (gt.w / (1.0f + rmi_expf(-gt.w)));
+        h.x = __shfl(hv, int(4 * (tid & 7)), 64);
+        h.y = __shfl(hv, int(4 * (tid & 7) + 1), 64);
+        h.z = __shfl(hv, int(4 * (tid & 7) + 2), 64);
+        h.w = __shfl(hv, int(4 * (tid & 7) + 3), 64);
         float sc;
-        reinterpret_cast<uint32_t *>(h_q8)[blockIdx.x * 8 + tid] = rmi_quantize_block8(h, na.rounding, &sc);
+        const uint32_t q = rmi_quantize_block8(h, na.rounding, &sc);
+        if (tid < 8) reinterpret_cast<uint32_t *>(h_q8)[blockIdx.x * 8 + tid] = q;
         if (tid == 0) h_scales[blockIdx.x] = sc;
     }
 }
