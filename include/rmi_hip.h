@@ -177,7 +177,9 @@ int rmi_hip_q6_k_forward_prequantized(const rmi_hip_weight *w, const uint8_t *in
 int rmi_hip_block_lanes_q6_k(const rmi_hip_weight *w, const int8_t *q8k_qs, const int16_t *q8k_bsums,
                              int32_t *lanes);
 
-/* ---- device-resident entry points (activations stay in HBM) ---------------*/
+/* ---- device-resident entry points (activations stay in HBM) ---------------
+ * Device pointers: activation quants (x_q8, q8k_qs) 16-byte aligned; scales, d, bsums and outputs 4-byte
+ * aligned (what rmi_hip_malloc returns is aligned for all of them).  Anything else is RMI_HIP_E_INVALID. */
 
 void *rmi_hip_malloc(size_t nbytes);
 void rmi_hip_free(void *dptr);
@@ -207,7 +209,7 @@ int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
  * integers, the f32 sums within rounding of the CPU kernels. */
 int rmi_hip_gemm_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
                               const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride, void *stream);
-/* Q4_0 weights, Q8_0 activations on the device (src/ops/kernel/q4_0/scalar.rs:13-52); x_q8 16-byte aligned. */
+/* Q4_0 weights, Q8_0 activations on the device (src/ops/kernel/q4_0/scalar.rs:13-52). */
 int rmi_hip_gemv_q4_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                           uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, void *stream);
 /* y[t*y_stride + r] = vec_dot_q6k_q8k(row r, Q8_K token t) for rows [row_start,row_end), 1..n tokens

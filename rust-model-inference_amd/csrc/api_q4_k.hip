@@ -198,6 +198,7 @@ int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
     if (row_end > w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) exceed n_out=%u", row_start, row_end, w->n_out);
     if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
     if (!q8k_d || !q8k_qs || !q8k_bsums || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (rmi_misaligned(q8k_qs, q8k_d, q8k_bsums, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
     return rmi_launch_gemv_q4_k(w, q8k_d, q8k_qs, q8k_bsums, y, n_tokens, y_stride, row_start, row_end,
                                 static_cast<hipStream_t>(stream));
 }
@@ -209,11 +210,7 @@ int rmi_hip_gemm_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
     if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
     if (y_stride < w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < n_out=%u", y_stride, w->n_out);
     if (!q8k_d || !q8k_qs || !q8k_bsums || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
-    if (w->n_units == 0) {
-        RMI_HIP_CHECK(hipMemset2DAsync(y, size_t(y_stride) * 4, 0, size_t(w->n_out) * 4, n_tokens,
-                                       static_cast<hipStream_t>(stream)));
-        return RMI_HIP_OK;
-    }
+    if (rmi_misaligned(q8k_qs, q8k_d, q8k_bsums, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
     return rmi_launch_gemm_q4_k(w, q8k_d, q8k_qs, q8k_bsums, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
 }
 
@@ -241,6 +238,11 @@ static rmi_hip_gemv_group *group_create_kquant(int dtype, uint32_t n_problems, c
         const rmi_hip_weight *w = weights[i];
         if (!w || w->dtype != dtype || !q8k_d[i] || !q8k_qs[i] || !q8k_bsums[i] || !y[i]) {
             rmi_set_error("gemv group problem %u: bad weight handle or null pointer", i);
+            delete g;
+            return nullptr;
+        }
+        if (rmi_misaligned(q8k_qs[i], q8k_d[i], q8k_bsums[i], y[i])) {
+            rmi_set_error("gemv group problem %u: " RMI_ALIGNMENT_MESSAGE, i);
             delete g;
             return nullptr;
         }
@@ -388,6 +390,7 @@ int rmi_hip_gemv_q6_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
     if (row_end > w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) exceed n_out=%u", row_start, row_end, w->n_out);
     if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
     if (!q8k_d || !q8k_qs || !q8k_bsums || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (rmi_misaligned(q8k_qs, q8k_d, q8k_bsums, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
     return rmi_launch_gemv_q6_k(w, q8k_d, q8k_qs, q8k_bsums, y, n_tokens, y_stride, row_start, row_end,
                                 static_cast<hipStream_t>(stream));
 }

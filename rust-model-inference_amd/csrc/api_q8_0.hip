@@ -255,6 +255,7 @@ int rmi_hip_gemv_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
     if (row_end > w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) exceed n_out=%u", row_start, row_end, w->n_out);
     if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
     if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (rmi_misaligned(x_q8, x_scales, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
     return gemv_tokens(w, x_q8, x_scales, y, n_tokens, y_stride, row_start, row_end, static_cast<hipStream_t>(stream));
 }
 
@@ -273,6 +274,7 @@ int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
     if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
     if (y_stride < w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < n_out=%u", y_stride, w->n_out);
     if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (rmi_misaligned(x_q8, x_scales, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
     return rmi_launch_gemm_q8_0(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
 }
 
@@ -307,6 +309,11 @@ rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip
         const rmi_hip_weight *w = weights[i];
         if (!w || w->dtype != g->dtype || !x_q8[i] || !x_scales[i] || !y[i]) {
             rmi_set_error("gemv group problem %u: bad weight handle or null pointer", i);
+            delete g;
+            return nullptr;
+        }
+        if (rmi_misaligned(x_q8[i], x_scales[i], y[i])) {
+            rmi_set_error("gemv group problem %u: " RMI_ALIGNMENT_MESSAGE, i);
             delete g;
             return nullptr;
         }
@@ -450,7 +457,7 @@ int rmi_hip_gemv_q4_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
     if (row_end > w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) exceed n_out=%u", row_start, row_end, w->n_out);
     if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
     if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
-    if (reinterpret_cast<uintptr_t>(x_q8) % 16) return rmi_fail(RMI_HIP_E_INVALID, "x_q8 must be 16-byte aligned");
+    if (rmi_misaligned(x_q8, x_scales, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
     return gemv_tokens(w, x_q8, x_scales, y, n_tokens, y_stride, row_start, row_end, static_cast<hipStream_t>(stream));
 }
 

@@ -85,6 +85,13 @@ bool rmi_ready();
                             __LINE__);                                                             \
     } while (0)
 
+// Activation quants are read with 16-byte loads; scales, sums and outputs with 4-byte ones.
+inline bool rmi_misaligned(const void *quants, const void *a = nullptr, const void *b = nullptr, const void *c = nullptr) {
+    return (reinterpret_cast<uintptr_t>(quants) & 15) != 0 ||
+           ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 3) != 0;
+}
+#define RMI_ALIGNMENT_MESSAGE "activation quants must be 16-byte aligned, scales / sums / outputs 4-byte aligned"
+
 #define RMI_REQUIRE_INIT()                                                             \
     do {                                                                               \
         if (!rmi_ready()) return rmi_fail(RMI_HIP_E_NOT_INIT, "rmi_hip_init has not succeeded"); \

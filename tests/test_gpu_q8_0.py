@@ -432,3 +432,24 @@ def test_error_codes(hip):
     # zero rows
     K.Q8Kernel(np.zeros(0, np.uint8), 64, 0).forward_prequantized(np.zeros(64, np.uint8), np.zeros(2, np.float32),
                                                                  out, 64, 0, 0, 1)
+
+
+def test_misaligned_device_pointers_are_refused(hip):
+    """The staging kernels read activation quants 16 bytes at a time and the rest 4 bytes at a time: a device
+    pointer that is not so aligned is an argument error, reported before anything is launched."""
+    H, K = hip.hip, hip.kernel
+    q8 = K.Q8Kernel(gen.make_q8_0_weight(16, 256, 3), 256, 16)
+    q4k = K.Q4_KKernel(hip.synth.q4_k_weight(5, 16, 256), 256, 16)
+    buf, y = H.DeviceBuffer(4096), H.DeviceBuffer(4096)
+    ok = H.lib.rmi_hip_gemv_q8_0_dev(q8.w.handle, buf.ptr, buf.ptr + 1024, y.ptr, 1, 16, 0, 16, None)
+    assert ok == 0, H.last_error()
+    for dq, ds, dy in ((4, 0, 0), (0, 2, 0), (0, 0, 2)):
+        rc = H.lib.rmi_hip_gemv_q8_0_dev(q8.w.handle, buf.ptr + dq, buf.ptr + 1024 + ds, y.ptr + dy, 1, 16, 0, 16, None)
+        assert rc == -1 and "aligned" in H.last_error(), (dq, ds, dy)
+        rc = H.lib.rmi_hip_gemm_q8_0_dev(q8.w.handle, buf.ptr + dq, buf.ptr + 1024 + ds, y.ptr + dy, 1, 16, None)
+        assert rc == -1 and "aligned" in H.last_error(), (dq, ds, dy)
+    rc = H.lib.rmi_hip_gemv_q4_k_q8k_dev(q4k.w.handle, buf.ptr, buf.ptr + 1024 + 8, buf.ptr + 2048, y.ptr, 1, 16, 0, 16, None)
+    assert rc == -1 and "aligned" in H.last_error()
+    rc = H.lib.rmi_hip_gemv_q4_k_q8k_dev(q4k.w.handle, buf.ptr, buf.ptr + 1024, buf.ptr + 2048 + 2, y.ptr, 1, 16, 0, 16, None)
+    assert rc == -1 and "aligned" in H.last_error()
+    H.check(H.lib.rmi_hip_synchronize())
