@@ -46,11 +46,7 @@ struct StepParams {
     uint32_t n_prompt;  // steps below n_prompt - 1 read their token from the prompt
 };
 
-__device__ __forceinline__ double wave_sum(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
+__device__ __forceinline__ double wave_sum(double v) { return wave_sum_f64(v); }
 
 // x[e] = d * q of row `token` of a Q8_0 weight in the GEMV tile stream
 __global__ __launch_bounds__(256) void embed_q8_0_kernel(const uint8_t *__restrict__ w, uint32_t n_oct,
@@ -304,8 +300,8 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
                     sum = __builtin_fma(double(h2f(kw[j] >> 16)), qq[8 * c + 2 * j + 1], sum);
                 }
             }
-            sum += __shfl_xor(sum, 1, 64);
-            sum += __shfl_xor(sum, 2, 64);
+            sum += dpp_f64<kDppQuadXor1>(sum);
+            sum += dpp_f64<kDppQuadXor2>(sum);
             if (t < n_keys) {
                 const float s = float(sum) * kq_scale;
                 if (lane4 == 0) scores[t] = s;
@@ -329,8 +325,8 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
                     sum = __builtin_fma(double(h2f(kw[j] >> 16)), qq[d + 2 * j + 1], sum);
                 }
             }
-            sum += __shfl_xor(sum, 1, 64);
-            sum += __shfl_xor(sum, 2, 64);
+            sum += dpp_f64<kDppQuadXor1>(sum);
+            sum += dpp_f64<kDppQuadXor2>(sum);
             if (live) {
                 const float s = float(sum) * kq_scale;
                 if (lane4 == 0) scores[t] = s;
@@ -338,8 +334,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_quant_kernel(
             }
         }
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) my_max = fmaxf(my_max, __shfl_xor(my_max, off, 64));
+    my_max = wave_max_f32(my_max);
     if ((tid & 63) == 0) red_f[tid >> 6] = my_max;
     __syncthreads();
     float max_val = red_f[0];
@@ -518,8 +513,7 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
 #pragma unroll
         for (int c = 0; c < 4; c++) kk[c] = kn[c];
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) my_max = fmaxf(my_max, __shfl_xor(my_max, off, 64));
+    my_max = wave_max_f32(my_max);
     if ((tid & 63) == 0) red_f[tid >> 6] = my_max;
     if (tid < 32) exp_tab[tid] = tab_entry;
     __syncthreads();

@@ -46,13 +46,76 @@ __device__ __forceinline__ int dot4_i8(int a, int b) {
     return __builtin_amdgcn_sdot4(a, b, 0, false);
 }
 
+// ---- values of other lanes without an address register: DPP where the pattern exists, else the LDS crossbar
+// with a constant pattern (ds_swizzle).  All 64 lanes must be active wherever these are used.
+constexpr int kDppQuadXor1 = 1 | (0 << 2) | (3 << 4) | (2 << 6);  // quad_perm [1,0,3,2]: lane ^ 1
+constexpr int kDppQuadXor2 = 2 | (3 << 2) | (0 << 4) | (1 << 6);  // quad_perm [2,3,0,1]: lane ^ 2
+constexpr int kDppRowHalfMirror = 0x141;                          // lane i <-> 7 - i of each 8 lanes
+constexpr int kDppRowMirror = 0x140;                              // lane i <-> 15 - i of each 16 lanes
+constexpr int kDppRowBcast15 = 0x142;                             // lane 15 of a row to the whole next row
+constexpr int kDppRowBcast31 = 0x143;                             // lane 31 to rows 2 and 3
+constexpr int kSwizzleXor4 = 0x1f | (4 << 10);                    // bit-mask mode: and 0x1f, or 0, xor 4
+constexpr int kSwizzleFirstOf8 = 0x18;                            // bit-mask mode: lane & ~7
+
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {  // rows outside ROW_MASK read 0
+    return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), CTRL, ROW_MASK, 0xf, ROW_MASK == 0xf));
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, dpp_u32<CTRL, ROW_MASK>(__builtin_bit_cast(uint32_t, v)));
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ double dpp_f64(double v) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint64_t lo = dpp_u32<CTRL, ROW_MASK>(uint32_t(b)), hi = dpp_u32<CTRL, ROW_MASK>(uint32_t(b >> 32));
+    return __builtin_bit_cast(double, lo | (hi << 32));
+}
+
 // ((l0+l4)+(l1+l5))+((l2+l6)+(l3+l7)) of the eight lanes of a row (src/ops/dot.rs:447-456); every lane of the
-// row ends up with the sum (a + b and b + a are the same bits)
+// row ends up with the sum (a + b and b + a are the same bits).
 __device__ __forceinline__ float hsum8_lanes(float a) {
-    a = a + __shfl_xor(a, 4, 64);
-    a = a + __shfl_xor(a, 1, 64);
-    a = a + __shfl_xor(a, 2, 64);
+    a = a + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, a), kSwizzleXor4));
+    a = a + dpp_f32<kDppQuadXor1>(a);
+    a = a + dpp_f32<kDppQuadXor2>(a);
     return a;
+}
+
+// the largest of the eight lanes' values, in all eight
+__device__ __forceinline__ float max8_lanes(float a) {
+    a = fmaxf(a, dpp_f32<kDppQuadXor1>(a));
+    a = fmaxf(a, dpp_f32<kDppQuadXor2>(a));
+    return fmaxf(a, dpp_f32<kDppRowHalfMirror>(a));
+}
+
+// Sum of the wave's 64 values, the same in every lane (it comes back through a scalar register): quads, halves
+// of eight, rows of sixteen, then row to row; the total forms in lane 63.  For f64 sums of exact terms, where
+// the order of the additions is free.
+__device__ __forceinline__ double wave_sum_f64(double v) {
+    v += dpp_f64<kDppQuadXor1>(v);
+    v += dpp_f64<kDppQuadXor2>(v);
+    v += dpp_f64<kDppRowHalfMirror>(v);
+    v += dpp_f64<kDppRowMirror>(v);
+    v += dpp_f64<kDppRowBcast15, 0xa>(v);
+    v += dpp_f64<kDppRowBcast31, 0xc>(v);
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint64_t lo = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(b)), 63));
+    const uint64_t hi = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(b >> 32)), 63));
+    return __builtin_bit_cast(double, lo | (hi << 32));
+}
+
+// Largest of the wave's 64 values, the same in every lane (rows a broadcast does not write keep their own value).
+__device__ __forceinline__ float wave_max_f32(float v) {
+    v = fmaxf(v, dpp_f32<kDppQuadXor1>(v));
+    v = fmaxf(v, dpp_f32<kDppQuadXor2>(v));
+    v = fmaxf(v, dpp_f32<kDppRowHalfMirror>(v));
+    v = fmaxf(v, dpp_f32<kDppRowMirror>(v));
+    // row to row with the old value kept where the broadcast does not write
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                       kDppRowBcast15, 0xa, 0xf, false)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                       kDppRowBcast31, 0xc, 0xf, false)));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 #endif  // RMI_DEVICE_COMMON_H

@@ -9,14 +9,13 @@
 #include <cstdint>
 
 #include "../../include/rmi_hip.h"
+#include "device_common.h"
 
 // Returns the four quants packed little-endian; *scale is f32(f16(amax/127)), valid in all 8 lanes.
 // The 8 lanes of a block must be consecutive lanes of one wave, aligned to 8, and all active.
 __device__ __forceinline__ uint32_t rmi_quantize_block8(float4 v, int rounding, float *scale) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    amax = max8_lanes(amax);
     const float d = amax == 0.0f ? 0.0f : amax / 127.0f;
     float r0, r1, r2, r3;
     if (rounding == RMI_HIP_ROUND_TIES_EVEN) {

@@ -276,8 +276,7 @@ __global__ __launch_bounds__(64) void gemv_q8_0_norm_deep_kernel(RmiGemvProblem 
 #pragma unroll
         for (int j = 0; j < NOCT; j++) reinterpret_cast<float4 *>(na.x_out)[lane + 64 * j] = v[j];
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+    part = wave_sum_f64(part);
     const float mean_sq = float(part / double(NOCT * 256));
     const float scale = 1.0f / sqrtf(mean_sq + na.eps);
     uint32_t *dq = reinterpret_cast<uint32_t *>(lds);
@@ -351,8 +350,7 @@ __global__ __launch_bounds__(512) void gemv_q8_0_norm_silu_kernel(const uint8_t 
         part += double(s1);
         part += double(s2);
         part += double(s3);
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        part = wave_sum_f64(part);
         if (lane == 0) red[wave] = part;
     }
     __syncthreads();
@@ -469,8 +467,7 @@ __global__ __launch_bounds__(512) void gemv_q8_0_norm_rope_kernel(const uint8_t 
         part += double(s1);
         part += double(s2);
         part += double(s3);
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        part = wave_sum_f64(part);
         if (lane == 0) red[wave] = part;
     }
     __syncthreads();
@@ -517,8 +514,7 @@ __global__ __launch_bounds__(512) void gemv_q8_0_norm_rope_kernel(const uint8_t 
         const float q0 = x0r * x0r, q1 = x1r * x1r;
         double part = double(q0);
         part += double(q1);
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        part = wave_sum_f64(part);
         const float mean_sq = float(part / 128.0);
         const float sc = 1.0f / sqrtf(mean_sq + ra.eps);
         x0 = (x0r * sc) * w0;

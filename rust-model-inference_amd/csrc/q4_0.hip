@@ -143,7 +143,8 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_0_kernel(RmiGemvProblem single, 
             float y[B];
 #pragma unroll
             for (int t = 0; t < B; t++) {
-                y[t] = __shfl(acc[t], int(lane & ~7u), 64);  // the row's chain ends in its lane 0
+                // the row's chain ends in its lane 0
+                y[t] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, acc[t]), kSwizzleFirstOf8));
                 acc[t] = 0.0f;
             }
             o = 0;

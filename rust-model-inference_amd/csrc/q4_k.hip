@@ -95,7 +95,10 @@ template <int B>
 __device__ __forceinline__ void super_fma(float (&acc)[B], float (&acc_m)[B], const SuperRegs &g,
                                           const uint32_t *lds_dw, uint32_t n_sb, uint32_t sb, uint32_t T) {
     const float wd = h2f(g.hdr.x & 0xffffu), wdmin = h2f(g.hdr.x >> 16);
-    const uint4 sm = unpack_scales(g.hdr.y, g.hdr.z, g.hdr.w);
+    uint4 sm = unpack_scales(g.hdr.y, g.hdr.z, g.hdr.w);
+    // the eight scales stay whole bytes of two registers: the multiplies below then select their byte themselves
+    // (SDWA) instead of a bit-field extract per scale from the packed source
+    asm("" : "+v"(sm.x), "+v"(sm.y));
     const uint32_t qd[4] = {g.qv.x, g.qv.y, g.qv.z, g.qv.w};
     // mins 2T and 2T+1 (mod 8) are neighbours in one dword of the unpacked eight
     const uint32_t mn_dw = (T & 2) ? sm.w : sm.z;
@@ -187,8 +190,8 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_kernel(RmiQ4kProblem single, c
             for (int t = 0; t < B; t++) {
                 const float main_val = hsum8_lanes(acc[t]);
                 float m = acc_m[t];  // lanes T and T + 4 hold the same acc_m
-                m = m + __shfl_xor(m, 2, 64);
-                m = m + __shfl_xor(m, 1, 64);
+                m = m + dpp_f32<kDppQuadXor2>(m);
+                m = m + dpp_f32<kDppQuadXor1>(m);
                 y[t] = main_val + m;  // the same in the row's eight lanes
                 acc[t] = acc_m[t] = 0.0f;
             }
