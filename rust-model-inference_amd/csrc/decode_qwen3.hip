@@ -432,6 +432,11 @@ __device__ __forceinline__ double quad_sum(double v) {  // (l0 + l1) + (l2 + l3)
     v += __hiloint2double(__builtin_amdgcn_mov_dpp(hi, 0x4E, 0xf, 0xf, true), __builtin_amdgcn_mov_dpp(lo, 0x4E, 0xf, 0xf, true));
     return v;
 }
+__device__ __forceinline__ double swizzle_xor16_f64(double v) {  // the value of lane ^ 16
+    constexpr int kXor16 = 0x1f | (16 << 10);
+    return __hiloint2double(__builtin_amdgcn_ds_swizzle(__double2hiint(v), kXor16),
+                            __builtin_amdgcn_ds_swizzle(__double2loint(v), kXor16));
+}
 __host__ __device__ inline size_t attn128_lds_bytes(uint32_t n_keys) {
     const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
     return n_pad * 12 + (kA128Threads / 64) * 128 * 8;
@@ -494,17 +499,17 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
 #pragma unroll
             for (int c = 0; c < 4; c++) kn[c] = key[4 * c];
         }
-        double sum = 0.0;
+        double s4[4] = {0.0, 0.0, 0.0, 0.0};  // four chains of eight adds, not one of thirty-two
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             const half8 kh = as_half8(kk[c]), qh = as_half8(qv[c]);
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const float prod = __builtin_fmaf(float(kh[j]), float(qh[j]), 0.0f);  // exact
-                sum += double(prod);
+                s4[c] += double(prod);
             }
         }
-        sum = quad_sum(sum);
+        double sum = quad_sum((s4[0] + s4[1]) + (s4[2] + s4[3]));
         if (t < n_keys) {
             const float sc = float(sum) * kq_scale;
             if (lane4 == 0) scores[t] = sc;
@@ -600,7 +605,7 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     }
 #pragma unroll
     for (int d = 0; d < 8; d++) {  // the four slices of a wave: lanes 16 apart
-        acc[d] += __shfl_xor(acc[d], 16, 64);
+        acc[d] += swizzle_xor16_f64(acc[d]);
         acc[d] += __shfl_xor(acc[d], 32, 64);
     }
     if ((tid & 63) < 16) {
