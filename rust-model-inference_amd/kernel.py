@@ -181,11 +181,31 @@ class Q8Kernel(Kernel):
         x = as_f32(input)
         check(lib.rmi_hip_matmul_q8_0_f32(self.w.handle, ptr(x, _f32p), ptr(_out(output, n_out), _f32p), n_in, n_out))
 
+    def matmul_q8_0_via_q8(self, input, output, n_in, n_out, q8_buf, scale_buf, rounding=hip.ROUND_TIES_EVEN):
+        """`matmul_q8_0_via_q8` (src/ops/kernel/q8_0/legacy.rs:27-83): quantize the f32 input into the caller's
+        scratch (which keeps the quants and scales afterwards, as in the reference), then the prequantized GEMV."""
+        quantize_q8_0_into(input, n_in, q8_buf, scale_buf, rounding)
+        self.forward_prequantized(q8_buf, scale_buf, output, n_in, n_out, 0, 1)
+
     def block_dots(self, input_q8):
         q8 = as_u8(input_q8)
         dots = np.zeros((self.w.n_out, self.w.n_in // 32), np.int32)
         check(lib.rmi_hip_block_dots_q8_0(self.w.handle, ptr(q8, _u8p), ptr(dots, _i32p)))
         return dots
+
+
+class MatmulTask:
+    """One f32-input matmul of a batch (`MatmulTask`, src/ops/kernel/q8_0/batch.rs:20-26); `weight` is a Q8Kernel."""
+
+    def __init__(self, weight, input, output, n_in, n_out):
+        self.weight, self.input, self.output, self.n_in, self.n_out = weight, input, output, n_in, n_out
+
+
+def matmul_q8_0_batch(tasks):
+    """`matmul_q8_0_batch` (batch.rs:32-79): every task is the f32-activation matmul over all of its rows; the
+    reference's 128-row chunks are a scheduling detail and leave each row's result unchanged."""
+    for t in tasks:
+        t.weight.matmul_q8_0(t.input, t.output, t.n_in, t.n_out)
 
 
 class Q4_0Kernel(Kernel):

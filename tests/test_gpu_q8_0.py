@@ -414,6 +414,30 @@ def test_legacy_f32_matmul_bit_exact(hip, oracle):
         assert np.array_equal(bits(out), bits(oracle.matmul_q8_0_f32(w, x[0], n_in, n_out, A)))
 
 
+def test_legacy_via_q8_and_batch(hip, oracle):
+    """`matmul_q8_0_via_q8` (legacy.rs:27-83) quantizes into the caller's scratch and runs the prequantized
+    GEMV; `matmul_q8_0_batch` (batch.rs:32-79) runs a list of f32-activation matmuls."""
+    K = hip.kernel
+    n_out, n_in = 200, 768
+    w, x = _case(hip, 1400, n_out, n_in)
+    kernel = K.Q8Kernel(w, n_in, n_out)
+    out = np.zeros(n_out, np.float32)
+    q8_buf, scale_buf = np.zeros(n_in, np.uint8), np.zeros(n_in // 32, np.float32)
+    kernel.matmul_q8_0_via_q8(x[0], out, n_in, n_out, q8_buf, scale_buf)
+    ref_q8, ref_sc = oracle.quantize_q8_0(x[0], A)
+    assert np.array_equal(q8_buf.view(np.int8), np.asarray(ref_q8).view(np.int8).reshape(-1))
+    assert np.array_equal(bits(scale_buf), bits(ref_sc))
+    assert np.array_equal(bits(out), bits(oracle.q8_0_forward_batched(w, x, n_in, n_out, A)[0]))
+    tasks, refs = [], []
+    for i, (no, ni) in enumerate([(64, 512), (130, 96), (257, 1024)]):
+        wi, xi = _case(hip, 1410 + i, no, ni)
+        tasks.append(K.MatmulTask(K.Q8Kernel(wi, ni, no), xi[0], np.zeros(no, np.float32), ni, no))
+        refs.append(oracle.matmul_q8_0_f32(wi, xi[0], ni, no, A))
+    K.matmul_q8_0_batch(tasks)
+    for t, r in zip(tasks, refs):
+        assert np.array_equal(bits(t.output), bits(r))
+
+
 def test_error_codes(hip):
     H, K = hip.hip, hip.kernel
     kernel = K.Q8Kernel(gen.make_q8_0_weight(4, 64, 0), 64, 4)
