@@ -264,7 +264,8 @@ int rmi_hip_expf_dev(const float *x, float *y, size_t n, void *stream);
 
 typedef struct {
     uint32_t n_embd, n_layer, n_head, n_head_kv, head_dim_k, head_dim_v, n_ff, vocab;
-    uint32_t capacity; /* positions the KV cache holds (prompt + generated) */
+    uint32_t capacity; /* positions the KV cache holds (prompt + generated); about 12 900 at most: one head's
+                        * scores and weights of all positions stay in a workgroup's LDS */
     float eps, freq_base;
     int32_t has_qk_norm;
     int32_t rounding; /* RMI_HIP_ROUND_* of the activation quantizer */

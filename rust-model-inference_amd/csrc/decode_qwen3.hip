@@ -629,6 +629,22 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     }
 }
 
+// Dynamic LDS an attention launch may use: 64 KiB unless more has been asked for, which is done once, for both
+// kernels; then what a compute unit has (160 KiB) less the kernels' static arrays (under 1 KiB).  With 12 bytes
+// per key that is about 13 000 keys.
+size_t attn_lds_limit() {
+    static const size_t limit = [] {
+        constexpr size_t kWant = 159 * 1024;
+        const bool ok = hipFuncSetAttribute(reinterpret_cast<const void *>(attention128_quant_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(kWant)) == hipSuccess &&
+                        hipFuncSetAttribute(reinterpret_cast<const void *>(attention_quant_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(kWant)) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+        return ok ? kWant : size_t(64 * 1024);
+    }();
+    return limit;
+}
+
 // gu = [W_gate x ; W_up x]: h = (W_up x) * silu(W_gate x), quantized to Q8_0
 __global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float *__restrict__ gu, uint32_t n_ff,
                                                              int8_t *__restrict__ q8, float *__restrict__ scales,
@@ -954,7 +970,7 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
         return rmi_fail(RMI_HIP_E_INVALID, "bad attention shape");
     const bool d128 = head_dim_k == 128 && head_dim_v == 128;
     const size_t lds = d128 ? attn128_lds_bytes(n_keys) : attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
-    if (lds > 64 * 1024) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
+    if (lds > attn_lds_limit()) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
     if (d128)
         hipLaunchKernelGGL(attention128_quant_kernel, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
                            q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding);
@@ -998,7 +1014,7 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
     }
     // attention keeps the scores of one head in LDS
     if ((c.head_dim_k == 128 && c.head_dim_v == 128 ? attn128_lds_bytes(c.capacity)
-                                                    : attn_lds_bytes(c.capacity, c.head_dim_k, c.head_dim_v)) > 64 * 1024) {
+                                                    : attn_lds_bytes(c.capacity, c.head_dim_k, c.head_dim_v)) > attn_lds_limit()) {
         rmi_set_error("capacity %u exceeds what the attention kernel holds in LDS", c.capacity);
         return nullptr;
     }
