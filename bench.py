@@ -117,11 +117,12 @@ def build_projection_set(pkg, batch, keep_host):
     return problems
 
 
-def make_group(H, recs, batch):
+def make_group(H, recs, batch, order="avx2"):
     n = len(recs)
     arr = lambda vals: (C.c_void_p * n)(*vals)  # noqa: E731
-    g = H.lib.rmi_hip_gemv_group_create(n, arr([r["kernel"].w.handle for r in recs]), arr([r["d_q8"].ptr for r in recs]),
-                                        arr([r["d_sc"].ptr for r in recs]), arr([r["d_y"].ptr for r in recs]), batch)
+    create = H.lib.rmi_hip_gemv_group_create_neon if order == "neon" else H.lib.rmi_hip_gemv_group_create
+    g = create(n, arr([r["kernel"].w.handle for r in recs]), arr([r["d_q8"].ptr for r in recs]),
+               arr([r["d_sc"].ptr for r in recs]), arr([r["d_y"].ptr for r in recs]), batch)
     if not g:
         raise RuntimeError(H.last_error())
     return g
@@ -134,7 +135,7 @@ def group_maxt(H, g):
     return "64" if waves.value == 1 else "512"
 
 
-def layer_groups(H, problems, batch):
+def layer_groups(H, problems, batch, order="avx2"):
     """[q,k,v] [o] [gate,up] [down] per layer, then lm_head: what a dependent decode step can fuse."""
     groups = []
     by_layer = {}
@@ -143,8 +144,8 @@ def layer_groups(H, problems, batch):
     for layer in sorted(k for k in by_layer if k >= 0):
         rs = {r["name"].split(".")[-1]: r for r in by_layer[layer]}
         for names in (("attn_q", "attn_k", "attn_v"), ("attn_output",), ("ffn_gate", "ffn_up"), ("ffn_down",)):
-            groups.append(make_group(H, [rs[n] for n in names], batch))
-    groups.append(make_group(H, by_layer[-1], batch))
+            groups.append(make_group(H, [rs[n] for n in names], batch, order))
+    groups.append(make_group(H, by_layer[-1], batch, order))
     return groups
 
 
@@ -242,21 +243,23 @@ def run_projection_set(args, pkg, ev):
     H, synth = pkg.hip, pkg.synth
     dev_name, cus, hbm = H.device_info()
     batch = args.batch
-    want_cpu = not args.no_cpu_baseline
+    neon = args.order == "neon"  # the small-batch MFMA kernel; the CPU leg below restates the AVX2 order only
+    want_cpu = not args.no_cpu_baseline and not neon
     problems = build_projection_set(pkg, batch, keep_host=want_cpu)
     alg_bytes = sum(synth.q8_0_gemv_bytes(r["n_out"], r["n_in"], batch) for r in problems)
     flops = sum(2 * r["n_out"] * r["n_in"] * batch for r in problems)
 
-    group_all = make_group(H, problems, batch)
-    groups_layer = layer_groups(H, problems, batch)
+    group_all = make_group(H, problems, batch, args.order)
+    groups_layer = layer_groups(H, problems, batch, args.order)
+    gemv_dev = H.lib.rmi_hip_gemv_q8_0_neon_dev if neon else H.lib.rmi_hip_gemv_q8_0_dev
 
     def step_grouped():
         H.check(H.lib.rmi_hip_gemv_group_run_dev(group_all, None))
 
     def step_per_matmul():
         for r in problems:
-            H.check(H.lib.rmi_hip_gemv_q8_0_dev(r["kernel"].w.handle, r["d_q8"].ptr, r["d_sc"].ptr, r["d_y"].ptr, batch,
-                                                r["n_out"], 0, r["n_out"], None))
+            H.check(gemv_dev(r["kernel"].w.handle, r["d_q8"].ptr, r["d_sc"].ptr, r["d_y"].ptr, batch, r["n_out"], 0,
+                             r["n_out"], None))
 
     def step_layer():
         for g in groups_layer:
@@ -274,7 +277,8 @@ def run_projection_set(args, pkg, ev):
     result = base_result(args, "Q8_0 GEMV HBM GB/s, Qwen3-0.6B shapes, 1 GPU", "GB/s", round(value, 1), wall,
                          "int8 dot4 -> f32", {
         "workload": f"Qwen3-0.6B per-token projection set (7x28 + lm_head = 197 Q8_0 GEMVs, 633 MB of weights), "
-                    f"decode batch {batch}, launch mode {args.mode}",
+                    f"decode batch {batch}, launch mode {args.mode}"
+                    + (", NEON accumulation order on the matrix cores" if neon else ""),
         "batch": batch,
         "launches_per_step": launches,
         "algorithmic_bytes_per_step": alg_bytes,
@@ -288,7 +292,9 @@ def run_projection_set(args, pkg, ev):
         "gflops": round(flops / wall / 1e9, 1),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_q8_0_kernel<%d,%s,%s>" % (batch, "true" if args.mode != "per_matmul" else "false",
+            "kernel": ("gemv_q8_0_mfma_kernel<%d,%s>" % ((batch + 15) // 16, "true" if args.mode != "per_matmul" else "false"))
+                      if neon else
+                      "gemv_q8_0_kernel<%d,%s,%s>" % (batch, "true" if args.mode != "per_matmul" else "false",
                                                        group_maxt(H, group_all) if args.mode == "grouped" else "*"),
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
@@ -779,7 +785,10 @@ def main():
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
                          "q4_0: Q4_0 x Q8_0 decode GEMV; q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); qlinear: QuantizedLinear::forward (Q4_K dequantise-and-dot, f32 activation); decode: end-to-end device-resident greedy decode "
                          "(one step = one 639-token-step generation)")
-    ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens)")
+    ap.add_argument("--batch", type=int, default=1, help="decode batch (1..8 tokens; 1..64 with --order neon)")
+    ap.add_argument("--order", choices=["avx2", "neon"], default="avx2",
+                    help="projection_set: accumulation order of the reference's x86-64 kernel (GEMV, the default) or of "
+                         "its aarch64 kernel (small-batch kernel on the matrix cores)")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill tokens M for --workload gemm")
     ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
     ap.add_argument("--no-cpu-baseline", action="store_true")

@@ -198,6 +198,14 @@ int rmi_hip_gemv_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
                           uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, void *stream);
 int rmi_hip_quantize_q8_0_dev(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
                               int rounding, void *stream);
+/* The same product for a small batch, 1..64 tokens whose activations fit the kernel's LDS staging
+ * (n_in * 1.14 bytes a token, 159 KiB in all), in the accumulation order of the reference's NEON kernel:
+ * sum = fma(float(dot_b), f32(w.d_b) * x_scale_b, sum) block after block (matmul_q8_0_vs_q8_0_neon,
+ * src/ops/kernel/q8_0/neon.rs:49-73), bit for bit, through int8 MFMA with the weights streamed once.  The
+ * AVX2-order call above converts eight partial sums per block and is bound by the vector ALU from four tokens
+ * on; this one stays bound by HBM.  Results of the two orders differ in the last bits only. */
+int rmi_hip_gemv_q8_0_neon_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                               uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, void *stream);
 /* Y[t][:] = W . Q8_0(X[t][:]) for n_tokens >= 1 through int8 MFMA. */
 int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                           uint32_t n_tokens, uint32_t y_stride, void *stream);
@@ -230,6 +238,10 @@ typedef struct rmi_hip_gemv_group rmi_hip_gemv_group;
 rmi_hip_gemv_group *rmi_hip_gemv_group_create(uint32_t n_problems, const rmi_hip_weight *const *weights,
                                               const int8_t *const *x_q8, const float *const *x_scales,
                                               float *const *y, uint32_t n_tokens);
+/* The same list (Q8_0 weights only) for 1..64 tokens through rmi_hip_gemv_q8_0_neon_dev's kernel. */
+rmi_hip_gemv_group *rmi_hip_gemv_group_create_neon(uint32_t n_problems, const rmi_hip_weight *const *weights,
+                                                   const int8_t *const *x_q8, const float *const *x_scales,
+                                                   float *const *y, uint32_t n_tokens);
 /* The same for Q4_K weights with Q8_K activations (three arrays per problem). */
 rmi_hip_gemv_group *rmi_hip_gemv_group_create_q4_k(uint32_t n_problems, const rmi_hip_weight *const *weights,
                                                    const float *const *q8k_d, const int8_t *const *q8k_qs,

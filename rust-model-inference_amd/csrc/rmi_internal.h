@@ -179,6 +179,14 @@ int rmi_launch_gemv_q8_0_norm(const rmi_hip_weight *w, const float *x_in, const 
 // workgroup belong to one problem (count 0 pads)
 int rmi_launch_gemv_q8_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,
                                uint32_t max_n_oct, uint32_t n_tokens, hipStream_t s);
+// Small batches (1..kMfmaMaxTokens tokens) through int8 MFMA in the order of the reference's NEON kernel; the
+// problem records and run tables of the GEMV.  `fits`: the tokens' activations fit the LDS staging.
+constexpr uint32_t kMfmaMaxTokens = 64;
+bool rmi_gemv_q8_0_mfma_fits(uint32_t n_tokens, uint32_t max_n_oct);
+size_t rmi_gemv_q8_0_mfma_lds_bytes(uint32_t n_tokens, uint32_t max_n_oct);
+int rmi_launch_gemv_q8_0_mfma(const RmiGemvProblem *single, const RmiGemvProblem *d_list, const uint4 *d_runs,
+                              uint32_t n_waves, uint32_t wpg, uint32_t tiles_per_wave, uint32_t max_n_oct,
+                              uint32_t n_tokens, hipStream_t s);
 uint32_t rmi_gemv_waves_per_group(size_t lds_bytes, size_t run_bytes);
 uint32_t rmi_gemv_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles, uint32_t n_tokens);
 int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s);
@@ -244,4 +252,5 @@ struct rmi_hip_gemv_group {
     uint32_t wpg = 1;  // waves per workgroup
     uint32_t max_units = 0;
     uint32_t n_tokens = 0;
+    bool mfma = false;  // Q8_0 only: the small-batch MFMA kernel (NEON order) instead of the GEMV (AVX2 order)
 };

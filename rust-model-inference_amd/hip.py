@@ -101,6 +101,8 @@ SIGNATURES = {
     "rmi_hip_gemv_q6_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_quantize_row_q8_k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_group_create": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u32]),
+    "rmi_hip_gemv_group_create_neon": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u32]),
+    "rmi_hip_gemv_q8_0_neon_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_gemv_group_create_q4_k": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                              C.POINTER(_vp), _u32]),
     "rmi_hip_gemv_group_create_q6_k": (_vp, [_u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),

@@ -278,9 +278,9 @@ def test_prequantized_batch_bit_exact(hip, oracle, n_tokens):
         assert np.array_equal(bits(out[t]), bits(oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, A))), t
 
 
-@pytest.mark.parametrize("n_tokens", [1, 4, 8, 15])
+@pytest.mark.parametrize("n_tokens", [1, 4, 8])
 def test_forward_batched_small_is_gemv_order(hip, oracle, n_tokens):
-    """Kernel::forward_batched below the GEMM threshold: device quantizer + GEMV, bit-exact."""
+    """Kernel::forward_batched up to 8 tokens: device quantizer + GEMV in the AVX2 order, bit-exact."""
     n_out, n_in = 512, 1024
     w, x = _case(hip, 800 + n_tokens, n_out, n_in, n_tokens)
     out = np.zeros((n_tokens, n_out), np.float32)
