@@ -200,8 +200,14 @@ int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, fl
         rc = mfma_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
     else if (n_tokens >= kGemmMinTokens)
         rc = rmi_launch_gemm_q8_0(w, d_q8, d_sc, d_y, n_tokens, n_out, c->stream);
-    else
-        rc = gemv_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
+    else {  // 9..15 tokens of a row too long for that: the same kernel, as many tokens at a time as fit
+        uint32_t chunk = n_tokens;
+        while (chunk > 0 && !rmi_gemv_q8_0_mfma_fits(chunk, w->n_units)) chunk--;
+        if (chunk == 0) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u is too long for the small-batch staging", n_in);
+        for (uint32_t t0 = 0; t0 < n_tokens && rc == RMI_HIP_OK; t0 += chunk)
+            rc = mfma_tokens(w, d_q8 + size_t(t0) * n_in, d_sc + size_t(t0) * (n_in / 32), d_y + size_t(t0) * n_out,
+                             n_tokens - t0 < chunk ? n_tokens - t0 : chunk, n_out, 0, n_out, c->stream);
+    }
     if (rc != RMI_HIP_OK) return rc;
     return fetch(c, output, d_y, size_t(n_tokens) * n_out * 4, 1);
 }

@@ -142,6 +142,19 @@ def test_forward_batched_takes_this_path(hip, oracle, n_tokens):
     assert np.array_equal(bits(out), bits(ref))
 
 
+def test_forward_batched_wide_rows_stay_in_this_order(hip, oracle):
+    """11 tokens of 16384 elements do not fit the staging at once (and are too few for the tiled GEMM): they go
+    through the same kernel a few at a time, so the order does not depend on the width."""
+    n_tokens, n_out, n_in = 11, 24, 16384
+    w = hip.synth.q8_0_weight(700, n_out, n_in)
+    x = hip.synth.activations(701, n_tokens, n_in)
+    out = np.zeros((n_tokens, n_out), np.float32)
+    hip.kernel.Q8Kernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out)
+    per = [oracle.quantize_q8_0(x[t], A) for t in range(n_tokens)]
+    ref = np.stack([oracle.matmul_q8_0_quantized(w, per[t][0], per[t][1], n_in, n_out, N) for t in range(n_tokens)])
+    assert np.array_equal(bits(out), bits(ref))
+
+
 def test_limits(hip):
     H = hip.hip
     k = hip.kernel.Q8Kernel(hip.synth.q8_0_weight(1, 16, 256), 256, 16)
