@@ -61,9 +61,11 @@ int gemv_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scal
 // staging of the tokens, short enough to fill the chip.  Measured on the Qwen3-0.6B set at 8 / 16 / 32 tokens:
 // twice the GEMV's run length with eight waves per workgroup is within 1 % of the best of {1,2,4,8} x {2,4,8}.
 uint32_t mfma_tiles_per_wave(uint32_t n_oct, uint32_t launch_tiles, uint32_t n_tokens) {
-    uint32_t tpw = 2 * rmi_gemv_tiles_per_wave(n_oct, launch_tiles, n_tokens);
-    if (n_tokens > 16) tpw *= 2;
-    return (tpw + 1) & ~1u;
+    const uint32_t base = rmi_gemv_tiles_per_wave(n_oct, launch_tiles, n_tokens);
+    uint32_t mul = n_tokens > 16 ? 4 : 2;
+    const uint32_t fill = uint32_t(rmi_device_cus()) * 8;  // a launch too small to fill the chip keeps short runs
+    while (mul > 1 && launch_tiles / (base * mul) < fill) mul >>= 1;
+    return (base * mul + 1) & ~1u;
 }
 
 // 1..kMfmaMaxTokens tokens in one launch of the small-batch MFMA kernel (NEON order)
@@ -194,9 +196,12 @@ int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, fl
     if (rc != RMI_HIP_OK) return rc;
     // up to 8 tokens: the GEMV (AVX2 order); beyond, the NEON order: the small-batch MFMA kernel while the tokens
     // fit its LDS staging, the tiled GEMM for more
+    // (measured per launch: the small-batch kernel is level with the GEMM or ahead up to 16 tokens for any matrix
+    // and up to 32 for one of lm_head's size; the GEMM leads from 17 tokens on for matrices of a few MB)
+    const bool small_batch = n_tokens <= 16 || (n_tokens <= 32 && w->n_tiles >= 4096);
     if (n_tokens <= 8)
         rc = gemv_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
-    else if (rmi_gemv_q8_0_mfma_fits(n_tokens, w->n_units))
+    else if (small_batch && rmi_gemv_q8_0_mfma_fits(n_tokens, w->n_units))
         rc = mfma_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
     else if (n_tokens >= kGemmMinTokens)
         rc = rmi_launch_gemm_q8_0(w, d_q8, d_sc, d_y, n_tokens, n_out, c->stream);
