@@ -58,22 +58,34 @@ __device__ __forceinline__ void stage_tokens(uint8_t *lds_q, float *lds_s, const
     float sv[kS];
     uint32_t sd[kS];
     bool slive[kS];
+    // piece i = (token t, piece c of its row); from one piece of a thread to its next both move by the same
+    // amounts, so one division per call does
+    const uint32_t q_dt = n_threads / row_u4, q_dc = n_threads - q_dt * row_u4;
+    const uint32_t s_dt = n_threads / row_s, s_dc = n_threads - s_dt * row_s;
     auto load_q = [&](uint32_t base) {
+        uint32_t t = base / row_u4, c = base - t * row_u4;
 #pragma unroll
         for (int j = 0; j < kQ; j++) {
-            const uint32_t i = base + j * n_threads, t = i / row_u4, c = i - t * row_u4;
+            const uint32_t i = base + j * n_threads;
             qlive[j] = i < total && c < src_u4;
             qd[j] = i < total ? t * stride_u4 + c : ~0u;
             v[j] = xq[qlive[j] ? t * src_u4 + c : 0];
+            c += q_dc;
+            t += q_dt + (c >= row_u4 ? 1u : 0u);
+            c -= c >= row_u4 ? row_u4 : 0u;
         }
     };
     auto load_s = [&](uint32_t base) {
+        uint32_t t = base / row_s, c = base - t * row_s;
 #pragma unroll
         for (int j = 0; j < kS; j++) {
-            const uint32_t i = base + j * n_threads, t = i / row_s, c = i - t * row_s;
+            const uint32_t i = base + j * n_threads;
             slive[j] = i < total_s && c < nb;
             sd[j] = i < total_s ? t * stride_s + c : ~0u;
             sv[j] = xs[slive[j] ? t * nb + c : 0];
+            c += s_dc;
+            t += s_dt + (c >= row_s ? 1u : 0u);
+            c -= c >= row_s ? row_s : 0u;
         }
     };
     // the empty asm statements keep the compiler from moving a load into the guarded store that uses it, where it
