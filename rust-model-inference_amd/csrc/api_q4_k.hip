@@ -276,8 +276,8 @@ static rmi_hip_gemv_group *group_create_kquant(int dtype, uint32_t n_problems, c
         e = hipMemcpy(g->d_runs, runs.data(), sizeof(uint4) * runs.size(), hipMemcpyHostToDevice);
     if (e != hipSuccess) {
         rmi_set_error("gemv group upload failed: %s", hipGetErrorString(e));
-        if (g->d_list) hipFree(g->d_list);
-        if (g->d_runs) hipFree(g->d_runs);
+        if (g->d_list) (void)hipFree(g->d_list);
+        if (g->d_runs) (void)hipFree(g->d_runs);
         delete g;
         return nullptr;
     }

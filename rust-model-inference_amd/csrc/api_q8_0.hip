@@ -406,8 +406,8 @@ static rmi_hip_gemv_group *group_create_q8_0(uint32_t n_problems, const rmi_hip_
         e = hipMemcpy(g->d_runs, runs.data(), sizeof(uint4) * runs.size(), hipMemcpyHostToDevice);
     if (e != hipSuccess) {
         rmi_set_error("gemv group upload failed: %s", hipGetErrorString(e));
-        if (g->d_list) hipFree(g->d_list);
-        if (g->d_runs) hipFree(g->d_runs);
+        if (g->d_list) (void)hipFree(g->d_list);
+        if (g->d_runs) (void)hipFree(g->d_runs);
         delete g;
         return nullptr;
     }
@@ -435,8 +435,8 @@ int rmi_hip_gemv_group_shape(const rmi_hip_gemv_group *g, uint32_t *n_workgroups
 
 void rmi_hip_gemv_group_destroy(rmi_hip_gemv_group *g) {
     if (!g) return;
-    if (g->d_list) hipFree(g->d_list);
-    if (g->d_runs) hipFree(g->d_runs);
+    if (g->d_list) (void)hipFree(g->d_list);
+    if (g->d_runs) (void)hipFree(g->d_runs);
     delete g;
 }
 

@@ -62,8 +62,8 @@ void *rmi_dev_buf(RmiThreadCtx *c, int slot, size_t nbytes) {
     if (c->dev_cap[slot] >= nbytes) return c->dev[slot];
     if (c->dev[slot]) {
         // the stream may still read the old buffer
-        hipStreamSynchronize(c->stream);
-        hipFree(c->dev[slot]);
+        (void)hipStreamSynchronize(c->stream);
+        (void)hipFree(c->dev[slot]);
         c->dev[slot] = nullptr;
         c->dev_cap[slot] = 0;
     }
@@ -80,8 +80,8 @@ void *rmi_pin_buf(RmiThreadCtx *c, int slot, size_t nbytes) {
     if (nbytes == 0) nbytes = 16;
     if (c->pin_cap[slot] >= nbytes) return c->pin[slot];
     if (c->pin[slot]) {
-        hipStreamSynchronize(c->stream);
-        hipHostFree(c->pin[slot]);
+        (void)hipStreamSynchronize(c->stream);
+        (void)hipHostFree(c->pin[slot]);
         c->pin[slot] = nullptr;
         c->pin_cap[slot] = 0;
     }
@@ -124,24 +124,24 @@ int rmi_hip_init(int device) {
 void rmi_hip_shutdown(void) {
     std::lock_guard<std::mutex> lock(g_mutex);
     if (g_device < 0) return;
-    hipDeviceSynchronize();
+    (void)hipDeviceSynchronize();
     for (RmiThreadCtx *c : g_ctxs) {
         for (int i = 0; i < 6; i++) {
-            if (c->dev[i]) hipFree(c->dev[i]);
-            if (c->pin[i]) hipHostFree(c->pin[i]);
+            if (c->dev[i]) (void)hipFree(c->dev[i]);
+            if (c->pin[i]) (void)hipHostFree(c->pin[i]);
             c->dev[i] = nullptr;
             c->pin[i] = nullptr;
             c->dev_cap[i] = c->pin_cap[i] = 0;
         }
         for (int i = 0; i < 2; i++) {
-            if (c->up_pin[i]) hipHostFree(c->up_pin[i]);
-            if (c->up_dev[i]) hipFree(c->up_dev[i]);
-            if (c->up_done[i]) hipEventDestroy(c->up_done[i]);
+            if (c->up_pin[i]) (void)hipHostFree(c->up_pin[i]);
+            if (c->up_dev[i]) (void)hipFree(c->up_dev[i]);
+            if (c->up_done[i]) (void)hipEventDestroy(c->up_done[i]);
             c->up_pin[i] = c->up_dev[i] = nullptr;
             c->up_done[i] = nullptr;
         }
         c->up_cap = 0;
-        if (c->stream) hipStreamDestroy(c->stream);
+        if (c->stream) (void)hipStreamDestroy(c->stream);
         c->stream = nullptr;
     }
     // contexts stay allocated: their owning threads may still hold the pointer
@@ -172,7 +172,7 @@ void *rmi_hip_malloc(size_t nbytes) {
 }
 
 void rmi_hip_free(void *dptr) {
-    if (dptr) hipFree(dptr);
+    if (dptr) (void)hipFree(dptr);
 }
 
 int rmi_hip_memcpy_h2d(void *dst, const void *src, size_t nbytes) {
@@ -247,8 +247,8 @@ static int upload_staging(RmiThreadCtx *c, size_t tile_src_bytes) {
     if (c->up_cap >= want) return RMI_HIP_OK;
     RMI_HIP_CHECK(hipStreamSynchronize(c->stream));
     for (int i = 0; i < 2; i++) {
-        if (c->up_pin[i]) hipHostFree(c->up_pin[i]);
-        if (c->up_dev[i]) hipFree(c->up_dev[i]);
+        if (c->up_pin[i]) (void)hipHostFree(c->up_pin[i]);
+        if (c->up_dev[i]) (void)hipFree(c->up_dev[i]);
         c->up_pin[i] = c->up_dev[i] = nullptr;
     }
     c->up_cap = 0;
@@ -445,7 +445,7 @@ rmi_hip_weight *rmi_hip_fuse_vstack(const rmi_hip_weight *a, const rmi_hip_weigh
 
 void rmi_hip_free_weight(rmi_hip_weight *w) {
     if (!w) return;
-    if (w->data) hipFree(w->data);
+    if (w->data) (void)hipFree(w->data);
     delete w;
 }
 
