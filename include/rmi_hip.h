@@ -97,8 +97,9 @@ int rmi_hip_matmul_q8_0_quantized_range(const rmi_hip_weight *w, const uint8_t *
 int rmi_hip_matmul_q8_0_quantized_batch(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
                                         float *output, uint32_t n_in, uint32_t n_out, uint32_t n_tokens);
 /* Kernel::forward / forward_batched with f32 input (trait_.rs:59-109):
- * quantize each token row on the device (rounding as given), then GEMV
- * (n_tokens < gemm_min_tokens) or the MFMA GEMM. */
+ * quantize each token row on the device (rounding as given), then the GEMV in
+ * the x86-64 kernel's order (1..8 tokens) or, from 9 tokens on, the matrix cores
+ * in the aarch64 kernel's order (the small-batch kernel, the tiled GEMM beyond). */
 int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
                                  uint32_t n_out, uint32_t n_tokens, int rounding);
 /* quantize_q8_0_into (src/ops/quant/q8_0.rs:3-24) run on the device. */
