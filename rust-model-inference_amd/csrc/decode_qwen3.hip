@@ -49,11 +49,8 @@ struct StepParams {
 __device__ __forceinline__ double wave_sum(double v) { return wave_sum_f64(v); }
 
 // x[e] = d * q of row `token` of a Q8_0 weight in the GEMV tile stream
-__global__ __launch_bounds__(256) void embed_q8_0_kernel(const uint8_t *__restrict__ w, uint32_t n_oct,
-                                                          const uint32_t *__restrict__ tok,
-                                                          const StepParams *__restrict__ sp, uint32_t vocab,
-                                                          float *__restrict__ x, uint32_t n_embd) {
-    uint32_t token = tok[sp->step];
+__device__ __forceinline__ void embed_row(const uint8_t *__restrict__ w, uint32_t n_oct, uint32_t token, uint32_t vocab,
+                                          float *__restrict__ x, uint32_t n_embd) {
     if (token >= vocab) token = vocab - 1;  // ids are validated on the host; never read outside the weight
     const uint8_t *tile = w + size_t(token >> 3) * n_oct * kOctetBytes;
     const uint32_t r = token & 7;
@@ -64,6 +61,13 @@ __global__ __launch_bounds__(256) void embed_q8_0_kernel(const uint8_t *__restri
                                                            (k >> 2) * 16 + (b & 3) * 4 + (k & 3));
         x[e] = h2f(dh) * float(int(q));
     }
+}
+// the first step's embedding; every later one is written by the step before it (argmax_final_kernel)
+__global__ __launch_bounds__(256) void embed_q8_0_kernel(const uint8_t *__restrict__ w, uint32_t n_oct,
+                                                          const uint32_t *__restrict__ tok,
+                                                          const StepParams *__restrict__ sp, uint32_t vocab,
+                                                          float *__restrict__ x, uint32_t n_embd) {
+    embed_row(w, n_oct, tok[sp->step], vocab, x, n_embd);
 }
 
 // x += r (if r), then rms_norm(x, weight) quantized to Q8_0.  One workgroup of 256; R float4 per thread stay in
@@ -713,8 +717,11 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const Top *__restrict
                                                            StepParams *__restrict__ sp,
                                                            uint32_t *__restrict__ tok, uint32_t *__restrict__ step_argmax,
                                                            float *__restrict__ step_top2,
-                                                           uint32_t *__restrict__ nonfinite_steps) {
+                                                           uint32_t *__restrict__ nonfinite_steps,
+                                                           const uint8_t *__restrict__ w_embd, uint32_t n_oct,
+                                                           uint32_t vocab, float *__restrict__ x, uint32_t n_embd) {
     __shared__ Top sm[256];
+    __shared__ uint32_t next_token;
     Top t{-INFINITY, -INFINITY, 0xffffffffu, 1u};
     for (uint32_t i = threadIdx.x; i < n_partial; i += 256) t = top_merge(t, partial[i]);
     const Top r = top_block_reduce(t, sm);
@@ -724,9 +731,12 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const Top *__restrict
         step_top2[2 * step] = r.best;
         step_top2[2 * step + 1] = r.second;
         if (!r.finite) atomicAdd(nonfinite_steps, 1u);
-        if (step + 1 >= n_prompt) tok[step + 1] = r.id;  // the next step reads its token here
-        sp->step = step + 1;                             // last kernel of the step: the next one sees the new position
+        if (step + 1 >= n_prompt) tok[step + 1] = r.id;  // the next step's token
+        next_token = step + 1 >= n_prompt ? r.id : tok[step + 1];
+        sp->step = step + 1;  // last kernel of the step: the next one sees the new position
     }
+    __syncthreads();
+    embed_row(w_embd, n_oct, next_token, vocab, x, n_embd);  // the next step starts from its token's embedding
 }
 
 }  // namespace
@@ -804,8 +814,9 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
     const int rnd = c.rounding;
     StepParams *sp = static_cast<StepParams *>(s->params);
     const size_t attn_lds = attn_lds_bytes(step + 1, c.head_dim_k, c.head_dim_v);
-    hipLaunchKernelGGL(embed_q8_0_kernel, dim3(1), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, sp, c.vocab,
-                       s->x, c.n_embd);
+    if (step == 0)
+        hipLaunchKernelGGL(embed_q8_0_kernel, dim3(1), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, sp, c.vocab,
+                           s->x, c.n_embd);
     const float *pending = nullptr;  // matmul output still to be added to the residual stream
     // the residual stream alternates between two buffers where the norm is folded into the next product
     float *x = s->x, *x_other = s->x2;
@@ -866,7 +877,8 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxGroups), dim3(256), 0, st, s->logits, c.vocab,
                        static_cast<Top *>(s->partial));
     hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, static_cast<const Top *>(s->partial),
-                       kArgmaxGroups, sp, s->tok, s->step_argmax, s->step_top2, s->nonfinite);
+                       kArgmaxGroups, sp, s->tok, s->step_argmax, s->step_top2, s->nonfinite, s->embd->data,
+                       s->embd->n_units, c.vocab, s->x, c.n_embd);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
