@@ -188,6 +188,19 @@ int rmi_hip_memcpy_h2d(void *dst, const void *src, size_t nbytes);
 int rmi_hip_memcpy_d2h(void *dst, const void *src, size_t nbytes);
 int rmi_hip_synchronize(void);
 
+/* Kernel::forward / forward_batched of a Q8_0 weight on device pointers WITHOUT any allocation: x f32
+ * [n_tokens][n_in] is quantized (rounding as given) and multiplied as rmi_hip_q8_0_forward_batched does, bit for
+ * bit, into y[t * y_stride + row].  No counterpart in the reference: it exists for callers that cannot allocate
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The quantized
+ * activation lives in a fixed 288 KiB array inside the library's code object, one copy per GPU, held until the
+ * process ends: n_tokens * n_in may not exceed RMI_HIP_NOALLOC_MAX_ELEMS (RMI_HIP_E_INVALID beyond), and calls
+ * that overlap on one GPU (two streams, two threads) race on it -- order them on one stream.  The calling
+ * thread's current device must be the one given to rmi_hip_init.  Calls no hipMalloc / hipFree, creates no
+ * stream, does not synchronise. */
+#define RMI_HIP_NOALLOC_MAX_ELEMS 262144
+int rmi_hip_q8_0_forward_noalloc_dev(const rmi_hip_weight *w, const float *x, float *y, uint32_t n_tokens,
+                                     uint32_t y_stride, int rounding, void *stream);
+
 /* Plain device-to-device streaming copy kernel (nbytes a multiple of 16).  No
  * counterpart in the reference: it is the known-size kernel against which
  * hardware HBM-traffic counters are calibrated when profiling. */

@@ -41,9 +41,11 @@ uint32_t gemv_chunk(const rmi_hip_weight *w) {
     return c > 8 ? 8 : c;
 }
 
+}  // namespace
+
 // device pointers in, rows [row_start,row_end) of n_tokens tokens
-int gemv_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
-                uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s) {
+int rmi_gemv_q8_0_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
+                         uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s) {
     const uint32_t chunk = gemv_chunk(w);
     if (chunk == 0) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u is too long for the GEMV staging", w->n_in);
     const uint32_t nb = w->n_in / 32;
@@ -56,6 +58,8 @@ int gemv_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scal
     }
     return RMI_HIP_OK;
 }
+
+namespace {
 
 // Runs of an even number of tiles (the small-batch kernel takes them in pairs), long enough to amortise the
 // staging of the tokens, short enough to fill the chip.  Measured on the Qwen3-0.6B set at 8 / 16 / 32 tokens:
@@ -122,7 +126,7 @@ int host_gemv_range(const rmi_hip_weight *w, const uint8_t *input_q8, const floa
     float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, size_t(n_tokens) * n_rows * 4));
     if (!d_y) return RMI_HIP_E_RUNTIME;
     // device y holds only the row slice: y[t][row - row_start]
-    rc = gemv_tokens(w, x.d_q8, x.d_scales, d_y - row_start, n_tokens, n_rows, row_start, row_end, c->stream);
+    rc = rmi_gemv_q8_0_tokens(w, x.d_q8, x.d_scales, d_y - row_start, n_tokens, n_rows, row_start, row_end, c->stream);
     if (rc != RMI_HIP_OK) return rc;
     if (out_stride == n_rows) return fetch(c, out_row_start, d_y, size_t(n_tokens) * n_rows * 4, 1);
     float *pin = static_cast<float *>(rmi_pin_buf(c, 1, size_t(n_tokens) * n_rows * 4));
@@ -200,7 +204,7 @@ int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, fl
     // and up to 32 for one of lm_head's size; the GEMM leads from 17 tokens on for matrices of a few MB)
     const bool small_batch = n_tokens <= 16 || (n_tokens <= 32 && w->n_tiles >= 4096);
     if (n_tokens <= 8)
-        rc = gemv_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
+        rc = rmi_gemv_q8_0_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
     else if (small_batch && rmi_gemv_q8_0_mfma_fits(n_tokens, w->n_units))
         rc = mfma_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
     else if (n_tokens >= kGemmMinTokens)
@@ -293,7 +297,7 @@ int rmi_hip_gemv_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
     if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
     if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
     if (rmi_misaligned(x_q8, x_scales, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
-    return gemv_tokens(w, x_q8, x_scales, y, n_tokens, y_stride, row_start, row_end, static_cast<hipStream_t>(stream));
+    return rmi_gemv_q8_0_tokens(w, x_q8, x_scales, y, n_tokens, y_stride, row_start, row_end, static_cast<hipStream_t>(stream));
 }
 
 int rmi_hip_gemv_q8_0_neon_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
@@ -498,7 +502,7 @@ int rmi_hip_q4_0_forward_batched(const rmi_hip_weight *w, const float *input, fl
     RMI_HIP_CHECK(hipMemcpyAsync(d_x, pin, n_x * 4, hipMemcpyHostToDevice, c->stream));
     int rc = rmi_launch_quantize_q8_0(d_x, d_q8, d_sc, n_tokens, n_in, rounding, c->stream);
     if (rc != RMI_HIP_OK) return rc;
-    rc = gemv_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
+    rc = rmi_gemv_q8_0_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
     if (rc != RMI_HIP_OK) return rc;
     return fetch(c, output, d_y, size_t(n_tokens) * n_out * 4, 1);
 }
@@ -531,7 +535,7 @@ int rmi_hip_gemv_q4_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
     if (y_stride < row_end && n_tokens > 1) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < row_end=%u", y_stride, row_end);
     if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
     if (rmi_misaligned(x_q8, x_scales, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
-    return gemv_tokens(w, x_q8, x_scales, y, n_tokens, y_stride, row_start, row_end, static_cast<hipStream_t>(stream));
+    return rmi_gemv_q8_0_tokens(w, x_q8, x_scales, y, n_tokens, y_stride, row_start, row_end, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

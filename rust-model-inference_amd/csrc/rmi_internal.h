@@ -117,6 +117,9 @@ RmiThreadCtx *rmi_thread_ctx();
 void *rmi_dev_buf(RmiThreadCtx *c, int slot, size_t nbytes);
 void *rmi_pin_buf(RmiThreadCtx *c, int slot, size_t nbytes);
 int rmi_device_cus();
+int rmi_device();  // the device rmi_hip_init bound, -1 before
+// the device address of the no-allocation entry point's scratch array on `device`, which must be current
+int rmi_noalloc_setup(int device);
 
 // ------------------------------------------------- launchers (device ptrs)
 // repack tiles [tile0, tile0 + n_tiles) of w; src = the source rows from row tile0 * 8 on (device memory)
@@ -150,6 +153,10 @@ struct RmiGemvProblem {
     uint32_t reserved;
 };
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
+// rows [row_start,row_end) of n_tokens tokens of a Q8_0 or Q4_0 weight, as many GEMV launches (x86-64 order) as
+// the LDS staging of the tokens asks for; device pointers, nothing allocated
+int rmi_gemv_q8_0_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
+                         uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s);
 // the same problem record with w = a Q4_0 tile stream (Q8_0 activation)
 int rmi_launch_gemv_q4_0(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
 int rmi_launch_gemv_q4_0_group(const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_runs, uint32_t wpg,

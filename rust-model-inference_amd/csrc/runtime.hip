@@ -35,6 +35,7 @@ int rmi_fail(int code, const char *fmt, ...) {
 
 bool rmi_ready() { return g_device >= 0; }
 int rmi_device_cus() { return g_cus; }
+int rmi_device() { return g_device; }
 
 RmiThreadCtx *rmi_thread_ctx() {
     if (t_ctx) return t_ctx;
@@ -114,6 +115,8 @@ int rmi_hip_init(int device) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return rmi_fail(RMI_HIP_E_NO_DEVICE, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
     RMI_HIP_CHECK(hipSetDevice(device));
+    int rc = rmi_noalloc_setup(device);
+    if (rc != RMI_HIP_OK) return rc;
     g_cus = prop.multiProcessorCount;
     g_hbm = prop.totalGlobalMem;
     snprintf(g_name, sizeof(g_name), "%s (%s)", prop.name, prop.gcnArchName);

@@ -17,6 +17,7 @@ DTYPE_Q4_K = 12
 DTYPE_Q6_K = 14
 ROUND_HALF_AWAY = 0
 ROUND_TIES_EVEN = 1
+NOALLOC_MAX_ELEMS = 262144
 
 _u8p = C.POINTER(C.c_uint8)
 _i8p = C.POINTER(C.c_int8)
@@ -93,6 +94,7 @@ SIGNATURES = {
     "rmi_hip_synchronize": (C.c_int, []),
     "rmi_hip_copy_dev": (C.c_int, [_vp, _vp, _sz, _vp]),
     "rmi_hip_gemv_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "rmi_hip_q8_0_forward_noalloc_dev": (C.c_int, [_vp, _vp, _vp, _u32, _u32, C.c_int, _vp]),
     "rmi_hip_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, _u32, C.c_int, _vp]),
     "rmi_hip_gemm_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
