@@ -242,6 +242,14 @@ void rmi_ref_rms_norm(const float *input, const float *weight, float *output, si
 void rmi_ref_rope_neox(float *x, size_t pos, size_t head_dim, float freq_base);
 void rmi_ref_rope_angles(size_t pos, size_t head_dim, float freq_base, float *cos_out, float *sin_out);
 void rmi_ref_silu_mul(const float *gate_out, float *up_out, size_t n);
+/* src/ops/attention.rs:28-38 (the x86-64, non-parity-trace branch: f32 sum, one division per element) */
+void rmi_ref_softmax(float *x, size_t n);
+/* src/ops/dot.rs:99-119 (f64 sum of f32 products) */
+float rmi_ref_dot_f16(const uint16_t *a, const uint16_t *b, size_t n);
+/* src/ops/embedding.rs:12-22 */
+void rmi_ref_embedding_lookup_q8_0(const uint8_t *weight, uint32_t token_id, size_t n_embd, float *out);
+/* src/models/qwen3.rs:172-191: 0 and the first strict maximum, or -1 for empty or non-finite logits */
+int rmi_ref_greedy_token(const float *logits, size_t n, uint32_t *token_id);
 void rmi_ref_attention_f16(const float *q, const uint16_t *k_cache, const uint16_t *v_cache, size_t step,
                            size_t kv_stride, size_t n_head, size_t n_head_kv, size_t hk, size_t hv, float *attn_out);
 

@@ -146,6 +146,39 @@ def attention_f16(q, k_cache, v_cache, step, kv_stride, n_head, n_head_kv, hk, h
     return out
 
 
+def softmax(x):
+    x = np.array(x, np.float32)
+    lib.rmi_ref_softmax(_p(x, _f32p), C.c_size_t(x.size))
+    return x
+
+
+lib.rmi_ref_dot_f16.restype = C.c_float
+
+
+def dot_f16(a, b):
+    a, b = np.ascontiguousarray(a, np.uint16), np.ascontiguousarray(b, np.uint16)
+    u16p = C.POINTER(C.c_uint16)
+    return np.float32(lib.rmi_ref_dot_f16(a.ctypes.data_as(u16p), b.ctypes.data_as(u16p), C.c_size_t(min(a.size, b.size))))
+
+
+def embedding_lookup_q8_0(weight, token_id, n_embd):
+    weight = np.ascontiguousarray(weight, np.uint8)
+    out = np.zeros(n_embd, np.float32)
+    lib.rmi_ref_embedding_lookup_q8_0(_p(weight, _u8p), C.c_uint32(token_id), C.c_size_t(n_embd), _p(out, _f32p))
+    return out
+
+
+lib.rmi_ref_greedy_token.restype = C.c_int
+
+
+def greedy_token(logits):
+    """Token id of the first strict maximum; None for empty or non-finite logits (the reference's Err)."""
+    logits = np.ascontiguousarray(logits, np.float32)
+    tid = C.c_uint32(0)
+    rc = lib.rmi_ref_greedy_token(_p(logits, _f32p), C.c_size_t(logits.size), C.byref(tid))
+    return None if rc != 0 else int(tid.value)
+
+
 def expf_array(x, restated=False):
     """exp of an f32 array through the host libm's expf, or through the restated formula"""
     x = np.ascontiguousarray(x, np.float32)

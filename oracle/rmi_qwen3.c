@@ -12,10 +12,13 @@
  *   silu_mul_inplace    src/ops/activation/mod.rs:137-151
  *   embedding_lookup    src/ops/embedding.rs:12-22
  *   greedy_token        src/models/qwen3.rs:172-191
- * expf/cosf/sinf/powf come from this host's libm, Rust's from its platform
- * libm: their last-ulp behaviour is "parity unpinned".  Both runs that the
- * tests compare (CPU matmuls vs. GPU matmuls) share this file, so the
- * comparison isolates the matmul back end.
+ * Pins (tests/test_oracle_qwen3.py): rms_norm, rms_norm_inplace and rope_neox by the reference's own bit
+ * vectors (src/ops/matmul_tests.rs:127-198); silu_mul_inplace by the scalar-order bit vector of
+ * tests/quantized_inference.rs:21-29 and, for operand order, the fixture of src/ops/matmul_tests.rs:361-372;
+ * greedy_token by src/models/qwen3.rs:1519-1522; softmax, dot_f16, the attention block and embedding_lookup_q8_0
+ * (no reference vector exists for the x86-64 branch) by an independent numpy statement with every rounding
+ * point enumerated; the loop's wiring by a second composition of the pinned pieces written from qwen3.rs.
+ * expf/cosf/sinf/powf come from this host's libm, as Rust's f32::exp/cos/sin/powf do on the same platform.
  *
  * Built with -mf16c (hardware f16 conversions, as the reference with
  * target-cpu=native, src/ops/float.rs:177-207).
@@ -96,6 +99,52 @@ static float dot_f16(const uint16_t *a, const uint16_t *b, size_t n) {
     return (float)sum;
 }
 
+/* src/ops/activation/mod.rs:137-151 (the scalar loop; x86-64 has no vector variant) */
+static void silu_mul_inplace(const float *gate, float *up, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float g = gate[i];
+        float s = g / (1.0f + expf(-g));
+        up[i] *= s;
+    }
+}
+
+/* src/ops/embedding.rs:12-22 */
+static void embedding_lookup_q8_0(const uint8_t *weight, uint32_t token_id, size_t n_embd, float *out) {
+    size_t bpr = n_embd / 32;
+    const uint8_t *row = weight + (size_t)token_id * bpr * 34;
+    for (size_t b = 0; b < bpr; b++) {
+        uint16_t dh;
+        memcpy(&dh, row + b * 34, 2);
+        float d = h2f(dh);
+        for (int jx = 0; jx < 32; jx++) out[b * 32 + jx] = d * (float)(int8_t)row[b * 34 + 2 + jx];
+    }
+}
+
+/* greedy_token (src/models/qwen3.rs:172-191): the first strict maximum; returns 0 when the logits are empty or
+ * one of them is not finite (the reference's Err).  `second` is the largest of the others (not in the
+ * reference: the decode tests compare it). */
+static int greedy_top2(const float *logits, size_t n, uint32_t *best_id, float *best_out, float *second_out) {
+    if (n == 0) return 0;
+    uint32_t id = 0;
+    float best = logits[0], second = -INFINITY;
+    int finite = isfinite(best);
+    for (size_t i = 1; i < n && finite; i++) {
+        float l = logits[i];
+        if (!isfinite(l)) finite = 0;
+        if (l > best) {
+            second = best;
+            best = l;
+            id = (uint32_t)i;
+        } else if (l > second) {
+            second = l;
+        }
+    }
+    *best_id = id;
+    *best_out = best;
+    *second_out = second;
+    return finite;
+}
+
 typedef struct {
     const rmi_ref_qwen3_model *m;
     const float *q;
@@ -152,14 +201,17 @@ void rmi_ref_rope_angles(size_t pos, size_t head_dim, float freq_base, float *co
         theta *= theta_scale;
     }
 }
-/* silu_mul_inplace(&gate_out, &mut up_out): up_out[i] *= gate_out[i] / (1 + exp(-gate_out[i])) */
-void rmi_ref_silu_mul(const float *gate_out, float *up_out, size_t n) {
-    for (size_t i = 0; i < n; i++) {
-        float g = gate_out[i];
-        float s = g / (1.0f + expf(-g));
-        up_out[i] *= s;
-    }
+void rmi_ref_softmax(float *x, size_t n) { softmax(x, n); }
+float rmi_ref_dot_f16(const uint16_t *a, const uint16_t *b, size_t n) { return dot_f16(a, b, n); }
+void rmi_ref_embedding_lookup_q8_0(const uint8_t *weight, uint32_t token_id, size_t n_embd, float *out) {
+    embedding_lookup_q8_0(weight, token_id, n_embd, out);
 }
+int rmi_ref_greedy_token(const float *logits, size_t n, uint32_t *token_id) {
+    float best, second;
+    return greedy_top2(logits, n, token_id, &best, &second) ? 0 : -1;
+}
+/* silu_mul_inplace(&gate_out, &mut up_out): up_out[i] *= gate_out[i] / (1 + exp(-gate_out[i])) */
+void rmi_ref_silu_mul(const float *gate_out, float *up_out, size_t n) { silu_mul_inplace(gate_out, up_out, n); }
 /* attention of one token over keys 0..step of an F16 cache laid out [t][kv_stride] (qwen3.rs:876-933) */
 void rmi_ref_attention_f16(const float *q, const uint16_t *k_cache, const uint16_t *v_cache, size_t step,
                            size_t kv_stride, size_t n_head, size_t n_head_kv, size_t hk, size_t hv, float *attn_out) {
@@ -233,16 +285,7 @@ int rmi_ref_qwen3_generate(const rmi_ref_qwen3_model *m, rmi_ref_matmul_fn matmu
     for (size_t step = 0; step < steps; step++) {
         size_t position = step; /* text prompt: positions 0..n-1, then last+1+i */
         uint32_t token = step < n_prompt ? prompt[step] : generated[n_generated - 1];
-        { /* embedding_lookup_q8_0 */
-            size_t bpr = n_embd / 32;
-            const uint8_t *row = m->token_embd + (size_t)token * bpr * 34;
-            for (size_t b = 0; b < bpr; b++) {
-                uint16_t dh;
-                memcpy(&dh, row + b * 34, 2);
-                float d = h2f(dh);
-                for (int jx = 0; jx < 32; jx++) x[b * 32 + jx] = d * (float)(int8_t)row[b * 34 + 2 + jx];
-            }
-        }
+        embedding_lookup_q8_0(m->token_embd, token, n_embd, x);
         for (size_t layer = 0; layer < m->n_layer; layer++) {
             rms_norm(x, m->attn_norm[layer], normed, n_embd, m->eps);
             rmi_ref_quantize_q8_0(normed, n_embd, q8, sc, qv);
@@ -271,11 +314,7 @@ int rmi_ref_qwen3_generate(const rmi_ref_qwen3_model *m, rmi_ref_matmul_fn matmu
             /* w_gate's output lands in up_buf and w_up's in gate_buf (qwen3.rs:996-1015) */
             MATMUL(m->w_gate[layer], up_buf, n_embd, n_ff);
             MATMUL(m->w_up[layer], gate_buf, n_embd, n_ff);
-            for (size_t i = 0; i < n_ff; i++) { /* silu_mul_inplace(&up, &mut gate) */
-                float g = up_buf[i];
-                float s = g / (1.0f + expf(-g));
-                gate_buf[i] *= s;
-            }
+            silu_mul_inplace(up_buf, gate_buf, n_ff); /* silu_mul_inplace(&up_buf, &mut gate_buf) */
             rmi_ref_quantize_q8_0(gate_buf, n_ff, q8, sc, qv);
             MATMUL(m->w_down[layer], down, n_ff, n_embd);
             for (size_t i = 0; i < n_embd; i++) x[i] += down[i];
@@ -284,21 +323,9 @@ int rmi_ref_qwen3_generate(const rmi_ref_qwen3_model *m, rmi_ref_matmul_fn matmu
         rmi_ref_quantize_q8_0(normed, n_embd, q8, sc, qv);
         MATMUL(m->output, logits, n_embd, m->vocab);
 
-        /* greedy_token: first strict maximum; non-finite logits are an error */
         uint32_t best_id = 0;
-        float best = logits[0], second = -INFINITY;
-        int finite = isfinite(best);
-        for (uint32_t i = 1; i < m->vocab && finite; i++) {
-            float l = logits[i];
-            if (!isfinite(l)) finite = 0;
-            if (l > best) {
-                second = best;
-                best = l;
-                best_id = i;
-            } else if (l > second) {
-                second = l;
-            }
-        }
+        float best = 0.0f, second = 0.0f;
+        int finite = greedy_top2(logits, m->vocab, &best_id, &best, &second);
         if (step_hash) step_hash[step] = fnv1a(logits, (size_t)m->vocab * 4);
         if (step_argmax) step_argmax[step] = best_id;
         if (step_top2) {
