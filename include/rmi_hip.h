@@ -46,6 +46,7 @@ extern "C" {
  * architecture (src/ops/quant/q8_0.rs:3-24). */
 #define RMI_HIP_ROUND_HALF_AWAY 0 /* scalar path, :49-71: 1/d, round()        */
 #define RMI_HIP_ROUND_TIES_EVEN 1 /* AVX2 path, :176-230: 127/amax, rint()    */
+#define RMI_HIP_ROUND_NEON 2      /* NEON path, :75-164: 1/d, nearest-even, clamped to [-127, 127] */
 
 typedef struct rmi_hip_weight rmi_hip_weight;
 
@@ -54,6 +55,10 @@ typedef struct rmi_hip_weight rmi_hip_weight;
 int rmi_hip_init(int device);
 void rmi_hip_shutdown(void);
 const char *rmi_hip_last_error(void);
+/* Diagnostic, no counterpart in the reference: how many per-thread contexts (a stream plus staging buffers) the
+ * library holds.  A thread that exits hands its context to the next new thread, so this is the largest number
+ * of threads that were inside the library at once, not the number of threads ever seen. */
+size_t rmi_hip_thread_context_count(void);
 /* name/arch of the bound device, compute units, bytes of HBM */
 int rmi_hip_device_info(char *name, size_t name_len, int *compute_units, size_t *hbm_bytes);
 
@@ -84,7 +89,11 @@ const void *rmi_hip_weight_device_data(const rmi_hip_weight *w);
 
 /* Kernel::forward_prequantized for Q8Kernel (src/ops/kernel/q8_0/mod.rs:33-55)
  * = matmul_q8_0_quantized_parallel_rows (q8_0/parallel.rs:102-139): `output`
- * is the FULL n_out-long slice; only rows of partition (ith, nth) are written. */
+ * is the FULL n_out-long slice; only rows of partition (ith, nth) are written.
+ * Activation quants of -128: the integer dot is exact (the scalar kernel, scalar.rs:49-53).  The reference's
+ * AVX2 kernel negates the activation byte where the weight is negative, which wraps -(-128), and saturates pair
+ * sums to i16 (avx2.rs:128-147): it is wrong wherever a -128 activation quant meets a negative weight, and
+ * this library does not follow it there.  No quantizer of the reference emits -128 from finite input. */
 int rmi_hip_q8_0_forward_prequantized(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
                                       float *output, uint32_t n_in, uint32_t n_out, uint32_t ith, uint32_t nth);
 /* matmul_q8_0_quantized_range (q8_0/dispatch.rs:27-108), the slot the Vulkan
@@ -98,10 +107,18 @@ int rmi_hip_matmul_q8_0_quantized_batch(const rmi_hip_weight *w, const uint8_t *
                                         float *output, uint32_t n_in, uint32_t n_out, uint32_t n_tokens);
 /* Kernel::forward / forward_batched with f32 input (trait_.rs:59-109):
  * quantize each token row on the device (rounding as given), then the GEMV in
- * the x86-64 kernel's order (1..8 tokens) or, from 9 tokens on, the matrix cores
- * in the aarch64 kernel's order (the small-batch kernel, the tiled GEMM beyond). */
+ * the x86-64 kernel's order for every token, eight tokens a launch.  As in the
+ * reference, a token's result does not depend on the batch it arrives in:
+ * forward_batched(x)[t] == forward(x[t]) bit for bit. */
 int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
                                  uint32_t n_out, uint32_t n_tokens, int rounding);
+/* The same call on the matrix cores, in the aarch64 kernel's accumulation order (neon.rs:49-73) for every
+ * token count: the small-batch kernel up to 16 tokens (32 for very tall matrices), the tiled int8-MFMA GEMM
+ * beyond.  Batch-independent in the same sense; with RMI_HIP_ROUND_NEON it is what an aarch64 host computes
+ * end to end.  Differs from the call above in the last bits only (within 1e-4 + 1e-4 |ref|); prefill-sized
+ * batches run one to two orders of magnitude faster here. */
+int rmi_hip_q8_0_forward_batched_neon(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                      uint32_t n_out, uint32_t n_tokens, int rounding);
 /* quantize_q8_0_into (src/ops/quant/q8_0.rs:3-24) run on the device. */
 int rmi_hip_quantize_q8_0(const float *input, uint32_t n, uint8_t *q8, float *scales, int rounding);
 /* The per-block int32 dots of scalar.rs:49-53, dots[n_out][n_in/32], computed
@@ -120,9 +137,15 @@ int rmi_hip_q4_k_forward_prepared(const rmi_hip_weight *w, const float *q8k_d, c
                                   const int16_t *q8k_bsums, float *output, uint32_t n_in, uint32_t n_out, uint32_t ith,
                                   uint32_t nth);
 /* Same with f32 input: quantize_row_q8_k on the device (quant/mod.rs:140-200),
- * the `q8_k == None` branch of q4_k.rs:77-84; n_tokens rows, token-major out. */
+ * the `q8_k == None` branch of q4_k.rs:77-84; n_tokens rows, token-major out, every token through the GEMV in
+ * the x86-64 kernel's order (forward_batched(x)[t] == forward(x[t]) bit for bit, trait_.rs:78-109). */
 int rmi_hip_q4_k_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
                                  uint32_t n_out, uint32_t n_tokens);
+/* The same call with prefill-sized batches (16 tokens and more) on the int8 matrix cores: exact integers, the
+ * f32 sum of an output as one chain over the super-blocks instead of the AVX2 kernel's 8 + 4 lane chains, so
+ * results agree with the call above within 1e-4 + 1e-4 |ref|, not bit for bit. */
+int rmi_hip_q4_k_forward_batched_mfma(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                      uint32_t n_out, uint32_t n_tokens);
 /* quantize_row_q8_k (quant/mod.rs:42-59) run on the device. */
 int rmi_hip_quantize_row_q8_k(const float *input, uint32_t n, float *d, int8_t *qs, int16_t *bsums);
 /* Q4_KKernel::forward_prequantized (q4_k.rs:20-54): dequantise-and-dot with
@@ -353,9 +376,15 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
 /* Uploads and repacks the weights (host slices may be dropped afterwards), allocates the KV cache. */
 rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_hip_qwen3_weights *weights);
 void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s);
-/* Runs n_prompt + max_new - 1 steps, one token per step, positions 0.. (the prompt is fed token by
- * token as generate_inner does), greedy sampling, no EOS.  Per step the argmax and the two largest
- * logits; full logits of the steps listed in dump_steps.  One synchronisation at the end.
+/* Token ids that end generation (the tokenizer's EOS id and "im_end", src/models/qwen3.rs:1123-1130); none by
+ * default.  At most 16. */
+int rmi_hip_qwen3_set_stop_ids(rmi_hip_qwen3 *s, const uint32_t *ids, uint32_t n_ids);
+/* Runs up to n_prompt + max_new - 1 steps, one token per step, positions 0.. (the prompt is fed token by
+ * token as generate_inner does), greedy sampling (temperature 0, sample_token's argmax branch).  With stop
+ * ids set the run ends at the first sampled stop id, which is not part of the result, as in generate_inner
+ * (checked by the host every 32 generated steps, so up to 31 further steps may have run); without, all steps
+ * are enqueued at once and synchronised once at the end.  Per step run the argmax and the two largest
+ * logits; full logits of the steps listed in dump_steps.
  * Returns the number of generated tokens or a negative code (non-finite logits are an error). */
 int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_prompt, uint32_t max_new,
                            uint32_t *generated, uint32_t *step_argmax, float *step_top2, const uint32_t *dump_steps,

@@ -129,6 +129,12 @@ class Q8Kernel : public Kernel {
         check(rmi_hip_q8_0_forward_batched(w_->get(), input, output, uint32_t(n_in), uint32_t(n_out),
                                            uint32_t(n_tokens), RMI_HIP_ROUND_TIES_EVEN));
     }
+    // the prefill path: the same product on the int8 matrix cores in the aarch64 kernel's accumulation order
+    void forward_batched_matrix_cores(const float *input, size_t n_tokens, float *output, size_t n_in, size_t n_out,
+                                      int rounding = RMI_HIP_ROUND_TIES_EVEN) const {
+        check(rmi_hip_q8_0_forward_batched_neon(w_->get(), input, output, uint32_t(n_in), uint32_t(n_out),
+                                                uint32_t(n_tokens), rounding));
+    }
     const std::shared_ptr<DeviceWeight> &weight() const { return w_; }
 
   private:

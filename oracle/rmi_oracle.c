@@ -158,21 +158,26 @@ static void quantize_q8_0_avx2(const float *input, size_t n, uint8_t *q8,
     }
 }
 
+/* vmaxq_f32 / vmaxvq_f32 hand a NaN on, vcvtnq_s32_f32 turns one into 0 */
 static void quantize_q8_0_neon(const float *input, size_t n, uint8_t *q8,
                                float *scales) {
     size_t blocks = n / QK8_0;
     for (size_t b = 0; b < blocks; b++) {
         const float *v = input + b * QK8_0;
         float amax = 0.0f;
-        for (int k = 0; k < QK8_0; k++) amax = fmaxf(amax, fabsf(v[k]));
+        for (int k = 0; k < QK8_0; k++) amax = (isnan(v[k]) || isnan(amax)) ? NAN : fmaxf(amax, fabsf(v[k]));
         float scale = amax / 127.0f;
         float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
         scales[b] = rmi_ref_f16_to_f32(rmi_ref_f32_to_f16(scale));
         for (int k = 0; k < QK8_0; k++) {
-            float c = fminf(fmaxf(v[k] * inv, -127.0f), 127.0f);
-            int32_t i = (int32_t)nearbyintf(c);
-            if (i < -127) i = -127;
-            if (i > 127) i = 127;
+            float t = v[k] * inv;
+            int32_t i = 0;
+            if (!isnan(t)) {
+                float c = fminf(fmaxf(t, -127.0f), 127.0f);
+                i = (int32_t)nearbyintf(c);
+                if (i < -127) i = -127;
+                if (i > 127) i = 127;
+            }
             q8[b * QK8_0 + k] = (uint8_t)(int8_t)i;
         }
     }

@@ -80,8 +80,11 @@ int rmi_hip_q4_k_forward_prepared(const rmi_hip_weight *w, const float *q8k_d, c
     return fetch(c, output + start, d_y, size_t(end - start) * 4, 1);
 }
 
-int rmi_hip_q4_k_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
-                                 uint32_t n_out, uint32_t n_tokens) {
+// Kernel::forward_batched of a Q4_K weight.  gemm = false: every token through the GEMV in the x86-64 kernel's
+// order (8 at a time), so a token's result does not depend on its batch, as in trait_.rs:78-109.  gemm = true:
+// from 16 tokens on the matrix-core GEMM, whose f32 sums are one chain per output (no reference order).
+static int q4_k_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                uint32_t n_out, uint32_t n_tokens, bool gemm) {
     RMI_REQUIRE_INIT();
     int rc = check_q4k(w, n_in, n_out);
     if (rc != RMI_HIP_OK) return rc;
@@ -98,11 +101,21 @@ int rmi_hip_q4_k_forward_batched(const rmi_hip_weight *w, const float *input, fl
     if (!d_x || !d_qs || !d_bs || !d_d || !d_y) return RMI_HIP_E_RUNTIME;
     rc = rmi_launch_quantize_q8_k(d_x, d_d, d_qs, d_bs, n_tokens, n_in, c->stream);
     if (rc != RMI_HIP_OK) return rc;
-    // prefill: the matrix-core GEMM; a few tokens: the GEMV in the x86-64 kernel's order
-    rc = n_tokens >= kGemmMinTokens ? rmi_launch_gemm_q4_k(w, d_d, d_qs, d_bs, d_y, n_tokens, n_out, c->stream)
-                                    : rmi_launch_gemv_q4_k(w, d_d, d_qs, d_bs, d_y, n_tokens, n_out, 0, n_out, c->stream);
+    rc = gemm && n_tokens >= kGemmMinTokens
+             ? rmi_launch_gemm_q4_k(w, d_d, d_qs, d_bs, d_y, n_tokens, n_out, c->stream)
+             : rmi_launch_gemv_q4_k(w, d_d, d_qs, d_bs, d_y, n_tokens, n_out, 0, n_out, c->stream);
     if (rc != RMI_HIP_OK) return rc;
     return fetch(c, output, d_y, size_t(n_tokens) * n_out * 4, 1);
+}
+
+int rmi_hip_q4_k_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens) {
+    return q4_k_forward_batched(w, input, output, n_in, n_out, n_tokens, false);
+}
+
+int rmi_hip_q4_k_forward_batched_mfma(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                      uint32_t n_out, uint32_t n_tokens) {
+    return q4_k_forward_batched(w, input, output, n_in, n_out, n_tokens, true);
 }
 
 int rmi_hip_quantize_row_q8_k(const float *input, uint32_t n, float *d, int8_t *qs, int16_t *bsums) {

@@ -178,8 +178,12 @@ int rmi_hip_matmul_q8_0_quantized_batch(const rmi_hip_weight *w, const uint8_t *
     return host_gemv_range(w, input_q8, input_scales, output, n_tokens, n_out, 0, n_out);
 }
 
-int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
-                                 uint32_t n_out, uint32_t n_tokens, int rounding) {
+// Kernel::forward / forward_batched on host slices.  x86_order: every token through the GEMV in the x86-64 kernel's
+// order, so a token's result does not depend on the batch it arrives in (forward_batched(x)[t] == forward(x[t]), as
+// in trait_.rs:78-109).  Otherwise the aarch64 kernel's order on the matrix cores, equally batch-independent: the
+// small-batch kernel while the tokens fit its LDS staging, the tiled GEMM for more.
+static int forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in, uint32_t n_out,
+                           uint32_t n_tokens, int rounding, bool x86_order) {
     RMI_REQUIRE_INIT();
     int rc = check_q8(w, n_in, n_out);
     if (rc != RMI_HIP_OK) return rc;
@@ -198,18 +202,16 @@ int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, fl
     RMI_HIP_CHECK(hipMemcpyAsync(d_x, pin, n_x * 4, hipMemcpyHostToDevice, c->stream));
     rc = rmi_launch_quantize_q8_0(d_x, d_q8, d_sc, n_tokens, n_in, rounding, c->stream);
     if (rc != RMI_HIP_OK) return rc;
-    // up to 8 tokens: the GEMV (AVX2 order); beyond, the NEON order: the small-batch MFMA kernel while the tokens
-    // fit its LDS staging, the tiled GEMM for more
     // (measured per launch: the small-batch kernel is level with the GEMM or ahead up to 16 tokens for any matrix
     // and up to 32 for one of lm_head's size; the GEMM leads from 17 tokens on for matrices of a few MB)
     const bool small_batch = n_tokens <= 16 || (n_tokens <= 32 && w->n_tiles >= 4096);
-    if (n_tokens <= 8)
+    if (x86_order)
         rc = rmi_gemv_q8_0_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
     else if (small_batch && rmi_gemv_q8_0_mfma_fits(n_tokens, w->n_units))
         rc = mfma_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
     else if (n_tokens >= kGemmMinTokens)
         rc = rmi_launch_gemm_q8_0(w, d_q8, d_sc, d_y, n_tokens, n_out, c->stream);
-    else {  // 9..15 tokens of a row too long for that: the same kernel, as many tokens at a time as fit
+    else {  // up to 15 tokens of a row too long for that: the same kernel, as many tokens at a time as fit
         uint32_t chunk = n_tokens;
         while (chunk > 0 && !rmi_gemv_q8_0_mfma_fits(chunk, w->n_units)) chunk--;
         if (chunk == 0) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u is too long for the small-batch staging", n_in);
@@ -219,6 +221,16 @@ int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, fl
     }
     if (rc != RMI_HIP_OK) return rc;
     return fetch(c, output, d_y, size_t(n_tokens) * n_out * 4, 1);
+}
+
+int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                 uint32_t n_out, uint32_t n_tokens, int rounding) {
+    return forward_batched(w, input, output, n_in, n_out, n_tokens, rounding, true);
+}
+
+int rmi_hip_q8_0_forward_batched_neon(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                      uint32_t n_out, uint32_t n_tokens, int rounding) {
+    return forward_batched(w, input, output, n_in, n_out, n_tokens, rounding, false);
 }
 
 int rmi_hip_quantize_q8_0(const float *input, uint32_t n, uint8_t *q8, float *scales, int rounding) {

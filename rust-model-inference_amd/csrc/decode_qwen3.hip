@@ -759,6 +759,7 @@ struct rmi_hip_qwen3 {
     void *partial = nullptr;
     void *params = nullptr;              // StepParams in HBM
     std::vector<void *> owned;  // every other device allocation, freed with the session
+    std::vector<uint32_t> stop_ids;  // generation ends before the first of these (EOS, im_end)
 };
 
 namespace {
@@ -1016,11 +1017,32 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
         return nullptr;
     }
     const rmi_hip_qwen3_config &c = *cfg;
+    if (!wt->attn_norm || !wt->ffn_norm || !wt->wq || !wt->wk || !wt->wv || !wt->wo || !wt->w_gate || !wt->w_up ||
+        !wt->w_down || (c.has_qk_norm && (!wt->q_norm || !wt->k_norm))) {
+        rmi_set_error("null per-layer weight array");
+        return nullptr;
+    }
+    for (uint32_t l = 0; l < c.n_layer; l++)
+        if (!wt->attn_norm[l] || !wt->ffn_norm[l] || !wt->wq[l] || !wt->wk[l] || !wt->wv[l] || !wt->wo[l] ||
+            !wt->w_gate[l] || !wt->w_up[l] || !wt->w_down[l] || (c.has_qk_norm && (!wt->q_norm[l] || !wt->k_norm[l]))) {
+            rmi_set_error("null weights in layer %u", l);
+            return nullptr;
+        }
+    // widths and cache rows are 32-bit in the kernels (the reference's checked_product, src/models/qwen3.rs:96-121)
+    const uint64_t kMax32 = 0x7fffffffull;
+    const uint64_t wide_q = uint64_t(c.n_head) * c.head_dim_k, wide_attn = uint64_t(c.n_head) * c.head_dim_v;
+    const uint64_t wide_kv = uint64_t(c.n_head_kv) * (c.head_dim_k > c.head_dim_v ? c.head_dim_k : c.head_dim_v);
+    if (wide_q > kMax32 || wide_attn > kMax32 || uint64_t(c.n_ff) * 2 > kMax32 || wide_q + 2 * wide_kv > kMax32 ||
+        uint64_t(c.capacity) * wide_kv > 0xffffffffull ||
+        uint64_t(c.n_layer) * c.capacity * wide_kv > (uint64_t(1) << 40)) {
+        rmi_set_error("unsupported model shape: a width or the KV cache overflows");
+        return nullptr;
+    }
     if (c.n_embd == 0 || c.n_embd % 32 || c.n_ff == 0 || c.n_ff % 32 || c.n_layer == 0 || c.n_head == 0 ||
         c.n_head_kv == 0 || c.n_head % c.n_head_kv || c.head_dim_k == 0 || c.head_dim_k % 32 || c.head_dim_v == 0 ||
         c.head_dim_v % 32 || c.head_dim_k > 1024 || c.head_dim_v > 1024 || c.vocab == 0 || c.capacity == 0 ||
         c.n_embd > kNormMaxN ||
-        (c.rounding != RMI_HIP_ROUND_TIES_EVEN && c.rounding != RMI_HIP_ROUND_HALF_AWAY)) {
+        (c.rounding != RMI_HIP_ROUND_TIES_EVEN && c.rounding != RMI_HIP_ROUND_HALF_AWAY && c.rounding != RMI_HIP_ROUND_NEON)) {
         rmi_set_error("unsupported model shape");
         return nullptr;
     }
@@ -1146,19 +1168,48 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
     if (e == hipSuccess) e = hipMemsetAsync(s->nonfinite, 0, 4, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     const auto t0 = std::chrono::steady_clock::now();
-    for (uint32_t step = 0; e == hipSuccess && rc == RMI_HIP_OK && step < steps; step++) {
-        rc = enqueue_step(s, step, st);
-        for (uint32_t d = 0; rc == RMI_HIP_OK && d < n_dump; d++)
-            if (dump_steps[d] == step)
-                e = hipMemcpyAsync(d_dump + size_t(d) * c.vocab, s->logits, size_t(c.vocab) * 4, hipMemcpyDeviceToDevice, st);
+    // Without stop ids every step is enqueued at once.  With them the host looks at the tokens every
+    // kStopCheck generated steps (one small copy) and ends the run at the first stop id, which is not part of
+    // the result (src/models/qwen3.rs:1123-1130: the loop breaks before the token is pushed).
+    constexpr uint32_t kStopCheck = 32;
+    const bool stops = !s->stop_ids.empty() && max_new > 0;
+    uint32_t n_valid = max_new, steps_done = 0, checked = 0;
+    std::vector<uint32_t> seen(stops ? max_new : 0);
+    while (e == hipSuccess && rc == RMI_HIP_OK && steps_done < steps) {
+        uint32_t until = steps;
+        if (stops) {
+            const uint32_t base = steps_done < n_prompt - 1 ? n_prompt - 1 : steps_done;
+            until = steps - base > kStopCheck ? base + kStopCheck : steps;
+        }
+        for (uint32_t step = steps_done; e == hipSuccess && rc == RMI_HIP_OK && step < until; step++) {
+            rc = enqueue_step(s, step, st);
+            for (uint32_t d = 0; rc == RMI_HIP_OK && d < n_dump; d++)
+                if (dump_steps[d] == step)
+                    e = hipMemcpyAsync(d_dump + size_t(d) * c.vocab, s->logits, size_t(c.vocab) * 4, hipMemcpyDeviceToDevice, st);
+        }
+        steps_done = until;
+        if (!stops || e != hipSuccess || rc != RMI_HIP_OK) continue;
+        const uint32_t have = steps_done - (n_prompt - 1);  // tokens sampled so far
+        e = hipStreamSynchronize(st);
+        if (e == hipSuccess && have > checked)
+            e = hipMemcpy(seen.data() + checked, s->tok + n_prompt + checked, size_t(have - checked) * 4, hipMemcpyDeviceToHost);
+        bool hit = false;
+        for (; e == hipSuccess && checked < have && !hit; checked++)
+            for (uint32_t id : s->stop_ids)
+                if (seen[checked] == id) {
+                    n_valid = checked;
+                    hit = true;
+                    break;
+                }
+        if (hit) break;
     }
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     if (seconds) *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     uint32_t nonfinite = 0;
     if (e == hipSuccess && rc == RMI_HIP_OK) {
-        if (max_new) e = hipMemcpy(generated, s->tok + n_prompt, size_t(max_new) * 4, hipMemcpyDeviceToHost);
-        if (e == hipSuccess && step_argmax) e = hipMemcpy(step_argmax, s->step_argmax, size_t(steps) * 4, hipMemcpyDeviceToHost);
-        if (e == hipSuccess && step_top2) e = hipMemcpy(step_top2, s->step_top2, size_t(steps) * 8, hipMemcpyDeviceToHost);
+        if (n_valid) e = hipMemcpy(generated, s->tok + n_prompt, size_t(n_valid) * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess && step_argmax) e = hipMemcpy(step_argmax, s->step_argmax, size_t(steps_done) * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess && step_top2) e = hipMemcpy(step_top2, s->step_top2, size_t(steps_done) * 8, hipMemcpyDeviceToHost);
         if (e == hipSuccess && n_dump) e = hipMemcpy(dump_logits, d_dump, size_t(n_dump) * c.vocab * 4, hipMemcpyDeviceToHost);
         if (e == hipSuccess) e = hipMemcpy(&nonfinite, s->nonfinite, 4, hipMemcpyDeviceToHost);
     }
@@ -1166,7 +1217,14 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
     if (rc != RMI_HIP_OK) return rc;
     if (e != hipSuccess) return rmi_fail(RMI_HIP_E_RUNTIME, "decode failed: %s", hipGetErrorString(e));
     if (nonfinite) return rmi_fail(RMI_HIP_E_RUNTIME, "non-finite logits in %u steps", nonfinite);
-    return int(max_new);
+    return int(n_valid);
+}
+
+int rmi_hip_qwen3_set_stop_ids(rmi_hip_qwen3 *s, const uint32_t *ids, uint32_t n_ids) {
+    if (!s || (n_ids && !ids)) return rmi_fail(RMI_HIP_E_INVALID, "null session or ids");
+    if (n_ids > 16) return rmi_fail(RMI_HIP_E_INVALID, "at most 16 stop ids");
+    s->stop_ids.assign(ids, ids + n_ids);
+    return RMI_HIP_OK;
 }
 
 }  // extern "C"

@@ -1,6 +1,6 @@
 // Device-side pieces shared by the activation quantizer and the kernels that
 // quantize their own output (norm, attention, SiLU): quantize_q8_0_into
-// (src/ops/quant/q8_0.rs:49-71 scalar, :176-230 AVX2) for 8 consecutive lanes
+// (src/ops/quant/q8_0.rs:49-71 scalar, :176-230 AVX2, :75-164 NEON) for 8 consecutive lanes
 // that hold one 32-element block, 4 consecutive elements each.
 #pragma once
 
@@ -16,6 +16,23 @@
 __device__ __forceinline__ uint32_t rmi_quantize_block8(float4 v, int rounding, float *scale) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = max8_lanes(amax);
+    if (rounding == RMI_HIP_ROUND_NEON) {
+        // the aarch64 host: vmaxq / vmaxvq hand a NaN on (fmaxf drops it), scale = amax / 127 with no zero test,
+        // 1 / scale, clamp to [-127, 127] before and after vcvtnq (nearest, ties to even; NaN gives 0)
+        const bool nan_here = v.x != v.x || v.y != v.y || v.z != v.z || v.w != v.w;
+        if (max8_lanes(nan_here ? 1.0f : 0.0f) != 0.0f) amax = __builtin_nanf("");
+        const float d = amax / 127.0f;
+        const float inv = d > 0.0f ? 1.0f / d : 0.0f;
+        const float t[4] = {v.x * inv, v.y * inv, v.z * inv, v.w * inv};
+        uint32_t packed = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int q = t[k] != t[k] ? 0 : int(rintf(fminf(fmaxf(t[k], -127.0f), 127.0f)));
+            packed |= uint32_t(q & 0xff) << (8 * k);
+        }
+        *scale = float(_Float16(d));
+        return packed;
+    }
     const float d = amax == 0.0f ? 0.0f : amax / 127.0f;
     float r0, r1, r2, r3;
     if (rounding == RMI_HIP_ROUND_TIES_EVEN) {

@@ -807,6 +807,8 @@ int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int3
 int rmi_launch_quantize_q8_0(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
                              int rounding, hipStream_t s) {
     const uint64_t n_blocks = uint64_t(n_tokens) * (n_in / 32);
+    if (rounding != RMI_HIP_ROUND_HALF_AWAY && rounding != RMI_HIP_ROUND_TIES_EVEN && rounding != RMI_HIP_ROUND_NEON)
+        return rmi_fail(RMI_HIP_E_INVALID, "unknown activation rounding %d", rounding);
     if (n_blocks == 0) return RMI_HIP_OK;
     if (n_blocks * 8 > 0xffffffffull) return rmi_fail(RMI_HIP_E_INVALID, "activation too large for one launch");
     const uint32_t grid = uint32_t((n_blocks * 8 + 255) / 256);

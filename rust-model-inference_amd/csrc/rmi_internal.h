@@ -101,6 +101,7 @@ inline bool rmi_misaligned(const void *quants, const void *a = nullptr, const vo
 // One per calling host thread: its own stream plus device and pinned host
 // buffers that grow on demand, so concurrent Kernel calls never share state.
 struct RmiThreadCtx {
+    uint64_t generation = 0;  // the library generation (count of shutdowns) its stream and buffers belong to
     hipStream_t stream = nullptr;
     // weight upload: two pinned and two device staging chunks taken in turn, an event per pair
     void *up_pin[2] = {nullptr, nullptr};

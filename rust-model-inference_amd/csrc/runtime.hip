@@ -1,4 +1,5 @@
 // Context, error reporting, per-thread staging, weight upload / fusion.
+#include <atomic>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -13,8 +14,25 @@ int g_cus = 0;
 size_t g_hbm = 0;
 char g_name[128] = "";
 std::mutex g_mutex;
+// Every context ever made; shutdown empties them (stream and buffers) and leaves the objects, whose owning
+// threads may still hold the pointer.  g_generation counts shutdowns: a context of an older generation has no
+// stream any more and is rebuilt on its owner's next call.
 std::vector<RmiThreadCtx *> g_ctxs;
-thread_local RmiThreadCtx *t_ctx = nullptr;
+std::vector<RmiThreadCtx *> g_idle;  // contexts of threads that have exited, handed to the next new thread
+std::atomic<uint64_t> g_generation{1};
+
+// The calling thread's context.  When the thread exits its context goes to the idle list, buffers and all, for
+// the next thread that needs one: no HIP call runs inside a thread-exit destructor, and a pool that keeps
+// starting and ending threads holds as many contexts as it has threads at once, not as many as it ever had.
+struct ThreadSlot {
+    RmiThreadCtx *c = nullptr;
+    ~ThreadSlot() {
+        if (!c) return;
+        std::lock_guard<std::mutex> lock(g_mutex);
+        g_idle.push_back(c);
+    }
+};
+thread_local ThreadSlot t_slot;
 
 }  // namespace
 
@@ -38,23 +56,47 @@ int rmi_device_cus() { return g_cus; }
 int rmi_device() { return g_device; }
 
 RmiThreadCtx *rmi_thread_ctx() {
-    if (t_ctx) return t_ctx;
+    const uint64_t generation = g_generation.load(std::memory_order_acquire);
+    RmiThreadCtx *c = t_slot.c;
+    if (c && c->generation == generation && c->stream) return c;
     if (hipSetDevice(g_device) != hipSuccess) {
         rmi_set_error("hipSetDevice(%d) failed", g_device);
         return nullptr;
     }
-    RmiThreadCtx *c = new RmiThreadCtx();
-    // default priority: mixed-priority streams are not used anywhere
-    if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
-        rmi_set_error("hipStreamCreate failed");
-        delete c;
-        return nullptr;
+    bool fresh = false;
+    if (!c) {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        if (!g_idle.empty()) {
+            c = g_idle.back();
+            g_idle.pop_back();
+        }
     }
-    {
+    if (!c) {
+        c = new RmiThreadCtx();
+        fresh = true;
+    }
+    if (c->generation != generation || !c->stream) {
+        // new, or emptied by a shutdown since its last use: shutdown left no stream and no buffers behind
+        c->stream = nullptr;
+        // default priority: mixed-priority streams are not used anywhere
+        if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
+            rmi_set_error("hipStreamCreate failed");
+            c->stream = nullptr;
+            if (fresh) delete c;
+            else {
+                std::lock_guard<std::mutex> lock(g_mutex);
+                g_idle.push_back(c);
+            }
+            t_slot.c = nullptr;
+            return nullptr;
+        }
+        c->generation = generation;
+    }
+    if (fresh) {
         std::lock_guard<std::mutex> lock(g_mutex);
         g_ctxs.push_back(c);
     }
-    t_ctx = c;
+    t_slot.c = c;
     return c;
 }
 
@@ -147,8 +189,15 @@ void rmi_hip_shutdown(void) {
         if (c->stream) (void)hipStreamDestroy(c->stream);
         c->stream = nullptr;
     }
-    // contexts stay allocated: their owning threads may still hold the pointer
+    // contexts stay allocated: their owning threads may still hold the pointer; the new generation tells them
+    // that stream and buffers are gone
+    g_generation.fetch_add(1, std::memory_order_acq_rel);
     g_device = -1;
+}
+
+size_t rmi_hip_thread_context_count(void) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    return g_ctxs.size();
 }
 
 int rmi_hip_device_info(char *name, size_t name_len, int *compute_units, size_t *hbm_bytes) {

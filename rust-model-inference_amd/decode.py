@@ -72,6 +72,11 @@ class Qwen3Session:
             raise hip.RmiHipError(-1, hip.last_error())
         return self
 
+    def set_stop_ids(self, ids):
+        """The tokenizer's EOS / `im_end` ids (src/models/qwen3.rs:1123-1130): generation ends before the first."""
+        ids = np.ascontiguousarray(ids, np.uint32)
+        hip.check(hip.lib.rmi_hip_qwen3_set_stop_ids(self._h, hip.ptr(ids, hip._u32p), ids.size))
+
     def generate(self, prompt, max_new, dump_steps=()):
         prompt = np.ascontiguousarray(prompt, np.uint32)
         steps = prompt.size + max_new - 1

@@ -17,6 +17,7 @@ DTYPE_Q4_K = 12
 DTYPE_Q6_K = 14
 ROUND_HALF_AWAY = 0
 ROUND_TIES_EVEN = 1
+ROUND_NEON = 2
 NOALLOC_MAX_ELEMS = 262144
 
 _u8p = C.POINTER(C.c_uint8)
@@ -54,6 +55,7 @@ SIGNATURES = {
     "rmi_hip_init": (C.c_int, [C.c_int]),
     "rmi_hip_shutdown": (None, []),
     "rmi_hip_last_error": (C.c_char_p, []),
+    "rmi_hip_thread_context_count": (_sz, []),
     "rmi_hip_device_info": (C.c_int, [C.c_char_p, _sz, C.POINTER(C.c_int), C.POINTER(_sz)]),
     "rmi_hip_upload_q8_0": (_vp, [_u8p, _sz, _u32, _u32]),
     "rmi_hip_upload_q4_k": (_vp, [_u8p, _sz, _u32, _u32]),
@@ -70,11 +72,13 @@ SIGNATURES = {
     "rmi_hip_matmul_q8_0_quantized_range": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32]),
     "rmi_hip_matmul_q8_0_quantized_batch": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32]),
     "rmi_hip_q8_0_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32, C.c_int]),
+    "rmi_hip_q8_0_forward_batched_neon": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32, C.c_int]),
     "rmi_hip_quantize_q8_0": (C.c_int, [_f32p, _u32, _u8p, _f32p, C.c_int]),
     "rmi_hip_block_dots_q8_0": (C.c_int, [_vp, _u8p, _i32p]),
     "rmi_hip_matmul_q8_0_f32": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32]),
     "rmi_hip_q4_k_forward_prepared": (C.c_int, [_vp, _f32p, _i8p, _i16p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_q4_k_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32]),
+    "rmi_hip_q4_k_forward_batched_mfma": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32]),
     "rmi_hip_quantize_row_q8_k": (C.c_int, [_f32p, _u32, _f32p, _i8p, _i16p]),
     "rmi_hip_q4_k_forward_prequantized": (C.c_int, [_vp, _u8p, _f32p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_quantized_linear_forward": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32]),
@@ -122,6 +126,7 @@ SIGNATURES = {
                                                           C.c_int, _vp]),
     "rmi_hip_qwen3_create": (_vp, [C.POINTER(Qwen3Config), C.POINTER(Qwen3Weights)]),
     "rmi_hip_qwen3_destroy": (None, [_vp]),
+    "rmi_hip_qwen3_set_stop_ids": (C.c_int, [_vp, _u32p, _u32]),
     "rmi_hip_qwen3_generate": (C.c_int, [_vp, _u32p, _u32, _u32, _u32p, _u32p, _f32p, _u32p, _u32, _f32p,
                                          C.POINTER(C.c_double)]),
     "rmi_hip_gguf_open": (_vp, [C.c_char_p]),

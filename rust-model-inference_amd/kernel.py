@@ -8,7 +8,8 @@ the Rust traits so that tests read like the reference's own:
   Q4_KKernel             src/ops/kernel/q4_k.rs:7-93
   Q6_KKernel             src/ops/kernel/q6_k.rs:7-80
   QuantizedTensor        src/ops/kernel/quantized_tensor.rs:32-190  (from_bytes / into_kernel)
-  QTensorOwned.fuse_vstack  src/ops/kernel/qtensor_owned.rs:138-164
+  QTensorOwned           src/ops/kernel/qtensor_owned.rs:34-164 (constructors, fuse_vstack), :167-255 (Kernel),
+                         :374-471 (Q8_K matmuls), :533-589 (quantize_and_matmul_with_scratch)
   QuantizedLinear, Layer, ExecContext   src/core/model.rs:12-104, src/core/traits.rs:45-74
   quantize_q8_0_into, quantize_row_q8_k  src/ops/quant/q8_0.rs:3-24, src/ops/quant/mod.rs:42-59
 
@@ -154,13 +155,16 @@ class Q8Kernel(Kernel):
         check(lib.rmi_hip_q8_0_forward_batched(self.w.handle, ptr(x, _f32p), ptr(_out(output, n_out), _f32p), n_in,
                                                n_out, 1, rounding))
 
-    def forward_batched(self, input, output, n_in, n_out, rounding=hip.ROUND_TIES_EVEN):
+    def forward_batched(self, input, output, n_in, n_out, rounding=hip.ROUND_TIES_EVEN, matrix_cores=False):
+        """`Kernel::forward_batched`.  By default every token goes through the x86-64-order GEMV, so
+        `forward_batched(x)[t] == forward(x[t])` bit for bit as in the reference; `matrix_cores=True` asks for
+        the aarch64 kernel's order on int8 MFMA (the prefill path), equally batch-independent."""
         x = as_f32(input).reshape(-1)
         n_tokens = x.size // n_in
         assert x.size == n_tokens * n_in
-        check(lib.rmi_hip_q8_0_forward_batched(self.w.handle, ptr(x, _f32p),
-                                               ptr(_out(output, n_tokens * n_out), _f32p), n_in, n_out, n_tokens,
-                                               rounding))
+        fn = lib.rmi_hip_q8_0_forward_batched_neon if matrix_cores else lib.rmi_hip_q8_0_forward_batched
+        check(fn(self.w.handle, ptr(x, _f32p), ptr(_out(output, n_tokens * n_out), _f32p), n_in, n_out, n_tokens,
+                 rounding))
 
     # free functions of the reference that take the weight slice as first argument
     def matmul_q8_0_quantized_range(self, input_q8, input_scales, output, n_in, row_start, row_end):
@@ -256,11 +260,13 @@ class Q4_KKernel(Kernel):
         check(lib.rmi_hip_q4_k_forward_prepared(self.w.handle, ptr(d, _f32p), ptr(qs, _i8p), ptr(bs, _i16p),
                                                 ptr(_out(output, n_out), _f32p), n_in, n_out, ith, nth))
 
-    def forward_batched(self, input, output, n_in, n_out):
+    def forward_batched(self, input, output, n_in, n_out, matrix_cores=False):
+        """Every token through the x86-64-order GEMV (bit-exact, batch-independent); `matrix_cores=True` takes
+        the int8 MFMA GEMM from 16 tokens on (exact integers, f32 within 1e-4 + 1e-4 |ref|)."""
         x = as_f32(input).reshape(-1)
         n_tokens = x.size // n_in
-        check(lib.rmi_hip_q4_k_forward_batched(self.w.handle, ptr(x, _f32p),
-                                               ptr(_out(output, n_tokens * n_out), _f32p), n_in, n_out, n_tokens))
+        fn = lib.rmi_hip_q4_k_forward_batched_mfma if matrix_cores else lib.rmi_hip_q4_k_forward_batched
+        check(fn(self.w.handle, ptr(x, _f32p), ptr(_out(output, n_tokens * n_out), _f32p), n_in, n_out, n_tokens))
 
     def block_ints(self, q8_k):
         _, qs, bs = _q8k_arrays(q8_k)
@@ -341,6 +347,115 @@ def fuse_vstack(a, b):
     if not handle:
         return None
     return type(a)(None, a.w.n_in, a.w.n_out + b.w.n_out, _handle=handle)
+
+
+class QTensorOwned(Kernel):
+    """`QTensorOwned` (src/ops/kernel/qtensor_owned.rs): the owned weight of the Qwen3.5 path.  Here every weight
+    is owned by construction (the bytes are copied to HBM), so this is the same device kernel behind the owned
+    type's method names.  Q8_0, Q4_K and Q6_K are offered; F32 / F16 / Q5_K stay on the host crate's CPU kernels
+    (`from_bytes_owned` returns None for them, which is the caller's signal to keep its own)."""
+
+    _KERNELS = {GGML_TYPE_Q8_0: Q8Kernel, GGML_TYPE_Q4_K: Q4_KKernel, GGML_TYPE_Q6_K: Q6_KKernel}
+
+    def __init__(self, ggml_type, kernel):
+        self._type, self.kernel = ggml_type, kernel
+
+    @classmethod
+    def from_bytes_owned(cls, data, ggml_type, n_cols, n_rows):
+        if ggml_type not in cls._KERNELS:
+            return None
+        return cls(ggml_type, cls._KERNELS[ggml_type](data, n_cols, n_rows))
+
+    @classmethod
+    def from_quantized(cls, q):
+        """`from_quantized(QuantizedTensor)`; Q4_0 is not modelled by the owned type (qtensor_owned.rs:129-133)."""
+        if q.ggml_type == GGML_TYPE_Q4_0:
+            raise ValueError("Q4_0 / Q4_1 not yet supported in QTensorOwned")
+        return cls.from_bytes_owned(q.data, q.ggml_type, q.n_in(), q.n_out())
+
+    def n_in(self):
+        return self.kernel.w.n_in
+
+    n_cols = n_in
+
+    def n_rows(self):
+        return self.kernel.w.n_out
+
+    def ggml_type(self):
+        return self._type
+
+    @staticmethod
+    def fuse_vstack(a, b):
+        """None when dtype or n_cols differ (qtensor_owned.rs:139-141)."""
+        if a._type != b._type:
+            return None
+        fused = fuse_vstack(a.kernel, b.kernel)
+        return None if fused is None else QTensorOwned(a._type, fused)
+
+    # ---- Kernel (qtensor_owned.rs:167-255)
+    def forward_prequantized(self, input_q8, input_scales, output, n_in, n_out, ith, nth):
+        self.kernel.forward_prequantized(input_q8, input_scales, output, n_in, n_out, ith, nth)
+
+    def forward_prepared(self, input_f32, input_q8, input_scales, q8_k, output, n_in, n_out, ith, nth):
+        if self._type == GGML_TYPE_Q8_0:  # Q8_0 ignores q8_k
+            self.kernel.forward_prequantized(input_q8, input_scales, output, n_in, n_out, ith, nth)
+        else:
+            self.kernel.forward_prepared(input_f32, input_q8, input_scales, q8_k, output, n_in, n_out, ith, nth)
+
+    # ---- Q8_K matmuls (qtensor_owned.rs:374-471)
+    def matmul_into_with_q8k(self, q8k, output, row_start, row_end):
+        """Rows [row_start, row_end) into `output[0 .. row_end - row_start]`."""
+        if self._type == GGML_TYPE_Q8_0:
+            raise ValueError("matmul_with_q8k called on non-K-quant weight type")
+        n_rows = self.n_rows()
+        full = np.zeros(n_rows, np.float32)
+        self.kernel.forward_prepared(None, None, None, q8k, full, self.n_in(), n_rows, 0, 1)
+        _out(output, row_end - row_start)[:row_end - row_start] = full[row_start:row_end]
+
+    def matmul_with_q8k_into_buf(self, q8k, buf):
+        self.matmul_into_with_q8k(q8k, buf, 0, self.n_rows())
+
+    def matmul_with_q8k(self, q8k):
+        out = np.zeros(self.n_rows(), np.float32)
+        self.matmul_with_q8k_into_buf(q8k, out)
+        return out
+
+    def matmul_with_q8k_into_buf_pooled(self, q8k, buf, pool=None):
+        """The reference splits rows over its pool; one launch covers them all here."""
+        self.matmul_with_q8k_into_buf(q8k, buf)
+
+    def matmul_into(self, input, output, row_start, row_end):
+        """K-quants: quantize_row_q8_k, then the Q8_K dot (qtensor_owned.rs:325-371).  The Q8_0 / F32 / F16 arms of
+        the reference dequantise and call dot_f32 per block, an f32-activation fallback off the quantized path."""
+        if self._type == GGML_TYPE_Q8_0:
+            raise NotImplementedError("QTensorOwned::matmul_into of a Q8_0 weight is the CPU dequantise-and-dot fallback")
+        self.matmul_into_with_q8k(quantize_row_q8_k(as_f32(input)[:self.n_in()]), output, row_start, row_end)
+
+    def matmul(self, input):
+        out = np.zeros(self.n_rows(), np.float32)
+        self.matmul_into(input, out, 0, self.n_rows())
+        return out
+
+    # ---- quantize + matmul (qtensor_owned.rs:516-589)
+    def quantize_and_matmul_with_scratch(self, input, q8k_buf, q8_buf, scale_buf, buf, pool=None,
+                                         rounding=hip.ROUND_TIES_EVEN):
+        """K-quants: `quantize_row_q8_k_into(input, q8k_buf[..blocks])`, then the Q8_K matmul.  Q8_0:
+        `quantize_q8_0_into(input, n_cols, q8_buf, scale_buf)`, then `matmul_q8_0_quantized_parallel_rows`.  The
+        scratch buffers hold the quantized activation afterwards, as in the reference."""
+        n_cols, n_rows = self.n_in(), self.n_rows()
+        x = as_f32(input)[:n_cols]
+        if self._type == GGML_TYPE_Q8_0:
+            quantize_q8_0_into(x, n_cols, q8_buf, scale_buf, rounding)
+            self.kernel.forward_prequantized(q8_buf[:n_cols], scale_buf[:n_cols // 32], buf, n_cols, n_rows, 0, 1)
+        else:
+            blocks = n_cols // 256
+            q8k_buf[:blocks] = quantize_row_q8_k(x)
+            self.matmul_with_q8k_into_buf_pooled(q8k_buf[:blocks], buf, pool)
+
+    def quantize_and_matmul(self, input, q8k_buf, buf):
+        n = as_f32(input).size
+        self.quantize_and_matmul_with_scratch(input, q8k_buf, np.zeros(n, np.uint8), np.zeros((n + 31) // 32, np.float32),
+                                              buf, None)
 
 
 @dataclass

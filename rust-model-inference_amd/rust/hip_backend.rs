@@ -45,6 +45,13 @@ extern "C" {
         w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
         rounding: c_int,
     ) -> c_int;
+    fn rmi_hip_q8_0_forward_batched_neon(
+        w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
+        rounding: c_int,
+    ) -> c_int;
+    fn rmi_hip_q4_k_forward_batched_mfma(
+        w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
+    ) -> c_int;
     fn rmi_hip_q4_k_forward_prepared(
         w: *const RmiHipWeight, d: *const f32, qs: *const i8, bsums: *const i16, output: *mut f32,
         n_in: u32, n_out: u32, ith: u32, nth: u32,
@@ -200,6 +207,26 @@ impl Kernel for HipKernel {
                                                            n_in as u32, n_out as u32, n_tokens),
             }
         });
+    }
+}
+
+impl HipKernel {
+    /// Prefill: `forward_batched` on the int8 matrix cores.  Q8_0 results follow the aarch64 kernel's order
+    /// (neon.rs:49-73), Q4_K results one f32 chain per output; both within 1e-4 + 1e-4*|ref| of `forward_batched`,
+    /// which stays bit-identical to the x86-64 kernels for every token count.
+    pub fn forward_batched_matrix_cores(&self, input: &[f32], output: &mut [f32], n_in: usize, n_out: usize) {
+        let n_tokens = (input.len() / n_in) as u32;
+        match self.dtype {
+            Dtype::Q8_0 => expect_ok(unsafe {
+                rmi_hip_q8_0_forward_batched_neon(self.handle, input.as_ptr(), output.as_mut_ptr(), n_in as u32,
+                                                  n_out as u32, n_tokens, ROUND_TIES_EVEN)
+            }),
+            Dtype::Q4K => expect_ok(unsafe {
+                rmi_hip_q4_k_forward_batched_mfma(self.handle, input.as_ptr(), output.as_mut_ptr(), n_in as u32,
+                                                  n_out as u32, n_tokens)
+            }),
+            _ => self.forward_batched(input, output, n_in, n_out),
+        }
     }
 }
 

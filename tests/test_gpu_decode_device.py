@@ -78,6 +78,47 @@ def test_small_model_device_decode_matches_cpu(hip, oracle, tmp_path):
     pool.close()
 
 
+def test_stop_ids_end_the_generation_before_the_stop_token(hip, tmp_path):
+    """generate_inner breaks at EOS / im_end before pushing the token (src/models/qwen3.rs:1123-1130)."""
+    kw = dict(n_layer=2, n_embd=256, n_head=4, n_head_kv=2, head_dim=64, n_ff=512, vocab=1000, n_ctx=4096)
+    f = _write_model(hip, tmp_path, **kw)
+    sess = hip.decode.Qwen3Session(f.metadata, _tensors(f), capacity=128)
+    prompt = np.random.default_rng(8).integers(0, 1000, 10, dtype=np.uint32)
+    full = sess.generate(prompt, 100)
+    assert full["tokens"].size == 100
+    for cut in (0, 5, 31, 32, 70):  # before, on and after a host check boundary
+        stop = int(full["tokens"][cut])
+        first = int(np.flatnonzero(full["tokens"] == stop)[0])
+        sess.set_stop_ids([stop, 999999])
+        got = sess.generate(prompt, 100)
+        assert got["tokens"].size == first and np.array_equal(got["tokens"], full["tokens"][:first]), cut
+    sess.set_stop_ids([])
+    assert np.array_equal(sess.generate(prompt, 100)["tokens"], full["tokens"])
+    sess.close()
+
+
+def test_create_rejects_null_and_overflowing_shapes(hip):
+    import ctypes as C
+
+    H = hip.hip
+    c = H.Qwen3Config()
+    c.n_embd, c.n_layer, c.n_head, c.n_head_kv, c.head_dim_k, c.head_dim_v = 64, 2, 2, 1, 32, 32
+    c.n_ff, c.vocab, c.capacity, c.eps, c.freq_base, c.has_qk_norm, c.rounding = 64, 10, 16, 1e-6, 1e6, 1, 1
+    w = H.Qwen3Weights()
+    embd, norm = np.zeros(10 * 2 * 34, np.uint8), np.ones(64, np.float32)
+    w.token_embd, w.output_norm = H.ptr(embd, H._u8p), H.ptr(norm, H._f32p)
+    assert not H.lib.rmi_hip_qwen3_create(C.byref(c), C.byref(w)) and "per-layer" in H.last_error()
+    mats = (H._u8p * 2)(H.ptr(np.zeros(64 * 2 * 34, np.uint8), H._u8p), None)
+    norms = (H._f32p * 2)(H.ptr(norm, H._f32p), H.ptr(norm, H._f32p))
+    for field in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
+        setattr(w, field, mats)
+    for field in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+        setattr(w, field, norms)
+    assert not H.lib.rmi_hip_qwen3_create(C.byref(c), C.byref(w)) and "layer 1" in H.last_error()
+    c.n_head, c.n_head_kv, c.head_dim_k, c.head_dim_v, c.n_layer = 1 << 24, 1 << 24, 1024, 1024, 1
+    assert not H.lib.rmi_hip_qwen3_create(C.byref(c), C.byref(w)) and "overflow" in H.last_error()
+
+
 def test_full_qwen3_0_6b_device_decode_512_plus_128(hip, oracle, tmp_path):
     """512 prompt tokens + 128 greedy tokens = 639 steps of a random-init Qwen3-0.6B-architecture Q8_0 GGUF."""
     f = _write_model(hip, tmp_path)  # 28 layers, 1024 wide, vocab 151936

@@ -120,7 +120,7 @@ def test_q4k_partition_and_fusion(hip, oracle):
     assert K.fuse_vstack(kg, K.Q8Kernel(gen.make_q8_0_weight(4, n_in, 0), n_in, 4)) is None
 
 
-@pytest.mark.parametrize("n_tokens", [1, 3, 8, 12])
+@pytest.mark.parametrize("n_tokens", [1, 3, 8, 12, 16, 40])
 def test_q4k_forward_batched(hip, oracle, n_tokens):
     n_out, n_in = 512, 2048
     w = hip.synth.q4_k_weight(70, n_out, n_in)
@@ -135,7 +135,7 @@ def test_q4k_forward_batched(hip, oracle, n_tokens):
 
 
 @pytest.mark.parametrize("n_tokens,n_out,n_in", [(64, 1000, 512), (37, 45, 256), (130, 6144, 2048), (300, 200, 6144),
-                                                  (16, 8, 256)])
+                                                  (16, 8, 256), (512, 6144, 2048), (512, 2048, 6144)])
 def test_q4k_gemm_mfma_parity(hip, oracle, n_tokens, n_out, n_in):
     """Prefill (>= 16 tokens) goes through the matrix cores: the integers are exact, the f32 sums run in one
     chain per output instead of the AVX2 kernel's lane chains.  Within 1e-4 + 1e-4*|ref| of the AVX2-order
@@ -144,7 +144,7 @@ def test_q4k_gemm_mfma_parity(hip, oracle, n_tokens, n_out, n_in):
     w = hip.synth.q4_k_weight(80 + n_tokens, n_out, n_in)
     x = hip.synth.activations(81 + n_out, n_tokens, n_in)
     out = np.zeros((n_tokens, n_out), np.float32)
-    hip.kernel.Q4_KKernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out)
+    hip.kernel.Q4_KKernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out, matrix_cores=True)
     wr = w.reshape(n_out, -1, 144)
     wd = wr[:, :, 0:2].copy().view(np.float16)[:, :, 0].astype(np.float64)
     wdmin = wr[:, :, 2:4].copy().view(np.float16)[:, :, 0].astype(np.float64)

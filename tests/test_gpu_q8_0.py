@@ -92,6 +92,37 @@ def test_block_dots_extreme_quants(hip, oracle):
     assert np.array_equal(hip.kernel.Q8Kernel(w, n_in, n_out).block_dots(q8), oracle.block_dots_q8_0(w, q8, n_in, n_out))
 
 
+def test_activation_quants_of_minus_128_follow_the_exact_integer_dot(hip, oracle):
+    """Prequantized input that holds -128: the device sums the exact products (the scalar kernel,
+    src/ops/kernel/q8_0/scalar.rs:49-53).  The x86-64 kernel negates the activation byte where the weight is
+    negative, which wraps -(-128) to -128, and saturates pair sums to i16 (avx2.rs:128-147): it is wrong on every
+    row that meets such a quant with a negative weight, and the device does not follow it there."""
+    n_out, n_in = 16, 64
+    w = hip.synth.q8_0_weight(431, n_out, n_in).reshape(n_out, 2, 34).copy()
+    hot = [(0, 0), (0, 1), (1, 7)]  # (block, element) of the activation quants set to -128
+    for b, k in hot:
+        w[2:8, b, 2 + k] = np.abs(w[2:8, b, 2 + k].view(np.int8)).view(np.uint8)  # rows 2..7: weights >= 0 there
+    w[0, 0, 2:4] = 0x80      # row 0: a -128 weight pair against the -128 activation pair
+    w[1, 1, 2 + 7] = 0x85    # row 1: one negative weight against a -128
+    w = np.ascontiguousarray(w).reshape(-1)
+    q8 = np.random.default_rng(432).integers(-127, 128, n_in, dtype=np.int8)
+    for b, k in hot:
+        q8[32 * b + k] = -128
+    sc = np.array([0.5, 0.25], np.float32)
+    kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
+    dots = kernel.block_dots(q8.view(np.uint8))
+    assert np.array_equal(dots, oracle.block_dots_q8_0(w, q8.view(np.uint8), n_in, n_out))
+    wq = w.reshape(n_out, 2, 34)[:, :, 2:].view(np.int8).astype(np.int64)
+    assert np.array_equal(dots, np.einsum("rbk,bk->rb", wq, q8.reshape(2, 32).astype(np.int64)))
+    out = np.zeros(n_out, np.float32)
+    kernel.forward_prequantized(q8.view(np.uint8), sc, out, n_in, n_out, 0, 1)
+    ref_s = oracle.matmul_q8_0_quantized(w, q8.view(np.uint8), sc, n_in, n_out, S)
+    ref_a = oracle.matmul_q8_0_quantized(w, q8.view(np.uint8), sc, n_in, n_out, A)
+    assert np.all(np.abs(out - ref_s) <= TOL(ref_s))
+    assert np.array_equal(bits(out[2:8]), bits(ref_a[2:8]))  # no negative weight meets a -128: the x86-64 bits
+    assert not np.all(np.abs(ref_a[:2] - ref_s[:2]) <= TOL(ref_s[:2]))  # the x86-64 kernel is off on rows 0, 1
+
+
 # ------------------------------------------------------------------------- GEMV
 
 QWEN_SHAPES = [(3072, 1024), (2048, 1024), (1024, 1024), (1024, 2048), (1024, 3072)]
@@ -235,7 +266,7 @@ def test_fused_vstack_matches_separate(hip, oracle):
 
 # -------------------------------------------------------------------- quantizer
 
-@pytest.mark.parametrize("rounding,variant", [(1, A), (0, S)])
+@pytest.mark.parametrize("rounding,variant", [(1, A), (0, S), (2, N)])
 def test_device_quantizer_bit_exact(hip, oracle, rounding, variant):
     rng = np.random.default_rng(600)
     x = (rng.standard_normal(32 * 4096) * rng.choice([1e-6, 1e-3, 1.0, 50.0, 3e4], 32 * 4096)).astype(np.float32)
@@ -255,7 +286,7 @@ def test_device_quantizer_reference_kats(hip):
     x = np.zeros(32, np.float32)
     x[0] = 1.0
     x[1] = np.array([0x3D11213E], np.uint32).view(np.float32)[0]
-    for rounding in (0, 1):
+    for rounding in (0, 1, 2):
         q8, sc = hip.kernel.quantize_q8_0(x, 32, rounding)
         assert list(q8.view(np.int8)[:2]) == [127, 4] and int(bits(sc)[0]) == 0x3C010000
     x = np.zeros(32, np.float32)
@@ -263,6 +294,30 @@ def test_device_quantizer_reference_kats(hip):
     assert list(hip.kernel.quantize_q8_0(x, 32, 0)[0].view(np.int8)[:3]) == [127, 1, -1]
     x[1] = 34.5
     assert hip.kernel.quantize_q8_0(x, 32, 1)[0].view(np.int8)[1] == 34
+    assert hip.kernel.quantize_q8_0(x, 32, 2)[0].view(np.int8)[1] == 34  # src/ops/matmul_tests.rs:546-556
+    # src/ops/matmul_tests.rs:528-544: the NEON quantizer equals the scalar one on this input
+    x = np.array([((i % 17) - 8) * 0.125 for i in range(64)], np.float32)
+    qs, ss = hip.kernel.quantize_q8_0(x, 64, 0)
+    qn, sn = hip.kernel.quantize_q8_0(x, 64, 2)
+    assert np.array_equal(qs, qn) and np.array_equal(bits(ss), bits(sn))
+
+
+def test_device_quantizer_neon_clamps_and_non_finite(hip, oracle):
+    """The aarch64 quantizer never emits -128 and turns a block with a NaN or an infinity into zeros (vmaxq hands
+    the NaN on, 1/scale becomes 0 or the product NaN, vcvtnq of NaN is 0); the x86-64 one can emit -128."""
+    x = hip.synth.activations(5, 1, 32 * 64)[0]
+    x[40] = np.nan
+    x[70] = np.inf
+    x[100] = -np.inf
+    q8, sc = hip.kernel.quantize_q8_0(x, x.size, 2)
+    rq, rs = oracle.quantize_q8_0(x, N)
+    assert np.array_equal(q8, rq)
+    ok = np.isfinite(rs)
+    assert np.array_equal(bits(sc)[ok], bits(rs)[ok]) and np.array_equal(np.isnan(sc), np.isnan(rs))
+    assert not q8[32:64].any() and not q8[64:128].any() and np.isnan(sc[1]) and np.isinf(sc[2])
+    assert q8.view(np.int8).min() >= -127
+    assert hip.hip.lib.rmi_hip_quantize_q8_0(hip.hip.ptr(x, hip.hip._f32p), 32, hip.hip.ptr(q8, hip.hip._u8p),
+                                             hip.hip.ptr(sc, hip.hip._f32p), 7) == -1
 
 
 # ------------------------------------------------------------- batches and GEMM
@@ -295,7 +350,7 @@ def test_gemm_mfma_parity(hip, oracle, n_tokens, n_out, n_in):
     the fused sequential (NEON) order; within tolerance of the x86-64 (AVX2) order."""
     w, x = _case(hip, 900 + n_tokens + n_out, n_out, n_in, n_tokens)
     out = np.zeros((n_tokens, n_out), np.float32)
-    hip.kernel.Q8Kernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out)
+    hip.kernel.Q8Kernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out, matrix_cores=True)
     q8, sc = _quantize_rows(oracle, x)
     ref_n = np.stack([oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, N) for t in range(n_tokens)])
     assert np.array_equal(bits(out), bits(ref_n))
@@ -341,21 +396,77 @@ def test_gemm_special_scales(hip, oracle):
     assert np.count_nonzero((prod != 0) & (np.abs(prod) < 1.17549435e-38)) > 1000
 
 
-def test_gemm_full_size_properties(hip, oracle):
-    """M=2048 x (3072 x 1024): rows sampled against the checker; every token row equals
-    the same token run through a 64-token call (tile position must not change bits)."""
-    n_tokens, n_out, n_in = 2048, 3072, 1024
-    w, x = _case(hip, 1000, n_out, n_in, n_tokens)
+@pytest.mark.parametrize("n_tokens,n_out,n_in", [(2048, 3072, 1024), (2048, 1024, 3072), (512, 3072, 1024),
+                                                  (512, 1024, 3072)])
+def test_gemm_full_size_properties(hip, oracle, n_tokens, n_out, n_in):
+    """The prefill configuration at its stated sizes (M = 512 and 2048, the FFN up and down shapes): token rows
+    sampled against the checker's NEON order, bit for bit, and within tolerance of the x86-64 order; every token
+    row equals the same token run through a 64-token call (tile position must not change bits)."""
+    w, x = _case(hip, 1000 + n_tokens + n_in, n_out, n_in, n_tokens)
     kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
     out = np.zeros((n_tokens, n_out), np.float32)
-    kernel.forward_batched(x, out, n_in, n_out)
-    sample = [0, 1, 63, 64, 1023, 2047]
+    kernel.forward_batched(x, out, n_in, n_out, matrix_cores=True)
+    sample = [0, 1, 63, 64, n_tokens // 2 - 1, n_tokens - 1]
     q8, sc = _quantize_rows(oracle, x[sample])
     for i, t in enumerate(sample):
         assert np.array_equal(bits(out[t]), bits(oracle.matmul_q8_0_quantized(w, q8[i], sc[i], n_in, n_out, N)))
+        ref_a = oracle.matmul_q8_0_quantized(w, q8[i], sc[i], n_in, n_out, A)
+        assert np.all(np.abs(out[t] - ref_a) <= TOL(ref_a))
+    lo = n_tokens // 2 - 24
     part = np.zeros((64, n_out), np.float32)
-    kernel.forward_batched(x[1000:1064], part, n_in, n_out)
-    assert np.array_equal(bits(part), bits(out[1000:1064]))
+    kernel.forward_batched(x[lo:lo + 64], part, n_in, n_out, matrix_cores=True)
+    assert np.array_equal(bits(part), bits(out[lo:lo + 64]))
+
+
+@pytest.mark.parametrize("n_tokens", [9, 16, 17, 40])
+def test_forward_batched_does_not_depend_on_the_batch(hip, oracle, n_tokens):
+    """trait_.rs:78-109: every token goes through the same quantizer and kernel, so forward_batched(x)[t] ==
+    forward(x[t]) bit for bit, and both are the x86-64 kernel's result, for any token count."""
+    n_out, n_in = 520, 1024
+    w, x = _case(hip, 1900 + n_tokens, n_out, n_in, n_tokens)
+    kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
+    out = np.zeros((n_tokens, n_out), np.float32)
+    kernel.forward_batched(x, out, n_in, n_out)
+    for t in range(n_tokens):
+        one = np.zeros(n_out, np.float32)
+        kernel.forward(x[t], one, n_in, n_out)
+        assert np.array_equal(bits(out[t]), bits(one)), t
+    assert np.array_equal(bits(out), bits(oracle.q8_0_forward_batched(w, x, n_in, n_out, A)))
+    # the matrix-core path is batch-independent too, in its own (aarch64) order
+    mc = np.zeros((n_tokens, n_out), np.float32)
+    kernel.forward_batched(x, mc, n_in, n_out, matrix_cores=True)
+    one = np.zeros((1, n_out), np.float32)
+    kernel.forward_batched(x[n_tokens - 1], one, n_in, n_out, matrix_cores=True)
+    assert np.array_equal(bits(mc[n_tokens - 1]), bits(one[0]))
+
+
+@pytest.mark.parametrize("n_tokens", [1, 5, 16, 33, 100])
+def test_aarch64_host_end_to_end(hip, oracle, n_tokens):
+    """What an aarch64 host computes: its own quantizer (1/d, ties to even, clamp to [-127, 127],
+    src/ops/quant/q8_0.rs:75-164) and its kernel's order (neon.rs:49-73), for any token count."""
+    n_out, n_in = 264, 1024
+    w, x = _case(hip, 1950 + n_tokens, n_out, n_in, n_tokens)
+    out = np.zeros((n_tokens, n_out), np.float32)
+    hip.kernel.Q8Kernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out, rounding=hip.hip.ROUND_NEON,
+                                                        matrix_cores=True)
+    assert np.array_equal(bits(out), bits(oracle.q8_0_forward_batched(w, x, n_in, n_out, N)))
+
+
+def test_batch_8_on_the_lm_head(hip, oracle):
+    """Decode batch 8 on the 151 936-row head: rows sampled against the checker's x86-64 order."""
+    n_tokens, n_out, n_in = 8, 151936, 1024
+    w, x = _case(hip, 1990, n_out, n_in, n_tokens)
+    q8, sc = _quantize_rows(oracle, x)
+    out = np.zeros((n_tokens, n_out), np.float32)
+    kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
+    kernel.matmul_q8_0_quantized_batch(q8, sc, out, n_in, n_out, n_tokens)
+    rows = np.unique(np.concatenate([np.arange(0, 24), np.arange(n_out - 24, n_out),
+                                     np.random.default_rng(5).integers(0, n_out, 2000)]))
+    wr = np.ascontiguousarray(w.reshape(n_out, -1)[rows]).reshape(-1)
+    for t in range(n_tokens):
+        ref = oracle.matmul_q8_0_quantized(wr, q8[t], sc[t], n_in, rows.size, A)
+        assert np.array_equal(bits(out[t, rows]), bits(ref)), t
+    assert np.isfinite(out).all()
 
 
 # -------------------------------------------------------------- device-resident

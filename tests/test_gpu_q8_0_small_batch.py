@@ -131,12 +131,12 @@ def test_special_scales(hip, oracle):
 
 @pytest.mark.parametrize("n_tokens", [9, 15, 16, 40, 64])
 def test_forward_batched_takes_this_path(hip, oracle, n_tokens):
-    """Kernel::forward_batched from 9 tokens on is in the NEON order, whichever kernel runs."""
+    """The matrix-core variant of Kernel::forward_batched is in the NEON order, whichever kernel runs."""
     n_out, n_in = 520, 1024
     w = hip.synth.q8_0_weight(600 + n_tokens, n_out, n_in)
     x = hip.synth.activations(610 + n_tokens, n_tokens, n_in)
     out = np.zeros((n_tokens, n_out), np.float32)
-    hip.kernel.Q8Kernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out)
+    hip.kernel.Q8Kernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out, matrix_cores=True)
     per = [oracle.quantize_q8_0(x[t], A) for t in range(n_tokens)]
     ref = np.stack([oracle.matmul_q8_0_quantized(w, per[t][0], per[t][1], n_in, n_out, N) for t in range(n_tokens)])
     assert np.array_equal(bits(out), bits(ref))
@@ -149,7 +149,7 @@ def test_forward_batched_wide_rows_stay_in_this_order(hip, oracle):
     w = hip.synth.q8_0_weight(700, n_out, n_in)
     x = hip.synth.activations(701, n_tokens, n_in)
     out = np.zeros((n_tokens, n_out), np.float32)
-    hip.kernel.Q8Kernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out)
+    hip.kernel.Q8Kernel(w, n_in, n_out).forward_batched(x, out, n_in, n_out, matrix_cores=True)
     per = [oracle.quantize_q8_0(x[t], A) for t in range(n_tokens)]
     ref = np.stack([oracle.matmul_q8_0_quantized(w, per[t][0], per[t][1], n_in, n_out, N) for t in range(n_tokens)])
     assert np.array_equal(bits(out), bits(ref))
