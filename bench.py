@@ -84,6 +84,29 @@ def physical_cores():
     return os.cpu_count() or 1
 
 
+THREADS_OVERRIDE = None  # --threads
+
+
+def cpu_threads():
+    """Threads of the CPU legs: the host's physical core count, unless the job's own CPU share is smaller.  The
+    share is what OMP_NUM_THREADS says (the scheduler of a shared GPU host sets it to the cores that belong to the
+    job, and asks worker pools to stay within it whatever /proc/cpuinfo shows); --threads overrides both."""
+    detected = physical_cores()
+    info = {"physical_cores_detected": detected, "logical_cpus": os.cpu_count()}
+    if THREADS_OVERRIDE:
+        info.update(threads_used=THREADS_OVERRIDE, thread_cap=None, thread_cap_source="--threads")
+        return THREADS_OVERRIDE, info
+    cap = None
+    try:
+        cap = int(os.environ.get("OMP_NUM_THREADS", ""))
+    except ValueError:
+        pass
+    used = min(detected, cap) if cap and cap > 0 else detected
+    info.update(threads_used=used, thread_cap=cap,
+                thread_cap_source="OMP_NUM_THREADS: this job's share of the host's cores" if cap else None)
+    return used, info
+
+
 def build_projection_set(pkg, batch, keep_host):
     """Uploads the 197 weights and their quantized activations; returns problem records."""
     synth, K, H = pkg.synth, pkg.kernel, pkg.hip
@@ -157,7 +180,7 @@ def cpu_baseline(problems, batch, alg_bytes):
 
     if not oracle.have_avx2():
         return None
-    cores = min(16, physical_cores())
+    cores, core_info = cpu_threads()
     pool = oracle.Pool(cores)
     outs = [np.zeros((batch, r["n_out"]), np.float32) for r in problems]
 
@@ -188,19 +211,23 @@ def cpu_baseline(problems, batch, alg_bytes):
                   f"restated reference AVX2 kernels, (ith,nth) row partition over {cores} persistent threads",
         "ms_per_step": round(med * 1e3, 3),
         "token_steps_per_s": round(1.0 / med, 2),
+        **core_info,
     }, outs
 
 
 def read_traffic(name):
-    """HBM bytes per launch measured with rocprofv3 --pmc, recorded under profiles/<name>_pmc.txt."""
-    path = os.path.join(ROOT, "profiles", f"{name}_pmc.txt")
+    """HBM bytes per launch as rocprofv3 --pmc measured them when profiles/<name>_pmc.txt was recorded: a figure
+    read back from that file, not measured by this run.  Returns {"traffic": bytes or None, "traffic_source": ..}."""
+    rel = os.path.join("profiles", f"{name}_pmc.txt")
     try:
-        for line in open(path):
+        for line in open(os.path.join(ROOT, rel)):
             if line.startswith("traffic_bytes_per_launch:"):
-                return float(line.split(":")[1])
+                return {"traffic": float(line.split(":")[1]),
+                        "traffic_source": f"{rel} (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, recorded earlier; "
+                                          "not measured in this run)"}
     except OSError:
         pass
-    return None
+    return {"traffic": None, "traffic_source": None}
 
 
 def copy_calibration(H, args):
@@ -302,7 +329,9 @@ def run_projection_set(args, pkg, ev):
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
             "algorithmic_bytes_per_launch": round(alg_bytes / launches),
-            "traffic": read_traffic(f"gemv_q8_0_{args.mode}_qwen3_0.6b") if batch == 1 else None,
+            **(read_traffic(f"gemv_q8_0_{args.mode}_qwen3_0.6b") if batch == 1 and not neon else
+               read_traffic(f"gemv_q8_0_mfma_grouped_qwen3_0.6b_batch{batch}") if neon and args.mode == "grouped" else
+               {"traffic": None}),
         },
     })
 
@@ -332,6 +361,46 @@ def run_projection_set(args, pkg, ev):
         else:
             result["cpu_baseline"] = None
     return result
+
+
+def run_small_batches(args, pkg, ev):
+    """The projection set at decode batch 8 and 16 in one grouped launch each: the GEMV in the x86-64 kernel's
+    order at 8 tokens, the small-batch kernel on the matrix cores (aarch64 kernel's order) at 8 and 16."""
+    H, synth = pkg.hip, pkg.synth
+    problems = build_projection_set(pkg, 16, keep_host=False)  # batches of 8 use the first 8 tokens
+    out = {}
+    for label, order, batch in (("batch8_x86_order", "avx2", 8), ("batch8_aarch64_order", "neon", 8),
+                                ("batch16_aarch64_order", "neon", 16)):
+        group = make_group(H, problems, batch, order)
+
+        def step(g=group):
+            H.check(H.lib.rmi_hip_gemv_group_run_dev(g, None))
+
+        wall, dev_ms = time_region(H, ev, step, 30, 5)
+        alg = sum(synth.q8_0_gemv_bytes(r["n_out"], r["n_in"], batch) for r in problems)
+        achieved = alg / (dev_ms * 1e-3) / 1e9
+        out[label] = {
+            "workload": f"Qwen3-0.6B projection set (197 Q8_0 GEMVs), decode batch {batch}, one grouped launch, "
+                        + ("x86-64 accumulation order (GEMV)" if order == "avx2" else
+                           "aarch64 accumulation order (small-batch kernel on the matrix cores)"),
+            "value": round(alg / wall / 1e9, 1), "unit": "GB/s", "ms_per_step": round(wall * 1e3, 4),
+            "token_steps_per_s": round(batch / wall, 1), "algorithmic_bytes_per_step": alg,
+            "roofline": {"bound": "hbm",
+                         "kernel": "gemv_q8_0_kernel<%d,true,%s>" % (batch, group_maxt(H, group)) if order == "avx2"
+                                   else "gemv_q8_0_mfma_kernel<%d,true>" % ((batch + 15) // 16),
+                         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_us": round(dev_ms * 1e3, 3)}}
+        H.lib.rmi_hip_gemv_group_destroy(group)
+    return out
+
+
+def compact(r):
+    """A sub-record of the default line: the figure, its workload, its roofline and its CPU leg."""
+    keep = {"workload": r["config"]["workload"], "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+            "steps": r["steps"], "roofline": r["roofline"]}
+    if r.get("cpu_baseline"):
+        keep["cpu_baseline"] = r["cpu_baseline"]
+    return keep
 
 
 def run_gemm(args, pkg, ev):
@@ -369,12 +438,12 @@ def run_gemm(args, pkg, ev):
     result["roofline"] = {"bound": "mfma", "kernel": "gemm_q8_0_kernel", "achieved": round(achieved, 1), "peak": INT8_MFMA_PEAK_TOPS,
                           "unit": "TOP/s", "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
                           "avg_launch_us": round(dev_ms * 1e3 / 2, 3),
-                          "traffic": read_traffic(f"gemm_q8_0_m{M}_qwen3_0.6b_ffn")}
+                          **read_traffic(f"gemm_q8_0_m{M}_qwen3_0.6b_ffn")}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
         if oracle.have_avx2():
-            cores = min(16, physical_cores())
+            cores, core_info = cpu_threads()
             pool = oracle.Pool(cores)
             mt = min(M, 256)  # bounded sample: the first `mt` tokens of both products
             outs, qs = [], []
@@ -398,7 +467,7 @@ def run_gemm(args, pkg, ev):
                 gpu = r["d_y"].to_array(np.float32, (M, r["n_out"]))[:mt]
                 worst = max(worst, float(np.max(np.abs(gpu - out) / (1e-4 + 1e-4 * np.abs(out)))))
             result["cpu_baseline"] = {
-                "value": round(ops * mt / M / med / 1e12, 4), "unit": "TOP/s", "cores": cores, "kind": "port",
+                "value": round(ops * mt / M / med / 1e12, 4), "unit": "TOP/s", "cores": cores, **core_info, "kind": "port",
                 "sample": f"first {mt} of {M} tokens of both products, one GEMV per token (the reference has no GEMM), "
                           f"restated AVX2 kernels over {cores} threads, median of 3",
                 "max_err_over_tolerance": round(worst, 4)}
@@ -476,12 +545,12 @@ def run_kquant(args, pkg, ev, fmt):
                           "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(achieved / HBM_PEAK_GBS, 4),
                           "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
-                          "traffic": read_traffic(f"gemv_{fmt}_grouped_1.7b_ffn") if grouped and batch == 1 else None}
+                          **(read_traffic(f"gemv_{fmt}_grouped_1.7b_ffn") if grouped and batch == 1 else {"traffic": None})}
     if not args.no_cpu_baseline and batch == 1:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
         if oracle.have_avx2():
-            cores = min(16, physical_cores())
+            cores, core_info = cpu_threads()
             pool = oracle.Pool(cores)
             host = [(r["d_d"].to_array(np.float32, (r["n_in"] // 256,)), r["d_q"].to_array(np.int8, (r["n_in"],)),
                      r["d_b"].to_array(np.int16, (r["n_in"] // 16,)), np.zeros(r["n_out"], np.float32)) for r in recs]
@@ -497,7 +566,7 @@ def run_kquant(args, pkg, ev, fmt):
             H.check(H.lib.rmi_hip_synchronize())
             worst = max(int(np.count_nonzero(r["d_y"].to_array(np.float32, (r["n_out"],)).view(np.uint32)
                                              != out.view(np.uint32))) for r, (_, _, _, out) in zip(recs, host))
-            result["cpu_baseline"] = {"value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            result["cpu_baseline"] = {"value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, **core_info, "kind": "port",
                                       "sample": f"5 full steps (84 GEMVs, {alg / 1e6:.0f} MB), restated AVX2 "
                                                 f"vec_dot_{fmt.replace('_', '')}_q8k over {cores} threads, median",
                                       "gpu_outputs_differing_from_cpu": worst}
@@ -555,12 +624,12 @@ def run_q4_0(args, pkg, ev):
     result["roofline"] = {"bound": "hbm", "kernel": f"gemv_q4_0_kernel<{batch},{'true' if grouped else 'false'},{group_maxt(H, group) if grouped else '*'}>",
                           "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
-                          "traffic": read_traffic("gemv_q4_0_grouped_1.7b_ffn") if grouped and batch == 1 else None}
+                          **(read_traffic("gemv_q4_0_grouped_1.7b_ffn") if grouped and batch == 1 else {"traffic": None})}
     if not args.no_cpu_baseline and batch == 1:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
         if oracle.have_avx2():
-            cores = min(16, physical_cores())
+            cores, core_info = cpu_threads()
             pool = oracle.Pool(cores)
             host = [(r["d_q"].to_array(np.uint8, (r["n_in"],)), r["d_s"].to_array(np.float32, (r["n_in"] // 32,)),
                      np.zeros(r["n_out"], np.float32)) for r in recs]
@@ -576,7 +645,7 @@ def run_q4_0(args, pkg, ev):
             H.check(H.lib.rmi_hip_synchronize())
             worst = max(int(np.count_nonzero(r["d_y"].to_array(np.float32, (r["n_out"],)).view(np.uint32)
                                              != out.view(np.uint32))) for r, (_, _, out) in zip(recs, host))
-            result["cpu_baseline"] = {"value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            result["cpu_baseline"] = {"value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, **core_info, "kind": "port",
                                       "sample": f"5 full steps (84 GEMVs, {alg / 1e6:.0f} MB), restated AVX2 "
                                                 f"matmul_q4_0_vs_q8_0 over {cores} threads, median",
                                       "gpu_outputs_differing_from_cpu": worst}
@@ -671,12 +740,12 @@ def run_q4k_gemm(args, pkg, ev):
         "tokens": M, "launches_per_step": 3, "ops_per_step": ops, "device": dev_name.strip(), "compute_units": cus})
     result["roofline"] = {"bound": "mfma", "kernel": "gemm_q4_k_kernel", "achieved": round(achieved, 1),
                           "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s", "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
-                          "avg_launch_us": round(dev_ms * 1e3 / 3, 3), "traffic": None}
+                          "avg_launch_us": round(dev_ms * 1e3 / 3, 3), **read_traffic(f"gemm_q4_k_m{M}_1.7b_ffn")}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
         if oracle.have_avx2():
-            cores = min(16, physical_cores())
+            cores, core_info = cpu_threads()
             pool = oracle.Pool(cores)
             mt = min(M, 64)  # bounded sample: the first `mt` tokens of the three products
             t_cpu, worst = 0.0, 0.0
@@ -696,7 +765,7 @@ def run_q4k_gemm(args, pkg, ev):
             pool.close()
             ops_cpu = sum(2.0 * mt * r["n_in"] * r["n_out"] for r in recs)
             result["cpu_baseline"] = {"value": round(ops_cpu / t_cpu / 1e12, 4), "unit": "TOP/s", "cores": cores,
-                                      "kind": "port",
+                                      **core_info, "kind": "port",
                                       "sample": f"first {mt} of {M} tokens of the three products, one GEMV per token (the "
                                                 f"reference has no GEMM), restated AVX2 vec_dot_q4k_q8k over {cores} threads",
                                       "max_err_over_tolerance": round(worst, 4)}
@@ -754,12 +823,12 @@ def run_decode(args, pkg, ev):
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
         if oracle.have_avx2():
-            cores = min(16, physical_cores())
+            cores, core_info = cpu_threads()
             pool = oracle.Pool(cores)
             cpu = oracle.Qwen3Decoder(f.metadata, tensors, pool).generate(prompt, n_new)
             pool.close()
             result["cpu_baseline"] = {
-                "value": round(token_steps / cpu["seconds"], 1), "unit": "tok/s", "cores": cores, "kind": "port",
+                "value": round(token_steps / cpu["seconds"], 1), "unit": "tok/s", "cores": cores, **core_info, "kind": "port",
                 "sample": f"one full generation ({token_steps} token-steps) of the restated Qwen3Session loop with the "
                           f"restated AVX2 matmuls over {cores} threads",
                 "gpu_tokens_equal_cpu_tokens": bool(np.array_equal(cpu["tokens"], last["tokens"])),
@@ -798,7 +867,14 @@ def main():
     ap.add_argument("--extra", action="store_true", help="also time the other launch modes, outside the timed region")
     ap.add_argument("--no-decode", action="store_true",
                     help="projection_set only: skip the end-to-end decode figure that is attached to the JSON line")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="projection_set only: skip the sub-records of the other benchmark configurations (batch 8 / 16, "
+                         "prefill GEMM at M = 64 / 512 / 2048, Q4_K GEMV and GEMM) that the default run attaches")
+    ap.add_argument("--threads", type=int, default=0,
+                    help="threads of the CPU baseline legs (default: the host's physical cores, capped by OMP_NUM_THREADS)")
     args = ap.parse_args()
+    global THREADS_OVERRIDE
+    THREADS_OVERRIDE = args.threads or None
     long_run = args.workload in ("q4_0", "q4k", "q6k")
     if args.steps is None:
         args.steps = 500 if long_run else 50
@@ -823,6 +899,25 @@ def main():
         result["decode"] = {"value": d["value"], "unit": d["unit"], "ms_per_token_step": d["ms_per_token_step"],
                             "workload": d["config"]["workload"], "generations_timed": sub.steps,
                             "cpu_baseline": d.get("cpu_baseline")}
+    if args.workload == "projection_set" and not args.no_configs and args.batch == 1 and args.mode == "grouped" \
+            and args.order == "avx2":
+        # the other benchmark configurations, each measured like the headline (own warm-up, own timed steps between
+        # synchronisations, HIP events on the launch stream), after and outside the headline's timed region
+        configs = {}
+        t_cfg = time.time()
+        configs.update(run_small_batches(args, pkg, ev))
+        for m in (64, 512, 2048):
+            sub = argparse.Namespace(**vars(args))
+            sub.tokens, sub.steps, sub.warmup, sub.copy_calibration_mb = m, 50, 10, 0
+            configs[f"gemm_m{m}"] = compact(run_gemm(sub, pkg, ev))
+        sub = argparse.Namespace(**vars(args))
+        sub.steps, sub.warmup, sub.batch, sub.copy_calibration_mb = 300, 100, 1, 0
+        configs["q4k_gemv"] = compact(run_q4k(sub, pkg, ev))
+        sub = argparse.Namespace(**vars(args))
+        sub.tokens, sub.steps, sub.warmup, sub.copy_calibration_mb = 512, 50, 10, 0
+        configs["q4k_gemm_m512"] = compact(run_q4k_gemm(sub, pkg, ev))
+        result["configs"] = configs
+        log(f"[bench] other configurations measured in {time.time() - t_cfg:.1f}s")
     print(json.dumps(result), flush=True)
 
 
