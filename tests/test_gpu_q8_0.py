@@ -358,9 +358,12 @@ def test_gemm_mfma_parity(hip, oracle, n_tokens, n_out, n_in):
     assert np.all(np.abs(out - ref_a) <= TOL(ref_a))
 
 
-def test_gemm_special_scales(hip, oracle):
+@pytest.mark.parametrize("f16_token_scales", [False, True])
+def test_gemm_special_scales(hip, oracle, f16_token_scales):
     """Weight scales that are zero, negative zero, f16 subnormals, the largest f16, inf and NaN, against token
-    scales down to f32 subnormals: the scale products formed on the matrix cores must round like the f32 multiply."""
+    scales down to f32 subnormals (the f32 outer product on the matrix cores) or token scales that are f16 values,
+    as every quantizer of the reference writes them, down to f16 subnormals (the f16 one): either way the scale
+    products must round like the f32 multiply."""
     n_tokens, n_out, n_in = 96, 160, 320
     rng = np.random.default_rng(77)
     w = hip.synth.q8_0_weight(1234, n_out, n_in).reshape(n_out, n_in // 32, 34).copy()
@@ -377,6 +380,12 @@ def test_gemm_special_scales(hip, oracle):
         np.float32(10.0) ** rng.integers(-44, 3, (n_tokens, n_in // 32)).astype(np.float32)
     sc[rng.random(sc.shape) < 0.05] = 0.0
     sc = sc.astype(np.float32)
+    if f16_token_scales:
+        sc = (rng.random(sc.shape, dtype=np.float32) + 0.5) * np.float32(10.0) ** rng.integers(-8, 7, sc.shape).astype(np.float32)
+        sc[rng.random(sc.shape) < 0.05] = 0.0
+        with np.errstate(over="ignore"):
+            sc = sc.astype(np.float16).astype(np.float32)  # incl. f16 subnormals, zeros and inf
+        assert np.isinf(sc).any() and (np.abs(sc[sc != 0]) < 6.1e-5).any()
     H = hip.hip
     kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
     d_q8, d_sc = H.DeviceBuffer.from_array(q8), H.DeviceBuffer.from_array(sc)
@@ -393,7 +402,8 @@ def test_gemm_special_scales(hip, oracle):
     wd = scales.view(np.float16).astype(np.float32)
     with np.errstate(all="ignore"):
         prod = wd[:, None, :] * sc[None, :, :]
-    assert np.count_nonzero((prod != 0) & (np.abs(prod) < 1.17549435e-38)) > 1000
+    if not f16_token_scales:
+        assert np.count_nonzero((prod != 0) & (np.abs(prod) < 1.17549435e-38)) > 1000
 
 
 @pytest.mark.parametrize("n_tokens,n_out,n_in", [(2048, 3072, 1024), (2048, 1024, 3072), (512, 3072, 1024),
