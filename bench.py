@@ -772,6 +772,43 @@ def run_q4k_gemm(args, pkg, ev):
     return result
 
 
+def run_attention(args, pkg, ev):
+    """One attention launch of a Qwen3-0.6B layer over the F16 cache (16 query heads, 8 key/value heads, head
+    dimension 128; src/models/qwen3.rs:876-933), output quantized to Q8_0, at --keys cached positions.  One step =
+    one call of rmi_hip_attention_f16_quantize_q8_0_dev.  Neither HBM nor the matrix cores bound it: the reference's
+    f64 sums and its sequential f32 sum of the softmax weights do (about 8.4 clocks per key on one lane)."""
+    H = pkg.hip
+    dev_name, cus, hbm = H.device_info()
+    n_head, n_kv, hd, n_keys = 16, 8, 128, args.keys
+    kv_stride = n_kv * hd
+    rng = np.random.default_rng(1234)
+    q = rng.normal(0, 1, n_head * hd).astype(np.float16).view(np.uint16)
+    kc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+    vc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+    d_q, d_k, d_v = (H.DeviceBuffer.from_array(a) for a in (q, kc, vc))
+    d_o, d_s = H.DeviceBuffer(n_head * hd), H.DeviceBuffer(n_head * hd // 32 * 4)
+
+    def step():
+        H.check(H.lib.rmi_hip_attention_f16_quantize_q8_0_dev(d_q.ptr, d_k.ptr, d_v.ptr, n_keys, kv_stride, n_head, n_kv,
+                                                              hd, hd, d_o.ptr, d_s.ptr, 0, None))
+
+    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
+    alg = 2 * n_keys * kv_stride * 2 + n_head * hd * 2 + n_head * hd + n_head * hd // 32 * 4
+    achieved = alg / (dev_ms * 1e-3) / 1e9
+    result = base_result(args, "F16-KV attention launch, Qwen3-0.6B layer shape, keys per second, 1 GPU", "keys/s",
+                         round(n_keys / wall), wall, "f16 x f16 -> f64 sums, f32 softmax", {
+        "workload": f"attention over {n_keys} cached positions, 16 heads / 8 kv heads x 128, one launch per step",
+        "keys": n_keys, "algorithmic_bytes_per_step": alg, "device": dev_name.strip(), "compute_units": cus})
+    result["us_per_launch"] = round(dev_ms * 1e3, 3)
+    result["ns_per_key"] = round(dev_ms * 1e6 / n_keys, 2)
+    result["roofline"] = {"bound": "hbm", "kernel": "attention128_quant_kernel / attn128_scores_kernel + attn128_weights_pv_kernel",
+                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_us": round(dev_ms * 1e3, 3), "traffic": None,
+                          "limit": "the reference's sequential f32 sum of the softmax weights: "
+                                   f"{n_keys * 8.4 / 2.0e3:.1f} us at 8.4 clocks a key and 2.0 GHz, whatever the bandwidth"}
+    return result
+
+
 def run_decode(args, pkg, ev):
     """End-to-end greedy decode, device-resident: a random-init Qwen3-0.6B-architecture model written as a
     synthetic Q8_0 GGUF, 512 prompt tokens (fed one per step, as the reference's generate_inner does) plus 128
@@ -850,7 +887,7 @@ def main():
                     help="timed steps (default 50; 500 for the q4_0 / q4k / q6k GEMV workloads, whose compute-heavy kernels "
                          "read 10-15 %% slower until the clocks have settled, a few hundred launches in)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps before (default 10; 100 for q4_0 / q4k / q6k)")
-    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "qlinear", "decode"], default="projection_set",
+    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "qlinear", "attention", "decode"], default="projection_set",
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
                          "q4_0: Q4_0 x Q8_0 decode GEMV; q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); qlinear: QuantizedLinear::forward (Q4_K dequantise-and-dot, f32 activation); decode: end-to-end device-resident greedy decode "
                          "(one step = one 639-token-step generation)")
@@ -859,6 +896,7 @@ def main():
                     help="projection_set: accumulation order of the reference's x86-64 kernel (GEMV, the default) or of "
                          "its aarch64 kernel (small-batch kernel on the matrix cores)")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill tokens M for --workload gemm")
+    ap.add_argument("--keys", type=int, default=4096, help="cached positions for --workload attention")
     ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration-mb", type=int, default=0,
@@ -888,7 +926,7 @@ def main():
     pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
     ev = HipEvents()
     run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4_0": run_q4_0, "q4k": run_q4k, "q6k": run_q6k, "q4k_gemm": run_q4k_gemm, "qlinear": run_qlinear,
-           "decode": run_decode}[args.workload]
+           "attention": run_attention, "decode": run_decode}[args.workload]
     result = run(args, pkg, ev)
     if args.workload == "projection_set" and not args.no_decode and args.batch == 1:
         # the second half of the headline metric: end-to-end decode tok/s of the same model shape, measured

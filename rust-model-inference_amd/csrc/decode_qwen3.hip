@@ -443,7 +443,7 @@ __device__ __forceinline__ double swizzle_xor16_f64(double v) {  // the value of
 }
 __host__ __device__ inline size_t attn128_lds_bytes(uint32_t n_keys) {
     const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
-    return n_pad * 12 + (kA128Threads / 64) * 128 * 8;
+    return n_pad * 12 + (kA128Threads / 64) * 128 * 8 + 128;  // 32 floats of room behind the scores
 }
 __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
@@ -547,10 +547,10 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
                 acc += a[j].z;
                 acc += a[j].w;
             }
-            if (t + 64 < n_pad) {
+            // unconditional (the array has 32 floats of room behind n_pad): under a branch the registers would be
+            // copied every round, on the chain's own lane
 #pragma unroll
-                for (int j = 0; j < 8; j++) a[j] = reinterpret_cast<const float4 *>(scores + t + 64)[j];
-            }
+            for (int j = 0; j < 8; j++) a[j] = reinterpret_cast<const float4 *>(scores + t + 64)[j];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 acc += b[j].x;
@@ -633,6 +633,283 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     }
 }
 
+// ---- head dimension 128 over long contexts: a head's keys split over several workgroups, two launches.
+// One workgroup per head leaves most of the chip idle and costs about 54 clocks of one compute unit per key; of
+// the head's arithmetic only the f32 sum of the softmax weights has to run in key order (about 8 clocks a key
+// on one lane).  The scores and the p.v sums are f64 sums of exact terms, which are split over lanes already
+// and here over workgroups as well:
+//   attn128_scores_kernel    workgroup (head, part): the scores of its keys to HBM, and their maximum;
+//   attn128_weights_pv_kernel workgroup (head, part): the head's maximum, exp of every score of the head into
+//                            LDS, the sequential f32 sum (every part computes the same one: waiting for another
+//                            workgroup's would take as long), the f16 weights of its own keys, their p.v sums;
+//                            the part that finishes last adds the parts' sums in part order and quantizes.
+// Every f32 / f16 rounding point is that of attention128_quant_kernel.  Workgroup ids are head + n_head * part,
+// so with a multiple of 8 heads the parts of a head sit on one XCD and share its L2.
+constexpr uint32_t kAttnSplitThreads = 512;
+constexpr uint32_t kAttnSplitMaxParts = 16;
+struct AttnSplitScratch {  // device memory of one attention launch pair; the counters start, and are left, at zero
+    float *scores;      // [n_head][score_stride]
+    float *part_max;    // [n_head][kAttnSplitMaxParts]
+    double *part_sums;  // [n_head][kAttnSplitMaxParts][128]
+    uint32_t *arrived;  // [n_head]
+    uint32_t score_stride;
+};
+__host__ __device__ inline size_t attn128_split_lds_bytes(uint32_t n_keys, uint32_t keys_per_part) {
+    const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
+    return n_pad * 4 + size_t(keys_per_part) * 8 + (kAttnSplitThreads / 64) * 128 * 8 + 128;  // 32 floats of room behind e
+}
+__global__ __launch_bounds__(kAttnSplitThreads) void attn128_scores_kernel(
+    const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, uint32_t n_keys, uint32_t keys_per_part,
+    uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, AttnSplitScratch ws) {
+    __shared__ float red_f[kAttnSplitThreads / 64];
+    const uint32_t head = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+    const uint32_t kvh = head / (n_head / n_head_kv);
+    const uint32_t t_first = part * keys_per_part;
+    const uint32_t t_stop = t_first + keys_per_part < n_keys ? t_first + keys_per_part : n_keys;
+    const uint32_t row_u4 = kv_stride >> 3;
+    // four lanes per key, the 16-byte pieces interleaved as in attention128_quant_kernel
+    const uint32_t lane4 = tid & 3, key0 = t_first + (tid >> 2);
+    const uint4 *qp = reinterpret_cast<const uint4 *>(q16 + size_t(head) * 128) + lane4;
+    const uint4 *kbase = reinterpret_cast<const uint4 *>(k_cache + size_t(kvh) * 128) + lane4;
+    uint4 qv[4], kk[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) qv[c] = qp[4 * c];
+    {
+        const uint4 *key = kbase + size_t(key0 < n_keys ? key0 : n_keys - 1) * row_u4;
+#pragma unroll
+        for (int c = 0; c < 4; c++) kk[c] = key[4 * c];
+    }
+    const float kq_scale = 1.0f / sqrtf(128.0f);  // two f32 roundings, as the reference computes it
+    float my_max = -INFINITY;
+    float *scores = ws.scores + size_t(head) * ws.score_stride;
+    for (uint32_t t = key0; t - (tid >> 2) < t_stop; t += kAttnSplitThreads / 4) {
+        const uint32_t tn = t + kAttnSplitThreads / 4;
+        uint4 kn[4];  // the next round's keys, unconditionally (after the last round the last key again)
+        {
+            const uint4 *key = kbase + size_t(tn < n_keys ? tn : n_keys - 1) * row_u4;
+#pragma unroll
+            for (int c = 0; c < 4; c++) kn[c] = key[4 * c];
+        }
+        double s4[4] = {0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const half8 kh = as_half8(kk[c]), qh = as_half8(qv[c]);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float prod = __builtin_fmaf(float(kh[j]), float(qh[j]), 0.0f);  // exact
+                s4[c] += double(prod);
+            }
+        }
+        const double sum = quad_sum((s4[0] + s4[1]) + (s4[2] + s4[3]));
+        if (t < t_stop) {
+            const float sc = float(sum) * kq_scale;
+            if (lane4 == 0) scores[t] = sc;
+            my_max = fmaxf(my_max, sc);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) kk[c] = kn[c];
+    }
+    my_max = wave_max_f32(my_max);
+    if ((tid & 63) == 0) red_f[tid >> 6] = my_max;
+    __syncthreads();
+    if (tid == 0) {
+        float m = red_f[0];
+#pragma unroll
+        for (uint32_t i = 1; i < kAttnSplitThreads / 64; i++) m = fmaxf(m, red_f[i]);
+        ws.part_max[head * kAttnSplitMaxParts + part] = m;
+    }
+}
+
+__global__ __launch_bounds__(kAttnSplitThreads) void attn128_weights_pv_kernel(
+    const uint16_t *__restrict__ v_cache, uint32_t n_keys, uint32_t keys_per_part, uint32_t n_parts, uint32_t kv_stride,
+    uint32_t n_head, uint32_t n_head_kv, AttnSplitScratch ws, int8_t *__restrict__ q8, float *__restrict__ scales,
+    int rounding) {
+    extern __shared__ double lds_d[];
+    __shared__ float red_f[2];
+    __shared__ uint64_t exp_tab[32];
+    const uint32_t head = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+    const uint32_t kvh = head / (n_head / n_head_kv);
+    const uint32_t n_pad = (n_keys + kAttnPad - 1) / kAttnPad * kAttnPad;
+    const uint32_t t_first = part * keys_per_part;
+    const uint32_t t_stop = t_first + keys_per_part < n_keys ? t_first + keys_per_part : n_keys;
+    double *wd = lds_d;                                       // [keys_per_part] this part's weights (f16 values)
+    double *wave_sums = wd + keys_per_part;                   // [waves][128]
+    float *e = reinterpret_cast<float *>(wave_sums + (kAttnSplitThreads / 64) * 128);  // [n_pad] exp(score - max), 0 beyond n_keys
+    const uint32_t row_u4 = kv_stride >> 3;
+    if (tid < 32) exp_tab[tid] = kRmiExp2fTab[tid];
+
+    // values: lane = (8 dimensions dg, key slice sl) of this part's keys; the first loads go out now
+    constexpr uint32_t kPre = 8;
+    const uint32_t dg = tid & 15, sl = tid >> 4;
+    const uint32_t n_mine = t_stop - t_first;
+    const uint32_t chunk = (n_mine + kAttnSplitThreads / 16 - 1) / (kAttnSplitThreads / 16);
+    const uint32_t t_begin = t_first + sl * chunk, t_end = t_begin + chunk < t_stop ? t_begin + chunk : t_stop;
+    const uint4 *vbase = reinterpret_cast<const uint4 *>(v_cache + size_t(kvh) * 128 + dg * 8);
+    uint4 vp[kPre];
+#pragma unroll
+    for (uint32_t j = 0; j < kPre; j++) {
+        if (j < chunk) {
+            const uint32_t t = t_begin + j < n_keys ? t_begin + j : n_keys - 1;
+            vp[j] = vbase[size_t(t) * row_u4];
+        }
+    }
+    // every score of the head, four per load and all loads out before the first is used: one memory round trip
+    // (n_pad, a multiple of 64 and at most 16 384: more would not fit the LDS anyway)
+    constexpr uint32_t kScoreLoads = 8;
+    const float *scores = ws.scores + size_t(head) * ws.score_stride;
+    float4 raw[kScoreLoads];
+#pragma unroll
+    for (uint32_t j = 0; j < kScoreLoads; j++) {
+        if (j * kAttnSplitThreads * 4 < n_pad) {  // uniform; past the end the last group of four is read again
+            const uint32_t t = (j * kAttnSplitThreads + tid) * 4;
+            raw[j] = *reinterpret_cast<const float4 *>(scores + (t < n_pad ? t : n_pad - 4));
+        }
+    }
+    float max_val = ws.part_max[head * kAttnSplitMaxParts];
+    for (uint32_t i = 1; i < n_parts; i++) max_val = fmaxf(max_val, ws.part_max[head * kAttnSplitMaxParts + i]);
+    __syncthreads();  // exp_tab
+#pragma unroll
+    for (uint32_t j = 0; j < kScoreLoads; j++) {
+        const uint32_t t = (j * kAttnSplitThreads + tid) * 4;
+        if (j * kAttnSplitThreads * 4 < n_pad && t < n_pad) {
+            float4 ev;
+            ev.x = t + 0 < n_keys ? rmi_expf_tab(raw[j].x - max_val, exp_tab) : 0.0f;
+            ev.y = t + 1 < n_keys ? rmi_expf_tab(raw[j].y - max_val, exp_tab) : 0.0f;
+            ev.z = t + 2 < n_keys ? rmi_expf_tab(raw[j].z - max_val, exp_tab) : 0.0f;
+            ev.w = t + 3 < n_keys ? rmi_expf_tab(raw[j].w - max_val, exp_tab) : 0.0f;
+            *reinterpret_cast<float4 *>(e + t) = ev;
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {  // the reference adds the weights one after the other in f32; the padding zeros change nothing
+        float acc = 0.0f;
+        float4 a[8], b[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) a[j] = reinterpret_cast<const float4 *>(e)[j];
+        for (uint32_t t = 0; t < n_pad; t += 64) {  // n_pad is a multiple of 64
+#pragma unroll
+            for (int j = 0; j < 8; j++) b[j] = reinterpret_cast<const float4 *>(e + t + 32)[j];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc += a[j].x;
+                acc += a[j].y;
+                acc += a[j].z;
+                acc += a[j].w;
+            }
+            // unconditional (the array has 32 floats of room behind n_pad): under a branch the registers would be
+            // copied every round, on the chain's own lane
+#pragma unroll
+            for (int j = 0; j < 8; j++) a[j] = reinterpret_cast<const float4 *>(e + t + 64)[j];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc += b[j].x;
+                acc += b[j].y;
+                acc += b[j].z;
+                acc += b[j].w;
+            }
+        }
+        red_f[0] = acc;
+    }
+    __syncthreads();
+    const float total = red_f[0];
+    for (uint32_t t = t_first + tid; t < t_stop; t += kAttnSplitThreads) {
+        const float ev = e[t];
+        wd[t - t_first] = double(h2f(f2h(total > 0.0f ? ev / total : ev)));
+    }
+    __syncthreads();
+
+    double acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) acc[j] = 0.0;
+#pragma unroll
+    for (uint32_t j = 0; j < kPre; j++) {
+        if (t_begin + j < t_end) {
+            const double w = wd[t_begin + j - t_first];
+            const half8 vh = as_half8(vp[j]);
+#pragma unroll
+            for (int d = 0; d < 8; d++) acc[d] = __builtin_fma(double(float(vh[d])), w, acc[d]);
+        }
+    }
+    if (t_begin + kPre < t_end) {  // longer slices: batches of 8 keys, the next one in flight while one is added
+        uint4 cur[8], nxt[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; j++) {
+            const uint32_t t = t_begin + kPre + j;
+            cur[j] = vbase[size_t(t < n_keys ? t : n_keys - 1) * row_u4];
+        }
+        for (uint32_t t0 = t_begin + kPre; t0 < t_end; t0 += 8) {
+#pragma unroll
+            for (uint32_t j = 0; j < 8; j++) {
+                const uint32_t t = t0 + 8 + j;
+                nxt[j] = vbase[size_t(t < n_keys ? t : n_keys - 1) * row_u4];
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < 8; j++) {
+                if (t0 + j < t_end) {
+                    const double w = wd[t0 + j - t_first];
+                    const half8 vh = as_half8(cur[j]);
+#pragma unroll
+                    for (int d = 0; d < 8; d++) acc[d] = __builtin_fma(double(float(vh[d])), w, acc[d]);
+                }
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < 8; j++) cur[j] = nxt[j];
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < 8; d++) {  // the four slices of a wave: lanes 16 apart
+        acc[d] += swizzle_xor16_f64(acc[d]);
+        acc[d] += __shfl_xor(acc[d], 32, 64);
+    }
+    if ((tid & 63) < 16) {
+        double *dst = wave_sums + (tid >> 6) * 128 + dg * 8;
+#pragma unroll
+        for (int d = 0; d < 8; d++) dst[d] = acc[d];
+    }
+    __syncthreads();
+    // The first wave alone hands the part's sums over: its stores, one release (the other waves have nothing in
+    // flight that anybody reads), its count.  The part that counts last has every part's sums in reach after one
+    // acquire, adds them in part order and quantizes.  Nobody waits for anybody.
+    if (tid >= 64) return;
+    double *mine = ws.part_sums + (size_t(head) * kAttnSplitMaxParts + part) * 128;
+#pragma unroll
+    for (uint32_t d = tid; d < 128; d += 64) {
+        double o = wave_sums[d];
+        for (uint32_t w = 1; w < kAttnSplitThreads / 64; w++) o += wave_sums[w * 128 + d];
+        mine[d] = o;
+    }
+    __threadfence();
+    uint32_t before = 0;
+    if (tid == 0) before = __hip_atomic_fetch_add(ws.arrived + head, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = uint32_t(__builtin_amdgcn_readfirstlane(int(before)));
+    if (before + 1 != n_parts) return;
+    if (tid == 0) __hip_atomic_store(ws.arrived + head, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence();
+    if (tid < 32) {  // four dimensions per lane: whole 8-lane groups for the quantizer
+        const double *all = ws.part_sums + size_t(head) * kAttnSplitMaxParts * 128 + tid * 4;
+        double v[kAttnSplitMaxParts][4];  // every part's sums on their way before the first is added
+#pragma unroll
+        for (uint32_t p = 0; p < kAttnSplitMaxParts; p++) {
+            if (p < n_parts) {
+#pragma unroll
+                for (int d = 0; d < 4; d++) v[p][d] = __builtin_nontemporal_load(all + p * 128 + d);
+            }
+        }
+        double o[4] = {v[0][0], v[0][1], v[0][2], v[0][3]};
+#pragma unroll
+        for (uint32_t p = 1; p < kAttnSplitMaxParts; p++) {
+            if (p < n_parts) {
+#pragma unroll
+                for (int d = 0; d < 4; d++) o[d] += v[p][d];
+            }
+        }
+        const float4 of = make_float4(float(o[0]), float(o[1]), float(o[2]), float(o[3]));
+        float sc;
+        reinterpret_cast<uint32_t *>(q8)[(size_t(head) * 128 >> 2) + tid] = rmi_quantize_block8(of, rounding, &sc);
+        if ((tid & 7) == 0) scales[(size_t(head) * 128 >> 5) + (tid >> 3)] = sc;
+    }
+}
+
 // Dynamic LDS an attention launch may use: 64 KiB unless more has been asked for, which is done once, for both
 // kernels; then what a compute unit has (160 KiB) less the kernels' static arrays (under 1 KiB).  With 12 bytes
 // per key that is about 13 000 keys.
@@ -642,11 +919,64 @@ size_t attn_lds_limit() {
         const bool ok = hipFuncSetAttribute(reinterpret_cast<const void *>(attention128_quant_kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, int(kWant)) == hipSuccess &&
                         hipFuncSetAttribute(reinterpret_cast<const void *>(attention_quant_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(kWant)) == hipSuccess &&
+                        hipFuncSetAttribute(reinterpret_cast<const void *>(attn128_weights_pv_kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, int(kWant)) == hipSuccess;
         if (!ok) (void)hipGetLastError();
         return ok ? kWant : size_t(64 * 1024);
     }();
     return limit;
+}
+
+// From this many keys on a head's keys are split over workgroups (measured: below, the second launch and the
+// hand-over through HBM cost more than the other compute units save).
+#ifndef RMI_ATTN_SPLIT_MIN_KEYS
+#define RMI_ATTN_SPLIT_MIN_KEYS 768
+#endif
+constexpr uint32_t kAttnSplitMinKeys = RMI_ATTN_SPLIT_MIN_KEYS;
+inline bool attn128_use_split(uint32_t n_keys, uint32_t n_head);
+// bytes of the scratch of one launch pair for n_head heads and up to max_keys keys, and its layout
+inline uint32_t attn_split_score_stride(uint32_t max_keys) { return (max_keys + kAttnPad - 1) / kAttnPad * kAttnPad; }
+constexpr uint32_t kAttnSplitMaxHeads = 1024;  // the arrival counters sit in front, wherever the head count puts the rest
+inline size_t attn_split_scratch_bytes(uint32_t n_head, uint32_t max_keys) {
+    return size_t(kAttnSplitMaxHeads) * 4 +
+           size_t(n_head) * (size_t(attn_split_score_stride(max_keys)) * 4 + kAttnSplitMaxParts * 4 +
+                             size_t(kAttnSplitMaxParts) * 128 * 8);
+}
+inline AttnSplitScratch attn_split_scratch_at(void *base, uint32_t n_head, uint32_t max_keys) {
+    AttnSplitScratch ws;
+    ws.score_stride = attn_split_score_stride(max_keys);
+    uint8_t *p = static_cast<uint8_t *>(base);
+    ws.arrived = reinterpret_cast<uint32_t *>(p);
+    p += size_t(kAttnSplitMaxHeads) * 4;
+    ws.part_sums = reinterpret_cast<double *>(p);
+    p += size_t(n_head) * kAttnSplitMaxParts * 128 * 8;
+    ws.scores = reinterpret_cast<float *>(p);
+    p += size_t(n_head) * ws.score_stride * 4;
+    ws.part_max = reinterpret_cast<float *>(p);
+    return ws;
+}
+inline bool attn128_use_split(uint32_t n_keys, uint32_t n_head) {
+    return n_keys >= kAttnSplitMinKeys && n_head <= kAttnSplitMaxHeads;
+}
+// keys 0..n_keys-1 of every head, split; ws.arrived must be zero (the launch leaves it zero)
+int launch_attention128_split(const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache, uint32_t n_keys,
+                              uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, const AttnSplitScratch &ws,
+                              int8_t *q8, float *scales, int rounding, hipStream_t st) {
+    // about 256 keys a part (two rounds of the score loop), at most kAttnSplitMaxParts parts of whole 64-key groups
+    uint32_t parts = (n_keys + 255) / 256;
+    if (parts > kAttnSplitMaxParts) parts = kAttnSplitMaxParts;
+    if (parts < 2) parts = 2;
+    const uint32_t keys_per_part = ((n_keys + parts - 1) / parts + kAttnPad - 1) / kAttnPad * kAttnPad;
+    parts = (n_keys + keys_per_part - 1) / keys_per_part;
+    const size_t lds = attn128_split_lds_bytes(n_keys, keys_per_part);
+    if (lds > attn_lds_limit() || n_keys > ws.score_stride || n_keys > 8 * kAttnSplitThreads * 4)
+        return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the attention kernels hold", n_keys);
+    hipLaunchKernelGGL(attn128_scores_kernel, dim3(n_head, parts), dim3(kAttnSplitThreads), 0, st, q16, k_cache, n_keys,
+                       keys_per_part, kv_stride, n_head, n_head_kv, ws);
+    hipLaunchKernelGGL(attn128_weights_pv_kernel, dim3(n_head, parts), dim3(kAttnSplitThreads), lds, st, v_cache, n_keys,
+                       keys_per_part, parts, kv_stride, n_head, n_head_kv, ws, q8, scales, rounding);
+    return RMI_HIP_OK;
 }
 
 // gu = [W_gate x ; W_up x]: h = (W_up x) * silu(W_gate x), quantized to Q8_0
@@ -757,6 +1087,7 @@ struct rmi_hip_qwen3 {
     uint32_t *tok = nullptr, *step_argmax = nullptr, *nonfinite = nullptr;
     float *step_top2 = nullptr;
     void *partial = nullptr;
+    void *attn_split = nullptr;          // scratch of the split attention launches (head dimension 128)
     void *params = nullptr;              // StepParams in HBM
     std::vector<void *> owned;  // every other device allocation, freed with the session
     std::vector<uint32_t> stop_ids;  // generation ends before the first of these (EOS, im_end)
@@ -849,7 +1180,12 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                                s->cos_t, s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head,
                                c.n_head_kv, c.head_dim_k, c.head_dim_v, c.eps);
         }
-        if (c.head_dim_k == 128 && c.head_dim_v == 128)
+        if (c.head_dim_k == 128 && c.head_dim_v == 128 && s->attn_split && attn128_use_split(step + 1, c.n_head)) {
+            rc = launch_attention128_split(s->q16, s->k_cache + layer_base, s->v_cache + layer_base, step + 1, s->kv_stride,
+                                           c.n_head, c.n_head_kv, attn_split_scratch_at(s->attn_split, c.n_head, c.capacity),
+                                           s->act_q8, s->act_scales, rnd, st);
+            if (rc != RMI_HIP_OK) return rc;
+        } else if (c.head_dim_k == 128 && c.head_dim_v == 128)
             hipLaunchKernelGGL(attention128_quant_kernel, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kA128Threads), attn128_lds_bytes(step + 1),
                                st, s->q16, s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride,
                                c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd);
@@ -984,6 +1320,27 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     const bool d128 = head_dim_k == 128 && head_dim_v == 128;
     const size_t lds = d128 ? attn128_lds_bytes(n_keys) : attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
     if (lds > attn_lds_limit()) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
+    if (d128 && attn128_use_split(n_keys, n_head)) {
+        // The scratch of the two launches is the calling thread's (slot 5 of its staging buffers, never used by
+        // the host-slice entry points): calls of one thread that overlap on different streams would share it.
+        RmiThreadCtx *c = rmi_thread_ctx();
+        if (!c) return RMI_HIP_E_RUNTIME;
+        constexpr int kSlot = 5;
+        const uint32_t max_keys = n_keys < 16384 ? 16384 : n_keys;  // sized once for any context the kernels hold
+        const size_t need = attn_split_scratch_bytes(n_head, max_keys);
+        if (c->dev_cap[kSlot] < need) {
+            RMI_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));  // it may still read the old one
+            void *fresh = rmi_dev_buf(c, kSlot, need);
+            if (!fresh) return RMI_HIP_E_RUNTIME;
+            RMI_HIP_CHECK(hipMemset(fresh, 0, c->dev_cap[kSlot]));  // the arrival counters start at zero
+        }
+        const int rc = launch_attention128_split(q16, k_cache, v_cache, n_keys, kv_stride, n_head, n_head_kv,
+                                                 attn_split_scratch_at(c->dev[kSlot], n_head, max_keys), q8, scales,
+                                                 rounding, static_cast<hipStream_t>(stream));
+        if (rc != RMI_HIP_OK) return rc;
+        RMI_HIP_CHECK(hipGetLastError());
+        return RMI_HIP_OK;
+    }
     if (d128)
         hipLaunchKernelGGL(attention128_quant_kernel, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
                            q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding);
@@ -1129,6 +1486,8 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
          (s->step_top2 = dev_alloc<float>(s, size_t(2) * c.capacity, true)) &&
          (s->nonfinite = dev_alloc<uint32_t>(s, 1, true)) && (s->partial = dev_alloc<Top>(s, kArgmaxGroups)) &&
          (s->params = dev_alloc<StepParams>(s, 1, true));
+    if (ok && c.head_dim_k == 128 && c.head_dim_v == 128 && attn128_use_split(c.capacity, c.n_head))
+        ok = (s->attn_split = dev_alloc<uint8_t>(s, attn_split_scratch_bytes(c.n_head, c.capacity), true)) != nullptr;
     if (ok && hipStreamSynchronize(rmi_thread_ctx()->stream) != hipSuccess) {  // the uploads enqueued above
         rmi_set_error("weight upload failed");
         ok = false;

@@ -119,6 +119,26 @@ def test_create_rejects_null_and_overflowing_shapes(hip):
     assert not H.lib.rmi_hip_qwen3_create(C.byref(c), C.byref(w)) and "overflow" in H.last_error()
 
 
+def test_long_context_device_decode_crosses_the_attention_split(hip, oracle, tmp_path):
+    """From 768 cached positions on, the head-dimension-128 attention of the device-resident step runs as two
+    launches with a head's keys split over workgroups; logits before, at and after the switch equal the CPU loop's."""
+    kw = dict(n_layer=2, n_embd=256, n_head=4, n_head_kv=2, head_dim=128, n_ff=512, vocab=2000, n_ctx=4096)
+    f = _write_model(hip, tmp_path, **kw)
+    pool = oracle.Pool(8)
+    prompt = np.random.default_rng(9).integers(0, 2000, 700, dtype=np.uint32)
+    steps = [0, 699, 765, 766, 767, 768, 769, 832, 833, 899]
+    cpu = oracle.Qwen3Decoder(f.metadata, _tensors(f), pool).generate(prompt, 201, dump_steps=steps)
+    sess = hip.decode.Qwen3Session(f.metadata, _tensors(f), capacity=901)
+    gpu = sess.generate(prompt, 201, dump_steps=steps)
+    assert gpu["steps"] == 900
+    worst, same = _compare(cpu, gpu, "long context")
+    print(f"\nlong context: {same}/{len(steps)} dumped steps bit-identical, worst error {worst:.3g} of tolerance")
+    again = sess.generate(prompt, 201, dump_steps=steps)  # the split's arrival counters were left at zero
+    assert np.array_equal(again["dump"].view(np.uint32), gpu["dump"].view(np.uint32))
+    sess.close()
+    pool.close()
+
+
 def test_full_qwen3_0_6b_device_decode_512_plus_128(hip, oracle, tmp_path):
     """512 prompt tokens + 128 greedy tokens = 639 steps of a random-init Qwen3-0.6B-architecture Q8_0 GGUF."""
     f = _write_model(hip, tmp_path)  # 28 layers, 1024 wide, vocab 151936

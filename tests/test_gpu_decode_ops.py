@@ -217,8 +217,9 @@ def test_attention_f16_quantize(hip, oracle, hk, n_head, n_kv):
     rng = np.random.default_rng(hk + 1)
     hv = hk
     kv_stride = n_kv * hk
-    # 5000 and 12000 keys take more than the default 64 KiB of LDS per workgroup
-    for n_keys in [1, 2, 7, 8, 9, 36, 63, 64, 255, 256, 257, 640, 5000, 12000]:
+    # 5000 and 12000 keys take more than the default 64 KiB of LDS per workgroup; from 768 keys on, head dimension
+    # 128 goes through the launches that split a head's keys over workgroups (2 to 16 parts of whole 64-key groups)
+    for n_keys in [1, 2, 7, 8, 9, 36, 63, 64, 255, 256, 257, 383, 640, 767, 768, 769, 833, 1025, 2048, 4097, 5000, 12000]:
         for trial in range(3 if n_keys < 1000 else 1):
             scale = rng.choice([0.3, 1.0, 3.0])
             q = (rng.normal(0, 1, n_head * hk) * scale).astype(np.float32)
