@@ -164,6 +164,29 @@ def test_q4k_gemm_mfma_parity(hip, oracle, n_tokens, n_out, n_in):
             assert abs(float(out[t, r]) - exact) <= 2e-6 * scale + 1e-30, (t, r)
 
 
+@pytest.mark.parametrize("n_tokens,n_out,n_in", [(70, 300, 768), (33, 129, 256), (200, 1024, 2048)])
+def test_q4k_gemm_both_token_tile_widths(hip, oracle, monkeypatch, n_tokens, n_out, n_in):
+    """The GEMM has a 32-token and a 64-token tile; the launcher picks by problem size.  Forced either way the
+    integers are the same and the f32 chain is the same, so the two agree bit for bit with each other and to
+    rounding with the AVX2-order result; ragged row and token tiles included."""
+    w = hip.synth.q4_k_weight(90 + n_tokens, n_out, n_in)
+    x = hip.synth.activations(91 + n_out, n_tokens, n_in)
+    kernel = hip.kernel.Q4_KKernel(w, n_in, n_out)
+    outs = {}
+    for tile in ("1", "2"):
+        monkeypatch.setenv("RMI_Q4K_GEMM_TTW", tile)
+        out = np.full((n_tokens, n_out), np.nan, np.float32)
+        kernel.forward_batched(x, out, n_in, n_out, matrix_cores=True)
+        outs[tile] = out
+    assert np.array_equal(bits(outs["1"]), bits(outs["2"]))
+    out = outs["1"]
+    for t in np.unique(np.linspace(0, n_tokens - 1, 9).astype(int)):
+        d, qs, bs = oracle.quantize_row_q8_k(x[t], A)
+        ref = np.zeros(n_out, np.float32)
+        oracle.q4k_forward_prepared(w, d, qs, bs, ref, n_in, n_out, 0, 1, A)
+        assert np.all(np.abs(out[t] - ref) <= 1e-4 + 1e-4 * np.abs(ref)), t
+
+
 # ----------------------------------------------------------------- dequant paths
 
 def test_q4k_grouped_launch_bit_exact(hip, oracle):
