@@ -367,7 +367,12 @@ int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const fl
                                  const float *sin_row, uint16_t *q16, uint16_t *k_row, uint16_t *v_row, uint32_t n_head,
                                  uint32_t n_head_kv, uint32_t head_dim_k, uint32_t head_dim_v, float eps, void *stream);
 /* Attention of one token over keys 0..n_keys-1 of an F16 cache [t][kv_stride] (src/models/qwen3.rs:876-933,
- * dot_f16 src/ops/dot.rs:99-119, softmax src/ops/attention.rs:28-38); the output leaves quantized to Q8_0. */
+ * dot_f16 src/ops/dot.rs:99-119, softmax src/ops/attention.rs:28-38); the output leaves quantized to Q8_0.
+ * Head dimension 128 and 768 keys or more: a head's keys are spread over up to 16 workgroups in two launches
+ * (scores; then weights and p.v, the parts meeting in the workgroup that arrives last).  The softmax sum is still
+ * the reference's sequential f32 sum; results have the same bits as the one-workgroup-per-head kernel.  The
+ * hand-over uses a scratch region of the calling host thread (allocated at the first such call, which also
+ * synchronises `stream` once): calls of one host thread that overlap on different streams would share it. */
 int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache,
                                             uint32_t n_keys, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv,
                                             uint32_t head_dim_k, uint32_t head_dim_v, int8_t *q8, float *scales,

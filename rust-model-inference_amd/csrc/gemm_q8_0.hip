@@ -68,7 +68,8 @@ __device__ __forceinline__ uint32_t voff(uint32_t &o) {
 
 // RAGGED: n_in / 32 is not a multiple of 4 (the last quad is partly padding) or the token scales are not
 // 16-byte aligned; token scales are then read one by one and indices past the row end are clamped.
-// PER_CU workgroups are to fit a compute unit at once (it bounds the registers a thread may take).
+// PER_CU bounds the registers a thread may take: it is the number of waves that are to share a SIMD (the second
+// argument of __launch_bounds__), which for these four-wave workgroups is also the workgroups per compute unit.
 template <int NTW, int TTW, int WN, int WT, int PER_CU, bool RAGGED>
 __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ x_q8,
                                                                  const float *__restrict__ x_scales, float *__restrict__ y,
