@@ -187,6 +187,30 @@ def test_q4k_gemm_both_token_tile_widths(hip, oracle, monkeypatch, n_tokens, n_o
         assert np.all(np.abs(out[t] - ref) <= 1e-4 + 1e-4 * np.abs(ref)), t
 
 
+def test_q4k_gemm_ragged_shapes_both_widths(hip, oracle, monkeypatch):
+    """Row counts around the 8-row tile and the 128-row workgroup, token counts around the 32- and 64-token tiles,
+    one to three super-blocks: both tile widths against the AVX2-order result, every output."""
+    shapes = [(17, 1, 256), (31, 7, 256), (32, 8, 512), (33, 9, 256), (63, 127, 256), (64, 128, 768), (65, 129, 512),
+              (96, 136, 256), (127, 250, 512), (129, 64, 256)]
+    for i, (n_tokens, n_out, n_in) in enumerate(shapes):
+        w = hip.synth.q4_k_weight(400 + i, n_out, n_in)
+        x = hip.synth.activations(420 + i, n_tokens, n_in)
+        kernel = hip.kernel.Q4_KKernel(w, n_in, n_out)
+        ref = np.zeros((n_tokens, n_out), np.float32)
+        for t in range(n_tokens):
+            d, qs, bs = oracle.quantize_row_q8_k(x[t], A)
+            oracle.q4k_forward_prepared(w, d, qs, bs, ref[t], n_in, n_out, 0, 1, A)
+        outs = []
+        for tile in ("1", "2"):
+            monkeypatch.setenv("RMI_Q4K_GEMM_TTW", tile)
+            out = np.full((n_tokens + 1, n_out), np.nan, np.float32)  # one row more: nothing may be written past the end
+            kernel.forward_batched(x, out[:n_tokens], n_in, n_out, matrix_cores=True)
+            assert np.all(np.isnan(out[n_tokens])), (n_tokens, n_out, n_in, tile)
+            assert np.all(np.abs(out[:n_tokens] - ref) <= 1e-4 + 1e-4 * np.abs(ref)), (n_tokens, n_out, n_in, tile)
+            outs.append(out[:n_tokens].copy())
+        assert np.array_equal(bits(outs[0]), bits(outs[1])), (n_tokens, n_out, n_in)
+
+
 # ----------------------------------------------------------------- dequant paths
 
 def test_q4k_grouped_launch_bit_exact(hip, oracle):
