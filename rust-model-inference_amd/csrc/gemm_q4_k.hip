@@ -31,13 +31,13 @@
 // requested and its registers take the piece of the super-block after at once.
 //
 // What bounds it, by the kernel's own clock stamps around the parts of a super-block (two waves a SIMD): a wave's
-// MFMAs and the vector instructions behind them do not overlap, only those of different waves do; with TTW = 2 the
-// eight calls (32 MFMAs) take about 2300 clocks for the two waves of a SIMD, which is their MFMAs back to back,
-// the fold and the next scales 1200, which is their vector instructions back to back, the barrier 300: the two
-// workgroups of a compute unit stay in step, so the halves add up instead of overlapping (a late start of one of
-// them does not last).  Folding a super-block between the MFMAs of the next one needs the chains twice: 64 more
-// registers, which TTW = 2 does not have at two waves a SIMD (it stands at 254) and which did not pay with TTW = 1
-// (half the MFMAs for the same vector work: the vector ALU is then the bound either way).
+// MFMAs and the vector instructions behind them do not overlap; with TTW = 2 the eight calls (32 MFMAs) take about
+// 2300 clocks for the two waves of a SIMD, which is their MFMAs back to back, the fold and the next scales 1200,
+// which is their vector instructions back to back, the barrier 300: the matrix-core half and the vector half add
+// up.  Putting the two waves of a SIMD into opposite halves (a late start of every second workgroup; an eight-wave
+// workgroup whose second four waves fold a super-block at the start of the next) changed nothing.  Folding a
+// super-block between the MFMAs of the next one needs the chains twice: 64 more registers, which TTW = 2 does not
+// have at two waves a SIMD (it stands at 254) and which did not pay with TTW = 1.
 #include <type_traits>
 
 #include "rmi_internal.h"
