@@ -237,3 +237,28 @@ def test_attention_f16_quantize(hip, oracle, hk, n_head, n_kv):
                                   s_ref.view(np.uint32)), (n_keys, trial)
             for b in (d_q, d_k, d_v, d_o, d_s):
                 b.free()
+
+
+def test_attention_split_mixed_head_counts(hip, oracle):
+    """Head dimension 128 from 768 keys on: launches with different head counts and key counts in turn share the
+    calling thread's scratch region (partial sums, arrival counters); every result has the checker's bits."""
+    H = hip.hip
+    rng = np.random.default_rng(77)
+    hk = hv = 128
+    for n_head, n_kv, n_keys in [(32, 8, 4097), (6, 2, 1500), (16, 8, 769), (32, 4, 768), (6, 6, 2300), (16, 8, 640), (32, 8, 1024)]:
+        kv_stride = n_kv * hk
+        q = rng.normal(0, 1, n_head * hk).astype(np.float32)
+        kc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+        vc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+        d_q, d_k, d_v = _dev(H, q.astype(np.float16).view(np.uint16)), _dev(H, kc), _dev(H, vc)
+        d_o, d_s = H.DeviceBuffer(n_head * hv), H.DeviceBuffer(n_head * hv // 32 * 4)
+        for _ in range(2):  # the second call meets the counters as the first left them
+            H.check(H.lib.rmi_hip_attention_f16_quantize_q8_0_dev(d_q.ptr, d_k.ptr, d_v.ptr, n_keys, kv_stride, n_head,
+                                                                  n_kv, hk, hv, d_o.ptr, d_s.ptr, A, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        ref = oracle.attention_f16(q, kc, vc, n_keys - 1, kv_stride, n_head, n_kv, hk, hv)
+        q_ref, s_ref = _quant(oracle, ref)
+        assert np.array_equal(d_o.to_array(np.int8, (n_head * hv,)), q_ref), (n_head, n_kv, n_keys)
+        assert np.array_equal(d_s.to_array(np.float32, (n_head * hv // 32,)).view(np.uint32), s_ref.view(np.uint32)), (n_head, n_kv, n_keys)
+        for b in (d_q, d_k, d_v, d_o, d_s):
+            b.free()
