@@ -41,6 +41,26 @@ __device__ __forceinline__ float h2f_times(uint32_t bits16, float x) {
     return h2f(bits16) * x;
 }
 
+// ---- which tile of a GEMM a workgroup takes.  Workgroups are handed to the 8 XCDs round-robin, each XCD with its
+// own L2, so the tiles are renumbered per XCD.  split_n = 0: an XCD's workgroups are consecutive tiles, running
+// fastest along the smaller operand; every XCD then fetches that operand whole and its own eighth of the larger one.
+// split_n = 2 or 4 (the tile grid divides evenly): the XCDs form a split_n x (8 / split_n) grid over the tile grid,
+// so every XCD fetches 1 / split_n of the weights and split_n / 8 of the tokens.
+__device__ __forceinline__ void rmi_gemm_tile_of(uint32_t lin, uint32_t grid_n, uint32_t grid_t, uint32_t t_fastest,
+                                                 uint32_t split_n, uint32_t &n_tile, uint32_t &t_tile) {
+    const uint32_t xcd = lin & 7, slot = lin >> 3;
+    if (split_n == 0) {
+        const uint32_t n_groups = grid_n * grid_t;
+        const uint32_t tile_id = xcd * (n_groups >> 3) + (xcd < (n_groups & 7) ? xcd : (n_groups & 7)) + slot;
+        n_tile = t_fastest ? tile_id / grid_t : tile_id % grid_n;
+        t_tile = t_fastest ? tile_id % grid_t : tile_id / grid_n;
+    } else {
+        const uint32_t sub_n = grid_n / split_n, sub_t = grid_t / (8 / split_n);
+        n_tile = (xcd % split_n) * sub_n + (t_fastest ? slot / sub_t : slot % sub_n);
+        t_tile = (xcd / split_n) * sub_t + (t_fastest ? slot % sub_t : slot / sub_n);
+    }
+}
+
 // signed 4 x int8 dot from zero (the build turns v_dot4c off, so this is one v_dot4_i32_i8 with a literal 0)
 __device__ __forceinline__ int dot4_i8(int a, int b) {
     return __builtin_amdgcn_sdot4(a, b, 0, false);

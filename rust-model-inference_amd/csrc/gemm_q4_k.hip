@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
                                                                          const int16_t *__restrict__ q8bs, float *__restrict__ y,
                                                                          uint32_t n_out, uint32_t n_sb, uint32_t n_tiles,
                                                                          uint32_t n_tokens, uint32_t y_stride, uint32_t grid_n,
-                                                                         uint32_t grid_t, uint32_t t_fastest) {
+                                                                         uint32_t grid_t, uint32_t t_fastest, uint32_t xcd_split) {
     constexpr int kTileN = 128, kTileT = 32 * TTW;
     constexpr int kXPieces = kTileT * 16 / 256;  // 16-byte pieces of the token tile per thread and super-block
     constexpr int kXBuf = kTileT * kXRow, kBBuf = kTileT * kBRow, kWBuf = kTileN * kWRow;
@@ -124,12 +124,9 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = uint32_t(__builtin_amdgcn_readfirstlane(int(tid >> 6)));
     const uint32_t c = lane & 31, h = lane >> 5;
     const uint32_t n_off = wave * 32;
-    // one XCD's workgroups are consecutive tiles, fastest along the smaller operand (see gemm_q8_0.hip)
-    const uint32_t n_groups = grid_n * grid_t, lin = blockIdx.x;
-    const uint32_t xcd = lin & 7, slot = lin >> 3;
-    const uint32_t tile_id = xcd * (n_groups >> 3) + (xcd < (n_groups & 7) ? xcd : (n_groups & 7)) + slot;
-    const uint32_t n0 = (t_fastest ? tile_id / grid_t : tile_id % grid_n) * kTileN;
-    const uint32_t t0 = (t_fastest ? tile_id % grid_t : tile_id / grid_n) * kTileT;
+    uint32_t n_tile, t_tile;  // one XCD's workgroups take neighbouring tiles
+    rmi_gemm_tile_of(blockIdx.x, grid_n, grid_t, t_fastest, xcd_split, n_tile, t_tile);
+    const uint32_t n0 = n_tile * kTileN, t0 = t_tile * kTileT;
     const uint32_t n_in = n_sb * 256;
     const uint32_t sb_last = n_sb - 1;
     auto clampsb = [&](uint32_t sb) __attribute__((always_inline)) { return sb < sb_last ? sb : sb_last; };
@@ -396,8 +393,9 @@ template <int TTW, int WAVES_PER_SIMD>
 void launch(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bs, float *y, uint32_t n_tokens,
             uint32_t y_stride, hipStream_t s) {
     const uint32_t grid_n = (w->n_out + 127) / 128, grid_t = (n_tokens + 32 * TTW - 1) / (32 * TTW);
+    const uint32_t xcd_split = rmi_gemm_xcd_split(grid_n, grid_t, double(w->n_out) * w->n_units * 144.0, double(n_tokens) * w->n_units * 292.0);
     hipLaunchKernelGGL((gemm_q4_k_kernel<TTW, WAVES_PER_SIMD>), dim3(grid_n * grid_t), dim3(256), 0, s, w->data, d, qs, bs, y,
-                       w->n_out, w->n_units, w->n_tiles, n_tokens, y_stride, grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u);
+                       w->n_out, w->n_units, w->n_tiles, n_tokens, y_stride, grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
 }
 
 }  // namespace

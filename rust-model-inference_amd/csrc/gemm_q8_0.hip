@@ -75,7 +75,7 @@ __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const u
                                                                  const float *__restrict__ x_scales, float *__restrict__ y,
                                                                  uint32_t n_out, uint32_t n_in, uint32_t n_oct,
                                                                  uint32_t n_tiles, uint32_t n_tokens, uint32_t y_stride,
-                                                                 uint32_t grid_n, uint32_t grid_t, uint32_t t_fastest) {
+                                                                 uint32_t grid_n, uint32_t grid_t, uint32_t t_fastest, uint32_t xcd_split) {
     constexpr int kThreads = 64 * WN * WT;
     constexpr int kTileN = 32 * NTW * WN, kTileT = 32 * TTW * WT;
     constexpr int kWPieces = kTileN * 8 / kThreads;  // 16-byte pieces of the weight tile per thread
@@ -90,14 +90,9 @@ __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const u
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = uint32_t(__builtin_amdgcn_readfirstlane(int(tid >> 6)));
     const uint32_t c = lane & 31, h = lane >> 5;
     const uint32_t n_off = (wave % WN) * 32 * NTW, t_off = (wave / WN) * 32 * TTW;
-    // Workgroups are handed to the 8 XCDs round-robin, each XCD with its own L2.  Renumber them so that the
-    // workgroups of one XCD are consecutive tiles, running fastest along the smaller operand: every XCD then
-    // fetches that operand whole and only its own eighth of the larger one.
-    const uint32_t n_groups = grid_n * grid_t, lin = blockIdx.x;
-    const uint32_t xcd = lin & 7, slot = lin >> 3;
-    const uint32_t tile_id = xcd * (n_groups >> 3) + (xcd < (n_groups & 7) ? xcd : (n_groups & 7)) + slot;
-    const uint32_t n0 = (t_fastest ? tile_id / grid_t : tile_id % grid_n) * kTileN;
-    const uint32_t t0 = (t_fastest ? tile_id % grid_t : tile_id / grid_n) * kTileT;
+    uint32_t n_tile, t_tile;  // one XCD's workgroups take neighbouring tiles
+    rmi_gemm_tile_of(blockIdx.x, grid_n, grid_t, t_fastest, xcd_split, n_tile, t_tile);
+    const uint32_t n0 = n_tile * kTileN, t0 = t_tile * kTileT;
     const uint32_t nb = n_in >> 5, n_quads = (nb + 3) >> 2;
     const uint32_t t_last = n_tokens - 1 - t0;  // last token of the input, counted from this tile's first
 
@@ -409,14 +404,15 @@ void launch_gemm(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_sca
                  uint32_t y_stride, bool ragged, hipStream_t s) {
     constexpr uint32_t tile_n = 32 * NTW * WN, tile_t = 32 * TTW * WT;
     const uint32_t grid_n = (w->n_out + tile_n - 1) / tile_n, grid_t = (n_tokens + tile_t - 1) / tile_t;
+    const uint32_t xcd_split = rmi_gemm_xcd_split(grid_n, grid_t, double(w->n_out) * w->n_in * (34.0 / 32.0), double(n_tokens) * w->n_in * (36.0 / 32.0));
     if (ragged)
         hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, PER_CU, true>), dim3(grid_n * grid_t), dim3(64 * WN * WT), 0, s,
                            w->data, x_q8, x_scales, y, w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride,
-                           grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u);
+                           grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
     else
         hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, PER_CU, false>), dim3(grid_n * grid_t), dim3(64 * WN * WT), 0, s,
                            w->data, x_q8, x_scales, y, w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride,
-                           grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u);
+                           grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
 }
 
 // A tile shape: rows x tokens of a workgroup, sub-tiles per wave, waves, how many workgroups a compute unit holds

@@ -92,6 +92,24 @@ inline bool rmi_misaligned(const void *quants, const void *a = nullptr, const vo
 }
 #define RMI_ALIGNMENT_MESSAGE "activation quants must be 16-byte aligned, scales / sums / outputs 4-byte aligned"
 
+// How the 8 XCDs divide a GEMM's grid_n x grid_t tiles (rmi_gemm_tile_of, device_common.h): the split along the rows
+// that makes the XCDs together fetch the fewest operand bytes, 8 * (w_bytes / split + x_bytes * split / 8), among
+// those that divide the tile grid evenly; 0 = the one-dimensional renumbering, which takes any grid.
+inline uint32_t rmi_gemm_xcd_split(uint32_t grid_n, uint32_t grid_t, double w_bytes, double x_bytes) {
+    const double one_dim = w_bytes < x_bytes ? 8.0 * w_bytes + x_bytes : w_bytes + 8.0 * x_bytes;
+    uint32_t best = 0;
+    double best_cost = one_dim;
+    for (uint32_t split : {2u, 4u}) {
+        if (grid_n % split != 0 || grid_t % (8 / split) != 0) continue;
+        const double cost = w_bytes * (8 / split) + x_bytes * split;
+        if (cost < best_cost * 0.95) {
+            best_cost = cost;
+            best = split;
+        }
+    }
+    return best;
+}
+
 #define RMI_REQUIRE_INIT()                                                             \
     do {                                                                               \
         if (!rmi_ready()) return rmi_fail(RMI_HIP_E_NOT_INIT, "rmi_hip_init has not succeeded"); \
