@@ -119,6 +119,34 @@ int main() {
         CK(hipFree(p));
     }
 
+    // ---- 1b. the same chain with kernels that do a small GEMV's worth of reading (3 MB each, 64 buffers in turn)
+    {
+        const size_t bytes = 3u << 20, n16 = bytes / 16;
+        const int N = 144, REP = 100;
+        uint4 *pool;
+        uint32_t *sink;
+        CK(hipMalloc(&pool, bytes * 64));
+        CK(hipMemset(pool, 1, bytes * 64));
+        CK(hipMalloc(&sink, 4));
+        for (int wgs : {64, 256, 1024}) {
+            auto enqueue = [&]() { for (int i = 0; i < N; i++) hipLaunchKernelGGL(read_kernel, dim3(wgs), dim3(256), 0, st, pool + size_t(i % 64) * n16, n16, sink); };
+            enqueue(); CK(hipStreamSynchronize(st));
+            CK(hipEventRecord(e0, st)); for (int r = 0; r < REP; r++) enqueue(); CK(hipEventRecord(e1, st)); CK(hipEventSynchronize(e1));
+            CK(hipEventElapsedTime(&ms, e0, e1));
+            printf("chain of %d 3 MB reads, %4d workgroups each: stream launches %.2f us per kernel", N, wgs, ms * 1e3 / (N * REP));
+            hipGraph_t graph; hipGraphExec_t exec;
+            CK(hipStreamBeginCapture(st, hipStreamCaptureModeGlobal)); enqueue(); CK(hipStreamEndCapture(st, &graph));
+            CK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+            for (int r = 0; r < 3; r++) CK(hipGraphLaunch(exec, st));
+            CK(hipStreamSynchronize(st));
+            CK(hipEventRecord(e0, st)); for (int r = 0; r < REP; r++) CK(hipGraphLaunch(exec, st)); CK(hipEventRecord(e1, st)); CK(hipEventSynchronize(e1));
+            CK(hipEventElapsedTime(&ms, e0, e1));
+            printf(", graph replay %.2f us per kernel\n", ms * 1e3 / (N * REP));
+            CK(hipGraphExecDestroy(exec)); CK(hipGraphDestroy(graph));
+        }
+        CK(hipFree(pool)); CK(hipFree(sink));
+    }
+
     // ---- 2. a grid-wide barrier among co-resident workgroups (at most one per compute unit)
     {
         uint32_t *counter, *flag;
