@@ -96,7 +96,10 @@ inline bool rmi_misaligned(const void *quants, const void *a = nullptr, const vo
 // that makes the XCDs together fetch the fewest operand bytes, 8 * (w_bytes / split + x_bytes * split / 8), among
 // those that divide the tile grid evenly; 0 = the one-dimensional renumbering, which takes any grid.
 inline uint32_t rmi_gemm_xcd_split(uint32_t grid_n, uint32_t grid_t, double w_bytes, double x_bytes) {
-    if (const char *e = getenv("RMI_GEMM_XCD_SPLIT")) return uint32_t(atoi(e)) & 6u;  // 0, 2 or 4: for measurements
+    if (const char *e = getenv("RMI_GEMM_XCD_SPLIT")) {  // for measurements: 2 or 4 where the grid allows it, else 0
+        const uint32_t f = uint32_t(atoi(e));
+        return (f == 2 || f == 4) && grid_n % f == 0 && grid_t % (8 / f) == 0 ? f : 0u;
+    }
     const double one_dim = w_bytes < x_bytes ? 8.0 * w_bytes + x_bytes : w_bytes + 8.0 * x_bytes;
     uint32_t best = 0;
     double best_cost = one_dim;
