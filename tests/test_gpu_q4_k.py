@@ -211,6 +211,26 @@ def test_q4k_gemm_ragged_shapes_both_widths(hip, oracle, monkeypatch):
         assert np.array_equal(bits(outs[0]), bits(outs[1])), (n_tokens, n_out, n_in)
 
 
+@pytest.mark.parametrize("n_tokens,n_out,n_in", [(256, 1024, 512), (128, 512, 256), (70, 300, 768)])
+def test_q4k_gemm_tile_to_xcd_assignment_changes_no_bit(hip, oracle, monkeypatch, n_tokens, n_out, n_in):
+    """The Q4_K prefill GEMM with the assignment of tiles to XCDs forced each way: the same bits."""
+    w = hip.synth.q4_k_weight(500 + n_tokens, n_out, n_in)
+    x = hip.synth.activations(501 + n_out, n_tokens, n_in)
+    kernel = hip.kernel.Q4_KKernel(w, n_in, n_out)
+    outs = []
+    for split in (None, "0", "2", "4"):
+        if split is None:
+            monkeypatch.delenv("RMI_GEMM_XCD_SPLIT", raising=False)
+        else:
+            monkeypatch.setenv("RMI_GEMM_XCD_SPLIT", split)
+        out = np.full((n_tokens, n_out), np.nan, np.float32)
+        kernel.forward_batched(x, out, n_in, n_out, matrix_cores=True)
+        outs.append(out)
+    assert not np.any(np.isnan(outs[0]))
+    for o in outs[1:]:
+        assert np.array_equal(bits(o), bits(outs[0]))
+
+
 # ----------------------------------------------------------------- dequant paths
 
 def test_q4k_grouped_launch_bit_exact(hip, oracle):

@@ -428,6 +428,30 @@ def test_gemm_full_size_properties(hip, oracle, n_tokens, n_out, n_in):
     assert np.array_equal(bits(part), bits(out[lo:lo + 64]))
 
 
+@pytest.mark.parametrize("n_tokens,n_out,n_in", [(512, 768, 512), (256, 1536, 256), (130, 200, 320)])
+def test_gemm_tile_to_xcd_assignment_changes_no_bit(hip, oracle, monkeypatch, n_tokens, n_out, n_in):
+    """Which XCD takes which tile of the prefill GEMM (one-dimensional renumbering, 2 x 4 or 4 x 2 grids of XCDs) is a
+    matter of cache traffic: forced each way, where the tile grid allows it and where it does not, every output has the
+    same bits, and those of the checker's NEON order."""
+    w, x = _case(hip, 3000 + n_tokens, n_out, n_in, n_tokens)
+    kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
+    outs = []
+    for split in (None, "0", "2", "4"):
+        if split is None:
+            monkeypatch.delenv("RMI_GEMM_XCD_SPLIT", raising=False)
+        else:
+            monkeypatch.setenv("RMI_GEMM_XCD_SPLIT", split)
+        out = np.full((n_tokens, n_out), np.nan, np.float32)
+        kernel.forward_batched(x, out, n_in, n_out, matrix_cores=True)
+        outs.append(out)
+    for o in outs[1:]:
+        assert np.array_equal(bits(o), bits(outs[0]))
+    sample = [0, n_tokens // 3, n_tokens - 1]
+    q8, sc = _quantize_rows(oracle, x[sample])
+    for i, t in enumerate(sample):
+        assert np.array_equal(bits(outs[0][t]), bits(oracle.matmul_q8_0_quantized(w, q8[i], sc[i], n_in, n_out, N)))
+
+
 @pytest.mark.parametrize("n_tokens", [9, 16, 17, 40])
 def test_forward_batched_does_not_depend_on_the_batch(hip, oracle, n_tokens):
     """trait_.rs:78-109: every token goes through the same quantizer and kernel, so forward_batched(x)[t] ==
