@@ -15,8 +15,9 @@
 // those with odd L tile B's, then the other way round, and each destination lane sorts the two arrivals into
 // low and high dword.  The activations sit in LDS in natural order, one row per token (rows 32 bytes apart from
 // a multiple of 256, which spreads the 8-byte reads of a quarter wave over all banks), with their block scales.
-// Lane 16g + m receives the dots of rows 4g..4g+3 of the pair for token m: it loads those rows' f16 scales
-// itself (16 bytes a row and octet, the same address for the 16 lanes of a g).
+// Lane 16g + m receives the dots of rows 4g..4g+3 of the pair for token m.  Those rows' f16 scales (64 bytes an
+// octet, the same for the 16 lanes of a g) are loaded a dword a lane and shared by DPP row broadcasts.  A lane's
+// four rows are neighbours in y and leave as one 16-byte store, two pairs of tiles at a time.
 #include "rmi_internal.h"
 
 #include "device_common.h"
@@ -24,18 +25,34 @@
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef f32x4 __attribute__((address_space(1))) *gptr_f32x4_w;
 
 constexpr uint32_t kRowPadBytes = 32;   // added to a token's row of quants in LDS
 constexpr uint32_t kScalePadFloats = 4; // added to a token's row of block scales in LDS
+// Results of this many pairs of tiles are kept before they are stored: a token's 32 rows then leave together and
+// fill a 128-byte line of y.  (Stores that reach HBM are dear next to the weight stream: with 8 tokens they are 3 %
+// of the bytes and cost 10 % of the time; 4-byte stores, one row a lane, cost 15 %.)
+constexpr int kHoldPairs = 2;
 
 __host__ __device__ inline size_t mfma_lds_bytes(uint32_t n_tokens, uint32_t n_oct) {
     return size_t(n_tokens) * (size_t(n_oct) * 256 + kRowPadBytes) +
            size_t(n_tokens) * (size_t(n_oct) * 8 + kScalePadFloats) * 4;
 }
 
+// Lane K of every sixteen lanes, to all of the sixteen (DPP row_newbcast).
+template <int K>
+__device__ __forceinline__ uint32_t row_bcast(uint32_t x) {
+    return uint32_t(__builtin_amdgcn_update_dpp(0, int(x), 0x150 + K, 0xf, 0xf, false));
+}
+
 struct PairRegs {        // one octet of two tiles
     u32x4 qa[2], qb[2];  // [tile]: blocks 8o..8o+3 and 8o+4..8o+7, bytes 4L..4L+3 of each, of row r
-    u32x4 sc[4];         // the octet's 8 f16 block scales of rows 4g..4g+3 of the pair
+    // Block scales of rows 4g..4g+3 of the pair: 64 bytes that all sixteen lanes of a g need.  Each lane loads one
+    // dword of them, lane 16g + m the f16 scales of blocks 2(m&3), 2(m&3)+1 of row 4g + (m>>2), and the sixteen
+    // share them by row broadcasts when they are used: one load instruction an octet instead of four, 1 register
+    // instead of 16.
+    uint32_t sc1;
 };
 
 // The activations of the n_tokens tokens into LDS: quants in natural order, a row per token, then the block
@@ -162,8 +179,7 @@ __global__ __launch_bounds__(512) void gemv_q8_0_mfma_kernel(RmiGemvProblem sing
             R.qa[1] = __builtin_nontemporal_load(qb);
             R.qb[1] = __builtin_nontemporal_load(qb + 64);
             gptr_u4 sc = (g >> 1 ? tile_b : tile_a) + o * 8 + 4 * (g & 1);
-#pragma unroll
-            for (int i = 0; i < 4; i++) R.sc[i] = sc[i];
+            R.sc1 = reinterpret_cast<gptr_u32>(sc)[lane & 15];
         }
         __device__ __forceinline__ void step() {
             if (++o == n_oct) {
@@ -215,7 +231,39 @@ __global__ __launch_bounds__(512) void gemv_q8_0_mfma_kernel(RmiGemvProblem sing
         for (int v = 0; v < 4; v++) acc[tt][v] = 0.0f;
     uint32_t o = 0, pair = 0;
     gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && (p.y_stride & 3) == 0;
 
+    // finished pairs wait here (consecutive pairs of the run: rows first_row0 + 16 j) and are stored together; only
+    // the run's last pair can lack its second tile
+    float hold[TT][kHoldPairs][4];
+    uint32_t held = 0, first_row0 = 0;
+    bool last_has_b = true;
+    auto flush = [&]() {
+#pragma unroll
+        for (int j = 0; j < kHoldPairs; j++) {
+            if (uint32_t(j) < held) {
+                const uint32_t row0 = first_row0 + 16 * j;
+                const bool has_b = uint32_t(j) + 1 < held || last_has_b;
+                const bool whole = vec_ok && row0 >= p.row_start && row0 + 4 <= p.row_end;
+#pragma unroll
+                for (int tt = 0; tt < TT; tt++) {
+                    const uint32_t token = tt * 16 + m;
+                    if (token < n_tokens && (g < 2 || has_b)) {
+                        if (whole) {
+                            const f32x4 out = {hold[tt][j][0], hold[tt][j][1], hold[tt][j][2], hold[tt][j][3]};
+                            *reinterpret_cast<gptr_f32x4_w>(yp + size_t(token) * p.y_stride + row0) = out;
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 4; v++)
+                                if (row0 + v >= p.row_start && row0 + v < p.row_end)
+                                    yp[size_t(token) * p.y_stride + row0 + v] = hold[tt][j][v];
+                        }
+                    }
+                }
+            }
+        }
+        held = 0;
+    };
     auto consume = [&](const PairRegs &R) {
         float4 xs[TT][2];  // this lane's token's eight block scales of the octet
 #pragma unroll
@@ -226,8 +274,11 @@ __global__ __launch_bounds__(512) void gemv_q8_0_mfma_kernel(RmiGemvProblem sing
         }
         const uint32_t wq[2][8] = {{R.qa[0].x, R.qa[0].y, R.qa[0].z, R.qa[0].w, R.qb[0].x, R.qb[0].y, R.qb[0].z, R.qb[0].w},
                                    {R.qa[1].x, R.qa[1].y, R.qa[1].z, R.qa[1].w, R.qb[1].x, R.qb[1].y, R.qb[1].z, R.qb[1].w}};
-        const uint32_t scw[4][4] = {{R.sc[0].x, R.sc[0].y, R.sc[0].z, R.sc[0].w}, {R.sc[1].x, R.sc[1].y, R.sc[1].z, R.sc[1].w},
-                                    {R.sc[2].x, R.sc[2].y, R.sc[2].z, R.sc[2].w}, {R.sc[3].x, R.sc[3].y, R.sc[3].z, R.sc[3].w}};
+        // [row v][block pair]: lane 4v + pair of this lane's sixteen holds it
+        const uint32_t scw[4][4] = {{row_bcast<0>(R.sc1), row_bcast<1>(R.sc1), row_bcast<2>(R.sc1), row_bcast<3>(R.sc1)},
+                                    {row_bcast<4>(R.sc1), row_bcast<5>(R.sc1), row_bcast<6>(R.sc1), row_bcast<7>(R.sc1)},
+                                    {row_bcast<8>(R.sc1), row_bcast<9>(R.sc1), row_bcast<10>(R.sc1), row_bcast<11>(R.sc1)},
+                                    {row_bcast<12>(R.sc1), row_bcast<13>(R.sc1), row_bcast<14>(R.sc1), row_bcast<15>(R.sc1)}};
 #pragma unroll
         for (int b = 0; b < 8; b++) {
             const int first = int(l_even ? wq[0][b] : wq[1][b]), second = int(l_even ? wq[1][b] : wq[0][b]);
@@ -249,18 +300,19 @@ __global__ __launch_bounds__(512) void gemv_q8_0_mfma_kernel(RmiGemvProblem sing
             }
         }
         if (++o == n_oct) {  // the pair is done: rows 4g..4g+3 of it, token m of each sixteen
-            const bool has_b = 2 * pair + 1 < run_tiles;
+            if (held == 0) first_row0 = (p.tile0 + k + 2 * pair) * kTileRows + 4 * g;
 #pragma unroll
-            for (int tt = 0; tt < TT; tt++) {
-                const uint32_t token = tt * 16 + m;
+            for (int tt = 0; tt < TT; tt++)
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const uint32_t row = (p.tile0 + k + 2 * pair) * kTileRows + 4 * g + v;
-                    if (token < n_tokens && (g < 2 || has_b) && row >= p.row_start && row < p.row_end)
-                        yp[size_t(token) * p.y_stride + row] = acc[tt][v];
+#pragma unroll
+                    for (int j = 0; j < kHoldPairs; j++)
+                        if (held == uint32_t(j)) hold[tt][j][v] = acc[tt][v];
                     acc[tt][v] = 0.0f;
                 }
-            }
+            last_has_b = 2 * pair + 1 < run_tiles;
+            held++;
+            if (held == kHoldPairs) flush();
             o = 0;
             pair++;
         }
@@ -271,6 +323,7 @@ __global__ __launch_bounds__(512) void gemv_q8_0_mfma_kernel(RmiGemvProblem sing
         fetch(R0);
         if (u + 1 < n_units) consume(R1);
     }
+    if (held) flush();
 }
 
 size_t mfma_lds_limit();
