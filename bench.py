@@ -376,7 +376,9 @@ def run_small_batches(args, pkg, ev):
         def step(g=group):
             H.check(H.lib.rmi_hip_gemv_group_run_dev(g, None))
 
-        wall, dev_ms = time_region(H, ev, step, 30, 5)
+        # a step is 0.13 ms: 200 of them after 50 untimed ones, so that the figure is the steady state
+        steps, warmup = 200, 50
+        wall, dev_ms = time_region(H, ev, step, steps, warmup)
         alg = sum(synth.q8_0_gemv_bytes(r["n_out"], r["n_in"], batch) for r in problems)
         achieved = alg / (dev_ms * 1e-3) / 1e9
         out[label] = {
@@ -384,7 +386,7 @@ def run_small_batches(args, pkg, ev):
                         + ("x86-64 accumulation order (GEMV)" if order == "avx2" else
                            "aarch64 accumulation order (small-batch kernel on the matrix cores)"),
             "value": round(alg / wall / 1e9, 1), "unit": "GB/s", "ms_per_step": round(wall * 1e3, 4),
-            "token_steps_per_s": round(batch / wall, 1), "algorithmic_bytes_per_step": alg,
+            "steps": steps, "warmup": warmup, "token_steps_per_s": round(batch / wall, 1), "algorithmic_bytes_per_step": alg,
             "roofline": {"bound": "hbm",
                          "kernel": "gemv_q8_0_kernel<%d,true,%s>" % (batch, group_maxt(H, group)) if order == "avx2"
                                    else "gemv_q8_0_mfma_kernel<%d,true>" % ((batch + 15) // 16),
