@@ -69,6 +69,33 @@ def test_row_ranges_and_stride(hip, oracle):
     _run(hip, oracle, 503, n_out, n_in, 4, r0=500, r1=500)  # empty: nothing is written
 
 
+def test_output_store_paths(hip, oracle):
+    """The kernel stores a lane's four neighbouring rows as one 16-byte piece where y allows it (base 16-byte
+    aligned, stride a multiple of four floats, the four rows inside the row range) and row by row elsewhere: a
+    row range that cuts groups of four at both ends on an aligned stride, the same on a base that is 4 bytes off,
+    and an odd number of tile pairs so that the last stores hold one pair."""
+    H = hip.hip
+    n_out, n_in, n_tokens = 8 * 37, 512, 11
+    w = hip.synth.q8_0_weight(610, n_out, n_in)
+    k = hip.kernel.Q8Kernel(w, n_in, n_out)
+    q8, sc = _acts(hip, oracle, 611, n_tokens, n_in)
+    d_q8, d_sc = H.DeviceBuffer.from_array(q8), H.DeviceBuffer.from_array(sc)
+    ref = _ref(oracle, w, q8, sc, n_in, n_out)
+    for stride, shift, r0, r1 in ((n_out + 8, 0, 13, n_out - 5), (n_out + 8, 1, 13, n_out - 5), (n_out, 0, 0, n_out),
+                                  (n_out + 4, 1, 0, n_out), (n_out + 8, 0, 4, 8)):
+        sentinel = np.full(n_tokens * stride + 4, np.float32(-3.75))
+        d_y = H.DeviceBuffer.from_array(sentinel)
+        H.check(H.lib.rmi_hip_gemv_q8_0_neon_dev(k.w.handle, d_q8.ptr, d_sc.ptr, d_y.ptr + 4 * shift, n_tokens, stride,
+                                                 r0, r1, None))
+        H.check(H.lib.rmi_hip_synchronize())
+        flat = d_y.to_array(np.float32, (n_tokens * stride + 4,))
+        got = flat[shift:shift + n_tokens * stride].reshape(n_tokens, stride)
+        assert np.array_equal(bits(got[:, r0:r1]), bits(ref[:, r0:r1])), (stride, shift, r0, r1)
+        keep = np.ones(flat.shape, bool)
+        keep[shift:shift + n_tokens * stride].reshape(n_tokens, stride)[:, r0:r1] = False
+        assert np.all(flat[keep] == np.float32(-3.75)), ("outside the row range", stride, shift, r0, r1)
+
+
 @pytest.mark.parametrize("seed", [1, 2])
 def test_grouped_launch(hip, oracle, seed):
     """One launch over a list of matrices of unlike widths and heights, 3 / 16 / 40 tokens."""
