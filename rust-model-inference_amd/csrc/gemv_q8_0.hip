@@ -82,9 +82,81 @@ __device__ __forceinline__ void stage_token(uint32_t *dq, const int8_t *x_q8, co
     }
 }
 
+// acc = fma(s of lane K of this lane's quad, p, acc): v_fmac_f32 takes its first factor through DPP, so the
+// broadcast costs no instruction of its own.  (The compiler does not fold a DPP move into the VOP3 fma it selects.)
+template <int K>
+__device__ __forceinline__ void fmac_quad(float &acc, float s, float p);
+template <>
+__device__ __forceinline__ void fmac_quad<0>(float &acc, float s, float p) {
+    asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(s), "v"(p));
+}
+template <>
+__device__ __forceinline__ void fmac_quad<1>(float &acc, float s, float p) {
+    asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(s), "v"(p));
+}
+template <>
+__device__ __forceinline__ void fmac_quad<2>(float &acc, float s, float p) {
+    asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(s), "v"(p));
+}
+template <>
+__device__ __forceinline__ void fmac_quad<3>(float &acc, float s, float p) {
+    asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(s), "v"(p));
+}
+__device__ __forceinline__ void fmac_quad_k(float &acc, float s, float p, int k) {  // k is a constant once unrolled
+    if (k == 0) fmac_quad<0>(acc, s, p);
+    else if (k == 1) fmac_quad<1>(acc, s, p);
+    else if (k == 2) fmac_quad<2>(acc, s, p);
+    else fmac_quad<3>(acc, s, p);
+}
+
 template <int B>
 __device__ __forceinline__ void octet_fma(float (&acc)[B], const OctetRegs &g, const uint4 *lds, uint32_t tok_u4,
                                           uint32_t n_oct, uint32_t o, uint32_t L) {
+    if constexpr (B >= 2) {
+        // The scale product of (row, block, token) is the same in the row's eight lanes: each lane of a quad
+        // multiplies it for token (lane & 3) and token (lane & 3) + 4 only, and the fma takes it from there.
+        const uint32_t q = L & 3;
+        const uint4 *x0 = lds + (q < B ? q : 0) * tok_u4, *x1 = lds + (q + 4 < B ? q + 4 : 0) * tok_u4;
+        const float4 a0 = reinterpret_cast<const float4 *>(x0 + n_oct * 16)[2 * o];
+        const float4 a1 = reinterpret_cast<const float4 *>(x0 + n_oct * 16)[2 * o + 1];
+        const float xs0[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        float xs1[8];
+        if constexpr (B > 4) {
+            const float4 b0 = reinterpret_cast<const float4 *>(x1 + n_oct * 16)[2 * o];
+            const float4 b1 = reinterpret_cast<const float4 *>(x1 + n_oct * 16)[2 * o + 1];
+            xs1[0] = b0.x, xs1[1] = b0.y, xs1[2] = b0.z, xs1[3] = b0.w, xs1[4] = b1.x, xs1[5] = b1.y, xs1[6] = b1.z, xs1[7] = b1.w;
+        }
+        const uint32_t scw[4] = {g.sc.x, g.sc.y, g.sc.z, g.sc.w};
+        float s0[8], s1[8];
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const float wd = h2f((b & 1) ? scw[b >> 1] >> 16 : scw[b >> 1] & 0xffffu);
+            s0[b] = wd * xs0[b];
+            if constexpr (B > 4) s1[b] = wd * xs1[b];
+        }
+        // a DPP read of a register needs two wait states after the vector instruction that wrote it, and the
+        // compiler does not look into the asm statements below: all products pass this point first
+        if constexpr (B > 4)
+            asm volatile("s_nop 1" : "+v"(s0[0]), "+v"(s0[1]), "+v"(s0[2]), "+v"(s0[3]), "+v"(s0[4]), "+v"(s0[5]), "+v"(s0[6]), "+v"(s0[7]),
+                                     "+v"(s1[0]), "+v"(s1[1]), "+v"(s1[2]), "+v"(s1[3]), "+v"(s1[4]), "+v"(s1[5]), "+v"(s1[6]), "+v"(s1[7]));
+        else
+            asm volatile("s_nop 1" : "+v"(s0[0]), "+v"(s0[1]), "+v"(s0[2]), "+v"(s0[3]), "+v"(s0[4]), "+v"(s0[5]), "+v"(s0[6]), "+v"(s0[7]));
+        const int wq[8] = {int(g.qa.x), int(g.qa.y), int(g.qa.z), int(g.qa.w), int(g.qb.x), int(g.qb.y), int(g.qb.z), int(g.qb.w)};
+#pragma unroll
+        for (int t = 0; t < B; t++) {
+            const uint4 *xt = lds + t * tok_u4;
+            const uint4 xa = xt[(2 * o) * 8 + L];
+            const uint4 xb = xt[(2 * o + 1) * 8 + L];
+            const int xq[8] = {int(xa.x), int(xa.y), int(xa.z), int(xa.w), int(xb.x), int(xb.y), int(xb.z), int(xb.w)};
+            float a = acc[t];
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                fmac_quad_k(a, t < 4 ? s0[b] : s1[b], float(dot4_i8(wq[b], xq[b])), t & 3);
+            }
+            acc[t] = a;
+        }
+        return;
+    }
 #pragma unroll
     for (int t = 0; t < B; t++) {
         const uint4 *xt = lds + t * tok_u4;

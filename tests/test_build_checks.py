@@ -1,0 +1,55 @@
+"""The build-time check for hand-written DPP instructions (rust-model-inference_amd/csrc/check_dpp_hazards.py)
+flags what it is there to flag.  The compiler's hazard recogniser does not look into inline asm: a DPP operand read
+within two wait states of the vector instruction that wrote it, or within five of a vector write of EXEC, returns
+stale data on the GPU without any error, so the check must not pass such code."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CHECK = os.path.join(HERE, "..", "rust-model-inference_amd", "csrc", "check_dpp_hazards.py")
+
+FMAC = "v_fmac_f32_dpp v10, v3, v7 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf"
+
+
+def _run(tmp_path, body, *args):
+    f = tmp_path / "k.s"
+    f.write_text("\t.text\nkernel:\n" + "".join("\t%s\n" % line for line in body) + "\ts_endpgm\n")
+    return subprocess.run([sys.executable, CHECK, str(f), *args], capture_output=True, text=True)
+
+
+def test_clean_code_passes(tmp_path):
+    r = _run(tmp_path, ["v_mul_f32_e32 v3, v1, v2", "v_add_u32_e32 v20, v21, v22", "v_cvt_f32_i32_e32 v7, v8", FMAC], "1")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "1 v_fmac_f32_dpp), 0 hazards" in r.stdout
+
+
+def test_write_right_before_the_dpp_read_fails(tmp_path):
+    r = _run(tmp_path, ["v_mul_f32_e32 v3, v1, v2", FMAC])
+    assert r.returncode == 1 and "hazard: 0 wait state(s)" in r.stdout
+    r = _run(tmp_path, ["v_mul_f32_e32 v3, v1, v2", "v_cvt_f32_i32_e32 v7, v8", FMAC])
+    assert r.returncode == 1 and "hazard: 1 wait state(s)" in r.stdout
+    r = _run(tmp_path, ["v_pk_mul_lo_u16 v[2:3], v[4:5], v[6:7]", FMAC])  # a register pair that holds the operand
+    assert r.returncode == 1
+
+
+def test_s_nop_counts_its_wait_states(tmp_path):
+    assert _run(tmp_path, ["v_mul_f32_e32 v3, v1, v2", "s_nop 0", FMAC]).returncode == 1
+    assert _run(tmp_path, ["v_mul_f32_e32 v3, v1, v2", "s_nop 1", FMAC]).returncode == 0
+
+
+def test_other_registers_and_non_dpp_sources_do_not_matter(tmp_path):
+    # v7 is the plain second factor and v10 the accumulator: neither goes through the DPP path
+    assert _run(tmp_path, ["v_cvt_f32_i32_e32 v7, v8", FMAC]).returncode == 0
+    assert _run(tmp_path, ["v_mul_f32_e32 v10, v1, v2", FMAC]).returncode == 0
+
+
+def test_vector_write_of_exec_fails(tmp_path):
+    r = _run(tmp_path, ["v_cmpx_lt_u32_e32 v1, v2", "s_nop 2", FMAC])
+    assert r.returncode == 1
+    assert _run(tmp_path, ["v_cmpx_lt_u32_e32 v1, v2", "s_nop 4", FMAC]).returncode == 0
+
+
+def test_missing_instructions_fail(tmp_path):
+    """The build names how many v_fmac_f32_dpp it expects: a compile that silently dropped them does not pass."""
+    assert _run(tmp_path, ["v_mul_f32_e32 v3, v1, v2"], "1000").returncode == 1

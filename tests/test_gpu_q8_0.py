@@ -187,6 +187,41 @@ def test_gemv_tiny_and_huge_scales(hip, oracle):
         assert np.array_equal(bits(out), bits(ref)), s
 
 
+@pytest.mark.parametrize("n_tokens", [2, 3, 4, 5, 7, 8])
+def test_gemv_batched_tiny_and_huge_scales(hip, oracle, n_tokens):
+    """Several tokens a launch share their scale products between lanes: weight scales that are zero, f16
+    subnormals, the largest f16, inf and NaN against token scales from f32 subnormals to large, a different one per
+    token and block, must give the single-token kernel's bits for every token."""
+    n_out, n_in = 8 * 5 + 3, 768
+    rng = np.random.default_rng(4100 + n_tokens)
+    w = hip.synth.q8_0_weight(410, n_out, n_in).reshape(n_out, -1, 34).copy()
+    special = np.array([0x0000, 0x8000, 0x0001, 0x03FF, 0x0400, 0x8001, 0x7BFF, 0xFBFF, 0x7C00, 0x7E00], np.uint16)
+    pick = special[rng.integers(0, special.size, (n_out, n_in // 32))]
+    keep = rng.random((n_out, n_in // 32)) < 0.6
+    own = w[:, :, :2].copy().view(np.uint16)[:, :, 0]
+    w[:, :, :2] = np.where(keep, own, pick).astype(np.uint16)[:, :, None].view(np.uint8)
+    w = np.ascontiguousarray(w).reshape(-1)
+    q8 = rng.integers(-127, 128, (n_tokens, n_in), dtype=np.int8)
+    sc = rng.choice(np.array([0.0, 1e-41, 1e-30, 6e-8, 1.0, 3e4, 2e38], np.float32), (n_tokens, n_in // 32)).astype(np.float32)
+    H = hip.hip
+    kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
+    d_q8, d_sc = H.DeviceBuffer.from_array(q8), H.DeviceBuffer.from_array(sc)
+    d_y = H.DeviceBuffer(n_tokens * n_out * 4)
+    H.check(H.lib.rmi_hip_gemv_q8_0_dev(kernel.w.handle, d_q8.ptr, d_sc.ptr, d_y.ptr, n_tokens, n_out, 0, n_out, None))
+    H.check(H.lib.rmi_hip_synchronize())
+    out = d_y.to_array(np.float32, (n_tokens, n_out))
+    with np.errstate(all="ignore"):
+        ref = np.stack([oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, A) for t in range(n_tokens)])
+    nan_o, nan_r = np.isnan(out), np.isnan(ref)
+    assert np.array_equal(nan_o, nan_r) and nan_r.any() and not nan_r.all()
+    assert np.array_equal(bits(out)[~nan_o], bits(ref)[~nan_r])
+    # products below the normal range were exercised
+    wd = np.where(keep, own, pick).astype(np.uint16).view(np.float16).astype(np.float32)
+    with np.errstate(all="ignore"):
+        prod = wd[:, None, :] * sc[None, :, :]
+    assert np.count_nonzero((prod != 0) & (np.abs(prod) < 1.17549435e-38)) > 100
+
+
 @pytest.mark.parametrize("nth", [1, 2, 3, 4, 8, 16])
 def test_thread_partition_bit_exact(hip, oracle, nth):
     """tests/q8_0_parallel_matmul.rs:82-145: every (ith, nth) slice of the full output."""
