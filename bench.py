@@ -309,12 +309,15 @@ def run_projection_set(args, pkg, ev):
         "batch": batch,
         "launches_per_step": launches,
         "algorithmic_bytes_per_step": alg_bytes,
+        # the reference's own count (src/bin/micro_bench.rs:170-171, 203-204): weights + 5 bytes per input element
+        "reference_convention_bytes_per_step": sum(r["n_out"] * (r["n_in"] // 32 * 34) + 5 * r["n_in"] * batch for r in problems),
         "flops_per_step": flops,
         "device": dev_name.strip(),
         "compute_units": cus,
     })
     result.update({
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "gbs_by_reference_convention": round(result["config"]["reference_convention_bytes_per_step"] / wall / 1e9, 1),
         "token_steps_per_s": round(1.0 / wall, 1),
         "gflops": round(flops / wall / 1e9, 1),
         "roofline": {
@@ -364,12 +367,22 @@ def run_projection_set(args, pkg, ev):
 
 
 def run_small_batches(args, pkg, ev):
-    """The projection set at decode batch 8 and 16 in one grouped launch each: the GEMV in the x86-64 kernel's
-    order at 8 tokens, the small-batch kernel on the matrix cores (aarch64 kernel's order) at 8 and 16."""
+    """The projection set at decode batch 2, 4, 8 and 16 in one grouped launch each: the GEMV in the x86-64 kernel's
+    order at 2, 4 and 8 tokens (what Kernel::forward_batched runs by default), the small-batch kernel on the matrix
+    cores (aarch64 kernel's order) at 8 and 16.  After each timed region every output of the launch is compared
+    with the CPU checker's result in the same order, bit for bit."""
     H, synth = pkg.hip, pkg.synth
-    problems = build_projection_set(pkg, 16, keep_host=False)  # batches of 8 use the first 8 tokens
+    check = not args.no_cpu_baseline
+    problems = build_projection_set(pkg, 16, keep_host=check)  # smaller batches use the first tokens
+    oracle = None
+    if check:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import rmi_oracle as oracle
+        from concurrent.futures import ThreadPoolExecutor
+        cores, _ = cpu_threads()
     out = {}
-    for label, order, batch in (("batch8_x86_order", "avx2", 8), ("batch8_aarch64_order", "neon", 8),
+    for label, order, batch in (("batch2_x86_order", "avx2", 2), ("batch4_x86_order", "avx2", 4),
+                                ("batch8_x86_order", "avx2", 8), ("batch8_aarch64_order", "neon", 8),
                                 ("batch16_aarch64_order", "neon", 16)):
         group = make_group(H, problems, batch, order)
 
@@ -392,8 +405,98 @@ def run_small_batches(args, pkg, ev):
                                    else "gemv_q8_0_mfma_kernel<%d,true>" % ((batch + 15) // 16),
                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_us": round(dev_ms * 1e3, 3)}}
+        if oracle is not None and (order == "neon" or oracle.have_avx2()):
+            variant = oracle.NEON if order == "neon" else oracle.AVX2
+
+            H.check(H.lib.rmi_hip_synchronize())
+            gpu_outs = [r["d_y"].to_array(np.float32, (batch, r["n_out"])) for r in problems]
+
+            def differing(pair, batch=batch, variant=variant):
+                r, gpu = pair
+                worst = 0
+                for t in range(batch):
+                    ref = oracle.matmul_q8_0_quantized(r["w"], r["q8"][t], r["sc"][t], r["n_in"], r["n_out"], variant)
+                    worst = max(worst, int(np.count_nonzero(gpu[t].view(np.uint32) != ref.view(np.uint32))))
+                return worst
+
+            with ThreadPoolExecutor(cores) as ex:  # the checker's C loops release the interpreter lock
+                out[label]["gpu_outputs_differing_from_cpu"] = max(ex.map(differing, zip(problems, gpu_outs)))
         H.lib.rmi_hip_gemv_group_destroy(group)
     return out
+
+
+def run_single_gemv(args, pkg, ev):
+    """One Q8_0 GEMV per launch, W[3072 x 1024], decode batch 1: the reference's own micro-benchmark case
+    (src/bin/micro_bench.rs:154-175).  A 3.3 MB weight would stay in the 256 MB last-level cache if launched again
+    and again, so the launches walk a pool of 160 separate copies in HBM (535 MB) in turn and every launch streams
+    its weight from HBM; one step = one launch, its time = the span between two HIP events on the launch stream
+    divided by the launches between them."""
+    H, synth, K = pkg.hip, pkg.synth, pkg.kernel
+    dev_name, cus, hbm = H.device_info()
+    n_out, n_in, copies = 3072, 1024, 160
+    w = synth.q8_0_weight(synth.seed_for(0, 0), n_out, n_in)
+    x = synth.activations(synth.seed_for(0, 0x8000), 1, n_in)
+    kernels = [K.Q8Kernel(w, n_in, n_out) for _ in range(copies)]
+    d_x = H.DeviceBuffer.from_array(x)
+    d_q8, d_sc, d_y = H.DeviceBuffer(n_in), H.DeviceBuffer(n_in // 32 * 4), H.DeviceBuffer(n_out * 4)
+    H.check(H.lib.rmi_hip_quantize_q8_0_dev(d_x.ptr, d_q8.ptr, d_sc.ptr, 1, n_in, H.ROUND_TIES_EVEN, None))
+    H.check(H.lib.rmi_hip_synchronize())
+    state = {"i": 0}
+
+    def step():
+        k = kernels[state["i"] % copies]
+        state["i"] += 1
+        H.check(H.lib.rmi_hip_gemv_q8_0_dev(k.w.handle, d_q8.ptr, d_sc.ptr, d_y.ptr, 1, n_out, 0, n_out, None))
+
+    steps, warmup = max(args.steps, 4 * copies), copies
+    wall, dev_ms = time_region(H, ev, step, steps, warmup)
+    alg = synth.q8_0_gemv_bytes(n_out, n_in, 1)
+    ref_bytes = n_out * (n_in // 32 * 34) + 5 * n_in  # the reference's own count, micro_bench.rs:170-171, 203-204
+    achieved = alg / (dev_ms * 1e-3) / 1e9
+    timed = argparse.Namespace(steps=steps, warmup=warmup)
+    result = base_result(timed, "Q8_0 GEMV HBM GB/s, single 3072x1024 matrix per launch, 1 GPU", "GB/s",
+                         round(alg / wall / 1e9, 1), wall, "int8 dot4 -> f32", {
+        "workload": f"single Q8_0 GEMV W[{n_out}x{n_in}], decode batch 1, one launch per step over a pool of {copies} "
+                    f"separate weight copies in HBM ({copies * synth.q8_0_weight_bytes(n_out, n_in) / 1e6:.0f} MB) taken in turn",
+        "launches_per_step": 1, "algorithmic_bytes_per_step": alg, "reference_convention_bytes_per_step": ref_bytes,
+        "device": dev_name.strip(), "compute_units": cus})
+    result["gbs_by_reference_convention"] = round(ref_bytes / wall / 1e9, 1)
+    result["gflops"] = round(2.0 * n_in * n_out / wall / 1e9, 1)
+    result["roofline"] = {"bound": "hbm", "kernel": "gemv_q8_0_deep_kernel<4>", "achieved": round(achieved, 1),
+                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                          "avg_launch_us": round(dev_ms * 1e3, 3), "algorithmic_bytes_per_launch": alg, "traffic": None,
+                          "limit": "0.42 us of HBM time per launch against the 2.4 us a launch costs in a stream of "
+                                   "back-to-back launches: launch-bound; the grouped launch of the headline is the remedy"}
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import rmi_oracle as oracle
+        if oracle.have_avx2():
+            cores, core_info = cpu_threads()
+            pool = oracle.Pool(cores)
+            q8, sc = d_q8.to_array(np.uint8, (1, n_in)), d_sc.to_array(np.float32, (1, n_in // 32))
+            out = np.zeros((1, n_out), np.float32)
+            for _ in range(10):
+                pool.matmul_q8_0(w, q8, sc, out, n_in, n_out, 1)
+            samples = []
+            for _ in range(15):
+                t0 = time.perf_counter()
+                for _ in range(20):
+                    pool.matmul_q8_0(w, q8, sc, out, n_in, n_out, 1)
+                samples.append((time.perf_counter() - t0) / 20)
+            pool.close()
+            med = statistics.median(samples)
+            step()
+            H.check(H.lib.rmi_hip_synchronize())
+            gpu = d_y.to_array(np.float32, (1, n_out))
+            result["cpu_baseline"] = {
+                "value": round(alg / med / 1e9, 2), "unit": "GB/s", "cores": cores, **core_info, "kind": "port",
+                "sample": "10 warm-ups, 15 samples of 20 calls, median (micro_bench.rs:32-33, 94-152); the one weight "
+                          "stays in the CPU's caches between calls, as in the reference's own run",
+                "us_per_call": round(med * 1e6, 2), "gbs_by_reference_convention": round(ref_bytes / med / 1e9, 2),
+                "gpu_outputs_differing_from_cpu": int(np.count_nonzero(gpu.view(np.uint32) != out.view(np.uint32)))}
+    for k in kernels:
+        k.w.free()
+    return result
 
 
 def compact(r):
@@ -889,7 +992,7 @@ def main():
                     help="timed steps (default 50; 500 for the q4_0 / q4k / q6k GEMV workloads, whose compute-heavy kernels "
                          "read 10-15 %% slower until the clocks have settled, a few hundred launches in)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps before (default 10; 100 for q4_0 / q4k / q6k)")
-    ap.add_argument("--workload", choices=["projection_set", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "qlinear", "attention", "decode"], default="projection_set",
+    ap.add_argument("--workload", choices=["projection_set", "single_gemv", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "qlinear", "attention", "decode"], default="projection_set",
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
                          "q4_0: Q4_0 x Q8_0 decode GEMV; q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); qlinear: QuantizedLinear::forward (Q4_K dequantise-and-dot, f32 activation); decode: end-to-end device-resident greedy decode "
                          "(one step = one 639-token-step generation)")
@@ -927,7 +1030,7 @@ def main():
     pkg = importlib.import_module("rust-model-inference_amd")
     pkg.init(int(os.environ.get("LOCAL_RANK", "0")))
     ev = HipEvents()
-    run = {"projection_set": run_projection_set, "gemm": run_gemm, "q4_0": run_q4_0, "q4k": run_q4k, "q6k": run_q6k, "q4k_gemm": run_q4k_gemm, "qlinear": run_qlinear,
+    run = {"projection_set": run_projection_set, "single_gemv": run_single_gemv, "gemm": run_gemm, "q4_0": run_q4_0, "q4k": run_q4k, "q6k": run_q6k, "q4k_gemm": run_q4k_gemm, "qlinear": run_qlinear,
            "attention": run_attention, "decode": run_decode}[args.workload]
     result = run(args, pkg, ev)
     if args.workload == "projection_set" and not args.no_decode and args.batch == 1:
@@ -938,13 +1041,16 @@ def main():
         d = run_decode(sub, pkg, ev)
         result["decode"] = {"value": d["value"], "unit": d["unit"], "ms_per_token_step": d["ms_per_token_step"],
                             "workload": d["config"]["workload"], "generations_timed": sub.steps,
-                            "cpu_baseline": d.get("cpu_baseline")}
+                            "roofline": d["roofline"], "cpu_baseline": d.get("cpu_baseline")}
     if args.workload == "projection_set" and not args.no_configs and args.batch == 1 and args.mode == "grouped" \
             and args.order == "avx2":
         # the other benchmark configurations, each measured like the headline (own warm-up, own timed steps between
         # synchronisations, HIP events on the launch stream), after and outside the headline's timed region
         configs = {}
         t_cfg = time.time()
+        sub = argparse.Namespace(**vars(args))
+        sub.copy_calibration_mb = 0
+        configs["single_gemv_3072x1024"] = compact(run_single_gemv(sub, pkg, ev))
         configs.update(run_small_batches(args, pkg, ev))
         for m in (64, 512, 2048):
             sub = argparse.Namespace(**vars(args))

@@ -127,6 +127,11 @@ int rmi_hip_block_dots_q8_0(const rmi_hip_weight *w, const uint8_t *input_q8, in
 /* ops::matmul_q8_0 (q8_0/parallel.rs:317-341): f32 activations used as they
  * are, no activation quantisation. */
 int rmi_hip_matmul_q8_0_f32(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in, uint32_t n_out);
+/* matmul_q8_0_fallback_range (src/ops/kernel/q8_0/scalar.rs:3-29), the same product on hosts without AVX2: per
+ * row one f32 chain, local += float(q)*x over the 32 elements of a block in order, sum += d*local block after
+ * block.  output has row_end - row_start entries.  Differs from the AVX2 order in the last bits only. */
+int rmi_hip_matmul_q8_0_fallback_range(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                       uint32_t row_start, uint32_t row_end);
 
 /* ---- Q4_K, host slices ---------------------------------------------------*/
 
@@ -254,6 +259,12 @@ int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
  * integers, the f32 sums within rounding of the CPU kernels. */
 int rmi_hip_gemm_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
                               const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride, void *stream);
+/* The integers of rmi_hip_gemm_q4_k_q8k_dev as they leave the matrix cores, per token, row and super-block:
+ * ints[((t * n_out + n) * (n_in / 256) + sb) * 2 + 0] = sum_j scale_j * dot_j (the sum of the eight lane integers
+ * of src/ops/quant/mod.rs:701-799), + 1 = sum_j min_j * bsum_j.  Same kernel, same tile width as the product takes
+ * for this problem; writes no y (debug / parity entry point). */
+int rmi_hip_gemm_block_ints_q4_k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                                     const int16_t *q8k_bsums, int32_t *ints, uint32_t n_tokens, void *stream);
 /* Q4_0 weights, Q8_0 activations on the device (src/ops/kernel/q4_0/scalar.rs:13-52). */
 int rmi_hip_gemv_q4_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                           uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, void *stream);

@@ -573,6 +573,19 @@ void rmi_ref_q4k_q8k_block_ints(const uint8_t *w, size_t nb, const int8_t *qs,
     }
 }
 
+/* the same integers for every row of a weight against one token: ints[n_out][nb][2] = {isum, msum} */
+void rmi_ref_q4k_q8k_block_ints_matrix(const uint8_t *w, size_t n_out, size_t nb, const int8_t *qs,
+                                       const int16_t *bsums, int32_t *ints) {
+    for (size_t r = 0; r < n_out; r++) {
+        int32_t isum[nb], msum[nb];
+        rmi_ref_q4k_q8k_block_ints(w + r * nb * Q4K_BLOCK, nb, qs, bsums, isum, msum);
+        for (size_t i = 0; i < nb; i++) {
+            ints[(r * nb + i) * 2] = isum[i];
+            ints[(r * nb + i) * 2 + 1] = msum[i];
+        }
+    }
+}
+
 void rmi_ref_dequantize_row_q4_k(const uint8_t *blocks, float *output, size_t n) {
     size_t nb = n / QK_K;
     for (size_t bi = 0; bi < nb; bi++) {

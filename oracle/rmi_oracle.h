@@ -106,6 +106,8 @@ float rmi_ref_vec_dot_q4k_q8k(const uint8_t *q4k_row, size_t n_blocks,
 void rmi_ref_q4k_q8k_block_ints(const uint8_t *q4k_row, size_t n_blocks,
                                 const int8_t *qs, const int16_t *bsums,
                                 int32_t *isum, int32_t *msum);
+void rmi_ref_q4k_q8k_block_ints_matrix(const uint8_t *q4k_weight, size_t n_out, size_t n_blocks, const int8_t *qs,
+                                       const int16_t *bsums, int32_t *ints);
 
 /* src/ops/quant/mod.rs:456-490, 492-508 */
 void rmi_ref_dequantize_row_q4_k(const uint8_t *blocks, float *output,

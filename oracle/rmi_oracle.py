@@ -52,6 +52,7 @@ def _load():
         "rmi_ref_unpack_scales_kmask": (None, [_u8p, _u8p]),
         "rmi_ref_vec_dot_q4k_q8k": (C.c_float, [_u8p, _sz, _f32p, _i8p, _i16p, C.c_int]),
         "rmi_ref_q4k_q8k_block_ints": (None, [_u8p, _sz, _i8p, _i16p, _i32p, _i32p]),
+        "rmi_ref_q4k_q8k_block_ints_matrix": (None, [_u8p, _sz, _sz, _i8p, _i16p, _i32p]),
         "rmi_ref_dequantize_row_q4_k": (None, [_u8p, _f32p, _sz]),
         "rmi_ref_q4k_forward_prepared": (None, [_u8p, _f32p, _i8p, _i16p, _f32p, _sz, _sz, _sz, _sz, C.c_int]),
         "rmi_ref_q4k_forward_prequantized": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz, _sz]),
@@ -307,6 +308,17 @@ def q4k_q8k_block_ints(row, qs, bsums):
     msum = np.zeros(nb, np.int32)
     lib.rmi_ref_q4k_q8k_block_ints(_p(row, _u8p), nb, _p(qs, _i8p), _p(bsums, _i16p), _p(isum, _i32p), _p(msum, _i32p))
     return isum, msum
+
+
+def q4k_q8k_block_ints_matrix(w, n_out, qs, bsums):
+    """`q4k_q8k_block_ints` for every row of a weight against one token: int32[n_out][n_in/256][2] = {isum, msum}."""
+    w = _u8(w)
+    qs = np.ascontiguousarray(qs, np.int8)
+    bsums = np.ascontiguousarray(bsums, np.int16)
+    nb = qs.size // 256
+    ints = np.zeros((n_out, nb, 2), np.int32)
+    lib.rmi_ref_q4k_q8k_block_ints_matrix(_p(w, _u8p), n_out, nb, _p(qs, _i8p), _p(bsums, _i16p), _p(ints, _i32p))
+    return ints
 
 
 def dequantize_row_q4_k(blocks, n):

@@ -50,6 +50,8 @@ int rmi_hip_q8_0_forward_noalloc_dev(const rmi_hip_weight *w, const float *x, fl
                         "%u tokens x %u elements = %llu exceed the fixed scratch of %zu elements; use "
                         "rmi_hip_q8_0_forward_batched or split the batch",
                         n_tokens, w->n_in, (unsigned long long)n_x, kNoAllocMaxElems);
+    // checked here, before the quantizer is enqueued: a refused call leaves the shared array as it was
+    if (!rmi_gemv_q8_0_tokens_fits(w)) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u is too long for the GEMV staging", w->n_in);
     int device = -1;
     RMI_HIP_CHECK(hipGetDevice(&device));
     if (device != rmi_device())

@@ -227,6 +227,16 @@ int rmi_hip_gemm_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const
     return rmi_launch_gemm_q4_k(w, q8k_d, q8k_qs, q8k_bsums, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
 }
 
+int rmi_hip_gemm_block_ints_q4_k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
+                                     const int16_t *q8k_bsums, int32_t *ints, uint32_t n_tokens, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q4_K) return rmi_fail(RMI_HIP_E_INVALID, "not a Q4_K weight handle");
+    if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
+    if (!q8k_d || !q8k_qs || !q8k_bsums || !ints) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (rmi_misaligned(q8k_qs, q8k_d, q8k_bsums, ints)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
+    return rmi_launch_gemm_q4_k_block_ints(w, q8k_d, q8k_qs, q8k_bsums, ints, n_tokens, static_cast<hipStream_t>(stream));
+}
+
 static rmi_hip_gemv_group *group_create_kquant(int dtype, uint32_t n_problems, const rmi_hip_weight *const *weights,
                                                const float *const *q8k_d, const int8_t *const *q8k_qs,
                                                const int16_t *const *q8k_bsums, float *const *y, uint32_t n_tokens) {

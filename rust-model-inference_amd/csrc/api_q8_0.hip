@@ -43,6 +43,10 @@ uint32_t gemv_chunk(const rmi_hip_weight *w) {
 
 }  // namespace
 
+// whether rmi_gemv_q8_0_tokens can stage a row of this weight at all (callers that must not enqueue anything
+// before every check has passed ask first)
+bool rmi_gemv_q8_0_tokens_fits(const rmi_hip_weight *w) { return gemv_chunk(w) != 0; }
+
 // device pointers in, rows [row_start,row_end) of n_tokens tokens
 int rmi_gemv_q8_0_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
                          uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s) {
@@ -296,6 +300,29 @@ int rmi_hip_matmul_q8_0_f32(const rmi_hip_weight *w, const float *input, float *
     rc = rmi_launch_matmul_q8_0_f32(w, d_x, d_y, c->stream);
     if (rc != RMI_HIP_OK) return rc;
     return fetch(c, output, d_y, size_t(n_out) * 4, 1);
+}
+
+int rmi_hip_matmul_q8_0_fallback_range(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
+                                       uint32_t row_start, uint32_t row_end) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (n_in != w->n_in) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u, the weight has %u", n_in, w->n_in);
+    if (row_start > row_end || row_end > w->n_out)
+        return rmi_fail(RMI_HIP_E_INVALID, "rows [%u,%u) outside 0..%u", row_start, row_end, w->n_out);
+    if (row_end == row_start) return RMI_HIP_OK;
+    if (!input || !output) return rmi_fail(RMI_HIP_E_INVALID, "null slice");
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    const size_t n_rows = row_end - row_start;
+    float *pin = static_cast<float *>(rmi_pin_buf(c, 0, size_t(n_in) * 4));
+    float *d_x = static_cast<float *>(rmi_dev_buf(c, 0, size_t(n_in) * 4));
+    float *d_y = static_cast<float *>(rmi_dev_buf(c, 1, n_rows * 4));
+    if (!pin || !d_x || !d_y) return RMI_HIP_E_RUNTIME;
+    memcpy(pin, input, size_t(n_in) * 4);
+    RMI_HIP_CHECK(hipMemcpyAsync(d_x, pin, size_t(n_in) * 4, hipMemcpyHostToDevice, c->stream));
+    int rc = rmi_launch_matmul_q8_0_f32_scalar(w, d_x, d_y, row_start, row_end, c->stream);
+    if (rc != RMI_HIP_OK) return rc;
+    return fetch(c, output, d_y, n_rows * 4, 1);
 }
 
 // ------------------------------------------------------ device-resident

@@ -106,7 +106,10 @@ __device__ __forceinline__ uint32_t bytes_to_f16_pair(uint32_t w) {
 }
 
 // WAVES_PER_SIMD bounds the registers of a thread: that many waves are to share a SIMD.
-template <int TTW, int WAVES_PER_SIMD>
+// DUMP (parity only): instead of folding them, the kernel writes the integers of every super-block as they leave
+// the matrix cores, sumi = 8 * D_hi + D_lo and prod (the min term's f16 MFMA result, an integer below 2^24), to
+// reinterpret_cast<int32_t *>(y)[((t * n_out + n) * n_sb + sb) * 2 + {0, 1}].
+template <int TTW, int WAVES_PER_SIMD, bool DUMP>
 __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const uint8_t *__restrict__ w, const float *__restrict__ q8d,
                                                                          const int8_t *__restrict__ q8qs,
                                                                          const int16_t *__restrict__ q8bs, float *__restrict__ y,
@@ -355,6 +358,18 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
         for (int tt = 0; tt < TTW; tt++) {
             const v32f sc = __builtin_amdgcn_mfma_f32_32x32x1f32(xd[tt], wd, zero32, 0, 0, 0);
             const v16f pm = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, xbv[tt]), __builtin_bit_cast(v8h, mins), zero16f, 0, 0, 0);
+            if constexpr (DUMP) {
+                const uint32_t n = n0 + n_off + c;
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const uint32_t t = t0 + tt * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
+                    if (n < n_out && t < n_tokens) {
+                        int32_t *dst = reinterpret_cast<int32_t *>(y) + ((size_t(t) * n_out + n) * n_sb + sb) * 2;
+                        dst[0] = d_hi[tt][i] * 8 + d_lo[tt][i];
+                        dst[1] = int32_t(pm[i]);
+                    }
+                }
+            }
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 acc[tt][i] = __builtin_fmaf(sc[i], float(d_hi[tt][i] * 8 + d_lo[tt][i]), acc[tt][i]);
@@ -378,7 +393,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     if (sb < n_sb) stage(sb, std::integral_constant<int, 0>{});
     // ---- results: lane (c, h) holds row n = c of 16 tokens
     const uint32_t n = n0 + n_off + c;
-    if (n < n_out) {
+    if (!DUMP && n < n_out) {
 #pragma unroll
         for (int tt = 0; tt < TTW; tt++)
 #pragma unroll
@@ -389,28 +404,48 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     }
 }
 
-template <int TTW, int WAVES_PER_SIMD>
+template <int TTW, int WAVES_PER_SIMD, bool DUMP = false>
 void launch(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bs, float *y, uint32_t n_tokens,
             uint32_t y_stride, hipStream_t s) {
     const uint32_t grid_n = (w->n_out + 127) / 128, grid_t = (n_tokens + 32 * TTW - 1) / (32 * TTW);
     const uint32_t xcd_split = rmi_gemm_xcd_split(grid_n, grid_t, double(w->n_out) * w->n_units * 144.0, double(n_tokens) * w->n_units * 292.0);
-    hipLaunchKernelGGL((gemm_q4_k_kernel<TTW, WAVES_PER_SIMD>), dim3(grid_n * grid_t), dim3(256), 0, s, w->data, d, qs, bs, y,
+    hipLaunchKernelGGL((gemm_q4_k_kernel<TTW, WAVES_PER_SIMD, DUMP>), dim3(grid_n * grid_t), dim3(256), 0, s, w->data, d, qs, bs, y,
                        w->n_out, w->n_units, w->n_tiles, n_tokens, y_stride, grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
 }
 
 }  // namespace
 
+// token tile width (in units of 32) the launcher takes for this problem; RMI_Q4K_GEMM_TTW = 1 or 2 forces one
+static int gemm_q4_k_ttw(const rmi_hip_weight *w, uint32_t n_tokens) {
+    const uint64_t groups64 = uint64_t((w->n_out + 127) / 128) * ((n_tokens + 63) / 64);
+    const char *e = getenv("RMI_Q4K_GEMM_TTW");
+    const int force = e ? atoi(e) : 0;
+    return force == 2 || (force != 1 && groups64 >= 2 * uint64_t(rmi_device_cus())) ? 2 : 1;
+}
+
+// The same kernel, same tile width as the product would take, writing its per-super-block integers instead of y:
+// ints[n_tokens][n_out][n_sb][2] = {sumi, prod} (parity entry point).
+int rmi_launch_gemm_q4_k_block_ints(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums,
+                                    int32_t *ints, uint32_t n_tokens, hipStream_t s) {
+    if (n_tokens == 0 || w->n_out == 0 || w->n_units == 0) return RMI_HIP_OK;
+    if (uint64_t((w->n_out + 127) / 128) * ((n_tokens + 31) / 32) > 0x7fffffffull)
+        return rmi_fail(RMI_HIP_E_INVALID, "GEMM too large for one launch");
+    if (gemm_q4_k_ttw(w, n_tokens) == 2)
+        launch<2, 2, true>(w, d, qs, bsums, reinterpret_cast<float *>(ints), n_tokens, w->n_out, s);
+    else
+        launch<1, 2, true>(w, d, qs, bsums, reinterpret_cast<float *>(ints), n_tokens, w->n_out, s);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
 int rmi_launch_gemm_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
                          uint32_t n_tokens, uint32_t y_stride, hipStream_t s) {
     if (n_tokens == 0 || w->n_out == 0 || w->n_units == 0) return RMI_HIP_OK;
-    const uint64_t groups64 = uint64_t((w->n_out + 127) / 128) * ((n_tokens + 63) / 64);
     const uint64_t groups32 = uint64_t((w->n_out + 127) / 128) * ((n_tokens + 31) / 32);
     if (groups32 > 0x7fffffffull) return rmi_fail(RMI_HIP_E_INVALID, "GEMM too large for one launch");
     // 64-token tiles halve the vector work per output but want two workgroups on every compute unit;
     // RMI_Q4K_GEMM_TTW = 1 or 2 forces a width (the parity tests run both)
-    const char *e = getenv("RMI_Q4K_GEMM_TTW");
-    const int force = e ? atoi(e) : 0;
-    if (force == 2 || (force != 1 && groups64 >= 2 * uint64_t(rmi_device_cus())))
+    if (gemm_q4_k_ttw(w, n_tokens) == 2)
         launch<2, 2>(w, d, qs, bsums, y, n_tokens, y_stride, s);
     else
         launch<1, 2>(w, d, qs, bsums, y, n_tokens, y_stride, s);

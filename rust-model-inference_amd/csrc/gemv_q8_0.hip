@@ -736,6 +736,41 @@ __global__ __launch_bounds__(64) void matmul_q8_0_f32_kernel(const uint8_t *__re
     if (i == 0 && row < n_out) y[row] = s;
 }
 
+// ---- matmul_q8_0_fallback_range (scalar.rs:3-29): the f32-activation product on hosts without AVX2.  Per row
+// one chain: local = 0; local += float(q[k]) * x[k] for the 32 elements of a block in order (product and sum
+// rounded separately); sum += d * local block after block.  The eight lanes of a row each make the four products
+// of their slice; the adds are one dependent chain, so every lane of the row runs it on values read from the
+// other lanes (only lane 0's copy is stored). ----
+__global__ __launch_bounds__(64) void matmul_q8_0_f32_scalar_kernel(const uint8_t *__restrict__ w,
+                                                                     const float *__restrict__ x, float *__restrict__ y,
+                                                                     uint32_t row_start, uint32_t row_end, uint32_t nb,
+                                                                     uint32_t n_oct, uint32_t tile0) {
+    const uint32_t lane = threadIdx.x, r = lane >> 3, i = lane & 7;
+    const uint32_t tile_idx = tile0 + blockIdx.x;
+    const uint8_t *tile = w + size_t(tile_idx) * n_oct * kOctetBytes;
+    const uint8_t *quants = tile + size_t(n_oct) * 128;
+    float sum = 0.0f;
+    for (uint32_t b = 0; b < nb; b++) {
+        const float d = h2f(reinterpret_cast<const uint16_t *>(tile + size_t(b >> 3) * 128 + r * 16)[b & 7]);
+        const uint32_t qw = *reinterpret_cast<const uint32_t *>(quants + size_t(b >> 2) * 1024 + r * 128 + i * 16 + (b & 3) * 4);
+        const float4 xv = *reinterpret_cast<const float4 *>(x + size_t(b) * 32 + i * 4);
+        float p[4];
+        p[0] = float(int(int8_t(qw & 0xff))) * xv.x;
+        p[1] = float(int(int8_t((qw >> 8) & 0xff))) * xv.y;
+        p[2] = float(int(int8_t((qw >> 16) & 0xff))) * xv.z;
+        p[3] = float(int(int8_t(qw >> 24))) * xv.w;
+        float local = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) local = local + __shfl(p[j], k, 8);
+        }
+        sum = sum + d * local;
+    }
+    const uint32_t row = tile_idx * kTileRows + r;
+    if (i == 0 && row >= row_start && row < row_end) y[row - row_start] = sum;
+}
+
 // plain streaming copy: the known-size kernel that HBM traffic counters are scaled against
 __global__ __launch_bounds__(256) void copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
     for (size_t i = blockIdx.x * size_t(blockDim.x) + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x)
@@ -885,6 +920,16 @@ int rmi_launch_quantize_q8_0(const float *x, int8_t *q8, float *scales, uint32_t
     if (n_blocks * 8 > 0xffffffffull) return rmi_fail(RMI_HIP_E_INVALID, "activation too large for one launch");
     const uint32_t grid = uint32_t((n_blocks * 8 + 255) / 256);
     hipLaunchKernelGGL(quantize_q8_0_kernel, dim3(grid), dim3(256), 0, s, x, q8, scales, uint32_t(n_blocks), rounding);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int rmi_launch_matmul_q8_0_f32_scalar(const rmi_hip_weight *w, const float *x, float *y, uint32_t row_start,
+                                      uint32_t row_end, hipStream_t s) {
+    if (row_end <= row_start) return RMI_HIP_OK;
+    const uint32_t tile0 = row_start / kTileRows, n_tiles = (row_end + kTileRows - 1) / kTileRows - tile0;
+    hipLaunchKernelGGL(matmul_q8_0_f32_scalar_kernel, dim3(n_tiles), dim3(64), 0, s, w->data, x, y, row_start, row_end,
+                       w->n_in / 32, w->n_units, tile0);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }

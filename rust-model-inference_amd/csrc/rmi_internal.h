@@ -178,6 +178,7 @@ struct RmiGemvProblem {
 int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
 // rows [row_start,row_end) of n_tokens tokens of a Q8_0 or Q4_0 weight, as many GEMV launches (x86-64 order) as
 // the LDS staging of the tokens asks for; device pointers, nothing allocated
+bool rmi_gemv_q8_0_tokens_fits(const rmi_hip_weight *w);
 int rmi_gemv_q8_0_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
                          uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s);
 // the same problem record with w = a Q4_0 tile stream (Q8_0 activation)
@@ -224,6 +225,8 @@ int rmi_launch_block_dots_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, int3
 int rmi_launch_quantize_q8_0(const float *x, int8_t *q8, float *scales, uint32_t n_tokens, uint32_t n_in,
                              int rounding, hipStream_t s);
 int rmi_launch_matmul_q8_0_f32(const rmi_hip_weight *w, const float *x, float *y, hipStream_t s);
+int rmi_launch_matmul_q8_0_f32_scalar(const rmi_hip_weight *w, const float *x, float *y, uint32_t row_start,
+                                      uint32_t row_end, hipStream_t s);
 int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                          uint32_t n_tokens, uint32_t y_stride, hipStream_t s);
 
@@ -251,6 +254,8 @@ int rmi_launch_gemv_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *
                          uint32_t n_tokens, uint32_t y_stride, uint32_t row_start, uint32_t row_end, hipStream_t s);
 int rmi_launch_gemm_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums, float *y,
                          uint32_t n_tokens, uint32_t y_stride, hipStream_t s);
+int rmi_launch_gemm_q4_k_block_ints(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bsums,
+                                    int32_t *ints, uint32_t n_tokens, hipStream_t s);
 int rmi_launch_block_ints_q4_k(const rmi_hip_weight *w, const int8_t *qs, const int16_t *bsums, int32_t *isum,
                                int32_t *msum, hipStream_t s);
 // mode 0: x = q8 * scale rebuilt per element (Q4_KKernel::forward_prequantized)

@@ -76,6 +76,7 @@ SIGNATURES = {
     "rmi_hip_quantize_q8_0": (C.c_int, [_f32p, _u32, _u8p, _f32p, C.c_int]),
     "rmi_hip_block_dots_q8_0": (C.c_int, [_vp, _u8p, _i32p]),
     "rmi_hip_matmul_q8_0_f32": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32]),
+    "rmi_hip_matmul_q8_0_fallback_range": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32]),
     "rmi_hip_q4_k_forward_prepared": (C.c_int, [_vp, _f32p, _i8p, _i16p, _f32p, _u32, _u32, _u32, _u32]),
     "rmi_hip_q4_k_forward_batched": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32]),
     "rmi_hip_q4_k_forward_batched_mfma": (C.c_int, [_vp, _f32p, _f32p, _u32, _u32, _u32]),
@@ -103,6 +104,7 @@ SIGNATURES = {
     "rmi_hip_gemm_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemv_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_gemm_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp]),
+    "rmi_hip_gemm_block_ints_q4_k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp]),
     "rmi_hip_gemv_q4_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_gemv_q6_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rmi_hip_quantize_row_q8_k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),

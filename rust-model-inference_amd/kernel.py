@@ -185,6 +185,14 @@ class Q8Kernel(Kernel):
         x = as_f32(input)
         check(lib.rmi_hip_matmul_q8_0_f32(self.w.handle, ptr(x, _f32p), ptr(_out(output, n_out), _f32p), n_in, n_out))
 
+    def matmul_q8_0_fallback_range(self, input, output, n_in, row_start, row_end):
+        """`matmul_q8_0_fallback_range` (src/ops/kernel/q8_0/scalar.rs:3-29): the f32-activation product in the
+        scalar kernel's order, rows [row_start, row_end) into `output[0 .. row_end - row_start)`."""
+        x = as_f32(input)
+        check(lib.rmi_hip_matmul_q8_0_fallback_range(self.w.handle, ptr(x, _f32p),
+                                                     ptr(_out(output, row_end - row_start), _f32p), n_in, row_start,
+                                                     row_end))
+
     def matmul_q8_0_via_q8(self, input, output, n_in, n_out, q8_buf, scale_buf, rounding=hip.ROUND_TIES_EVEN):
         """`matmul_q8_0_via_q8` (src/ops/kernel/q8_0/legacy.rs:27-83): quantize the f32 input into the caller's
         scratch (which keeps the quants and scales afterwards, as in the reference), then the prequantized GEMV."""

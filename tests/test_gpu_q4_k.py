@@ -332,3 +332,70 @@ def test_q4k_errors(hip):
     with pytest.raises(H.RmiHipError):
         kernel.forward_prequantized(np.zeros(512, np.uint8), np.zeros(16, np.float32), np.zeros(2, np.float32), 512, 2,
                                     0, 1)
+
+
+def _gemm_block_ints(hip, kernel, x, n_tokens, n_in, n_out):
+    """Q8_K-quantizes x on the device and returns what the GEMM's matrix-core chains deliver per super-block,
+    int32[n_tokens][n_out][n_in/256][2], plus the quantized activation."""
+    H = hip.hip
+    d_x = H.DeviceBuffer.from_array(H.as_f32(x))
+    d_d, d_q, d_b = H.DeviceBuffer(n_tokens * n_in // 256 * 4), H.DeviceBuffer(n_tokens * n_in), H.DeviceBuffer(n_tokens * n_in // 16 * 2)
+    H.check(H.lib.rmi_hip_quantize_row_q8_k_dev(d_x.ptr, d_d.ptr, d_q.ptr, d_b.ptr, n_tokens, n_in, None))
+    d_i = H.DeviceBuffer.from_array(np.full(n_tokens * n_out * (n_in // 256) * 2, -1, np.int32))
+    H.check(H.lib.rmi_hip_gemm_block_ints_q4_k_dev(kernel.w.handle, d_d.ptr, d_q.ptr, d_b.ptr, d_i.ptr, n_tokens, None))
+    H.check(H.lib.rmi_hip_synchronize())
+    ints = d_i.to_array(np.int32, (n_tokens, n_out, n_in // 256, 2))
+    qs = d_q.to_array(np.int8, (n_tokens, n_in))
+    bs = d_b.to_array(np.int16, (n_tokens, n_in // 16))
+    for b in (d_x, d_d, d_q, d_b, d_i):
+        b.free()
+    return ints, qs, bs
+
+
+@pytest.mark.parametrize("n_tokens,n_out,n_in", [(512, 6144, 2048), (512, 2048, 6144)])
+def test_q4k_gemm_block_ints_bit_exact_full_size(hip, oracle, n_tokens, n_out, n_in):
+    """The per-super-block integers of the prefill GEMM (8 * D_hi + D_lo from the two int8 MFMA chains, the min
+    term from the f16 MFMA) against the checker's scalar integers (quant/mod.rs:210-289), every token, row and
+    super-block of the 1.7B-class FFN shapes at M = 512."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    print(f"q4k gemm block ints: {n_tokens} tokens, {n_out}x{n_in}", flush=True)
+    w = hip.synth.q4_k_weight(300 + n_out, n_out, n_in)
+    x = hip.synth.activations(301 + n_in, n_tokens, n_in)
+    kernel = hip.kernel.Q4_KKernel(w, n_in, n_out)
+    ints, qs, bs = _gemm_block_ints(hip, kernel, x, n_tokens, n_in, n_out)
+
+    def bad(t):
+        return int(np.count_nonzero(ints[t] != oracle.q4k_q8k_block_ints_matrix(w, n_out, qs[t], bs[t])))
+
+    with ThreadPoolExecutor(8) as ex:
+        assert sum(ex.map(bad, range(n_tokens))) == 0
+    assert np.abs(ints[..., 0]).max() > 10_000  # integers of the size a rounding tolerance would hide an error in
+
+
+@pytest.mark.parametrize("ttw", ["1", "2"])
+def test_q4k_gemm_block_ints_both_tile_widths_ragged_and_extreme(hip, oracle, monkeypatch, ttw):
+    """Both token tile widths on ragged row and token tiles; and the largest integers the format allows (all
+    nibbles 15, all scales and mins 63, all quants +-127), where 8 * D_hi + D_lo reaches 256 * 15 * 63 * 127."""
+    monkeypatch.setenv("RMI_Q4K_GEMM_TTW", ttw)
+    n_tokens, n_out, n_in = 70, 300, 768
+    w = hip.synth.q4_k_weight(310, n_out, n_in)
+    x = hip.synth.activations(311, n_tokens, n_in)
+    kernel = hip.kernel.Q4_KKernel(w, n_in, n_out)
+    ints, qs, bs = _gemm_block_ints(hip, kernel, x, n_tokens, n_in, n_out)
+    for t in range(n_tokens):
+        assert np.array_equal(ints[t], oracle.q4k_q8k_block_ints_matrix(w, n_out, qs[t], bs[t])), t
+    # extremes: header = d, dmin, then twelve 0xff bytes (every 6-bit scale and min 63), nibbles all 15
+    n_out, n_in, n_tokens = 40, 512, 33
+    wx = np.full((n_out, n_in // 256, 144), 0xFF, np.uint8)
+    wx[:, :, 0:4] = np.array([0x00, 0x3C, 0x00, 0x3C], np.uint8)  # d = dmin = 1.0
+    # constant rows quantize to -127 everywhere (Q8_K's scale takes the sign of the largest element); every
+    # third token alternates the sign from element to element instead
+    xx = np.ones((n_tokens, n_in), np.float32)
+    xx[::3, 1::2] = -1.0
+    kx = hip.kernel.Q4_KKernel(wx.reshape(-1), n_in, n_out)
+    ints, qs, bs = _gemm_block_ints(hip, kx, xx, n_tokens, n_in, n_out)
+    assert set(np.unique(qs).tolist()) == {-127, 127}
+    for t in range(n_tokens):
+        assert np.array_equal(ints[t], oracle.q4k_q8k_block_ints_matrix(wx.reshape(-1), n_out, qs[t], bs[t])), t
+    assert np.abs(ints[..., 0]).max() == 256 * 15 * 63 * 127

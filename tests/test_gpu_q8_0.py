@@ -594,6 +594,29 @@ def test_legacy_f32_matmul_bit_exact(hip, oracle):
         assert np.array_equal(bits(out), bits(oracle.matmul_q8_0_f32(w, x[0], n_in, n_out, A)))
 
 
+def test_legacy_f32_matmul_scalar_order_bit_exact(hip, oracle):
+    """`matmul_q8_0_fallback_range` (scalar.rs:3-29): one f32 chain per row, products and sums rounded separately;
+    whole matrices, ragged shapes, and row ranges that start and end inside a tile."""
+    for n_out, n_in in [(64, 512), (13, 96), (1024, 1024), (203, 3072)]:
+        w, x = _case(hip, 1350 + n_out, n_out, n_in)
+        kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
+        ref = oracle.matmul_q8_0_f32(w, x[0], n_in, n_out, S)
+        out = np.zeros(n_out, np.float32)
+        kernel.matmul_q8_0_fallback_range(x[0], out, n_in, 0, n_out)
+        assert np.array_equal(bits(out), bits(ref))
+        # not the AVX2 order's bits (the two differ in the last places on data like this)
+        assert not np.array_equal(bits(out), bits(oracle.matmul_q8_0_f32(w, x[0], n_in, n_out, A)))
+        for lo, hi in [(3, n_out - 2), (n_out // 2, n_out // 2), (0, 1)]:
+            part = np.full(max(hi - lo, 1), np.nan, np.float32)
+            kernel.matmul_q8_0_fallback_range(x[0], part, n_in, lo, hi)
+            assert np.array_equal(bits(part[:hi - lo]), bits(ref[lo:hi]))
+    H = hip.hip
+    kernel = hip.kernel.Q8Kernel(*_case(hip, 1360, 16, 64)[:1], 64, 16)
+    out = np.zeros(16, np.float32)
+    with pytest.raises(H.RmiHipError):
+        kernel.matmul_q8_0_fallback_range(np.zeros(64, np.float32), out, 64, 4, 17)
+
+
 def test_legacy_via_q8_and_batch(hip, oracle):
     """`matmul_q8_0_via_q8` (legacy.rs:27-83) quantizes into the caller's scratch and runs the prequantized
     GEMV; `matmul_q8_0_batch` (batch.rs:32-79) runs a list of f32-activation matmuls."""

@@ -228,3 +228,16 @@ def test_dequant_path_against_f64(oracle, rmi):
     part = np.zeros(n_out, np.float32)
     oracle.q4k_forward_prequantized(w, q8, sc, part, n_in, n_out, 1, 4)
     assert np.array_equal(bits(part[3:6]), bits(out[3:6])) and not part[:3].any() and not part[6:].any()
+
+
+def test_block_ints_matrix_is_the_per_row_function_row_by_row(oracle):
+    rng = np.random.default_rng(77)
+    n_out, n_in = 9, 768
+    w = rng.integers(0, 256, n_out * (n_in // 256) * 144, dtype=np.uint8)
+    qs = rng.integers(-127, 128, n_in, dtype=np.int8)
+    bs = qs.reshape(-1, 16).astype(np.int32).sum(axis=1).astype(np.int16)
+    ints = oracle.q4k_q8k_block_ints_matrix(w, n_out, qs, bs)
+    wr = w.reshape(n_out, -1)
+    for r in range(n_out):
+        isum, msum = oracle.q4k_q8k_block_ints(wr[r], qs, bs)
+        assert np.array_equal(ints[r, :, 0], isum) and np.array_equal(ints[r, :, 1], msum)

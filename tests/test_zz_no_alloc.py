@@ -59,34 +59,57 @@ def test_noalloc_rejects_sizes_beyond_the_scratch(hip):
     d_y.free()
 
 
-def test_shutdown_then_init_rebuilds_the_calling_threads_stream(hip, oracle):
-    """After rmi_hip_shutdown and a new rmi_hip_init the same host thread gets a fresh stream and staging instead of
-    running on the emptied ones; threads that come and go reuse each other's contexts.  (Here, in the file that
-    runs last, because shutdown frees every thread's staging.)"""
+def test_noalloc_allocates_nothing_and_builds_no_thread_context(hip):
+    """The property the entry point is named for: across a call made from a host thread that has never called the
+    library (so it owns no stream and no staging), the device's free memory and the number of thread contexts are
+    what they were.  The buffers are made before the first reading; the HIP runtime's own calls are the meter."""
+    import ctypes
     import threading
 
     H = hip.hip
-    n_out, n_in = 264, 512
-    w = hip.synth.q8_0_weight(950, n_out, n_in)
-    x = hip.synth.activations(951, 1, n_in)[0]
-    q8, sc = oracle.quantize_q8_0(x, 1)
-    ref = oracle.matmul_q8_0_quantized(w, q8, sc, n_in, n_out, 1)
+    rt = ctypes.CDLL("libamdhip64.so")
+    rt.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
 
-    def run():
-        out = np.zeros(n_out, np.float32)
-        hip.kernel.Q8Kernel(w, n_in, n_out).forward_prequantized(q8, sc, out, n_in, n_out, 0, 1)
-        return np.array_equal(bits(out), bits(ref))
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert rt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
 
-    assert run()
-    H.lib.rmi_hip_shutdown()
-    assert H.lib.rmi_hip_synchronize() == -3
-    H.init(0)
-    assert run() and run()
-    before = H.lib.rmi_hip_thread_context_count()
-    results = []
-    for _ in range(6):  # six threads one after the other: at most one more context than before
-        t = threading.Thread(target=lambda: results.append(run()))
-        t.start()
-        t.join()
-    assert results == [True] * 6
-    assert H.lib.rmi_hip_thread_context_count() <= before + 1
+    n_out, n_in, n_tokens = 1024, 2048, 8
+    kernel = hip.kernel.Q8Kernel(hip.synth.q8_0_weight(960, n_out, n_in), n_in, n_out)
+    x = hip.synth.activations(961, n_tokens, n_in)
+    d_x = H.DeviceBuffer.from_array(H.as_f32(x))
+    d_y = H.DeviceBuffer.from_array(np.zeros((n_tokens, n_out), np.float32))
+    H.check(H.lib.rmi_hip_synchronize())
+    seen = {}
+
+    def call():
+        seen["ctx_before"] = H.lib.rmi_hip_thread_context_count()
+        seen["free_before"] = free_bytes()
+        seen["rc"] = H.lib.rmi_hip_q8_0_forward_noalloc_dev(kernel.w.handle, d_x.ptr, d_y.ptr, n_tokens, n_out,
+                                                            H.ROUND_TIES_EVEN, None)
+        seen["free_after"] = free_bytes()
+        seen["ctx_after"] = H.lib.rmi_hip_thread_context_count()
+
+    t = threading.Thread(target=call)
+    t.start()
+    t.join()
+    H.check(H.lib.rmi_hip_synchronize())
+    assert seen["rc"] == 0
+    assert seen["free_after"] == seen["free_before"]
+    assert seen["ctx_after"] == seen["ctx_before"]
+    assert np.abs(d_y.to_array(np.float32, (n_tokens, n_out))).max() > 0
+    d_x.free()
+    d_y.free()
+
+
+def test_noalloc_refuses_a_row_too_long_for_the_staging_before_it_enqueues_anything(hip):
+    H = hip.hip
+    n_in, n_out = 65536, 8  # 256 octets: beyond what the GEMV stages in LDS, within the scratch array's size
+    kernel = hip.kernel.Q8Kernel(hip.synth.q8_0_weight(970, n_out, n_in), n_in, n_out)
+    d_x = H.DeviceBuffer(n_in * 4)
+    d_y = H.DeviceBuffer(n_out * 4)
+    rc = H.lib.rmi_hip_q8_0_forward_noalloc_dev(kernel.w.handle, d_x.ptr, d_y.ptr, 1, n_out, H.ROUND_TIES_EVEN, None)
+    assert rc == -1 and "too long for the GEMV staging" in H.last_error()
+    d_x.free()
+    d_y.free()
