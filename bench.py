@@ -503,6 +503,8 @@ def compact(r):
     """A sub-record of the default line: the figure, its workload, its roofline and its CPU leg."""
     keep = {"workload": r["config"]["workload"], "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
             "steps": r["steps"], "roofline": r["roofline"]}
+    if r.get("other_mode"):
+        keep["other_mode"] = r["other_mode"]
     if r.get("cpu_baseline"):
         keep["cpu_baseline"] = r["cpu_baseline"]
     return keep
@@ -525,10 +527,15 @@ def run_gemm(args, pkg, ev):
         H.check(H.lib.rmi_hip_synchronize())
         recs.append(dict(w=w, x=x, k=k, d_q8=d_q8, d_sc=d_sc, d_y=d_y, n_out=n_out, n_in=n_in))
 
-    def step():
+    # "fast": the library picks, per product, the k-split kernel (few tokens, long rows) or the tiled kernel; every
+    # output within the reference's tolerance.  "exact": always the tiled kernel, the aarch64 kernel's single chain.
+    fast = args.gemm_mode == "fast"
+    entry = H.lib.rmi_hip_gemm_q8_0_fast_dev if fast else H.lib.rmi_hip_gemm_q8_0_dev
+    other = H.lib.rmi_hip_gemm_q8_0_dev if fast else H.lib.rmi_hip_gemm_q8_0_fast_dev
+
+    def step(fn=entry):
         for r in recs:
-            H.check(H.lib.rmi_hip_gemm_q8_0_dev(r["k"].w.handle, r["d_q8"].ptr, r["d_sc"].ptr, r["d_y"].ptr, M,
-                                                r["n_out"], None))
+            H.check(fn(r["k"].w.handle, r["d_q8"].ptr, r["d_sc"].ptr, r["d_y"].ptr, M, r["n_out"], None))
 
     copy_calibration(H, args)
     wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
@@ -538,12 +545,18 @@ def run_gemm(args, pkg, ev):
     result = base_result(args, "Q8_0 prefill GEMM TOP/s (int8 MFMA), Qwen3-0.6B FFN shapes, 1 GPU", "TOP/s",
                          round(value, 1), wall, "int8 MFMA -> f32", {
         "workload": f"Q8_0 GEMM M={M} tokens: X[Mx1024].W[3072x1024]^T and X[Mx3072].W[1024x3072]^T, "
-                    f"per-block f32 rescale, 2 launches per step",
+                    f"per-block f32 rescale, 2 launches per step, "
+                    + ("kernel chosen per product (k-split or tiled), outputs within 1e-4 + 1e-4|ref|" if fast else
+                       "tiled kernel, aarch64 accumulation order bit for bit"),
         "tokens": M, "launches_per_step": 2, "ops_per_step": ops, "device": dev_name.strip(), "compute_units": cus})
-    result["roofline"] = {"bound": "mfma", "kernel": "gemm_q8_0_kernel", "achieved": round(achieved, 1), "peak": INT8_MFMA_PEAK_TOPS,
+    result["roofline"] = {"bound": "mfma", "kernel": "gemm_q8_0_ksplit_kernel / gemm_q8_0_kernel" if fast else "gemm_q8_0_kernel",
+                          "achieved": round(achieved, 1), "peak": INT8_MFMA_PEAK_TOPS,
                           "unit": "TOP/s", "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
                           "avg_launch_us": round(dev_ms * 1e3 / 2, 3),
                           **read_traffic(f"gemm_q8_0_m{M}_qwen3_0.6b_ffn")}
+    w2, d2 = time_region(H, ev, lambda: step(other), args.steps, args.warmup)
+    result["other_mode"] = {"mode": "exact (tiled kernel, single chain)" if fast else "fast (kernel chosen per product)",
+                            "value": round(ops / w2 / 1e12, 1), "unit": "TOP/s", "avg_launch_us": round(d2 * 1e3 / 2, 3)}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
@@ -1001,6 +1014,10 @@ def main():
                     help="projection_set: accumulation order of the reference's x86-64 kernel (GEMV, the default) or of "
                          "its aarch64 kernel (small-batch kernel on the matrix cores)")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill tokens M for --workload gemm")
+    ap.add_argument("--gemm-mode", choices=["fast", "exact"], default="fast",
+                    help="gemm: 'fast' lets the library split the blocks of a row over the waves of a workgroup where the "
+                         "tile grid is smaller than the chip (outputs within the reference's tolerance); 'exact' keeps the "
+                         "aarch64 kernel's single f32 chain per output, bit for bit")
     ap.add_argument("--keys", type=int, default=4096, help="cached positions for --workload attention")
     ap.add_argument("--mode", choices=["grouped", "per_matmul", "layer"], default="grouped")
     ap.add_argument("--no-cpu-baseline", action="store_true")

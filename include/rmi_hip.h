@@ -251,6 +251,23 @@ int rmi_hip_gemv_q8_0_neon_dev(const rmi_hip_weight *w, const int8_t *x_q8, cons
 /* Y[t][:] = W . Q8_0(X[t][:]) for n_tokens >= 1 through int8 MFMA. */
 int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                           uint32_t n_tokens, uint32_t y_stride, void *stream);
+/* The same product for few tokens, for callers that ask for the reference's tolerance rather than one host's bits
+ * (Kernel::forward_batched, src/ops/kernel/trait_.rs:78-109: every token is an independent GEMV; outputs within
+ * 1e-4 + 1e-4 |ref| of either CPU kernel).  rmi_hip_gemm_q8_0_dev keeps the aarch64 kernel's single f32 chain per
+ * output, which leaves most of the chip idle below a few hundred tokens; here a workgroup is one 32 x 32 tile whose
+ * waves split the blocks of a row into runs of rmi_hip_gemm_q8_0_ksplit_quads_per_part(n_in) quads (128 elements
+ * each): every per-block int32 dot is exact, every run is added from zero in block order, the runs' sums are added
+ * in run order.  Deterministic, the same for a token whatever batch it arrives in, not bit-identical to the single
+ * chain.  No workspace, no allocation, no synchronisation. */
+int rmi_hip_gemm_q8_0_ksplit_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                                 uint32_t n_tokens, uint32_t y_stride, void *stream);
+uint32_t rmi_hip_gemm_q8_0_ksplit_quads_per_part(uint32_t n_in);
+/* Whichever of the two kernels above the library expects to be faster for this product (the k-split one for few
+ * tokens and long rows, the tiled one once the tiles fill the chip).  Every output within the reference's tolerance
+ * of the CPU kernels and built from exact integer block dots; which of the two chains a token's result follows
+ * depends on the token count of the call. */
+int rmi_hip_gemm_q8_0_fast_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                               uint32_t n_tokens, uint32_t y_stride, void *stream);
 int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,
                               const int16_t *q8k_bsums, float *y, uint32_t n_tokens, uint32_t y_stride,
                               uint32_t row_start, uint32_t row_end, void *stream);

@@ -291,6 +291,33 @@ void rmi_ref_matmul_q8_0_quantized_range(const uint8_t *weight,
     }
 }
 
+/* Not a function of the reference: the aarch64 kernel's chain (neon.rs:49-73) cut into runs of quads_per_part whole
+ * quads (4 blocks), each run summed in block order from zero, the runs' sums added in run order.  It is what the
+ * device's split-K GEMM promises to compute; one run is row_dot_neon itself, and tests hold every split to the
+ * reference orders within the reference's own tolerance. */
+void rmi_ref_matmul_q8_0_neon_split(const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
+                                    float *output, size_t n_in, size_t n_out, size_t quads_per_part) {
+    size_t blocks = n_in / QK8_0, quads = (blocks + 3) / 4;
+    size_t per = quads_per_part ? quads_per_part : 1;
+    size_t k_parts = (quads + per - 1) / per;
+    if (k_parts == 0) k_parts = 1;
+    for (size_t r = 0; r < n_out; r++) {
+        const uint8_t *row = weight + r * blocks * Q8_0_BLOCK;
+        float total = 0.0f;
+        for (size_t p = 0; p < k_parts; p++) {
+            size_t b0 = p * per * 4, b1 = (p + 1) * per * 4;
+            if (b1 > blocks) b1 = blocks;
+            float sum = 0.0f;
+            for (size_t b = b0; b < b1; b++) {
+                const uint8_t *blk = row + b * Q8_0_BLOCK;
+                sum = fmaf((float)block_dot_i8(blk + 2, input_q8 + b * QK8_0), load_f16(blk) * input_scales[b], sum);
+            }
+            total = p == 0 ? sum : total + sum;
+        }
+        output[r] = total;
+    }
+}
+
 void rmi_ref_matmul_q8_0_quantized_parallel_rows(
     const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
     float *output, size_t n_in, size_t n_out, size_t ith, size_t nth,

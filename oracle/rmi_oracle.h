@@ -62,6 +62,10 @@ void rmi_ref_matmul_q8_0_quantized_parallel_rows(
     int variant);
 
 /* The "per-block int32 dot" of scalar.rs:49-53: dots[row*n_in/32 + block]. */
+/* the aarch64 chain cut into runs of quads_per_part whole quads (128 elements each), runs summed in order (the
+ * device's split-K GEMM; not a function of the reference) */
+void rmi_ref_matmul_q8_0_neon_split(const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
+                                    float *output, size_t n_in, size_t n_out, size_t quads_per_part);
 void rmi_ref_block_dots_q8_0(const uint8_t *weight, const uint8_t *input_q8,
                              int32_t *dots, size_t n_in, size_t n_out);
 

@@ -373,6 +373,37 @@ int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
     return rmi_launch_gemm_q8_0(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
 }
 
+int rmi_hip_gemm_q8_0_ksplit_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                                 uint32_t n_tokens, uint32_t y_stride, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
+    if (y_stride < w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < n_out=%u", y_stride, w->n_out);
+    if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (rmi_misaligned(x_q8, x_scales, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
+    return rmi_launch_gemm_q8_0_ksplit(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
+}
+
+int rmi_hip_gemm_q8_0_fast_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                               uint32_t n_tokens, uint32_t y_stride, void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0) return rmi_fail(RMI_HIP_E_INVALID, "not a Q8_0 weight handle");
+    if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
+    if (y_stride < w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < n_out=%u", y_stride, w->n_out);
+    if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
+    if (rmi_misaligned(x_q8, x_scales, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
+    const double tiled = rmi_gemm_q8_0_cost_us(w, n_tokens);
+    if (tiled < 0.0 || rmi_gemm_q8_0_ksplit_cost_us(w, n_tokens) < tiled)
+        return rmi_launch_gemm_q8_0_ksplit(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
+    return rmi_launch_gemm_q8_0(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
+}
+
+uint32_t rmi_hip_gemm_q8_0_ksplit_quads_per_part(uint32_t n_in) {
+    uint32_t per = 1, n_waves = 1;
+    rmi_gemm_q8_0_ksplit_shape(n_in, &per, &n_waves);
+    return per;
+}
+
 int rmi_hip_copy_dev(void *dst, const void *src, size_t nbytes, void *stream) {
     RMI_REQUIRE_INIT();
     if (!dst || !src || nbytes % 16 != 0) return rmi_fail(RMI_HIP_E_INVALID, "copy needs non-null pointers and a multiple of 16 bytes");

@@ -438,22 +438,25 @@ GemmShape make_shape() {
 
 }  // namespace
 
-int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
-                         uint32_t n_tokens, uint32_t y_stride, hipStream_t s) {
-    if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
-    if (w->n_in < 32) return rmi_fail(RMI_HIP_E_INVALID, "GEMM needs at least one block per row");
-    // Every wave spends about the same time per sub-tile and block (the rescale on the VALU) and the waves of a SIMD
-    // share it, so a launch takes about (waves on the busiest SIMD) x (sub-tiles per wave) steps per block, round
-    // after round of workgroups, plus a fixed cost per round (first loads, last stores).  Measured on MI355X, a
-    // step: 90 ns with three or more waves on the SIMD or several sub-tiles per wave, 105 ns with two waves of one
-    // sub-tile, 125 ns for a wave alone; a round: about 3.5 us.  The shape with the smallest estimate is taken,
-    // the larger tile on a tie (less traffic): 96x128 (4 waves x 3 sub-tiles, two workgroups a compute unit) for
-    // large products, 64x128 and 64x64 where those would leave compute units idle.
+namespace {
+
+struct GemmPlan {
+    const GemmShape *shape;
+    double cost_us;
+};
+
+// Every wave spends about the same time per sub-tile and block (the rescale on the VALU) and the waves of a SIMD
+// share it, so a launch takes about (waves on the busiest SIMD) x (sub-tiles per wave) steps per block, round
+// after round of workgroups, plus a fixed cost per round (first loads, last stores).  Measured on MI355X, a
+// step: 90 ns with three or more waves on the SIMD or several sub-tiles per wave, 105 ns with two waves of one
+// sub-tile, 125 ns for a wave alone; a round: about 3.5 us.  The shape with the smallest estimate is taken,
+// the larger tile on a tie (less traffic): 96x128 (4 waves x 3 sub-tiles, two workgroups a compute unit) for
+// large products, 64x128 and 64x64 where those would leave compute units idle.
+GemmPlan plan_gemm(const rmi_hip_weight *w, uint32_t n_tokens) {
     static const GemmShape shapes[] = {make_shape<3, 1, 1, 4, 2>(), make_shape<2, 1, 1, 4, 2>(), make_shape<1, 1, 2, 2, 3>()};
     const uint64_t cus = uint64_t(rmi_device_cus() > 0 ? rmi_device_cus() : 1);
     const double nb = double(w->n_in / 32);
-    const GemmShape *best = nullptr;
-    double best_cost = 0.0;
+    GemmPlan best{nullptr, 0.0};
     for (const GemmShape &g : shapes) {
         const uint64_t groups = uint64_t((w->n_out + g.tile_n - 1) / g.tile_n) * ((n_tokens + g.tile_t - 1) / g.tile_t);
         if (groups > 0x7fffffffull) continue;
@@ -467,14 +470,28 @@ int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const floa
         };
         double cost = double(full) * round_us(uint64_t(g.per_cu));
         if (rest) cost += round_us((rest + cus - 1) / cus);
-        if (!best || cost < best_cost * 0.999) {
-            best_cost = cost;
-            best = &g;
-        }
+        if (!best.shape || cost < best.cost_us * 0.999) best = GemmPlan{&g, cost};
     }
-    if (!best) return rmi_fail(RMI_HIP_E_INVALID, "GEMM too large for one launch");
+    return best;
+}
+
+}  // namespace
+
+// the launch time the tile chooser expects for this product, in microseconds (a negative value: no shape fits)
+double rmi_gemm_q8_0_cost_us(const rmi_hip_weight *w, uint32_t n_tokens) {
+    if (n_tokens == 0 || w->n_out == 0 || w->n_in < 32) return 0.0;
+    const GemmPlan plan = plan_gemm(w, n_tokens);
+    return plan.shape ? plan.cost_us : -1.0;
+}
+
+int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                         uint32_t n_tokens, uint32_t y_stride, hipStream_t s) {
+    if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
+    if (w->n_in < 32) return rmi_fail(RMI_HIP_E_INVALID, "GEMM needs at least one block per row");
+    const GemmPlan plan = plan_gemm(w, n_tokens);
+    if (!plan.shape) return rmi_fail(RMI_HIP_E_INVALID, "GEMM too large for one launch");
     const bool ragged = (w->n_in / 32) % 4 != 0 || (reinterpret_cast<uintptr_t>(x_scales) & 15) != 0;
-    best->launch(w, x_q8, x_scales, y, n_tokens, y_stride, ragged, s);
+    plan.shape->launch(w, x_q8, x_scales, y, n_tokens, y_stride, ragged, s);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }

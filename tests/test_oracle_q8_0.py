@@ -300,3 +300,29 @@ def test_expf_restatement_equals_host_libm(oracle):
     assert oracle.lib.rmi_ref_expf_mismatches(int(np.float32(1.0).view(np.uint32)), 1, 1 << 22) == 0  # [1, 1.5)
     assert oracle.expf_restated(0.0) == 1.0 and oracle.expf_restated(-np.inf) == 0.0
     assert np.isnan(oracle.expf_restated(np.nan)) and oracle.expf_restated(89.0) == np.inf
+
+
+def test_neon_split_chain_is_the_neon_chain_for_one_part_and_within_tolerance_for_more(oracle):
+    """The checker's statement of the split-K GEMM: one run is the aarch64 chain bit for bit; several runs stay
+    within the reference's tolerance of every reference order and differ from the single chain somewhere (the
+    split is real)."""
+    n_out, n_in = 64, 3072
+    w = gen.q8_0_weight(4242, n_out, n_in) if hasattr(gen, "q8_0_weight") else None
+    if w is None:
+        rng = np.random.default_rng(4242)
+        blocks = np.zeros((n_out * n_in // 32, 34), np.uint8)
+        blocks[:, :2] = (np.abs(rng.normal(0, 0.02, (n_out * n_in // 32, 1))) / 127).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        blocks[:, 2:] = rng.integers(-127, 128, (n_out * n_in // 32, 32), dtype=np.int8).view(np.uint8)
+        w = blocks.reshape(-1)
+    x = np.random.default_rng(4243).normal(0, 1, n_in).astype(np.float32)
+    q8, sc = oracle.quantize_q8_0(x, oracle.AVX2)
+    neon = oracle.matmul_q8_0_quantized(w, q8, sc, n_in, n_out, oracle.NEON)
+    assert np.array_equal(bits(oracle.matmul_q8_0_neon_split(w, q8, sc, n_in, n_out, 24)), bits(neon))
+    avx2 = oracle.matmul_q8_0_quantized(w, q8, sc, n_in, n_out, oracle.AVX2)
+    differs = False
+    for per in (1, 2, 3, 5, 12, 23):
+        y = oracle.matmul_q8_0_neon_split(w, q8, sc, n_in, n_out, per)
+        for ref in (neon, avx2):
+            assert np.all(np.abs(y - ref) <= 1e-4 + 1e-4 * np.abs(ref))
+        differs |= not np.array_equal(bits(y), bits(neon))
+    assert differs
