@@ -406,6 +406,17 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
                                             uint32_t head_dim_k, uint32_t head_dim_v, int8_t *q8, float *scales,
                                             int rounding, void *stream);
 
+/* The two calls above in one launch, for head dimension 128 and contexts of up to 3392 keys: qkv is the f32
+ * [q ; k ; v] of the new token (position n_keys - 1); every head's workgroup norms and rotates its q and its
+ * key/value head's k, rounds them and v to f16, uses them from on-chip memory and writes k and v to row
+ * n_keys - 1 of the caches; keys 0..n_keys-2 are read from the caches (src/models/qwen3.rs:776-933).  Same bits
+ * as the two calls.  It lets the q/k/v product in front be a plain GEMV over the whole chip. */
+int rmi_hip_qkv_attention_f16_quantize_q8_0_dev(const float *qkv, const float *q_norm, const float *k_norm,
+                                                const float *cos_row, const float *sin_row, uint16_t *k_cache,
+                                                uint16_t *v_cache, uint32_t n_keys, uint32_t kv_stride, uint32_t n_head,
+                                                uint32_t n_head_kv, float eps, int8_t *q8, float *scales, int rounding,
+                                                void *stream);
+
 /* Uploads and repacks the weights (host slices may be dropped afterwards), allocates the KV cache. */
 rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_hip_qwen3_weights *weights);
 void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s);

@@ -445,16 +445,33 @@ __host__ __device__ inline size_t attn128_lds_bytes(uint32_t n_keys) {
     const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
     return n_pad * 12 + (kA128Threads / 64) * 128 * 8 + 128;  // 32 floats of room behind the scores
 }
+// FROM_QKV: the launch also does what qk_norm_rope_store_kernel does for this step, so that the q/k/v product in
+// front of it can be a plain GEMV spread over the whole chip (a head per workgroup there means 139 KB of weights
+// through one compute unit).  fq points at the step's f32 [q ; k ; v] and the norm weights and angles; waves 0, 1
+// and 2 turn the head's q, its key/value head's new k and new v into f16 while the first cached keys are on their
+// way, the new key and value are used from LDS (and written to their cache row by the first query head of each
+// key/value head), the keys 0..step-1 come from the cache as before.
+struct AttnFromQkv {
+    const float *qkv;                // [n_head * 128 q | n_head_kv * 128 k | n_head_kv * 128 v]
+    const float *q_norm, *k_norm;    // [128] each, or null
+    const float *cos_row, *sin_row;  // [64] each: the angles of this position
+    uint16_t *k_row, *v_row;         // the cache rows of this position, [n_head_kv][128] each
+    float eps;
+};
+template <bool FROM_QKV>
 __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
     uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, int8_t *__restrict__ q8,
-    float *__restrict__ scales, int rounding) {
+    float *__restrict__ scales, int rounding, AttnFromQkv fq) {
     extern __shared__ double lds_d[];
     __shared__ float red_f[kA128Threads / 64];
     __shared__ uint64_t exp_tab[32];
+    __shared__ __attribute__((aligned(16))) uint16_t new16[3][128];  // this step's q, k, v as f16
     // grid = (query heads per key/value head, key/value heads)
     const uint32_t kvh = blockIdx.y, head = blockIdx.y * gridDim.x + blockIdx.x, tid = threadIdx.x;
     const uint32_t n_keys = step + 1;
+    // keys that come from the cache, and the last row there that may be read
+    const uint32_t n_cached = FROM_QKV ? step : n_keys, last_row = n_cached ? n_cached - 1 : 0;
     const uint32_t n_pad = (n_keys + kAttnPad - 1) / kAttnPad * kAttnPad;
     double *wd = lds_d;                                        // [n_pad] softmax weights (f16 values), 0 beyond n_keys
     double *part = wd + n_pad;                                 // [waves][128]
@@ -469,26 +486,83 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     const uint4 *qp = reinterpret_cast<const uint4 *>(q16 + size_t(head) * 128) + lane4;
     const uint4 *kbase = reinterpret_cast<const uint4 *>(k_cache + size_t(kvh) * 128) + lane4;
     uint4 qv[4], kk[4];
+    float raw0 = 0.0f, raw1 = 0.0f, nw0 = 1.0f, nw1 = 1.0f, cos_a = 0.0f, sin_a = 0.0f;
+    if constexpr (FROM_QKV) {
+        if (tid < 192) {  // wave 0: q of this head, wave 1: the new k, wave 2: the new v; lane i owns (i, i + 64)
+            const uint32_t lane = tid & 63;
+            const float *src = tid < 64 ? fq.qkv + size_t(head) * 128
+                                        : fq.qkv + size_t(n_head) * 128 + (tid < 128 ? size_t(kvh) : size_t(n_head_kv) + kvh) * 128;
+            raw0 = src[lane];
+            raw1 = src[lane + 64];
+            if (tid < 128) {
+                cos_a = fq.cos_row[lane];
+                sin_a = fq.sin_row[lane];
+                const float *nw = tid < 64 ? fq.q_norm : fq.k_norm;
+                if (nw) {
+                    nw0 = nw[lane];
+                    nw1 = nw[lane + 64];
+                }
+            }
+        }
+    } else {
 #pragma unroll
-    for (int c = 0; c < 4; c++) qv[c] = qp[4 * c];
+        for (int c = 0; c < 4; c++) qv[c] = qp[4 * c];
+    }
     {
-        const uint4 *key = kbase + __umul24(key0 < n_keys ? key0 : n_keys - 1, row_u4);
+        const uint4 *key = kbase + __umul24(key0 < n_cached ? key0 : last_row, row_u4);
 #pragma unroll
         for (int c = 0; c < 4; c++) kk[c] = key[4 * c];
     }
     // values: lane = (8 dimensions dg, key slice sl): 16 consecutive lanes read the 256 bytes of one row
     constexpr uint32_t kPre = kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40);
     const uint32_t dg = tid & 15, sl = tid >> 4;
-    const uint32_t chunk = (n_keys + kA128Threads / 16 - 1) / (kA128Threads / 16);
-    const uint32_t t_begin = sl * chunk, t_end = t_begin + chunk < n_keys ? t_begin + chunk : n_keys;
+    const uint32_t chunk = (n_cached + kA128Threads / 16 - 1) / (kA128Threads / 16);
+    const uint32_t t_begin = sl * chunk, t_end = t_begin + chunk < n_cached ? t_begin + chunk : n_cached;
     const uint4 *vbase = reinterpret_cast<const uint4 *>(v_cache + size_t(kvh) * 128 + dg * 8);
     uint4 vp[kPre];
 #pragma unroll
     for (uint32_t j = 0; j < kPre; j++) {  // j < chunk is uniform: no lane waits on a guarded load of its own
         if (j < chunk) {
-            const uint32_t t = t_begin + j < n_keys ? t_begin + j : n_keys - 1;
+            const uint32_t t = t_begin + j < n_cached ? t_begin + j : last_row;
             vp[j] = vbase[__umul24(t, row_u4)];
         }
+    }
+    if constexpr (FROM_QKV) {
+        // head norm (when the model has the weights), NeoX rotation, rounding to f16: src/models/qwen3.rs:776-874
+        if (tid < 192) {
+            const uint32_t lane = tid & 63, which = tid >> 6;
+            uint16_t h0, h1;
+            if (which == 2) {
+                h0 = f2h(raw0);
+                h1 = f2h(raw1);
+            } else {
+                float x0 = raw0, x1 = raw1;
+                if (which == 0 ? fq.q_norm != nullptr : fq.k_norm != nullptr) {
+                    const float q0 = raw0 * raw0, q1 = raw1 * raw1;
+                    double part = double(q0);
+                    part += double(q1);
+                    part = wave_sum_f64(part);
+                    const float mean_sq = float(part / 128.0);
+                    const float sc = 1.0f / sqrtf(mean_sq + fq.eps);
+                    x0 = (raw0 * sc) * nw0;
+                    x1 = (raw1 * sc) * nw1;
+                }
+                const float ta = x1 * -sin_a;
+                const float tb = x1 * cos_a;
+                h0 = f2h(__builtin_fmaf(x0, cos_a, ta));
+                h1 = f2h(__builtin_fmaf(x0, sin_a, tb));
+            }
+            new16[which][lane] = h0;
+            new16[which][lane + 64] = h1;
+            if (which && blockIdx.x == 0) {  // the first query head of the key/value head fills the cache row
+                uint16_t *dst = (which == 1 ? fq.k_row : fq.v_row) + size_t(kvh) * 128;
+                dst[lane] = h0;
+                dst[lane + 64] = h1;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 4; c++) qv[c] = reinterpret_cast<const uint4 *>(new16[0])[lane4 + 4 * c];
     }
     const float kq_scale = 1.0f / sqrtf(128.0f);  // two f32 roundings, as the reference computes it
     float my_max = -INFINITY;
@@ -499,9 +573,15 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
         // for this round's keys would have to drain them, too.
         uint4 kn[4];
         {
-            const uint4 *key = kbase + __umul24(tn < n_keys ? tn : n_keys - 1, row_u4);
+            const uint4 *key = kbase + __umul24(tn < n_cached ? tn : last_row, row_u4);
 #pragma unroll
             for (int c = 0; c < 4; c++) kn[c] = key[4 * c];
+        }
+        if constexpr (FROM_QKV) {
+            if (t == n_cached) {  // this step's key: not in the cache yet for this launch, in LDS
+#pragma unroll
+                for (int c = 0; c < 4; c++) kk[c] = reinterpret_cast<const uint4 *>(new16[1])[lane4 + 4 * c];
+            }
         }
         double s4[4] = {0.0, 0.0, 0.0, 0.0};  // four chains of eight adds, not one of thirty-two
 #pragma unroll
@@ -586,13 +666,13 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
 #pragma unroll
         for (uint32_t j = 0; j < 8; j++) {
             const uint32_t t = t_begin + kPre + j;
-            cur[j] = vbase[__umul24(t < n_keys ? t : n_keys - 1, row_u4)];
+            cur[j] = vbase[__umul24(t < n_cached ? t : last_row, row_u4)];
         }
         for (uint32_t t0 = t_begin + kPre; t0 < t_end; t0 += 8) {
 #pragma unroll
             for (uint32_t j = 0; j < 8; j++) {
                 const uint32_t t = t0 + 8 + j;
-                nxt[j] = vbase[__umul24(t < n_keys ? t : n_keys - 1, row_u4)];
+                nxt[j] = vbase[__umul24(t < n_cached ? t : last_row, row_u4)];
             }
 #pragma unroll
             for (uint32_t j = 0; j < 8; j++) {
@@ -605,6 +685,14 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
             }
 #pragma unroll
             for (uint32_t j = 0; j < 8; j++) cur[j] = nxt[j];
+        }
+    }
+    if constexpr (FROM_QKV) {
+        if (sl == 0) {  // this step's value, from LDS: one more exact term of the f64 sums
+            const double w = wd[n_cached];
+            const half8 vh = as_half8(reinterpret_cast<const uint4 *>(new16[2])[dg]);
+#pragma unroll
+            for (int d = 0; d < 8; d++) acc[d] = __builtin_fma(double(float(vh[d])), w, acc[d]);
         }
     }
 #pragma unroll
@@ -916,7 +1004,7 @@ __global__ __launch_bounds__(kAttnSplitThreads) void attn128_weights_pv_kernel(
 size_t attn_lds_limit() {
     static const size_t limit = [] {
         constexpr size_t kWant = 159 * 1024;
-        const bool ok = hipFuncSetAttribute(reinterpret_cast<const void *>(attention128_quant_kernel),
+        const bool ok = hipFuncSetAttribute(reinterpret_cast<const void *>(attention128_quant_kernel<false>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, int(kWant)) == hipSuccess &&
                         hipFuncSetAttribute(reinterpret_cast<const void *>(attention_quant_kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, int(kWant)) == hipSuccess &&
@@ -1165,7 +1253,22 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
         int rc;
         const size_t layer_base = size_t(l) * c.capacity * s->kv_stride, row = layer_base + size_t(step) * s->kv_stride;
         const float *qn = c.has_qk_norm ? s->q_norm[l] : nullptr, *kn = c.has_qk_norm ? s->k_norm[l] : nullptr;
-        if (rmi_gemv_q8_0_norm_rope_fusable(s->w_qkv[l], c.n_head, c.n_head_kv, c.head_dim_k, c.head_dim_v)) {
+        const bool d128 = c.head_dim_k == 128 && c.head_dim_v == 128;
+        const bool split = d128 && s->attn_split && attn128_use_split(step + 1, c.n_head);
+        // Short contexts: the q/k/v product as a plain GEMV behind the norm, one wave a tile over the whole chip, and
+        // the head norms, the rotation and the cache row inside the attention launch.
+        const bool qkv_in_attention = d128 && !split && rmi_gemv_q8_0_norm_fusable(s->w_qkv[l]) &&
+                                      attn128_lds_bytes(step + 1) <= 48 * 1024;
+        if (qkv_in_attention) {
+            rc = norm_gemv(s->w_qkv[l], pending, s->attn_norm[l], s->qkv);
+            if (rc != RMI_HIP_OK) return rc;
+            const size_t half = 64;
+            const AttnFromQkv fq{s->qkv, qn, kn, s->cos_t + size_t(step) * half, s->sin_t + size_t(step) * half,
+                                 s->k_cache + row, s->v_cache + row, c.eps};
+            hipLaunchKernelGGL(attention128_quant_kernel<true>, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kA128Threads),
+                               attn128_lds_bytes(step + 1), st, static_cast<const uint16_t *>(nullptr), s->k_cache + layer_base,
+                               s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd, fq);
+        } else if (rmi_gemv_q8_0_norm_rope_fusable(s->w_qkv[l], c.n_head, c.n_head_kv, c.head_dim_k, c.head_dim_v)) {
             // norm, q/k/v products, head norms, rotation and the cache row in one launch
             const size_t half = c.head_dim_k / 2;
             rc = rmi_launch_gemv_q8_0_norm_rope(s->w_qkv[l], x, pending, s->attn_norm[l], x_other, c.eps, rnd, qn, kn,
@@ -1180,15 +1283,17 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                                s->cos_t, s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head,
                                c.n_head_kv, c.head_dim_k, c.head_dim_v, c.eps);
         }
-        if (c.head_dim_k == 128 && c.head_dim_v == 128 && s->attn_split && attn128_use_split(step + 1, c.n_head)) {
+        if (qkv_in_attention) {
+            // done above
+        } else if (split) {
             rc = launch_attention128_split(s->q16, s->k_cache + layer_base, s->v_cache + layer_base, step + 1, s->kv_stride,
                                            c.n_head, c.n_head_kv, attn_split_scratch_at(s->attn_split, c.n_head, c.capacity),
                                            s->act_q8, s->act_scales, rnd, st);
             if (rc != RMI_HIP_OK) return rc;
-        } else if (c.head_dim_k == 128 && c.head_dim_v == 128)
-            hipLaunchKernelGGL(attention128_quant_kernel, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kA128Threads), attn128_lds_bytes(step + 1),
+        } else if (d128)
+            hipLaunchKernelGGL(attention128_quant_kernel<false>, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kA128Threads), attn128_lds_bytes(step + 1),
                                st, s->q16, s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride,
-                               c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd);
+                               c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd, AttnFromQkv{});
         else
             hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(kAttnThreads), attn_lds, st, s->q16,
                                s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head,
@@ -1342,12 +1447,35 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
         return RMI_HIP_OK;
     }
     if (d128)
-        hipLaunchKernelGGL(attention128_quant_kernel, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
-                           q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding);
+        hipLaunchKernelGGL(attention128_quant_kernel<false>, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
+                           q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding, AttnFromQkv{});
     else
         hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream),
                            q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8,
                            scales, rounding);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_qkv_attention_f16_quantize_q8_0_dev(const float *qkv, const float *q_norm, const float *k_norm,
+                                                const float *cos_row, const float *sin_row, uint16_t *k_cache,
+                                                uint16_t *v_cache, uint32_t n_keys, uint32_t kv_stride, uint32_t n_head,
+                                                uint32_t n_head_kv, float eps, int8_t *q8, float *scales, int rounding,
+                                                void *stream) {
+    RMI_REQUIRE_INIT();
+    if (!qkv || !cos_row || !sin_row || !k_cache || !v_cache || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
+    if (n_keys == 0 || n_head == 0 || n_head_kv == 0 || n_head % n_head_kv || kv_stride % 8 || kv_stride < n_head_kv * 128)
+        return rmi_fail(RMI_HIP_E_INVALID, "bad attention shape");
+    const size_t lds = attn128_lds_bytes(n_keys);
+    if (lds > 48 * 1024)
+        return rmi_fail(RMI_HIP_E_INVALID, "%u keys: beyond %u the rotation runs in its own launch "
+                        "(rmi_hip_qk_norm_rope_f16_dev, then rmi_hip_attention_f16_quantize_q8_0_dev)", n_keys,
+                        uint32_t((48 * 1024 - (kA128Threads / 64) * 128 * 8 - 128) / 12 / kAttnPad * kAttnPad));
+    const size_t row = size_t(n_keys - 1) * kv_stride;
+    const AttnFromQkv fq{qkv, q_norm, k_norm, cos_row, sin_row, k_cache + row, v_cache + row, eps};
+    hipLaunchKernelGGL(attention128_quant_kernel<true>, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(nullptr), k_cache, v_cache, n_keys - 1,
+                       kv_stride, n_head, n_head_kv, q8, scales, rounding, fq);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }

@@ -127,6 +127,8 @@ SIGNATURES = {
     "rmi_hip_silu_mul_quantize_q8_0_dev": (C.c_int, [_vp, _u32, _vp, _vp, C.c_int, _vp]),
     "rmi_hip_qk_norm_rope_f16_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32,
                                                C.c_float, _vp]),
+    "rmi_hip_qkv_attention_f16_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_float,
+                                                              _vp, _vp, C.c_int, _vp]),
     "rmi_hip_attention_f16_quantize_q8_0_dev": (C.c_int, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp,
                                                           C.c_int, _vp]),
     "rmi_hip_qwen3_create": (_vp, [C.POINTER(Qwen3Config), C.POINTER(Qwen3Weights)]),

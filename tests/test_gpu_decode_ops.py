@@ -262,3 +262,60 @@ def test_attention_split_mixed_head_counts(hip, oracle):
         assert np.array_equal(d_s.to_array(np.float32, (n_head * hv // 32,)).view(np.uint32), s_ref.view(np.uint32)), (n_head, n_kv, n_keys)
         for b in (d_q, d_k, d_v, d_o, d_s):
             b.free()
+
+
+@pytest.mark.parametrize("n_head,n_kv,with_norm", [(16, 8, True), (16, 8, False), (6, 6, True), (32, 4, True)])
+def test_qkv_attention_in_one_launch_equals_the_two_calls(hip, oracle, n_head, n_kv, with_norm):
+    """rmi_hip_qkv_attention_f16_quantize_q8_0_dev against rmi_hip_qk_norm_rope_f16_dev followed by
+    rmi_hip_attention_f16_quantize_q8_0_dev: the quantized output, its scales and the two cache rows of the new
+    position, bit for bit, from the first position (no cached key) to several hundred; the other cache rows
+    untouched.  The two calls are held to the checker elsewhere in this file."""
+    H = hip.hip
+    rng = np.random.default_rng(n_head * 31 + n_kv)
+    hd = 128
+    kv_stride = n_kv * hd + 8  # rows wider than the heads: the stride is not the width
+    for n_keys in [1, 2, 3, 16, 17, 33, 127, 128, 129, 257, 512, 640, 767, 1024]:
+        scale = rng.choice([0.3, 1.0, 3.0])
+        qkv = (rng.normal(0, 1, (n_head + 2 * n_kv) * hd) * scale).astype(np.float32)
+        qn = rng.normal(1, 0.2, hd).astype(np.float32)
+        kn = rng.normal(1, 0.2, hd).astype(np.float32)
+        ang = rng.uniform(-3, 3, 64)
+        cs, sn = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+        kc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+        vc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+        kc[-1] = 0x7e00  # the new position's rows hold NaN until the call fills them
+        vc[-1] = 0x7e00
+        d_qkv, d_qn, d_kn, d_cs, d_sn = (_dev(H, a) for a in (qkv, qn, kn, cs, sn))
+        outs = []
+        for fused in (False, True):
+            d_k, d_v = _dev(H, kc), _dev(H, vc)
+            d_o, d_s = H.DeviceBuffer(n_head * hd), H.DeviceBuffer(n_head * hd // 32 * 4)
+            row = (n_keys - 1) * kv_stride * 2
+            if fused:
+                H.check(H.lib.rmi_hip_qkv_attention_f16_quantize_q8_0_dev(
+                    d_qkv.ptr, d_qn.ptr if with_norm else None, d_kn.ptr if with_norm else None, d_cs.ptr, d_sn.ptr, d_k.ptr,
+                    d_v.ptr, n_keys, kv_stride, n_head, n_kv, 1e-6, d_o.ptr, d_s.ptr, A, None))
+            else:
+                d_q16 = H.DeviceBuffer(n_head * hd * 2)
+                H.check(H.lib.rmi_hip_qk_norm_rope_f16_dev(d_qkv.ptr, d_qn.ptr if with_norm else None,
+                                                          d_kn.ptr if with_norm else None, d_cs.ptr, d_sn.ptr, d_q16.ptr,
+                                                          d_k.ptr + row, d_v.ptr + row, n_head, n_kv, hd, hd, 1e-6, None))
+                H.check(H.lib.rmi_hip_attention_f16_quantize_q8_0_dev(d_q16.ptr, d_k.ptr, d_v.ptr, n_keys, kv_stride, n_head,
+                                                                      n_kv, hd, hd, d_o.ptr, d_s.ptr, A, None))
+            H.check(H.lib.rmi_hip_synchronize())
+            outs.append((d_o.to_array(np.int8, (n_head * hd,)), d_s.to_array(np.uint32, (n_head * hd // 32,)),
+                         d_k.to_array(np.uint16, (n_keys, kv_stride)), d_v.to_array(np.uint16, (n_keys, kv_stride))))
+            for b in (d_k, d_v, d_o, d_s):
+                b.free()
+        (o0, s0, k0, v0), (o1, s1, k1, v1) = outs
+        assert np.array_equal(k0, k1) and np.array_equal(v0, v1), n_keys
+        assert np.array_equal(k1[:-1], kc[:-1]) and np.array_equal(v1[:-1], vc[:-1]), n_keys
+        assert not (k1[-1, :n_kv * hd] == 0x7e00).any() and np.all(k1[-1, n_kv * hd:] == 0x7e00), n_keys
+        assert np.array_equal(o0, o1) and np.array_equal(s0, s1), n_keys
+        for b in (d_qkv, d_qn, d_kn, d_cs, d_sn):
+            b.free()
+    # beyond what it holds: refused with the way out named
+    d = H.DeviceBuffer(64)
+    rc = H.lib.rmi_hip_qkv_attention_f16_quantize_q8_0_dev(d.ptr, None, None, d.ptr, d.ptr, d.ptr, d.ptr, 5000, 1024, 16, 8,
+                                                           1e-6, d.ptr, d.ptr, A, None)
+    assert rc == -1 and "rmi_hip_qk_norm_rope_f16_dev" in H.last_error()
