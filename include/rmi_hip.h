@@ -262,10 +262,18 @@ int rmi_hip_gemm_q8_0_dev(const rmi_hip_weight *w, const int8_t *x_q8, const flo
 int rmi_hip_gemm_q8_0_ksplit_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                                  uint32_t n_tokens, uint32_t y_stride, void *stream);
 uint32_t rmi_hip_gemm_q8_0_ksplit_quads_per_part(uint32_t n_in);
-/* Whichever of the two kernels above the library expects to be faster for this product (the k-split one for few
- * tokens and long rows, the tiled one once the tiles fill the chip).  Every output within the reference's tolerance
- * of the CPU kernels and built from exact integer block dots; which of the two chains a token's result follows
- * depends on the token count of the call. */
+/* The prefill product for callers that ask for the reference's tolerance rather than one host's bits: the library
+ * takes what it expects to be fastest for this product, the k-split kernel above (few tokens, long rows), the tiled
+ * kernel of rmi_hip_gemm_q8_0_dev, or that kernel with two groups of waves per tile that take the even and the odd
+ * quads of a row (a chain per group, the groups' sums added in group order), which gives a product of a few hundred
+ * tokens larger tiles on every compute unit.  Every output is built from exact integer block dots, deterministic,
+ * and within 1e-4 + 1e-4 |ref| of the CPU kernels; which chain a token's result follows depends on the token count
+ * of the call.  rmi_hip_gemm_q8_0_fast_plan says which one a call would take: RMI_HIP_GEMM_PLAN_* and, in *param,
+ * the quads per run (k-split) or the number of interleaved groups (tiled). */
+#define RMI_HIP_GEMM_PLAN_TILED_SINGLE_CHAIN 0
+#define RMI_HIP_GEMM_PLAN_TILED_GROUPS 1
+#define RMI_HIP_GEMM_PLAN_KSPLIT 2
+int rmi_hip_gemm_q8_0_fast_plan(const rmi_hip_weight *w, uint32_t n_tokens, uint32_t *param);
 int rmi_hip_gemm_q8_0_fast_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                                uint32_t n_tokens, uint32_t y_stride, void *stream);
 int rmi_hip_gemv_q4_k_q8k_dev(const rmi_hip_weight *w, const float *q8k_d, const int8_t *q8k_qs,

@@ -318,6 +318,29 @@ void rmi_ref_matmul_q8_0_neon_split(const uint8_t *weight, const uint8_t *input_
     }
 }
 
+/* Not a function of the reference either: the chain cut into n_groups interleaved chains, group g taking the quads
+ * g, g + n_groups, g + 2 n_groups, ... in order from zero, the groups' sums added in group order (the device's tiled
+ * GEMM with groups of waves; n_groups = 1 is row_dot_neon). */
+void rmi_ref_matmul_q8_0_neon_interleaved(const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
+                                          float *output, size_t n_in, size_t n_out, size_t n_groups) {
+    size_t blocks = n_in / QK8_0;
+    if (n_groups == 0) n_groups = 1;
+    for (size_t r = 0; r < n_out; r++) {
+        const uint8_t *row = weight + r * blocks * Q8_0_BLOCK;
+        float total = 0.0f;
+        for (size_t g = 0; g < n_groups; g++) {
+            float sum = 0.0f;
+            for (size_t b = 0; b < blocks; b++) {
+                if ((b / 4) % n_groups != g) continue;
+                const uint8_t *blk = row + b * Q8_0_BLOCK;
+                sum = fmaf((float)block_dot_i8(blk + 2, input_q8 + b * QK8_0), load_f16(blk) * input_scales[b], sum);
+            }
+            total = g == 0 ? sum : total + sum;
+        }
+        output[r] = total;
+    }
+}
+
 void rmi_ref_matmul_q8_0_quantized_parallel_rows(
     const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
     float *output, size_t n_in, size_t n_out, size_t ith, size_t nth,

@@ -66,6 +66,10 @@ void rmi_ref_matmul_q8_0_quantized_parallel_rows(
  * device's split-K GEMM; not a function of the reference) */
 void rmi_ref_matmul_q8_0_neon_split(const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
                                     float *output, size_t n_in, size_t n_out, size_t quads_per_part);
+/* the aarch64 chain as n_groups interleaved chains of quads, the groups' sums added in order (the device's tiled
+ * GEMM with groups of waves; not a function of the reference) */
+void rmi_ref_matmul_q8_0_neon_interleaved(const uint8_t *weight, const uint8_t *input_q8, const float *input_scales,
+                                          float *output, size_t n_in, size_t n_out, size_t n_groups);
 void rmi_ref_block_dots_q8_0(const uint8_t *weight, const uint8_t *input_q8,
                              int32_t *dots, size_t n_in, size_t n_out);
 

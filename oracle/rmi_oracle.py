@@ -52,6 +52,7 @@ def _load():
         "rmi_ref_unpack_scales_kmask": (None, [_u8p, _u8p]),
         "rmi_ref_vec_dot_q4k_q8k": (C.c_float, [_u8p, _sz, _f32p, _i8p, _i16p, C.c_int]),
         "rmi_ref_matmul_q8_0_neon_split": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz]),
+        "rmi_ref_matmul_q8_0_neon_interleaved": (None, [_u8p, _u8p, _f32p, _f32p, _sz, _sz, _sz]),
         "rmi_ref_q4k_q8k_block_ints": (None, [_u8p, _sz, _i8p, _i16p, _i32p, _i32p]),
         "rmi_ref_q4k_q8k_block_ints_matrix": (None, [_u8p, _sz, _sz, _i8p, _i16p, _i32p]),
         "rmi_ref_dequantize_row_q4_k": (None, [_u8p, _f32p, _sz]),
@@ -243,6 +244,16 @@ def matmul_q8_0_neon_split(w, q8, sc, n_in, n_out, quads_per_part):
     w, q8, sc = _u8(w), _u8(q8), _f32(sc)
     out = np.zeros(n_out, np.float32)
     lib.rmi_ref_matmul_q8_0_neon_split(_p(w, _u8p), _p(q8, _u8p), _p(sc, _f32p), _p(out, _f32p), n_in, n_out, quads_per_part)
+    return out
+
+
+def matmul_q8_0_neon_interleaved(w, q8, sc, n_in, n_out, n_groups):
+    """The aarch64 kernel's chain as `n_groups` interleaved chains (group g: quads g, g + n_groups, ...), the groups'
+    sums added in group order: what the device's tiled GEMM computes with groups of waves (not a function of the
+    reference)."""
+    w, q8, sc = _u8(w), _u8(q8), _f32(sc)
+    out = np.zeros(n_out, np.float32)
+    lib.rmi_ref_matmul_q8_0_neon_interleaved(_p(w, _u8p), _p(q8, _u8p), _p(sc, _f32p), _p(out, _f32p), n_in, n_out, n_groups)
     return out
 
 

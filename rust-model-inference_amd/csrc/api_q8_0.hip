@@ -384,6 +384,29 @@ int rmi_hip_gemm_q8_0_ksplit_dev(const rmi_hip_weight *w, const int8_t *x_q8, co
     return rmi_launch_gemm_q8_0_ksplit(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
 }
 
+// which kernel rmi_hip_gemm_q8_0_fast_dev takes for this product, and how it cuts the chain
+static int fast_plan(const rmi_hip_weight *w, uint32_t n_tokens, uint32_t *param) {
+    uint32_t groups = 1;
+    const double tiled = rmi_gemm_q8_0_cost_us(w, n_tokens, false, &groups);
+    if (tiled < 0.0 || rmi_gemm_q8_0_ksplit_cost_us(w, n_tokens) < tiled) {
+        uint32_t per = 1, n_waves = 1;
+        rmi_gemm_q8_0_ksplit_shape(w->n_in, &per, &n_waves);
+        *param = per;
+        return RMI_HIP_GEMM_PLAN_KSPLIT;
+    }
+    *param = groups;
+    return groups > 1 ? RMI_HIP_GEMM_PLAN_TILED_GROUPS : RMI_HIP_GEMM_PLAN_TILED_SINGLE_CHAIN;
+}
+
+int rmi_hip_gemm_q8_0_fast_plan(const rmi_hip_weight *w, uint32_t n_tokens, uint32_t *param) {
+    uint32_t dummy = 0;
+    if (!w || w->dtype != RMI_HIP_DTYPE_Q8_0 || n_tokens == 0 || w->n_out == 0 || w->n_in < 32) {
+        if (param) *param = 1;
+        return RMI_HIP_GEMM_PLAN_TILED_SINGLE_CHAIN;
+    }
+    return fast_plan(w, n_tokens, param ? param : &dummy);
+}
+
 int rmi_hip_gemm_q8_0_fast_dev(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                                uint32_t n_tokens, uint32_t y_stride, void *stream) {
     RMI_REQUIRE_INIT();
@@ -392,10 +415,11 @@ int rmi_hip_gemm_q8_0_fast_dev(const rmi_hip_weight *w, const int8_t *x_q8, cons
     if (y_stride < w->n_out) return rmi_fail(RMI_HIP_E_INVALID, "y_stride=%u < n_out=%u", y_stride, w->n_out);
     if (!x_q8 || !x_scales || !y) return rmi_fail(RMI_HIP_E_INVALID, "null device pointer");
     if (rmi_misaligned(x_q8, x_scales, y)) return rmi_fail(RMI_HIP_E_INVALID, RMI_ALIGNMENT_MESSAGE);
-    const double tiled = rmi_gemm_q8_0_cost_us(w, n_tokens);
-    if (tiled < 0.0 || rmi_gemm_q8_0_ksplit_cost_us(w, n_tokens) < tiled)
+    if (w->n_in < 32) return rmi_fail(RMI_HIP_E_INVALID, "GEMM needs at least one block per row");
+    uint32_t param = 1;
+    if (fast_plan(w, n_tokens, &param) == RMI_HIP_GEMM_PLAN_KSPLIT)
         return rmi_launch_gemm_q8_0_ksplit(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
-    return rmi_launch_gemm_q8_0(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
+    return rmi_launch_gemm_q8_0_grouped(w, x_q8, x_scales, y, n_tokens, y_stride, static_cast<hipStream_t>(stream));
 }
 
 uint32_t rmi_hip_gemm_q8_0_ksplit_quads_per_part(uint32_t n_in) {

@@ -70,8 +70,14 @@ __device__ __forceinline__ uint32_t voff(uint32_t &o) {
 // 16-byte aligned; token scales are then read one by one and indices past the row end are clamped.
 // PER_CU bounds the registers a thread may take: it is the number of waves that are to share a SIMD (the second
 // argument of __launch_bounds__), which for these four-wave workgroups is also the workgroups per compute unit.
-template <int NTW, int TTW, int WN, int WT, int PER_CU, bool RAGGED>
-__global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ x_q8,
+// KS > 1 (not the aarch64 order any more, see rmi_launch_gemm_q8_0_fast): KS groups of WN x WT waves share the tile;
+// group ks takes the quads ks, ks + KS, ks + 2 KS, ... (n_in / 128 must be a multiple of KS), stages them in LDS of
+// its own and keeps its own f32 chain per output; at the end the groups' sums are added in group order.  With a
+// single workgroup per compute unit this puts two or four waves on every SIMD where the tile grid has only as many
+// tiles as the chip has compute units, and a compute unit draws only so many bytes a microsecond: fewer, larger
+// tiles per unit are what a product of a few hundred tokens needs.
+template <int NTW, int TTW, int WN, int WT, int PER_CU, bool RAGGED, int KS = 1>
+__global__ __launch_bounds__(64 * WN * WT * KS, PER_CU) void gemm_q8_0_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ x_q8,
                                                                  const float *__restrict__ x_scales, float *__restrict__ y,
                                                                  uint32_t n_out, uint32_t n_in, uint32_t n_oct,
                                                                  uint32_t n_tiles, uint32_t n_tokens, uint32_t y_stride,
@@ -84,16 +90,23 @@ __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const u
     constexpr int kSub = NTW * TTW, kSteps = 4 * kSub;
     constexpr int kPieces = kWPieces + kXPieces;
     constexpr int kWBuf = kTileN * kRowStride, kXBuf = kTileT * kRowStride;
-    __shared__ __attribute__((aligned(16))) uint8_t sm_w[2 * kWBuf];
-    __shared__ __attribute__((aligned(16))) uint8_t sm_x[2 * kXBuf];
+    static_assert(KS == 1 || !RAGGED, "the quads of a ragged row are not split");
+    static_assert(KS == 1 || (KS - 1) * kTileT * 4 <= KS * 2 * kRowStride, "the groups' sums meet in the weight buffers");
+    __shared__ __attribute__((aligned(16))) uint8_t sm_w_all[KS * 2 * kWBuf];
+    __shared__ __attribute__((aligned(16))) uint8_t sm_x_all[KS * 2 * kXBuf];
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = uint32_t(__builtin_amdgcn_readfirstlane(int(tid >> 6)));
+    // ks: this wave's group; tid, wave: position inside the group (a group is what the whole workgroup is for KS = 1)
+    const uint32_t ks = KS == 1 ? 0u : uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x / kThreads)));
+    uint8_t *const sm_w = sm_w_all + ks * 2 * kWBuf, *const sm_x = sm_x_all + ks * 2 * kXBuf;
+    const uint32_t tid = KS == 1 ? threadIdx.x : threadIdx.x % kThreads, lane = tid & 63,
+                   wave = uint32_t(__builtin_amdgcn_readfirstlane(int(tid >> 6)));
     const uint32_t c = lane & 31, h = lane >> 5;
     const uint32_t n_off = (wave % WN) * 32 * NTW, t_off = (wave / WN) * 32 * TTW;
     uint32_t n_tile, t_tile;  // one XCD's workgroups take neighbouring tiles
     rmi_gemm_tile_of(blockIdx.x, grid_n, grid_t, t_fastest, xcd_split, n_tile, t_tile);
     const uint32_t n0 = n_tile * kTileN, t0 = t_tile * kTileT;
-    const uint32_t nb = n_in >> 5, n_quads = (nb + 3) >> 2;
+    const uint32_t nb = n_in >> 5, n_quads = ((nb + 3) >> 2) / KS;  // quads of this group: q stands for quad q * KS + ks
+    auto realq = [&](uint32_t q) __attribute__((always_inline)) { return KS == 1 ? q : q * KS + ks; };
     const uint32_t t_last = n_tokens - 1 - t0;  // last token of the input, counted from this tile's first
 
     // ---- addresses: a workgroup-uniform base that moves with the quad, plus a 32-bit offset per thread.
@@ -146,14 +159,14 @@ __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const u
     };
     auto load_piece = [&](Stage &g, int pc, uint32_t q) __attribute__((always_inline)) {
         if (pc < kWPieces) {
-            g.w[pc] = *(gptr_u4)(sbase(wq_base + size_t(q) * 1024) + voff(w_off[pc]));
+            g.w[pc] = *(gptr_u4)(sbase(wq_base + size_t(realq(q)) * 1024) + voff(w_off[pc]));
         } else {
             const int i = pc - kWPieces;
             if (RAGGED) {
                 const uint32_t off = x_off[i] + q * 128;
                 g.x[i] = *reinterpret_cast<const u32x4 *>(x_base + (off < x_lim ? off : x_lim));
             } else {
-                g.x[i] = *(gptr_u4)(sbase(x_base + size_t(q) * 128) + voff(x_off[i]));
+                g.x[i] = *(gptr_u4)(sbase(x_base + size_t(realq(q)) * 128) + voff(x_off[i]));
             }
         }
     };
@@ -169,7 +182,8 @@ __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const u
             *reinterpret_cast<u32x4 *>(sm_x + buf * kXBuf + x_dst[i]) = g.x[i];
         }
     };
-    auto load_scales = [&](Scales &sc, uint32_t q) __attribute__((always_inline)) {
+    auto load_scales = [&](Scales &sc, uint32_t q_group) __attribute__((always_inline)) {
+        const uint32_t q = realq(q_group);
         // weight scales of padded blocks are zero in the stream; token scales past n_in/32 are not there
         const gptr_u8 wb = sbase(w_base + ((q >> 1) * 128 + (q & 1) * 8));
 #pragma unroll
@@ -342,6 +356,7 @@ __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const u
             v16f a = zero16f;
 #pragma unroll 1
             for (uint32_t b = 0; b < nb; b++) {
+                if (KS > 1 && (b >> 2) % KS != ks) continue;  // another group's quad
                 const uint8_t *wp = w_row + size_t(b >> 2) * 1024 + (b & 3) * 4;
                 const v4i wo = {int(*reinterpret_cast<const uint32_t *>(wp)), int(*reinterpret_cast<const uint32_t *>(wp + 16)),
                                 int(*reinterpret_cast<const uint32_t *>(wp + 32)), int(*reinterpret_cast<const uint32_t *>(wp + 48))};
@@ -364,6 +379,31 @@ __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const u
         }
     }
 
+    if constexpr (KS > 1) {
+        // the groups' sums: groups 1.. leave theirs in LDS, group 0 adds them in group order and stores
+        __syncthreads();  // nobody reads a staging buffer any more
+        float *comb = reinterpret_cast<float *>(sm_w_all);
+        if (ks != 0) {
+#pragma unroll
+            for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+                for (int tt = 0; tt < TTW; tt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++)
+                        comb[((((ks - 1) * WN * WT + wave) * kSub + nt * TTW + tt) * 16 + i) * 64 + lane] = acc[nt][tt][i];
+        }
+        __syncthreads();
+        if (ks != 0) return;
+#pragma unroll 1
+        for (uint32_t g = 1; g < KS; g++)
+#pragma unroll
+            for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+                for (int tt = 0; tt < TTW; tt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++)
+                        acc[nt][tt][i] += comb[((((g - 1) * WN * WT + wave) * kSub + nt * TTW + tt) * 16 + i) * 64 + lane];
+    }
     // ---- results: lane (c, h) holds row n = c of 16 tokens
     const uint32_t t_w = t0 + t_off, n_w = n0 + n_off;
     if (t_w + 32 * TTW <= n_tokens && n_w + 32 * NTW <= n_out) {
@@ -399,41 +439,45 @@ __global__ __launch_bounds__(64 * WN * WT, PER_CU) void gemm_q8_0_kernel(const u
 typedef void (*GemmLaunch)(const rmi_hip_weight *, const int8_t *, const float *, float *, uint32_t, uint32_t, bool,
                            hipStream_t);
 
-template <int NTW, int TTW, int WN, int WT, int PER_CU>
+template <int NTW, int TTW, int WN, int WT, int PER_CU, int KS>
 void launch_gemm(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
                  uint32_t y_stride, bool ragged, hipStream_t s) {
     constexpr uint32_t tile_n = 32 * NTW * WN, tile_t = 32 * TTW * WT;
     const uint32_t grid_n = (w->n_out + tile_n - 1) / tile_n, grid_t = (n_tokens + tile_t - 1) / tile_t;
     const uint32_t xcd_split = rmi_gemm_xcd_split(grid_n, grid_t, double(w->n_out) * w->n_in * (34.0 / 32.0), double(n_tokens) * w->n_in * (36.0 / 32.0));
-    if (ragged)
-        hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, PER_CU, true>), dim3(grid_n * grid_t), dim3(64 * WN * WT), 0, s,
-                           w->data, x_q8, x_scales, y, w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride,
-                           grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
-    else
-        hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, PER_CU, false>), dim3(grid_n * grid_t), dim3(64 * WN * WT), 0, s,
-                           w->data, x_q8, x_scales, y, w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride,
-                           grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
+    if constexpr (KS == 1) {
+        if (ragged) {
+            hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, PER_CU, true>), dim3(grid_n * grid_t), dim3(64 * WN * WT), 0, s,
+                               w->data, x_q8, x_scales, y, w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride,
+                               grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((gemm_q8_0_kernel<NTW, TTW, WN, WT, PER_CU, false, KS>), dim3(grid_n * grid_t), dim3(64 * WN * WT * KS), 0, s,
+                       w->data, x_q8, x_scales, y, w->n_out, w->n_in, w->n_units, w->n_tiles, n_tokens, y_stride,
+                       grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
 }
 
-// A tile shape: rows x tokens of a workgroup, sub-tiles per wave, waves, how many workgroups a compute unit holds
-// at once (asked of the runtime once: it knows the registers and the LDS the compiled kernel takes).
+// A tile shape: rows x tokens of a workgroup, sub-tiles per wave, waves of a group, groups that split the quads, how
+// many workgroups a compute unit holds at once (asked of the runtime once: it knows the registers and the LDS the
+// compiled kernel takes).
 struct GemmShape {
-    uint32_t tile_n, tile_t, sub, waves;
+    uint32_t tile_n, tile_t, sub, waves, ks;
     int per_cu;
     GemmLaunch launch;
 };
 
-template <int NTW, int TTW, int WN, int WT, int PER_CU>
+template <int NTW, int TTW, int WN, int WT, int PER_CU, int KS = 1>
 GemmShape make_shape() {
     int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_q8_0_kernel<NTW, TTW, WN, WT, PER_CU, false>, 64 * WN * WT, 0) !=
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_q8_0_kernel<NTW, TTW, WN, WT, PER_CU, false, KS>, 64 * WN * WT * KS, 0) !=
             hipSuccess ||
         per_cu < 1) {
         (void)hipGetLastError();
         per_cu = 1;
     }
-    return GemmShape{32u * NTW * WN, 32u * TTW * WT, uint32_t(NTW * TTW), uint32_t(WN * WT), per_cu,
-                     launch_gemm<NTW, TTW, WN, WT, PER_CU>};
+    return GemmShape{32u * NTW * WN, 32u * TTW * WT, uint32_t(NTW * TTW), uint32_t(WN * WT), uint32_t(KS), per_cu,
+                     launch_gemm<NTW, TTW, WN, WT, PER_CU, KS>};
 }
 
 }  // namespace
@@ -449,24 +493,40 @@ struct GemmPlan {
 // share it, so a launch takes about (waves on the busiest SIMD) x (sub-tiles per wave) steps per block, round
 // after round of workgroups, plus a fixed cost per round (first loads, last stores).  Measured on MI355X, a
 // step: 90 ns with three or more waves on the SIMD or several sub-tiles per wave, 105 ns with two waves of one
-// sub-tile, 125 ns for a wave alone; a round: about 3.5 us.  The shape with the smallest estimate is taken,
-// the larger tile on a tie (less traffic): 96x128 (4 waves x 3 sub-tiles, two workgroups a compute unit) for
-// large products, 64x128 and 64x64 where those would leave compute units idle.
-GemmPlan plan_gemm(const rmi_hip_weight *w, uint32_t n_tokens) {
-    static const GemmShape shapes[] = {make_shape<3, 1, 1, 4, 2>(), make_shape<2, 1, 1, 4, 2>(), make_shape<1, 1, 2, 2, 3>()};
+// sub-tile, 125 ns for a wave alone; a round: about 3.5 us.  A compute unit also draws only about 40 KB a
+// microsecond from L2 and memory, whatever its waves do, so a round takes at least its workgroups' operand bytes at
+// that rate.  The shape with the smallest estimate is taken, the larger tile on a tie (less traffic): 96x128
+// (4 waves x 3 sub-tiles, two workgroups a compute unit) for large products, 64x128 and 64x64 where those would
+// leave compute units idle.  single_chain: only the shapes that keep one f32 chain per output.
+GemmPlan plan_gemm(const rmi_hip_weight *w, uint32_t n_tokens, bool single_chain) {
+    static const GemmShape shapes[] = {make_shape<3, 1, 1, 4, 2>(),    make_shape<2, 1, 1, 4, 2>(),    make_shape<1, 1, 2, 2, 3>(),
+                                       make_shape<3, 1, 1, 4, 2, 2>(), make_shape<2, 1, 1, 4, 2, 2>(), make_shape<1, 1, 2, 2, 2, 2>()};
     const uint64_t cus = uint64_t(rmi_device_cus() > 0 ? rmi_device_cus() : 1);
-    const double nb = double(w->n_in / 32);
+    const uint32_t n_quads = (w->n_in / 32 + 3) / 4;
+    const bool whole_quads = (w->n_in / 32) % 4 == 0;
     GemmPlan best{nullptr, 0.0};
+    static const int forced = [] {  // measurements only: RMI_GEMM_SHAPE = index into the table above
+        const char *e = getenv("RMI_GEMM_SHAPE");
+        return e ? atoi(e) : -1;
+    }();
     for (const GemmShape &g : shapes) {
+        if (forced >= 0 && !single_chain && &g != &shapes[forced % 6]) continue;
+        // groups pay off on long rows only (measured: 1024 x 3072 gains 10-15 % from 768 tokens on, 3072 x 1024 loses
+        // 3-10 %: a group needs about eight quads to make up for its own first loads and the last add)
+        if (g.ks > 1 && (single_chain || !whole_quads || n_quads % g.ks != 0 || n_quads / g.ks < 8)) continue;
         const uint64_t groups = uint64_t((w->n_out + g.tile_n - 1) / g.tile_n) * ((n_tokens + g.tile_t - 1) / g.tile_t);
         if (groups > 0x7fffffffull) continue;
+        const double nb = double(w->n_in / 32) / double(g.ks);
         const uint64_t at_once = cus * uint64_t(g.per_cu);
         const uint64_t full = groups / at_once, rest = groups % at_once;
-        const uint64_t per_simd = (g.waves + 3) / 4;  // a workgroup's waves spread over the four SIMDs of its compute unit
+        const uint64_t per_simd = (g.waves * g.ks + 3) / 4;  // a workgroup's waves spread over the four SIMDs of its compute unit
+        const double wg_kb = double(g.tile_n + g.tile_t) * double(w->n_in) * (35.0 / 32.0) * 1e-3;
         auto round_us = [&](uint64_t groups_per_cu) __attribute__((always_inline)) {
             const uint64_t wps = groups_per_cu * per_simd;
             const double step_ns = wps == 1 ? 125.0 : (wps >= 3 || g.sub >= 2) ? 90.0 : 105.0;
-            return double(wps * g.sub) * nb * step_ns * 1e-3 + 3.5;
+            const double valu = double(wps * g.sub) * nb * step_ns * 1e-3;
+            const double mem = single_chain ? 0.0 : double(groups_per_cu) * wg_kb / 40.0;
+            return (valu > mem ? valu : mem) + 3.5 + (g.ks > 1 ? 0.5 : 0.0);
         };
         double cost = double(full) * round_us(uint64_t(g.per_cu));
         if (rest) cost += round_us((rest + cus - 1) / cus);
@@ -477,21 +537,38 @@ GemmPlan plan_gemm(const rmi_hip_weight *w, uint32_t n_tokens) {
 
 }  // namespace
 
-// the launch time the tile chooser expects for this product, in microseconds (a negative value: no shape fits)
-double rmi_gemm_q8_0_cost_us(const rmi_hip_weight *w, uint32_t n_tokens) {
+// the launch time the tile chooser expects for this product, in microseconds (a negative value: no shape fits), and
+// the number of groups that split the quads in the shape it takes
+double rmi_gemm_q8_0_cost_us(const rmi_hip_weight *w, uint32_t n_tokens, bool single_chain, uint32_t *groups) {
+    if (groups) *groups = 1;
     if (n_tokens == 0 || w->n_out == 0 || w->n_in < 32) return 0.0;
-    const GemmPlan plan = plan_gemm(w, n_tokens);
+    const GemmPlan plan = plan_gemm(w, n_tokens, single_chain);
+    if (plan.shape && groups) *groups = plan.shape->ks;
     return plan.shape ? plan.cost_us : -1.0;
 }
 
-int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
-                         uint32_t n_tokens, uint32_t y_stride, hipStream_t s) {
+static int launch_planned(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y, uint32_t n_tokens,
+                          uint32_t y_stride, bool single_chain, hipStream_t s) {
     if (n_tokens == 0 || w->n_out == 0) return RMI_HIP_OK;
     if (w->n_in < 32) return rmi_fail(RMI_HIP_E_INVALID, "GEMM needs at least one block per row");
-    const GemmPlan plan = plan_gemm(w, n_tokens);
+    const GemmPlan plan = plan_gemm(w, n_tokens, single_chain);
     if (!plan.shape) return rmi_fail(RMI_HIP_E_INVALID, "GEMM too large for one launch");
     const bool ragged = (w->n_in / 32) % 4 != 0 || (reinterpret_cast<uintptr_t>(x_scales) & 15) != 0;
+    if (ragged && plan.shape->ks > 1) return launch_planned(w, x_q8, x_scales, y, n_tokens, y_stride, true, s);  // unaligned scales
     plan.shape->launch(w, x_q8, x_scales, y, n_tokens, y_stride, ragged, s);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
+}
+
+// one f32 chain per output in block order: the aarch64 kernel's result bit for bit
+int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                         uint32_t n_tokens, uint32_t y_stride, hipStream_t s) {
+    return launch_planned(w, x_q8, x_scales, y, n_tokens, y_stride, true, s);
+}
+
+// the tiled kernel with the quads of a row split over two or four groups of waves where the chooser expects that to
+// be faster: a chain per group, the groups' sums added in group order (within rounding of the single chain)
+int rmi_launch_gemm_q8_0_grouped(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
+                                 uint32_t n_tokens, uint32_t y_stride, hipStream_t s) {
+    return launch_planned(w, x_q8, x_scales, y, n_tokens, y_stride, false, s);
 }

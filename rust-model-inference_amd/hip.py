@@ -106,6 +106,7 @@ SIGNATURES = {
     "rmi_hip_gemm_q4_k_q8k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemm_q8_0_ksplit_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
     "rmi_hip_gemm_q8_0_fast_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _vp]),
+    "rmi_hip_gemm_q8_0_fast_plan": (C.c_int, [_vp, _u32, C.POINTER(_u32)]),
     "rmi_hip_gemm_q8_0_ksplit_quads_per_part": (_u32, [_u32]),
     "rmi_hip_gemm_block_ints_q4_k_dev": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp]),
     "rmi_hip_gemv_q4_0_dev": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),

@@ -120,10 +120,14 @@ def test_ksplit_special_scales(hip, oracle):
     assert np.array_equal(bits(got)[~nan_g], bits(want)[~nan_w])
 
 
-@pytest.mark.parametrize("n_tokens,n_out,n_in", [(64, 1024, 3072), (512, 3072, 1024), (256, 1024, 3072), (2048, 3072, 1024)])
-def test_fast_entry_runs_one_of_the_two_kernels(hip, oracle, n_tokens, n_out, n_in):
-    """rmi_hip_gemm_q8_0_fast_dev picks a kernel per product: its output is, bit for bit, that of the k-split kernel
-    or that of the tiled kernel, and within tolerance of the x86-64 order on sampled tokens either way."""
+@pytest.mark.parametrize("n_tokens,n_out,n_in", [(64, 1024, 3072), (512, 3072, 1024), (512, 1024, 3072), (256, 1024, 3072),
+                                                  (2048, 3072, 1024), (2048, 1024, 3072), (300, 520, 1024), (200, 260, 1120)])
+def test_fast_entry_follows_its_plan(hip, oracle, n_tokens, n_out, n_in):
+    """rmi_hip_gemm_q8_0_fast_dev picks a kernel per product and rmi_hip_gemm_q8_0_fast_plan names it: sampled token
+    rows equal, bit for bit, the checker's statement of that plan (the single chain, the chain cut into runs of quads,
+    or interleaved groups of quads), every sampled row is within tolerance of both CPU orders, and a second call
+    gives the same bits."""
+    import ctypes as C
     H = hip.hip
     w = hip.synth.q8_0_weight(5300 + n_tokens, n_out, n_in)
     x = hip.synth.activations(5301 + n_tokens, n_tokens, n_in)
@@ -131,21 +135,29 @@ def test_fast_entry_runs_one_of_the_two_kernels(hip, oracle, n_tokens, n_out, n_
     d_x = H.DeviceBuffer.from_array(H.as_f32(x))
     d_q8, d_sc = H.DeviceBuffer(n_tokens * n_in), H.DeviceBuffer(n_tokens * (n_in // 32) * 4)
     H.check(H.lib.rmi_hip_quantize_q8_0_dev(d_x.ptr, d_q8.ptr, d_sc.ptr, n_tokens, n_in, H.ROUND_TIES_EVEN, None))
-    outs = {}
-    for name in ("fast", "ksplit", "tiled"):
-        fn = {"fast": H.lib.rmi_hip_gemm_q8_0_fast_dev, "ksplit": H.lib.rmi_hip_gemm_q8_0_ksplit_dev,
-              "tiled": H.lib.rmi_hip_gemm_q8_0_dev}[name]
+    param = C.c_uint32(0)
+    plan = H.lib.rmi_hip_gemm_q8_0_fast_plan(kernel.w.handle, n_tokens, C.byref(param))
+    print(f"fast plan for {n_tokens} x {n_out}x{n_in}: kind {plan}, param {param.value}", flush=True)
+    outs = []
+    for _ in range(2):
         d_y = H.DeviceBuffer.from_array(np.full(n_tokens * n_out, np.nan, np.float32))
-        H.check(fn(kernel.w.handle, d_q8.ptr, d_sc.ptr, d_y.ptr, n_tokens, n_out, None))
+        H.check(H.lib.rmi_hip_gemm_q8_0_fast_dev(kernel.w.handle, d_q8.ptr, d_sc.ptr, d_y.ptr, n_tokens, n_out, None))
         H.check(H.lib.rmi_hip_synchronize())
-        outs[name] = d_y.to_array(np.float32, (n_tokens, n_out))
+        outs.append(d_y.to_array(np.float32, (n_tokens, n_out)))
         d_y.free()
-    assert np.array_equal(bits(outs["fast"]), bits(outs["ksplit"])) or np.array_equal(bits(outs["fast"]), bits(outs["tiled"]))
+    assert np.array_equal(bits(outs[0]), bits(outs[1])) and not np.isnan(outs[0]).any()
     q8 = d_q8.to_array(np.uint8, (n_tokens, n_in))
     sc = d_sc.to_array(np.float32, (n_tokens, n_in // 32))
-    for t in (0, n_tokens // 2, n_tokens - 1):
-        ref = oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, A)
-        for name in ("fast", "ksplit", "tiled"):
-            assert np.all(np.abs(outs[name][t] - ref) <= TOL(ref)), (name, t)
+    for t in sorted({0, 1, 31, 32, 63, min(64, n_tokens - 1), n_tokens // 2, n_tokens - 2, n_tokens - 1}):
+        if plan == 2:
+            want = oracle.matmul_q8_0_neon_split(w, q8[t], sc[t], n_in, n_out, param.value)
+        elif plan == 1:
+            want = oracle.matmul_q8_0_neon_interleaved(w, q8[t], sc[t], n_in, n_out, param.value)
+        else:
+            want = oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, N)
+        assert np.array_equal(bits(outs[0][t]), bits(want)), t
+        for variant in (A, N):
+            ref = oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, variant)
+            assert np.all(np.abs(outs[0][t] - ref) <= TOL(ref)), (variant, t)
     for b in (d_x, d_q8, d_sc):
         b.free()

@@ -326,3 +326,9 @@ def test_neon_split_chain_is_the_neon_chain_for_one_part_and_within_tolerance_fo
             assert np.all(np.abs(y - ref) <= 1e-4 + 1e-4 * np.abs(ref))
         differs |= not np.array_equal(bits(y), bits(neon))
     assert differs
+    assert np.array_equal(bits(oracle.matmul_q8_0_neon_interleaved(w, q8, sc, n_in, n_out, 1)), bits(neon))
+    for groups in (2, 4):
+        y = oracle.matmul_q8_0_neon_interleaved(w, q8, sc, n_in, n_out, groups)
+        for ref in (neon, avx2):
+            assert np.all(np.abs(y - ref) <= 1e-4 + 1e-4 * np.abs(ref))
+        assert not np.array_equal(bits(y), bits(neon))
