@@ -109,8 +109,12 @@ __device__ __forceinline__ uint32_t bytes_to_f16_pair(uint32_t w) {
 // DUMP (parity only): instead of folding them, the kernel writes the integers of every super-block as they leave
 // the matrix cores, sumi = 8 * D_hi + D_lo and prod (the min term's f16 MFMA result, an integer below 2^24), to
 // reinterpret_cast<int32_t *>(y)[((t * n_out + n) * n_sb + sb) * 2 + {0, 1}].
-template <int TTW, int WAVES_PER_SIMD, bool DUMP>
-__global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const uint8_t *__restrict__ w, const float *__restrict__ q8d,
+// KS > 1: KS groups of four waves share the tile; group ks takes the super-blocks ks, ks + KS, ... (n_in / 256 must
+// be a multiple of KS), stages them in LDS of its own and keeps its own f32 chains; at the end the groups' results
+// are added in group order.  For launches with no more tiles than the chip has compute units (a long row, a few
+// hundred tokens): eight waves a compute unit instead of four, and half as many super-blocks in sequence.
+template <int TTW, int WAVES_PER_SIMD, bool DUMP, int KS = 1>
+__global__ __launch_bounds__(256 * KS, WAVES_PER_SIMD) void gemm_q4_k_kernel(const uint8_t *__restrict__ w, const float *__restrict__ q8d,
                                                                          const int8_t *__restrict__ q8qs,
                                                                          const int16_t *__restrict__ q8bs, float *__restrict__ y,
                                                                          uint32_t n_out, uint32_t n_sb, uint32_t n_tiles,
@@ -120,18 +124,24 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     constexpr int kXPieces = kTileT * 16 / 256;  // 16-byte pieces of the token tile per thread and super-block
     constexpr int kXBuf = kTileT * kXRow, kBBuf = kTileT * kBRow, kWBuf = kTileN * kWRow;
     static_assert(kXPieces <= 4, "the token pieces move to LDS in the first four calls of a super-block");
-    __shared__ __attribute__((aligned(16))) uint8_t sm_w[2 * kWBuf];
-    __shared__ __attribute__((aligned(16))) uint8_t sm_x[2 * kXBuf];
-    __shared__ __attribute__((aligned(16))) uint8_t sm_b[2 * kBBuf];
+    __shared__ __attribute__((aligned(16))) uint8_t sm_w_all[KS * 2 * kWBuf];
+    __shared__ __attribute__((aligned(16))) uint8_t sm_x_all[KS * 2 * kXBuf];
+    __shared__ __attribute__((aligned(16))) uint8_t sm_b_all[KS * 2 * kBBuf];
+    static_assert(KS == 1 || (KS - 1) * kTileT * 4 <= KS * 2 * kWRow, "the groups' results meet in the weight buffers");
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = uint32_t(__builtin_amdgcn_readfirstlane(int(tid >> 6)));
+    // ks: this wave's group; tid, wave: position inside the group (the whole workgroup for KS = 1)
+    const uint32_t ks = KS == 1 ? 0u : uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x >> 8)));
+    uint8_t *const sm_w = sm_w_all + ks * 2 * kWBuf, *const sm_x = sm_x_all + ks * 2 * kXBuf, *const sm_b = sm_b_all + ks * 2 * kBBuf;
+    const uint32_t tid = threadIdx.x & 255, lane = tid & 63, wave = uint32_t(__builtin_amdgcn_readfirstlane(int(tid >> 6)));
     const uint32_t c = lane & 31, h = lane >> 5;
     const uint32_t n_off = wave * 32;
     uint32_t n_tile, t_tile;  // one XCD's workgroups take neighbouring tiles
     rmi_gemm_tile_of(blockIdx.x, grid_n, grid_t, t_fastest, xcd_split, n_tile, t_tile);
     const uint32_t n0 = n_tile * kTileN, t0 = t_tile * kTileT;
     const uint32_t n_in = n_sb * 256;
-    const uint32_t sb_last = n_sb - 1;
+    // super-blocks of this group: sb stands for super-block sb * KS + ks
+    const uint32_t n_sb_group = n_sb / KS, sb_last = n_sb_group - 1;
+    auto realsb = [&](uint32_t sb) __attribute__((always_inline)) { return KS == 1 ? sb : sb * KS + ks; };
     auto clampsb = [&](uint32_t sb) __attribute__((always_inline)) { return sb < sb_last ? sb : sb_last; };
 
     // ---- addresses: a workgroup-uniform base that moves with the super-block, plus a 32-bit offset per thread.
@@ -194,16 +204,16 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     float wd;
 
     auto load_w = [&](int i, uint32_t sb) __attribute__((always_inline)) {
-        wst[i] = *(gptr_u4)(sbase(w_base + size_t(sb) * kQ4KSuperBytes + w_tile_off[i]) + voff(w_ld));
+        wst[i] = *(gptr_u4)(sbase(w_base + size_t(realsb(sb)) * kQ4KSuperBytes + w_tile_off[i]) + voff(w_ld));
     };
     auto store_w = [&](int i, int buf) __attribute__((always_inline)) {
         *reinterpret_cast<u32x4 *>(sm_w + buf * kWBuf + w_dst + i * 32 * kWRow) = wst[i];
     };
     auto load_hdr = [&](uint32_t sb) __attribute__((always_inline)) {
-        hdr_n = *(gptr_u4)(sbase(w_base + size_t(sb) * kQ4KSuperBytes) + voff(hd_off));
+        hdr_n = *(gptr_u4)(sbase(w_base + size_t(realsb(sb)) * kQ4KSuperBytes) + voff(hd_off));
 #pragma unroll
         for (int tt = 0; tt < TTW; tt++)
-            xd_n[tt] = __builtin_bit_cast(float, *(gptr_u32)(sbase(d_base + size_t(sb) * 4) + voff(d_off[tt])));
+            xd_n[tt] = __builtin_bit_cast(float, *(gptr_u32)(sbase(d_base + size_t(realsb(sb)) * 4) + voff(d_off[tt])));
     };
     auto take_hdr = [&]() __attribute__((always_inline)) {
         const uint4 s8 = unpack_scales(hdr_n.y, hdr_n.z, hdr_n.w);
@@ -220,7 +230,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     auto load_x = [&](int i, uint32_t sb) __attribute__((always_inline)) {
         uint32_t off = x_off + uint32_t(i) * 16 * n_in;
         off = off < x_lim ? off : x_lim;
-        xst[i] = *(gptr_u4)(sbase(x_base + size_t(sb) * 256) + voff(off));
+        xst[i] = *(gptr_u4)(sbase(x_base + size_t(realsb(sb)) * 256) + voff(off));
     };
     auto store_x = [&](int i, int buf) __attribute__((always_inline)) {
         uint8_t *dst = sm_x + buf * kXBuf + x_dst + i * 16 * kXRow;
@@ -231,7 +241,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     };
     auto load_bs = [&](uint32_t sb) __attribute__((always_inline)) {
 #pragma unroll
-        for (int tt = 0; tt < TTW; tt++) bst[tt] = *(gptr_u32)(sbase(bs_base + size_t(sb) * 32) + voff(bs_off[tt]));
+        for (int tt = 0; tt < TTW; tt++) bst[tt] = *(gptr_u32)(sbase(bs_base + size_t(realsb(sb)) * 32) + voff(bs_off[tt]));
     };
     auto store_bs = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -364,7 +374,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
                 for (int i = 0; i < 16; i++) {
                     const uint32_t t = t0 + tt * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
                     if (n < n_out && t < n_tokens) {
-                        int32_t *dst = reinterpret_cast<int32_t *>(y) + ((size_t(t) * n_out + n) * n_sb + sb) * 2;
+                        int32_t *dst = reinterpret_cast<int32_t *>(y) + ((size_t(t) * n_out + n) * n_sb + realsb(sb)) * 2;
                         dst[0] = d_hi[tt][i] * 8 + d_lo[tt][i];
                         dst[1] = int32_t(pm[i]);
                     }
@@ -386,11 +396,38 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     };
 
     uint32_t sb = 0;
-    for (; sb + 1 < n_sb; sb += 2) {
+    for (; sb + 1 < n_sb_group; sb += 2) {
         stage(sb, std::integral_constant<int, 0>{});
         stage(sb + 1, std::integral_constant<int, 1>{});
     }
-    if (sb < n_sb) stage(sb, std::integral_constant<int, 0>{});
+    if (sb < n_sb_group) stage(sb, std::integral_constant<int, 0>{});
+    if constexpr (KS > 1) {
+        // the groups' results (their two chains added): groups 1.. leave theirs in LDS, group 0 adds them in group
+        // order and stores
+        __syncthreads();  // the loop ends with reads ahead into the buffers; they are over before the results land there
+        float *comb = reinterpret_cast<float *>(sm_w_all);
+#pragma unroll
+        for (int tt = 0; tt < TTW; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[tt][i] += acc_m[tt][i];
+        if (ks != 0) {
+#pragma unroll
+            for (int tt = 0; tt < TTW; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) comb[((((ks - 1) * 4 + wave) * TTW + tt) * 16 + i) * 64 + lane] = acc[tt][i];
+        }
+        __syncthreads();
+        if (ks != 0) return;
+#pragma unroll 1
+        for (uint32_t g = 1; g < KS; g++)
+#pragma unroll
+            for (int tt = 0; tt < TTW; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    acc[tt][i] += comb[((((g - 1) * 4 + wave) * TTW + tt) * 16 + i) * 64 + lane];
+                    acc_m[tt][i] = 0.0f;
+                }
+    }
     // ---- results: lane (c, h) holds row n = c of 16 tokens
     const uint32_t n = n0 + n_off + c;
     if (!DUMP && n < n_out) {
@@ -404,16 +441,28 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void gemm_q4_k_kernel(const ui
     }
 }
 
-template <int TTW, int WAVES_PER_SIMD, bool DUMP = false>
+template <int TTW, int WAVES_PER_SIMD, bool DUMP = false, int KS = 1>
 void launch(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int16_t *bs, float *y, uint32_t n_tokens,
             uint32_t y_stride, hipStream_t s) {
     const uint32_t grid_n = (w->n_out + 127) / 128, grid_t = (n_tokens + 32 * TTW - 1) / (32 * TTW);
     const uint32_t xcd_split = rmi_gemm_xcd_split(grid_n, grid_t, double(w->n_out) * w->n_units * 144.0, double(n_tokens) * w->n_units * 292.0);
-    hipLaunchKernelGGL((gemm_q4_k_kernel<TTW, WAVES_PER_SIMD, DUMP>), dim3(grid_n * grid_t), dim3(256), 0, s, w->data, d, qs, bs, y,
+    hipLaunchKernelGGL((gemm_q4_k_kernel<TTW, WAVES_PER_SIMD, DUMP, KS>), dim3(grid_n * grid_t), dim3(256 * KS), 0, s, w->data, d, qs, bs, y,
                        w->n_out, w->n_units, w->n_tiles, n_tokens, y_stride, grid_n, grid_t, n_tokens < w->n_out ? 1u : 0u, xcd_split);
 }
 
 }  // namespace
+
+// Two groups of waves per tile, on the even and the odd super-blocks: where the 32-token tiles are no more than the
+// chip has compute units and each group still has eight super-blocks or more (measured at 2048 x 6144, 512 tokens:
+// 29.5 -> about 16 us).  RMI_Q4K_GEMM_GROUPS = 1 or 2 forces a count where the row allows it.
+static int gemm_q4_k_groups(const rmi_hip_weight *w, uint32_t n_tokens) {
+    const uint64_t groups32 = uint64_t((w->n_out + 127) / 128) * ((n_tokens + 31) / 32);
+    const char *e = getenv("RMI_Q4K_GEMM_GROUPS");
+    const int force = e ? atoi(e) : 0;
+    if (w->n_units % 2 != 0 || force == 1) return 1;
+    if (force == 2) return 2;
+    return groups32 <= uint64_t(rmi_device_cus()) && w->n_units >= 16 ? 2 : 1;
+}
 
 // token tile width (in units of 32) the launcher takes for this problem; RMI_Q4K_GEMM_TTW = 1 or 2 forces one
 static int gemm_q4_k_ttw(const rmi_hip_weight *w, uint32_t n_tokens) {
@@ -430,7 +479,9 @@ int rmi_launch_gemm_q4_k_block_ints(const rmi_hip_weight *w, const float *d, con
     if (n_tokens == 0 || w->n_out == 0 || w->n_units == 0) return RMI_HIP_OK;
     if (uint64_t((w->n_out + 127) / 128) * ((n_tokens + 31) / 32) > 0x7fffffffull)
         return rmi_fail(RMI_HIP_E_INVALID, "GEMM too large for one launch");
-    if (gemm_q4_k_ttw(w, n_tokens) == 2)
+    if (gemm_q4_k_groups(w, n_tokens) == 2)
+        launch<1, 2, true, 2>(w, d, qs, bsums, reinterpret_cast<float *>(ints), n_tokens, w->n_out, s);
+    else if (gemm_q4_k_ttw(w, n_tokens) == 2)
         launch<2, 2, true>(w, d, qs, bsums, reinterpret_cast<float *>(ints), n_tokens, w->n_out, s);
     else
         launch<1, 2, true>(w, d, qs, bsums, reinterpret_cast<float *>(ints), n_tokens, w->n_out, s);
@@ -445,7 +496,9 @@ int rmi_launch_gemm_q4_k(const rmi_hip_weight *w, const float *d, const int8_t *
     if (groups32 > 0x7fffffffull) return rmi_fail(RMI_HIP_E_INVALID, "GEMM too large for one launch");
     // 64-token tiles halve the vector work per output but want two workgroups on every compute unit;
     // RMI_Q4K_GEMM_TTW = 1 or 2 forces a width (the parity tests run both)
-    if (gemm_q4_k_ttw(w, n_tokens) == 2)
+    if (gemm_q4_k_groups(w, n_tokens) == 2)
+        launch<1, 2, false, 2>(w, d, qs, bsums, y, n_tokens, y_stride, s);
+    else if (gemm_q4_k_ttw(w, n_tokens) == 2)
         launch<2, 2>(w, d, qs, bsums, y, n_tokens, y_stride, s);
     else
         launch<1, 2>(w, d, qs, bsums, y, n_tokens, y_stride, s);

@@ -399,3 +399,33 @@ def test_q4k_gemm_block_ints_both_tile_widths_ragged_and_extreme(hip, oracle, mo
     for t in range(n_tokens):
         assert np.array_equal(ints[t], oracle.q4k_q8k_block_ints_matrix(wx.reshape(-1), n_out, qs[t], bs[t])), t
     assert np.abs(ints[..., 0]).max() == 256 * 15 * 63 * 127
+
+
+@pytest.mark.parametrize("groups", ["1", "2"])
+def test_q4k_gemm_groups_of_waves_on_alternate_super_blocks(hip, oracle, monkeypatch, groups):
+    """Long rows with few tiles run two groups of waves per tile, on the even and the odd super-blocks; forced either
+    way the per-super-block integers are the checker's, every output is within 1e-4 + 1e-4 |ref| of the AVX2-order
+    result and within 2e-6 of the f64 sum over the exact integers; ragged row and token tiles included."""
+    monkeypatch.setenv("RMI_Q4K_GEMM_GROUPS", groups)
+    for n_tokens, n_out, n_in in [(70, 300, 4096), (512, 2048, 6144)]:
+        print(f"q4k gemm groups={groups}: {n_tokens} tokens, {n_out}x{n_in}", flush=True)
+        w = hip.synth.q4_k_weight(320 + n_tokens, n_out, n_in)
+        x = hip.synth.activations(321 + n_tokens, n_tokens, n_in)
+        kernel = hip.kernel.Q4_KKernel(w, n_in, n_out)
+        out = np.zeros((n_tokens, n_out), np.float32)
+        kernel.forward_batched(x, out, n_in, n_out, matrix_cores=True)
+        ints, qs, bs = _gemm_block_ints(hip, kernel, x, n_tokens, n_in, n_out)
+        wr = w.reshape(n_out, -1, 144)
+        wd = wr[:, :, 0:2].copy().view(np.float16)[:, :, 0].astype(np.float64)
+        wdmin = wr[:, :, 2:4].copy().view(np.float16)[:, :, 0].astype(np.float64)
+        for t in np.unique(np.linspace(0, n_tokens - 1, 6).astype(int)):
+            d, rq, rb = oracle.quantize_row_q8_k(x[t], A)
+            assert np.array_equal(rq, qs[t]) and np.array_equal(rb, bs[t])
+            want = oracle.q4k_q8k_block_ints_matrix(w, n_out, qs[t], bs[t])
+            assert np.array_equal(ints[t], want), t
+            ref = np.zeros(n_out, np.float32)
+            oracle.q4k_forward_prepared(w, d, qs[t], bs[t], ref, n_in, n_out, 0, 1, A)
+            assert np.all(np.abs(out[t] - ref) <= 1e-4 + 1e-4 * np.abs(ref)), t
+            exact = np.sum(wd * d.astype(np.float64)[None, :] * want[:, :, 0] - wdmin * d.astype(np.float64)[None, :] * want[:, :, 1], axis=1)
+            scale = np.sum(np.abs(wd * d[None, :] * want[:, :, 0]) + np.abs(wdmin * d[None, :] * want[:, :, 1]), axis=1)
+            assert np.all(np.abs(out[t].astype(np.float64) - exact) <= 2e-6 * scale + 1e-30), t
