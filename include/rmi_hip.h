@@ -105,6 +105,21 @@ int rmi_hip_matmul_q8_0_quantized_range(const rmi_hip_weight *w, const uint8_t *
  * (the layout of Kernel::forward_batched, trait_.rs:78-109). */
 int rmi_hip_matmul_q8_0_quantized_batch(const rmi_hip_weight *w, const uint8_t *input_q8, const float *input_scales,
                                         float *output, uint32_t n_in, uint32_t n_out, uint32_t n_tokens);
+/* How rmi_hip_q8_0_forward_batched and rmi_hip_q4_k_forward_batched multiply a batch (process-wide; a caller that
+ * implements Kernel::forward_batched, src/ops/kernel/trait_.rs:78-109, on those two entry points chooses once at
+ * start-up instead of at every call site):
+ *   X86_ORDER (default)  every token through the GEMV in the x86-64 kernels' accumulation order: the bits of an
+ *                        x86-64 host for any token count, and the whole weight is read once per 8 tokens;
+ *   AARCH64_ORDER        Q8_0: the aarch64 kernel's order on the matrix cores (what the *_neon entry computes), bit
+ *                        for bit an aarch64 host; Q4_K: as FAST (its CPU kernels have one order);
+ *   FAST                 the fastest kernel per product, every output within 1e-4 + 1e-4 |ref| of the CPU kernels
+ *                        and built from exact integer block dots: up to 8 tokens the GEMV, then the small-batch
+ *                        kernel and rmi_hip_gemm_q8_0_fast_dev / the Q4_K GEMM. */
+#define RMI_HIP_BATCHED_X86_ORDER 0
+#define RMI_HIP_BATCHED_AARCH64_ORDER 1
+#define RMI_HIP_BATCHED_FAST 2
+int rmi_hip_set_forward_batched_mode(int mode);
+int rmi_hip_get_forward_batched_mode(void);
 /* Kernel::forward / forward_batched with f32 input (trait_.rs:59-109):
  * quantize each token row on the device (rounding as given), then the GEMV in
  * the x86-64 kernel's order for every token, eight tokens a launch.  As in the

@@ -110,7 +110,7 @@ static int q4_k_forward_batched(const rmi_hip_weight *w, const float *input, flo
 
 int rmi_hip_q4_k_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
                                  uint32_t n_out, uint32_t n_tokens) {
-    return q4_k_forward_batched(w, input, output, n_in, n_out, n_tokens, false);
+    return q4_k_forward_batched(w, input, output, n_in, n_out, n_tokens, rmi_batched_mode() != RMI_HIP_BATCHED_X86_ORDER);
 }
 
 int rmi_hip_q4_k_forward_batched_mfma(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,

@@ -187,7 +187,10 @@ int rmi_hip_matmul_q8_0_quantized_batch(const rmi_hip_weight *w, const uint8_t *
 // in trait_.rs:78-109).  Otherwise the aarch64 kernel's order on the matrix cores, equally batch-independent: the
 // small-batch kernel while the tokens fit its LDS staging, the tiled GEMM for more.
 static int forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in, uint32_t n_out,
-                           uint32_t n_tokens, int rounding, bool x86_order) {
+                           uint32_t n_tokens, int rounding, int mode) {
+    // FAST: up to 8 tokens the GEMV (one launch, the x86-64 order); beyond, the matrix cores
+    const bool x86_order = mode == RMI_HIP_BATCHED_X86_ORDER || (mode == RMI_HIP_BATCHED_FAST && n_tokens <= 8);
+    const bool fast = mode == RMI_HIP_BATCHED_FAST;
     RMI_REQUIRE_INIT();
     int rc = check_q8(w, n_in, n_out);
     if (rc != RMI_HIP_OK) return rc;
@@ -213,6 +216,8 @@ static int forward_batched(const rmi_hip_weight *w, const float *input, float *o
         rc = rmi_gemv_q8_0_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
     else if (small_batch && rmi_gemv_q8_0_mfma_fits(n_tokens, w->n_units))
         rc = mfma_tokens(w, d_q8, d_sc, d_y, n_tokens, n_out, 0, n_out, c->stream);
+    else if (n_tokens >= kGemmMinTokens && fast)
+        rc = rmi_hip_gemm_q8_0_fast_dev(w, d_q8, d_sc, d_y, n_tokens, n_out, c->stream);
     else if (n_tokens >= kGemmMinTokens)
         rc = rmi_launch_gemm_q8_0(w, d_q8, d_sc, d_y, n_tokens, n_out, c->stream);
     else {  // up to 15 tokens of a row too long for that: the same kernel, as many tokens at a time as fit
@@ -229,12 +234,12 @@ static int forward_batched(const rmi_hip_weight *w, const float *input, float *o
 
 int rmi_hip_q8_0_forward_batched(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
                                  uint32_t n_out, uint32_t n_tokens, int rounding) {
-    return forward_batched(w, input, output, n_in, n_out, n_tokens, rounding, true);
+    return forward_batched(w, input, output, n_in, n_out, n_tokens, rounding, rmi_batched_mode());
 }
 
 int rmi_hip_q8_0_forward_batched_neon(const rmi_hip_weight *w, const float *input, float *output, uint32_t n_in,
                                       uint32_t n_out, uint32_t n_tokens, int rounding) {
-    return forward_batched(w, input, output, n_in, n_out, n_tokens, rounding, false);
+    return forward_batched(w, input, output, n_in, n_out, n_tokens, rounding, RMI_HIP_BATCHED_AARCH64_ORDER);
 }
 
 int rmi_hip_quantize_q8_0(const float *input, uint32_t n, uint8_t *q8, float *scales, int rounding) {

@@ -141,6 +141,7 @@ void *rmi_dev_buf(RmiThreadCtx *c, int slot, size_t nbytes);
 void *rmi_pin_buf(RmiThreadCtx *c, int slot, size_t nbytes);
 int rmi_device_cus();
 int rmi_device();  // the device rmi_hip_init bound, -1 before
+int rmi_batched_mode();  // RMI_HIP_BATCHED_*: what rmi_hip_set_forward_batched_mode chose
 // the device address of the no-allocation entry point's scratch array on `device`, which must be current
 int rmi_noalloc_setup(int device);
 

@@ -137,6 +137,10 @@ void *rmi_pin_buf(RmiThreadCtx *c, int slot, size_t nbytes) {
     return c->pin[slot];
 }
 
+// How the forward_batched entry points of the Kernel trait multiply more than one token; process-wide, read at each call.
+static std::atomic<int> g_batched_mode{RMI_HIP_BATCHED_X86_ORDER};
+int rmi_batched_mode() { return g_batched_mode.load(std::memory_order_relaxed); }
+
 extern "C" {
 
 const char *rmi_hip_last_error(void) { return t_error; }
@@ -194,6 +198,15 @@ void rmi_hip_shutdown(void) {
     g_generation.fetch_add(1, std::memory_order_acq_rel);
     g_device = -1;
 }
+
+int rmi_hip_set_forward_batched_mode(int mode) {
+    if (mode != RMI_HIP_BATCHED_X86_ORDER && mode != RMI_HIP_BATCHED_AARCH64_ORDER && mode != RMI_HIP_BATCHED_FAST)
+        return rmi_fail(RMI_HIP_E_INVALID, "unknown forward_batched mode %d", mode);
+    g_batched_mode.store(mode, std::memory_order_relaxed);
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_get_forward_batched_mode(void) { return rmi_batched_mode(); }
 
 size_t rmi_hip_thread_context_count(void) {
     std::lock_guard<std::mutex> lock(g_mutex);

@@ -15,6 +15,7 @@ DTYPE_Q4_0 = 2
 DTYPE_Q8_0 = 8
 DTYPE_Q4_K = 12
 DTYPE_Q6_K = 14
+BATCHED_X86_ORDER, BATCHED_AARCH64_ORDER, BATCHED_FAST = 0, 1, 2
 ROUND_HALF_AWAY = 0
 ROUND_TIES_EVEN = 1
 ROUND_NEON = 2
@@ -56,6 +57,8 @@ SIGNATURES = {
     "rmi_hip_shutdown": (None, []),
     "rmi_hip_last_error": (C.c_char_p, []),
     "rmi_hip_thread_context_count": (_sz, []),
+    "rmi_hip_set_forward_batched_mode": (C.c_int, [C.c_int]),
+    "rmi_hip_get_forward_batched_mode": (C.c_int, []),
     "rmi_hip_device_info": (C.c_int, [C.c_char_p, _sz, C.POINTER(C.c_int), C.POINTER(_sz)]),
     "rmi_hip_upload_q8_0": (_vp, [_u8p, _sz, _u32, _u32]),
     "rmi_hip_upload_q4_k": (_vp, [_u8p, _sz, _u32, _u32]),

@@ -102,6 +102,16 @@ class Kernel:
             self.forward(x[t * n_in:(t + 1) * n_in], out[t], n_in, n_out)
 
 
+def set_forward_batched_mode(mode):
+    """How `Kernel::forward_batched` of the Q8_0 and Q4_K kernels multiplies a batch, for the whole process:
+    `hip.BATCHED_X86_ORDER` (default: the x86-64 kernels' bits for every token), `hip.BATCHED_AARCH64_ORDER` or
+    `hip.BATCHED_FAST` (the fastest kernel per product, within the reference's tolerance).  Returns the mode it
+    replaces."""
+    old = lib.rmi_hip_get_forward_batched_mode()
+    check(lib.rmi_hip_set_forward_batched_mode(mode))
+    return old
+
+
 class _DeviceWeight:
     def __init__(self, handle):
         if not handle:

@@ -161,3 +161,49 @@ def test_fast_entry_follows_its_plan(hip, oracle, n_tokens, n_out, n_in):
             assert np.all(np.abs(outs[0][t] - ref) <= TOL(ref)), (variant, t)
     for b in (d_x, d_q8, d_sc):
         b.free()
+
+
+def test_forward_batched_mode_selects_the_path_without_touching_call_sites(hip, oracle):
+    """rmi_hip_set_forward_batched_mode: the same Kernel::forward_batched call gives the x86-64 order's bits by
+    default, the aarch64 order's bits in AARCH64_ORDER, and in FAST the x86-64 bits up to 8 tokens and a result within
+    tolerance beyond; an unknown mode is refused and changes nothing; Q4_K follows the same switch."""
+    H, K = hip.hip, hip.kernel
+    n_out, n_in = 520, 1024
+    w = hip.synth.q8_0_weight(5400, n_out, n_in)
+    kernel = K.Q8Kernel(w, n_in, n_out)
+    assert H.lib.rmi_hip_get_forward_batched_mode() == H.BATCHED_X86_ORDER
+    try:
+        for n_tokens in (3, 8, 40, 200):
+            x = hip.synth.activations(5401 + n_tokens, n_tokens, n_in)
+            pairs = [oracle.quantize_q8_0(x[t], A) for t in range(n_tokens)]
+            ref = {v: np.stack([oracle.matmul_q8_0_quantized(w, p[0], p[1], n_in, n_out, v) for p in pairs]) for v in (A, N)}
+            outs = {}
+            for mode in (H.BATCHED_X86_ORDER, H.BATCHED_AARCH64_ORDER, H.BATCHED_FAST):
+                K.set_forward_batched_mode(mode)
+                outs[mode] = np.zeros((n_tokens, n_out), np.float32)
+                kernel.forward_batched(x, outs[mode], n_in, n_out)
+            assert np.array_equal(bits(outs[H.BATCHED_X86_ORDER]), bits(ref[A]))
+            assert np.array_equal(bits(outs[H.BATCHED_AARCH64_ORDER]), bits(ref[N]))
+            if n_tokens <= 8:
+                assert np.array_equal(bits(outs[H.BATCHED_FAST]), bits(ref[A]))
+            assert np.all(np.abs(outs[H.BATCHED_FAST] - ref[A]) <= TOL(ref[A]))
+        assert H.lib.rmi_hip_set_forward_batched_mode(7) == -1 and H.lib.rmi_hip_get_forward_batched_mode() == H.BATCHED_FAST
+        # Q4_K: X86_ORDER is the GEMV for every token (AVX2 order, bit for bit), the other two the GEMM from 16 tokens on
+        n_out, n_in, n_tokens = 300, 1024, 48
+        wk = hip.synth.q4_k_weight(5410, n_out, n_in)
+        xk = hip.synth.activations(5411, n_tokens, n_in)
+        kk = K.Q4_KKernel(wk, n_in, n_out)
+        want = np.zeros((n_tokens, n_out), np.float32)
+        for t in range(n_tokens):
+            d, qs, bs = oracle.quantize_row_q8_k(xk[t], A)
+            oracle.q4k_forward_prepared(wk, d, qs, bs, want[t], n_in, n_out, 0, 1, A)
+        got = {}
+        for mode in (H.BATCHED_X86_ORDER, H.BATCHED_FAST):
+            K.set_forward_batched_mode(mode)
+            got[mode] = np.zeros((n_tokens, n_out), np.float32)
+            kk.forward_batched(xk, got[mode], n_in, n_out)
+        assert np.array_equal(bits(got[H.BATCHED_X86_ORDER]), bits(want))
+        assert np.all(np.abs(got[H.BATCHED_FAST] - want) <= TOL(want))
+        assert not np.array_equal(bits(got[H.BATCHED_FAST]), bits(want))  # the matrix-core path did run
+    finally:
+        K.set_forward_batched_mode(H.BATCHED_X86_ORDER)
