@@ -66,6 +66,13 @@ inline std::vector<BlockQ8K> quantize_row_q8_k(const float *x, size_t n) {
     return out;
 }
 
+// How forward_batched of the Q8_0 and Q4_K kernels multiplies a batch, for the whole process: RMI_HIP_BATCHED_X86_ORDER
+// (default: an x86-64 host's bits for every token), RMI_HIP_BATCHED_AARCH64_ORDER, or RMI_HIP_BATCHED_FAST (the fastest
+// kernel per product, within the reference's tolerance).  Chosen once at start-up; no call site changes.
+inline void set_forward_batched_mode(int mode) {
+    if (rmi_hip_set_forward_batched_mode(mode) != RMI_HIP_OK) throw HipError(RMI_HIP_E_INVALID, rmi_hip_last_error());
+}
+
 class Kernel {
   public:
     virtual ~Kernel() = default;

@@ -45,6 +45,7 @@ extern "C" {
         w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
         rounding: c_int,
     ) -> c_int;
+    fn rmi_hip_set_forward_batched_mode(mode: c_int) -> c_int;
     fn rmi_hip_q8_0_forward_batched_neon(
         w: *const RmiHipWeight, input: *const f32, output: *mut f32, n_in: u32, n_out: u32, n_tokens: u32,
         rounding: c_int,
@@ -96,6 +97,17 @@ fn last_error() -> String {
 /// `Err` means "stay on the CPU kernels" (src/ops/float.rs:51-57).
 pub fn init(device: i32) -> Result<(), String> {
     if unsafe { rmi_hip_init(device) } == 0 { Ok(()) } else { Err(last_error()) }
+}
+
+/// How `Kernel::forward_batched` of the Q8_0 and Q4_K kernels multiplies a batch, for the whole process
+/// (`rmi_hip_set_forward_batched_mode`): the x86-64 kernels' bits for every token (the default), the aarch64
+/// kernel's bits, or the fastest kernel per product within the crate's own tolerance (exact integer block dots,
+/// f32 sums within 1e-4 + 1e-4 |ref|).  Chosen once at start-up; no call site changes.
+#[derive(Clone, Copy, PartialEq)]
+pub enum BatchedMode { X86Order = 0, Aarch64Order = 1, Fast = 2 }
+
+pub fn set_forward_batched_mode(mode: BatchedMode) -> Result<(), String> {
+    if unsafe { rmi_hip_set_forward_batched_mode(mode as c_int) } == 0 { Ok(()) } else { Err(last_error()) }
 }
 
 #[derive(Clone, Copy, PartialEq)]
