@@ -446,6 +446,11 @@ void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s);
 /* Token ids that end generation (the tokenizer's EOS id and "im_end", src/models/qwen3.rs:1123-1130); none by
  * default.  At most 16. */
 int rmi_hip_qwen3_set_stop_ids(rmi_hip_qwen3 *s, const uint32_t *ids, uint32_t n_ids);
+/* Prompt positions are known in advance, so rmi_hip_qwen3_generate takes them eight to a pass while it can (head
+ * dimension 128, contexts short of the split attention's 768 keys): every weight is read once for the eight, each
+ * position's logits, argmax and cache rows are what the step-by-step run gives, bit for bit.  On by default;
+ * enabled = 0 makes every position its own step. */
+int rmi_hip_qwen3_set_prompt_passes(rmi_hip_qwen3 *s, int enabled);
 /* Runs up to n_prompt + max_new - 1 steps, one token per step, positions 0.. (the prompt is fed token by
  * token as generate_inner does), greedy sampling (temperature 0, sample_token's argmax branch).  With stop
  * ids set the run ends at the first sampled stop id, which is not part of the result, as in generate_inner

@@ -73,13 +73,22 @@ __global__ __launch_bounds__(256) void embed_q8_0_kernel(const uint8_t *__restri
 // x += r (if r), then rms_norm(x, weight) quantized to Q8_0.  One workgroup of 256; R float4 per thread stay in
 // registers (n <= 1024 * R), and every load of the kernel goes out before the first wait, so the kernel sees
 // one memory round trip.  Sum of squares: per thread in ascending order, f64, then lanes and waves combined.
+// A launch of several workgroups does the same for as many tokens: token blockIdx.x, the arrays tok_stride.x/.y/.z
+// elements apart (x, r, q8; the scales q8's stride / 32).
+struct TokStride3 {
+    uint32_t x, y, z;
+};
 template <int R>
 __global__ __launch_bounds__(256) void add_rmsnorm_quant_kernel(float *__restrict__ x, const float *__restrict__ r,
                                                                  const float *__restrict__ weight, uint32_t n, float eps,
                                                                  int8_t *__restrict__ q8, float *__restrict__ scales,
-                                                                 int rounding) {
+                                                                 int rounding, TokStride3 tok_stride) {
     __shared__ double red[4];
     const uint32_t tid = threadIdx.x;
+    x += size_t(blockIdx.x) * tok_stride.x;
+    if (r) r += size_t(blockIdx.x) * tok_stride.y;
+    q8 += size_t(blockIdx.x) * tok_stride.z;
+    scales += size_t(blockIdx.x) * (tok_stride.z >> 5);
     float4 v[R], a[R], wv[R];
 #pragma unroll
     for (int j = 0; j < R; j++) {  // unconditional loads; a vector past the end re-reads the last one and is not used
@@ -131,17 +140,17 @@ __global__ __launch_bounds__(256) void add_rmsnorm_quant_kernel(float *__restric
 
 constexpr uint32_t kNormMaxN = 1024 * 16;
 void launch_add_rmsnorm_quant(float *x, const float *r, const float *weight, uint32_t n, float eps, int8_t *q8,
-                              float *scales, int rounding, hipStream_t st) {
+                              float *scales, int rounding, hipStream_t st, uint32_t n_tok = 1, TokStride3 ts = TokStride3{0, 0, 0}) {
     if (n <= 1024)
-        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<1>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<1>, dim3(n_tok), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding, ts);
     else if (n <= 2048)
-        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<2>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<2>, dim3(n_tok), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding, ts);
     else if (n <= 4096)
-        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<4>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<4>, dim3(n_tok), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding, ts);
     else if (n <= 8192)
-        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<8>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<8>, dim3(n_tok), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding, ts);
     else
-        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<16>, dim3(1), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding);
+        hipLaunchKernelGGL(add_rmsnorm_quant_kernel<16>, dim3(n_tok), dim3(256), 0, st, x, r, weight, n, eps, q8, scales, rounding, ts);
 }
 
 // Per head of the stacked q|k|v vector: q/k RMS norm, NeoX rotation, f16 rounding; k and v go to the cache row.
@@ -152,8 +161,15 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(const float *__r
                                                                 const float *__restrict__ sin_t, uint32_t pos,
                                                                 uint16_t *__restrict__ q16, uint16_t *__restrict__ k_row,
                                                                 uint16_t *__restrict__ v_row, uint32_t n_head,
-                                                                uint32_t n_head_kv, uint32_t hk, uint32_t hv, float eps) {
+                                                                uint32_t n_head_kv, uint32_t hk, uint32_t hv, float eps,
+                                                                TokStride3 tok_stride) {
     const uint32_t head = blockIdx.x, tid = threadIdx.x;
+    // token blockIdx.y of a launch over several: the next position, its qkv, q16 and cache rows tok_stride apart
+    qkv += size_t(blockIdx.y) * tok_stride.x;
+    q16 += size_t(blockIdx.y) * tok_stride.y;
+    k_row += size_t(blockIdx.y) * tok_stride.z;
+    v_row += size_t(blockIdx.y) * tok_stride.z;
+    pos += blockIdx.y;
     if (head >= n_head + n_head_kv) {  // v: rounding only
         const uint32_t kvh = head - n_head - n_head_kv;
         const float *src = qkv + size_t(n_head) * hk + size_t(n_head_kv) * hk + size_t(kvh) * hv;
@@ -462,11 +478,16 @@ template <bool FROM_QKV>
 __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
     uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, int8_t *__restrict__ q8,
-    float *__restrict__ scales, int rounding, AttnFromQkv fq) {
+    float *__restrict__ scales, int rounding, AttnFromQkv fq, uint32_t tok_q16_stride, uint32_t tok_out_stride) {
     extern __shared__ double lds_d[];
     __shared__ float red_f[kA128Threads / 64];
     __shared__ uint64_t exp_tab[32];
     __shared__ __attribute__((aligned(16))) uint16_t new16[3][128];  // this step's q, k, v as f16
+    // token blockIdx.z of a launch over several consecutive positions (their cache rows are filled already)
+    step += blockIdx.z;
+    q16 += size_t(blockIdx.z) * tok_q16_stride;
+    q8 += size_t(blockIdx.z) * tok_out_stride;
+    scales += size_t(blockIdx.z) * (tok_out_stride >> 5);
     // grid = (query heads per key/value head, key/value heads)
     const uint32_t kvh = blockIdx.y, head = blockIdx.y * gridDim.x + blockIdx.x, tid = threadIdx.x;
     const uint32_t n_keys = step + 1;
@@ -1070,7 +1091,10 @@ int launch_attention128_split(const uint16_t *q16, const uint16_t *k_cache, cons
 // gu = [W_gate x ; W_up x]: h = (W_up x) * silu(W_gate x), quantized to Q8_0
 __global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float *__restrict__ gu, uint32_t n_ff,
                                                              int8_t *__restrict__ q8, float *__restrict__ scales,
-                                                             int rounding) {
+                                                             int rounding, uint32_t tok_gu_stride, uint32_t tok_q_stride) {
+    gu += size_t(blockIdx.y) * tok_gu_stride;  // token blockIdx.y of a launch over several
+    q8 += size_t(blockIdx.y) * tok_q_stride;
+    scales += size_t(blockIdx.y) * (tok_q_stride >> 5);
     const uint32_t i = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= n_ff) return;  // n_ff is a multiple of 32: whole 8-lane groups leave together
     const float4 g = *reinterpret_cast<const float4 *>(gu + i);
@@ -1116,6 +1140,8 @@ __device__ __forceinline__ Top top_block_reduce(Top t, Top *sm) {
 __global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__restrict__ logits, uint32_t n,
                                                              Top *__restrict__ partial) {
     __shared__ Top sm[256];
+    logits += size_t(blockIdx.y) * n;  // token blockIdx.y of a launch over several: its logits, its partial results
+    partial += size_t(blockIdx.y) * gridDim.x;
     Top t{-INFINITY, -INFINITY, 0xffffffffu, 1u};
     for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
         const float l = logits[i];
@@ -1157,6 +1183,44 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const Top *__restrict
     embed_row(w_embd, n_oct, next_token, vocab, x, n_embd);  // the next step starts from its token's embedding
 }
 
+// ---- several prompt positions in one pass (rmi_hip_qwen3_generate while the tokens are known in advance)
+// the embeddings of the prompt tokens step0 .. step0 + gridDim.x - 1, n_embd apart
+__global__ __launch_bounds__(256) void embed_batch_kernel(const uint8_t *__restrict__ w, uint32_t n_oct,
+                                                          const uint32_t *__restrict__ tok, uint32_t step0, uint32_t vocab,
+                                                          float *__restrict__ x, uint32_t n_embd) {
+    embed_row(w, n_oct, tok[step0 + blockIdx.x], vocab, x + size_t(blockIdx.x) * n_embd, n_embd);
+}
+// argmax_final_kernel for position step0 + blockIdx.x of such a pass; the workgroup of the pass's last position also
+// advances the step counter and leaves the next token's embedding where a single step starts from
+__global__ __launch_bounds__(256) void argmax_final_batch_kernel(const Top *__restrict__ partial, uint32_t n_partial,
+                                                                 StepParams *__restrict__ sp, uint32_t step0,
+                                                                 uint32_t *__restrict__ tok, uint32_t *__restrict__ step_argmax,
+                                                                 float *__restrict__ step_top2,
+                                                                 uint32_t *__restrict__ nonfinite_steps,
+                                                                 const uint8_t *__restrict__ w_embd, uint32_t n_oct,
+                                                                 uint32_t vocab, float *__restrict__ x, uint32_t n_embd) {
+    __shared__ Top sm[256];
+    __shared__ uint32_t next_token;
+    partial += size_t(blockIdx.x) * n_partial;
+    Top t{-INFINITY, -INFINITY, 0xffffffffu, 1u};
+    for (uint32_t i = threadIdx.x; i < n_partial; i += 256) t = top_merge(t, partial[i]);
+    const Top r = top_block_reduce(t, sm);
+    const uint32_t step = step0 + blockIdx.x;
+    if (threadIdx.x == 0) {
+        const uint32_t n_prompt = sp->n_prompt;
+        step_argmax[step] = r.id;
+        step_top2[2 * step] = r.best;
+        step_top2[2 * step + 1] = r.second;
+        if (!r.finite) atomicAdd(nonfinite_steps, 1u);
+        if (step + 1 >= n_prompt) tok[step + 1] = r.id;  // the next step's token
+        next_token = step + 1 >= n_prompt ? r.id : tok[step + 1];
+    }
+    if (blockIdx.x + 1 != gridDim.x) return;
+    if (threadIdx.x == 0) sp->step = step + 1;
+    __syncthreads();
+    embed_row(w_embd, n_oct, next_token, vocab, x, n_embd);
+}
+
 }  // namespace
 
 // ------------------------------------------------------------------ session
@@ -1175,15 +1239,22 @@ struct rmi_hip_qwen3 {
     uint32_t *tok = nullptr, *step_argmax = nullptr, *nonfinite = nullptr;
     float *step_top2 = nullptr;
     void *partial = nullptr;
+    // the same buffers for kPromptBatch positions at once (prompt passes), token-major
+    float *xb = nullptr, *residb = nullptr, *qkvb = nullptr, *gub = nullptr, *logitsb = nullptr, *act_scalesb = nullptr;
+    uint16_t *q16b = nullptr;
+    int8_t *act_q8b = nullptr;
+    void *partialb = nullptr;
     void *attn_split = nullptr;          // scratch of the split attention launches (head dimension 128)
     void *params = nullptr;              // StepParams in HBM
     std::vector<void *> owned;  // every other device allocation, freed with the session
     std::vector<uint32_t> stop_ids;  // generation ends before the first of these (EOS, im_end)
+    bool prompt_passes = true;       // prompt positions eight to a pass (rmi_hip_qwen3_set_prompt_passes)
 };
 
 namespace {
 
 constexpr uint32_t kArgmaxGroups = 256;
+constexpr uint32_t kPromptBatch = 8;  // positions per prompt pass: what one GEMV launch takes
 
 template <typename T>
 T *dev_alloc(rmi_hip_qwen3 *s, size_t count, bool zero = false) {
@@ -1267,7 +1338,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
                                  s->k_cache + row, s->v_cache + row, c.eps};
             hipLaunchKernelGGL(attention128_quant_kernel<true>, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kA128Threads),
                                attn128_lds_bytes(step + 1), st, static_cast<const uint16_t *>(nullptr), s->k_cache + layer_base,
-                               s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd, fq);
+                               s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd, fq, 0u, 0u);
         } else if (rmi_gemv_q8_0_norm_rope_fusable(s->w_qkv[l], c.n_head, c.n_head_kv, c.head_dim_k, c.head_dim_v)) {
             // norm, q/k/v products, head norms, rotation and the cache row in one launch
             const size_t half = c.head_dim_k / 2;
@@ -1281,7 +1352,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
             if (rc != RMI_HIP_OK) return rc;
             hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv), dim3(64), 0, st, s->qkv, qn, kn,
                                s->cos_t, s->sin_t, step, s->q16, s->k_cache + row, s->v_cache + row, c.n_head,
-                               c.n_head_kv, c.head_dim_k, c.head_dim_v, c.eps);
+                               c.n_head_kv, c.head_dim_k, c.head_dim_v, c.eps, TokStride3{0, 0, 0});
         }
         if (qkv_in_attention) {
             // done above
@@ -1293,7 +1364,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
         } else if (d128)
             hipLaunchKernelGGL(attention128_quant_kernel<false>, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kA128Threads), attn128_lds_bytes(step + 1),
                                st, s->q16, s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride,
-                               c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd, AttnFromQkv{});
+                               c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd, AttnFromQkv{}, 0u, 0u);
         else
             hipLaunchKernelGGL(attention_quant_kernel, dim3(c.n_head), dim3(kAttnThreads), attn_lds, st, s->q16,
                                s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head,
@@ -1307,7 +1378,7 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
         } else {
             rc = norm_gemv(s->w_gu[l], s->resid, s->ffn_norm[l], s->gu);
             hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((c.n_ff + 1023) / 1024), dim3(256), 0, st, s->gu, c.n_ff,
-                               s->act_q8, s->act_scales, rnd);
+                               s->act_q8, s->act_scales, rnd, 0u, 0u);
         }
         if (rc != RMI_HIP_OK) return rc;
         rc = gemv(s->w_down[l], s->act_q8, s->act_scales, s->resid, st);
@@ -1321,6 +1392,71 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
     hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, static_cast<const Top *>(s->partial),
                        kArgmaxGroups, sp, s->tok, s->step_argmax, s->step_top2, s->nonfinite, s->embd->data,
                        s->embd->n_units, c.vocab, s->x, c.n_embd);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+// Whether the prompt positions step0 .. step0 + n - 1 can go through one pass: head dimension 128, every launch
+// of the pass within what the single-workgroup attention kernel holds, and short of the split's first position.
+bool prompt_pass_possible(const rmi_hip_qwen3 *s, uint32_t step0, uint32_t n) {
+    const rmi_hip_qwen3_config &c = s->cfg;
+    if (!s->xb || n == 0 || n > kPromptBatch) return false;
+    if (c.n_embd > kNormMaxN) return false;
+    if (s->attn_split && attn128_use_split(step0 + n, c.n_head)) return false;
+    return attn128_lds_bytes(step0 + n) <= 64 * 1024;
+}
+
+// n consecutive prompt positions from step0 on in one pass: every product reads its weight once for all of them
+// (the x86-64-order GEMV takes up to eight tokens a launch and gives each the bits it gets alone), the other
+// kernels run once per position inside one launch.  Position by position the arithmetic is that of enqueue_step's
+// separate-kernel path; a position's keys and values are in the cache before any attention launch of the pass
+// reads them.  Leaves every position's argmax and top-2 logits, the logits in logitsb, and, behind the last
+// position, the step counter and the next token's embedding as a single step expects them.
+int enqueue_prompt_pass(rmi_hip_qwen3 *s, uint32_t step0, uint32_t n, hipStream_t st) {
+    const rmi_hip_qwen3_config &c = s->cfg;
+    const int rnd = c.rounding;
+    StepParams *sp = static_cast<StepParams *>(s->params);
+    const uint32_t n_qkv = s->n_q + s->n_k + s->n_v;
+    hipLaunchKernelGGL(embed_batch_kernel, dim3(n), dim3(256), 0, st, s->embd->data, s->embd->n_units, s->tok, step0, c.vocab,
+                       s->xb, c.n_embd);
+    const float *pending = nullptr;  // matmul output still to be added to the residual stream
+    uint32_t pending_stride = 0;
+    int rc;
+    for (uint32_t l = 0; l < c.n_layer; l++) {
+        const size_t layer_base = size_t(l) * c.capacity * s->kv_stride, row = layer_base + size_t(step0) * s->kv_stride;
+        const float *qn = c.has_qk_norm ? s->q_norm[l] : nullptr, *kn = c.has_qk_norm ? s->k_norm[l] : nullptr;
+        launch_add_rmsnorm_quant(s->xb, pending, s->attn_norm[l], c.n_embd, c.eps, s->act_q8b, s->act_scalesb, rnd, st, n,
+                                 TokStride3{c.n_embd, pending_stride, c.n_embd});
+        rc = rmi_gemv_q8_0_tokens(s->w_qkv[l], s->act_q8b, s->act_scalesb, s->qkvb, n, n_qkv, 0, n_qkv, st);
+        if (rc != RMI_HIP_OK) return rc;
+        hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv, n), dim3(64), 0, st, s->qkvb, qn, kn,
+                           s->cos_t, s->sin_t, step0, s->q16b, s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv,
+                           c.head_dim_k, c.head_dim_v, c.eps, TokStride3{n_qkv, s->n_q, s->kv_stride});
+        hipLaunchKernelGGL(attention128_quant_kernel<false>, dim3(c.n_head / c.n_head_kv, c.n_head_kv, n), dim3(kA128Threads),
+                           attn128_lds_bytes(step0 + n), st, s->q16b, s->k_cache + layer_base, s->v_cache + layer_base, step0,
+                           s->kv_stride, c.n_head, c.n_head_kv, s->act_q8b, s->act_scalesb, rnd, AttnFromQkv{}, s->n_q, s->n_attn);
+        rc = rmi_gemv_q8_0_tokens(s->w_o[l], s->act_q8b, s->act_scalesb, s->residb, n, c.n_embd, 0, c.n_embd, st);
+        if (rc != RMI_HIP_OK) return rc;
+        launch_add_rmsnorm_quant(s->xb, s->residb, s->ffn_norm[l], c.n_embd, c.eps, s->act_q8b, s->act_scalesb, rnd, st, n,
+                                 TokStride3{c.n_embd, c.n_embd, c.n_embd});
+        rc = rmi_gemv_q8_0_tokens(s->w_gu[l], s->act_q8b, s->act_scalesb, s->gub, n, 2 * c.n_ff, 0, 2 * c.n_ff, st);
+        if (rc != RMI_HIP_OK) return rc;
+        hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((c.n_ff + 1023) / 1024, n), dim3(256), 0, st, s->gub, c.n_ff, s->act_q8b,
+                           s->act_scalesb, rnd, 2 * c.n_ff, c.n_ff);
+        rc = rmi_gemv_q8_0_tokens(s->w_down[l], s->act_q8b, s->act_scalesb, s->residb, n, c.n_embd, 0, c.n_embd, st);
+        if (rc != RMI_HIP_OK) return rc;
+        pending = s->residb;
+        pending_stride = c.n_embd;
+    }
+    launch_add_rmsnorm_quant(s->xb, pending, s->output_norm, c.n_embd, c.eps, s->act_q8b, s->act_scalesb, rnd, st, n,
+                             TokStride3{c.n_embd, pending_stride, c.n_embd});
+    rc = rmi_gemv_q8_0_tokens(s->head, s->act_q8b, s->act_scalesb, s->logitsb, n, c.vocab, 0, c.vocab, st);
+    if (rc != RMI_HIP_OK) return rc;
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxGroups, n), dim3(256), 0, st, s->logitsb, c.vocab,
+                       static_cast<Top *>(s->partialb));
+    hipLaunchKernelGGL(argmax_final_batch_kernel, dim3(n), dim3(256), 0, st, static_cast<const Top *>(s->partialb), kArgmaxGroups,
+                       sp, step0, s->tok, s->step_argmax, s->step_top2, s->nonfinite, s->embd->data, s->embd->n_units, c.vocab,
+                       s->x, c.n_embd);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -1395,7 +1531,7 @@ int rmi_hip_silu_mul_quantize_q8_0_dev(const float *gate_up, uint32_t n_ff, int8
     if (n_ff % 32 != 0) return rmi_fail(RMI_HIP_E_INVALID, "n_ff=%u is not a multiple of 32", n_ff);
     if (!gate_up || !q8 || !scales) return rmi_fail(RMI_HIP_E_INVALID, "null pointer");
     hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((n_ff + 1023) / 1024), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       gate_up, n_ff, q8, scales, rounding);
+                       gate_up, n_ff, q8, scales, rounding, 0u, 0u);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -1408,7 +1544,7 @@ int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const fl
     if (n_head == 0 || n_head_kv == 0 || head_dim_k % 2) return rmi_fail(RMI_HIP_E_INVALID, "bad head shape");
     hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(n_head + 2 * n_head_kv), dim3(64), 0,
                        static_cast<hipStream_t>(stream), qkv, q_norm, k_norm, cos_row, sin_row, 0u, q16, k_row, v_row,
-                       n_head, n_head_kv, head_dim_k, head_dim_v, eps);
+                       n_head, n_head_kv, head_dim_k, head_dim_v, eps, TokStride3{0, 0, 0});
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -1448,7 +1584,7 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     }
     if (d128)
         hipLaunchKernelGGL(attention128_quant_kernel<false>, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
-                           q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding, AttnFromQkv{});
+                           q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding, AttnFromQkv{}, 0u, 0u);
     else
         hipLaunchKernelGGL(attention_quant_kernel, dim3(n_head), dim3(kAttnThreads), lds, static_cast<hipStream_t>(stream),
                            q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, head_dim_k, head_dim_v, q8,
@@ -1475,7 +1611,7 @@ int rmi_hip_qkv_attention_f16_quantize_q8_0_dev(const float *qkv, const float *q
     const AttnFromQkv fq{qkv, q_norm, k_norm, cos_row, sin_row, k_cache + row, v_cache + row, eps};
     hipLaunchKernelGGL(attention128_quant_kernel<true>, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds,
                        static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(nullptr), k_cache, v_cache, n_keys - 1,
-                       kv_stride, n_head, n_head_kv, q8, scales, rounding, fq);
+                       kv_stride, n_head, n_head_kv, q8, scales, rounding, fq, 0u, 0u);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
@@ -1614,6 +1750,16 @@ rmi_hip_qwen3 *rmi_hip_qwen3_create(const rmi_hip_qwen3_config *cfg, const rmi_h
          (s->step_top2 = dev_alloc<float>(s, size_t(2) * c.capacity, true)) &&
          (s->nonfinite = dev_alloc<uint32_t>(s, 1, true)) && (s->partial = dev_alloc<Top>(s, kArgmaxGroups)) &&
          (s->params = dev_alloc<StepParams>(s, 1, true));
+    if (ok && c.head_dim_k == 128 && c.head_dim_v == 128)  // prompt passes of kPromptBatch positions (head dimension 128)
+        ok = (s->xb = dev_alloc<float>(s, size_t(kPromptBatch) * c.n_embd)) &&
+             (s->residb = dev_alloc<float>(s, size_t(kPromptBatch) * c.n_embd)) &&
+             (s->qkvb = dev_alloc<float>(s, size_t(kPromptBatch) * (size_t(s->n_q) + s->n_k + s->n_v))) &&
+             (s->q16b = dev_alloc<uint16_t>(s, size_t(kPromptBatch) * s->n_q)) &&
+             (s->gub = dev_alloc<float>(s, size_t(kPromptBatch) * 2 * c.n_ff)) &&
+             (s->logitsb = dev_alloc<float>(s, size_t(kPromptBatch) * c.vocab)) &&
+             (s->act_q8b = dev_alloc<int8_t>(s, size_t(kPromptBatch) * s->max_n_in)) &&
+             (s->act_scalesb = dev_alloc<float>(s, size_t(kPromptBatch) * s->max_n_in / 32)) &&
+             (s->partialb = dev_alloc<Top>(s, size_t(kPromptBatch) * kArgmaxGroups));
     if (ok && c.head_dim_k == 128 && c.head_dim_v == 128 && attn128_use_split(c.capacity, c.n_head))
         ok = (s->attn_split = dev_alloc<uint8_t>(s, attn_split_scratch_bytes(c.n_head, c.capacity), true)) != nullptr;
     if (ok && hipStreamSynchronize(rmi_thread_ctx()->stream) != hipSuccess) {  // the uploads enqueued above
@@ -1668,11 +1814,25 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
             const uint32_t base = steps_done < n_prompt - 1 ? n_prompt - 1 : steps_done;
             until = steps - base > kStopCheck ? base + kStopCheck : steps;
         }
-        for (uint32_t step = steps_done; e == hipSuccess && rc == RMI_HIP_OK && step < until; step++) {
+        for (uint32_t step = steps_done; e == hipSuccess && rc == RMI_HIP_OK && step < until;) {
+            // prompt positions go eight to a pass while they can (their tokens are known); the rest step by step
+            uint32_t n = step < n_prompt ? n_prompt - step : 0;
+            if (n > kPromptBatch) n = kPromptBatch;
+            if (n > until - step) n = until - step;
+            if (s->prompt_passes && n > 1 && prompt_pass_possible(s, step, n)) {
+                rc = enqueue_prompt_pass(s, step, n, st);
+                for (uint32_t d = 0; rc == RMI_HIP_OK && d < n_dump; d++)
+                    if (dump_steps[d] >= step && dump_steps[d] < step + n)
+                        e = hipMemcpyAsync(d_dump + size_t(d) * c.vocab, s->logitsb + size_t(dump_steps[d] - step) * c.vocab,
+                                           size_t(c.vocab) * 4, hipMemcpyDeviceToDevice, st);
+                step += n;
+                continue;
+            }
             rc = enqueue_step(s, step, st);
             for (uint32_t d = 0; rc == RMI_HIP_OK && d < n_dump; d++)
                 if (dump_steps[d] == step)
                     e = hipMemcpyAsync(d_dump + size_t(d) * c.vocab, s->logits, size_t(c.vocab) * 4, hipMemcpyDeviceToDevice, st);
+            step++;
         }
         steps_done = until;
         if (!stops || e != hipSuccess || rc != RMI_HIP_OK) continue;
@@ -1705,6 +1865,12 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
     if (e != hipSuccess) return rmi_fail(RMI_HIP_E_RUNTIME, "decode failed: %s", hipGetErrorString(e));
     if (nonfinite) return rmi_fail(RMI_HIP_E_RUNTIME, "non-finite logits in %u steps", nonfinite);
     return int(n_valid);
+}
+
+int rmi_hip_qwen3_set_prompt_passes(rmi_hip_qwen3 *s, int enabled) {
+    if (!s) return rmi_fail(RMI_HIP_E_INVALID, "null session");
+    s->prompt_passes = enabled != 0;
+    return RMI_HIP_OK;
 }
 
 int rmi_hip_qwen3_set_stop_ids(rmi_hip_qwen3 *s, const uint32_t *ids, uint32_t n_ids) {

@@ -77,6 +77,10 @@ class Qwen3Session:
         ids = np.ascontiguousarray(ids, np.uint32)
         hip.check(hip.lib.rmi_hip_qwen3_set_stop_ids(self._h, hip.ptr(ids, hip._u32p), ids.size))
 
+    def set_prompt_passes(self, enabled):
+        """Prompt positions eight to a pass (the default) or every position its own step; same results either way."""
+        hip.check(hip.lib.rmi_hip_qwen3_set_prompt_passes(self._h, 1 if enabled else 0))
+
     def generate(self, prompt, max_new, dump_steps=()):
         prompt = np.ascontiguousarray(prompt, np.uint32)
         steps = prompt.size + max_new - 1

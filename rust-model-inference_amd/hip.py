@@ -138,6 +138,7 @@ SIGNATURES = {
     "rmi_hip_qwen3_create": (_vp, [C.POINTER(Qwen3Config), C.POINTER(Qwen3Weights)]),
     "rmi_hip_qwen3_destroy": (None, [_vp]),
     "rmi_hip_qwen3_set_stop_ids": (C.c_int, [_vp, _u32p, _u32]),
+    "rmi_hip_qwen3_set_prompt_passes": (C.c_int, [_vp, C.c_int]),
     "rmi_hip_qwen3_generate": (C.c_int, [_vp, _u32p, _u32, _u32, _u32p, _u32p, _f32p, _u32p, _u32, _f32p,
                                          C.POINTER(C.c_double)]),
     "rmi_hip_gguf_open": (_vp, [C.c_char_p]),
