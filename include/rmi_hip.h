@@ -446,10 +446,13 @@ void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s);
 /* Token ids that end generation (the tokenizer's EOS id and "im_end", src/models/qwen3.rs:1123-1130); none by
  * default.  At most 16. */
 int rmi_hip_qwen3_set_stop_ids(rmi_hip_qwen3 *s, const uint32_t *ids, uint32_t n_ids);
-/* Prompt positions are known in advance, so rmi_hip_qwen3_generate takes them eight to a pass while it can (head
- * dimension 128, contexts short of the split attention's 768 keys): every weight is read once for the eight, each
- * position's logits, argmax and cache rows are what the step-by-step run gives, bit for bit.  On by default;
- * enabled = 0 makes every position its own step. */
+/* Prompt positions are known in advance, so rmi_hip_qwen3_generate takes them 128 to a pass while it can (head
+ * dimension 128, contexts short of the split attention's 768 keys): every product is one launch for all of them
+ * (eight tokens to a workgroup, the x86-64 order's bits for each), the other kernels run once per position inside
+ * one launch; each position's logits, argmax and cache rows are what the step-by-step run gives, bit for bit.
+ * enabled = 1 (the default): 128 positions a pass; 0: every position its own step; n > 1: n positions a pass (at
+ * most 128).  Measured on the 512-token prompt of a Qwen3-0.6B model: 0.73 ms a position step by step, 0.07 ms in
+ * passes of 128. */
 int rmi_hip_qwen3_set_prompt_passes(rmi_hip_qwen3 *s, int enabled);
 /* Runs up to n_prompt + max_new - 1 steps, one token per step, positions 0.. (the prompt is fed token by
  * token as generate_inner does), greedy sampling (temperature 0, sample_token's argmax branch).  With stop

@@ -53,7 +53,17 @@ int rmi_gemv_q8_0_tokens(const rmi_hip_weight *w, const int8_t *x_q8, const floa
     const uint32_t chunk = gemv_chunk(w);
     if (chunk == 0) return rmi_fail(RMI_HIP_E_INVALID, "n_in=%u is too long for the GEMV staging", w->n_in);
     const uint32_t nb = w->n_in / 32;
-    for (uint32_t t0 = 0; t0 < n_tokens; t0 += chunk) {
+    uint32_t t0 = 0;
+    if (w->dtype != RMI_HIP_DTYPE_Q4_0 && n_tokens >= 2 * chunk) {
+        // every full group of `chunk` tokens in one launch (the groups re-read the weight from L2), up to what a
+        // grid's second dimension holds
+        const uint32_t groups = n_tokens / chunk < 65535 ? n_tokens / chunk : 65535;
+        RmiGemvProblem p = make_problem(w, x_q8, x_scales, y, y_stride, row_start, row_end);
+        int rc = rmi_launch_gemv_q8_0_single(p, chunk, s, groups);
+        if (rc != RMI_HIP_OK) return rc;
+        t0 = groups * chunk;
+    }
+    for (; t0 < n_tokens; t0 += chunk) {
         const uint32_t nt = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
         RmiGemvProblem p = make_problem(w, x_q8 + size_t(t0) * w->n_in, x_scales + size_t(t0) * nb,
                                         y + size_t(t0) * y_stride, y_stride, row_start, row_end);

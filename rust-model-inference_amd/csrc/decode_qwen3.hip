@@ -1248,13 +1248,14 @@ struct rmi_hip_qwen3 {
     void *params = nullptr;              // StepParams in HBM
     std::vector<void *> owned;  // every other device allocation, freed with the session
     std::vector<uint32_t> stop_ids;  // generation ends before the first of these (EOS, im_end)
-    bool prompt_passes = true;       // prompt positions eight to a pass (rmi_hip_qwen3_set_prompt_passes)
+    uint32_t prompt_pass = 128;      // prompt positions per pass, 0 = every position its own step (rmi_hip_qwen3_set_prompt_passes)
 };
 
 namespace {
 
 constexpr uint32_t kArgmaxGroups = 256;
-constexpr uint32_t kPromptBatch = 8;  // positions per prompt pass: what one GEMV launch takes
+constexpr uint32_t kPromptBatch = 128;  // most positions a prompt pass takes (the buffers' size); kPromptPassDefault is what it takes
+constexpr uint32_t kPromptPassDefault = 128;
 
 template <typename T>
 T *dev_alloc(rmi_hip_qwen3 *s, size_t count, bool zero = false) {
@@ -1817,9 +1818,9 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
         for (uint32_t step = steps_done; e == hipSuccess && rc == RMI_HIP_OK && step < until;) {
             // prompt positions go eight to a pass while they can (their tokens are known); the rest step by step
             uint32_t n = step < n_prompt ? n_prompt - step : 0;
-            if (n > kPromptBatch) n = kPromptBatch;
+            if (n > s->prompt_pass) n = s->prompt_pass;
             if (n > until - step) n = until - step;
-            if (s->prompt_passes && n > 1 && prompt_pass_possible(s, step, n)) {
+            if (n > 1 && prompt_pass_possible(s, step, n)) {
                 rc = enqueue_prompt_pass(s, step, n, st);
                 for (uint32_t d = 0; rc == RMI_HIP_OK && d < n_dump; d++)
                     if (dump_steps[d] >= step && dump_steps[d] < step + n)
@@ -1869,7 +1870,8 @@ int rmi_hip_qwen3_generate(rmi_hip_qwen3 *s, const uint32_t *prompt, uint32_t n_
 
 int rmi_hip_qwen3_set_prompt_passes(rmi_hip_qwen3 *s, int enabled) {
     if (!s) return rmi_fail(RMI_HIP_E_INVALID, "null session");
-    s->prompt_passes = enabled != 0;
+    // 0: off; 1: the default size; more: that many positions a pass, up to the buffers' size
+    s->prompt_pass = enabled <= 0 ? 0u : enabled == 1 ? kPromptPassDefault : uint32_t(enabled) < kPromptBatch ? uint32_t(enabled) : kPromptBatch;
     return RMI_HIP_OK;
 }
 

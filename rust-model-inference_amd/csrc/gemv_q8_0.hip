@@ -205,6 +205,10 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
         k_end = run.y + run.z;
     } else {
         p = single;
+        // a launch may spread its tokens over workgroups (gridDim.y groups of B tokens each): the group's B tokens
+        p.x_q8 += size_t(blockIdx.y) * B * p.n_in;
+        p.x_scales += size_t(blockIdx.y) * B * (p.n_in >> 5);
+        p.y += size_t(blockIdx.y) * B * p.y_stride;
         k = w_idx * tiles_per_wave < p.n_tiles ? w_idx * tiles_per_wave : p.n_tiles;
         k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
     }
@@ -635,12 +639,12 @@ int dispatch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
 template <int B>
 int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_waves,
                 uint32_t wpg,
-                uint32_t tiles_per_wave, uint32_t max_n_oct, hipStream_t s) {
+                uint32_t tiles_per_wave, uint32_t max_n_oct, hipStream_t s, uint32_t token_groups = 1) {
     const size_t lds_bytes = size_t(B) * max_n_oct * 288;
     if (lds_bytes > 64 * 1024)
         return rmi_fail(RMI_HIP_E_INVALID, "activation of %d tokens x %u elements does not fit the LDS staging", B,
                         max_n_oct * 256);
-    const dim3 grid_single((n_waves + wpg - 1) / wpg), grid_group(n_waves / wpg), block(64 * wpg);
+    const dim3 grid_single((n_waves + wpg - 1) / wpg, token_groups), grid_group(n_waves / wpg), block(64 * wpg);
     // the grouped run table is padded to whole workgroups
     if (single && wpg == 1)
         hipLaunchKernelGGL((gemv_q8_0_kernel<B, false, 64>), grid_single, block, lds_bytes, s, *single, d_list, d_runs,
@@ -658,18 +662,20 @@ int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, cons
     return RMI_HIP_OK;
 }
 
+// token_groups > 1 (single problems only): n_tokens is the tokens of one group, the launch covers token_groups of them
 int dispatch_gemv(uint32_t n_tokens, const RmiGemvProblem *single, const RmiGemvProblem *d_list, const uint4 *d_runs,
-                  uint32_t n_waves, uint32_t wpg, uint32_t tiles_per_wave, uint32_t max_n_oct, hipStream_t s) {
+                  uint32_t n_waves, uint32_t wpg, uint32_t tiles_per_wave, uint32_t max_n_oct, hipStream_t s,
+                  uint32_t token_groups = 1) {
     if (n_waves == 0) return RMI_HIP_OK;
     switch (n_tokens) {
-        case 1: return launch_gemv<1>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s);
-        case 2: return launch_gemv<2>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s);
-        case 3: return launch_gemv<3>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s);
-        case 4: return launch_gemv<4>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s);
-        case 5: return launch_gemv<5>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s);
-        case 6: return launch_gemv<6>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s);
-        case 7: return launch_gemv<7>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s);
-        case 8: return launch_gemv<8>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s);
+        case 1: return launch_gemv<1>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s, token_groups);
+        case 2: return launch_gemv<2>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s, token_groups);
+        case 3: return launch_gemv<3>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s, token_groups);
+        case 4: return launch_gemv<4>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s, token_groups);
+        case 5: return launch_gemv<5>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s, token_groups);
+        case 6: return launch_gemv<6>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s, token_groups);
+        case 7: return launch_gemv<7>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s, token_groups);
+        case 8: return launch_gemv<8>(single, d_list, d_runs, n_waves, wpg, tiles_per_wave, max_n_oct, s, token_groups);
         default: return rmi_fail(RMI_HIP_E_INVALID, "gemv takes 1..8 tokens per launch, got %u", n_tokens);
     }
 }
@@ -813,12 +819,29 @@ int rmi_launch_copy(const void *src, void *dst, size_t nbytes, hipStream_t s) {
     return RMI_HIP_OK;
 }
 
-int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s) {
-    if (p.n_tiles == 0 || p.n_oct == 0) return RMI_HIP_OK;
-    if (n_tokens == 1 && p.n_oct <= kDeepMaxOct && p.n_tiles <= kDeepMaxTiles) return dispatch_gemv_deep(p, s);
+// token_groups groups of n_tokens tokens each (n_tokens <= 8), consecutive in x_q8, x_scales and y, in one launch
+int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s, uint32_t token_groups) {
+    if (p.n_tiles == 0 || p.n_oct == 0 || token_groups == 0) return RMI_HIP_OK;
+    if (n_tokens == 1 && token_groups == 1 && p.n_oct <= kDeepMaxOct && p.n_tiles <= kDeepMaxTiles) return dispatch_gemv_deep(p, s);
     const uint32_t tpw = rmi_gemv_tiles_per_wave(p.n_oct, p.n_tiles, n_tokens);
-    const uint32_t wpg = rmi_gemv_waves_per_group(size_t(n_tokens) * p.n_oct * 288, size_t(tpw) * p.n_oct * kOctetBytes);
-    return dispatch_gemv(n_tokens, &p, nullptr, nullptr, (p.n_tiles + tpw - 1) / tpw, wpg, tpw, p.n_oct, s);
+    const uint32_t n_waves = (p.n_tiles + tpw - 1) / tpw, cus = uint32_t(rmi_device_cus() > 0 ? rmi_device_cus() : 1);
+    {
+        // A matrix of a few MB at several tokens is a launch of a few hundred waves with a long instruction stream
+        // each (the x86-64 order costs about 30 vector instructions a token and octet): its tokens are spread over
+        // workgroups, two or four to each, which re-read the weight from L2 and finish in a half or a quarter of
+        // the time (every token's result is that of any other grouping: a token has its own accumulators).
+        uint32_t per_group = n_tokens, groups = token_groups;
+        while (per_group > 2 && per_group % 2 == 0 && n_waves * groups < 4 * cus) {
+            per_group >>= 1;
+            groups <<= 1;
+        }
+        if (groups > 1) return dispatch_gemv(per_group, &p, nullptr, nullptr, n_waves, 1, tpw, p.n_oct, s, groups);
+    }
+    uint32_t wpg = rmi_gemv_waves_per_group(size_t(n_tokens) * p.n_oct * 288, size_t(tpw) * p.n_oct * kOctetBytes);
+    // a launch with fewer waves than would give every compute unit a workgroup of that size is bound by latency,
+    // not by the staging it shares: smaller workgroups on more compute units
+    while (wpg > 1 && n_waves / wpg < cus) wpg >>= 1;
+    return dispatch_gemv(n_tokens, &p, nullptr, nullptr, n_waves, wpg, tpw, p.n_oct, s);
 }
 
 bool rmi_gemv_q8_0_norm_fusable(const rmi_hip_weight *w) {

@@ -176,7 +176,8 @@ struct RmiGemvProblem {
     uint32_t n_tiles;      // tiles touched
     uint32_t reserved;
 };
-int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s);
+// token_groups groups of n_tokens (<= 8) tokens each, consecutive in the problem's arrays, in one launch
+int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipStream_t s, uint32_t token_groups = 1);
 // rows [row_start,row_end) of n_tokens tokens of a Q8_0 or Q4_0 weight, as many GEMV launches (x86-64 order) as
 // the LDS staging of the tokens asks for; device pointers, nothing allocated
 bool rmi_gemv_q8_0_tokens_fits(const rmi_hip_weight *w);

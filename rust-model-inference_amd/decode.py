@@ -78,8 +78,9 @@ class Qwen3Session:
         hip.check(hip.lib.rmi_hip_qwen3_set_stop_ids(self._h, hip.ptr(ids, hip._u32p), ids.size))
 
     def set_prompt_passes(self, enabled):
-        """Prompt positions eight to a pass (the default) or every position its own step; same results either way."""
-        hip.check(hip.lib.rmi_hip_qwen3_set_prompt_passes(self._h, 1 if enabled else 0))
+        """Prompt positions 128 to a pass (True, the default), every position its own step (False), or that many to a
+        pass (an int above 1, at most 128); same results either way."""
+        hip.check(hip.lib.rmi_hip_qwen3_set_prompt_passes(self._h, int(enabled)))
 
     def generate(self, prompt, max_new, dump_steps=()):
         prompt = np.ascontiguousarray(prompt, np.uint32)

@@ -140,24 +140,24 @@ def test_long_context_device_decode_crosses_the_attention_split(hip, oracle, tmp
 
 
 def test_prompt_passes_change_no_bit(hip, oracle, tmp_path):
-    """Eight prompt positions to a pass against every position its own step: tokens, every step's argmax and top-2
-    logits and every dumped step's logits identical, for prompts that end inside a pass, on a pass boundary and
-    before the first pass is full; and equal to the CPU loop's."""
+    """Prompt positions 128 (or 7, 8, 16, 32) to a pass against every position its own step: tokens, every step's
+    argmax and top-2 logits and every dumped step's logits identical, for prompts that end inside a pass, on a pass
+    boundary and before the first pass is full; and equal to the CPU loop's."""
     kw = dict(n_layer=3, n_embd=512, n_head=8, n_head_kv=4, head_dim=128, n_ff=1024, vocab=5000, n_ctx=4096)
     f = _write_model(hip, tmp_path, **kw)
     pool = oracle.Pool(8)
     sess = hip.decode.Qwen3Session(f.metadata, _tensors(f), capacity=96)
-    for n_prompt in (1, 5, 8, 9, 40, 43):
+    for n_prompt, per_pass in ((1, True), (5, True), (8, 8), (9, 8), (32, 32), (33, 32), (40, 16), (43, 7), (70, True), (75, 32)):
         prompt = np.random.default_rng(60 + n_prompt).integers(0, 5000, n_prompt, dtype=np.uint32)
         steps = list(range(n_prompt + 11))
-        sess.set_prompt_passes(True)
+        sess.set_prompt_passes(per_pass)
         fast = sess.generate(prompt, 12, dump_steps=steps)
         sess.set_prompt_passes(False)
         slow = sess.generate(prompt, 12, dump_steps=steps)
         assert np.array_equal(fast["tokens"], slow["tokens"]), n_prompt
         assert np.array_equal(fast["argmax"], slow["argmax"]) and np.array_equal(fast["top2"].view(np.uint32), slow["top2"].view(np.uint32))
         assert np.array_equal(fast["dump"].view(np.uint32), slow["dump"].view(np.uint32)), n_prompt
-        if n_prompt in (9, 43):
+        if n_prompt in (9, 43, 75):
             cpu = oracle.Qwen3Decoder(f.metadata, _tensors(f), pool).generate(prompt, 12, dump_steps=steps)
             _compare(cpu, fast, f"prompt passes, {n_prompt} prompt tokens")
     sess.set_prompt_passes(True)
