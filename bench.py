@@ -215,13 +215,15 @@ def cpu_baseline(problems, batch, alg_bytes):
     }, outs
 
 
-def read_traffic(name):
+def read_traffic(name, case=""):
     """HBM bytes per launch as rocprofv3 --pmc measured them when profiles/<name>_pmc.txt was recorded: a figure
-    read back from that file, not measured by this run.  Returns {"traffic": bytes or None, "traffic_source": ..}."""
+    read back from that file, not measured by this run.  A file that covers several workloads names the case in the
+    key ("traffic_bytes_per_launch_m512:").  Returns {"traffic": bytes or None, "traffic_source": ..}."""
     rel = os.path.join("profiles", f"{name}_pmc.txt")
+    key = f"traffic_bytes_per_launch{'_' + case if case else ''}:"
     try:
         for line in open(os.path.join(ROOT, rel)):
-            if line.startswith("traffic_bytes_per_launch:"):
+            if line.startswith(key):
                 return {"traffic": float(line.split(":")[1]),
                         "traffic_source": f"{rel} (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, recorded earlier; "
                                           "not measured in this run)"}
@@ -553,7 +555,8 @@ def run_gemm(args, pkg, ev):
                           "achieved": round(achieved, 1), "peak": INT8_MFMA_PEAK_TOPS,
                           "unit": "TOP/s", "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
                           "avg_launch_us": round(dev_ms * 1e3 / 2, 3),
-                          **read_traffic(f"gemm_q8_0_m{M}_qwen3_0.6b_ffn")}
+                          **(read_traffic("gemm_q8_0_m2048_qwen3_0.6b_ffn") if M == 2048 else
+                             read_traffic("gemm_q8_0_m64_m512_qwen3_0.6b_ffn", f"m{M}"))}
     w2, d2 = time_region(H, ev, lambda: step(other), args.steps, args.warmup)
     result["other_mode"] = {"mode": "exact (tiled kernel, single chain)" if fast else "fast (kernel chosen per product)",
                             "value": round(ops / w2 / 1e12, 1), "unit": "TOP/s", "avg_launch_us": round(d2 * 1e3 / 2, 3)}
@@ -858,7 +861,7 @@ def run_q4k_gemm(args, pkg, ev):
         "tokens": M, "launches_per_step": 3, "ops_per_step": ops, "device": dev_name.strip(), "compute_units": cus})
     result["roofline"] = {"bound": "mfma", "kernel": "gemm_q4_k_kernel", "achieved": round(achieved, 1),
                           "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s", "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
-                          "avg_launch_us": round(dev_ms * 1e3 / 3, 3), **read_traffic(f"gemm_q4_k_m{M}_1.7b_ffn")}
+                          "avg_launch_us": round(dev_ms * 1e3 / 3, 3), **read_traffic("gemm_q4_k_m512_m2048_1.7b_ffn", f"m{M}")}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
@@ -970,15 +973,19 @@ def run_decode(args, pkg, ev):
     result["ms_per_token_step"] = round(per_token * 1e3, 4)
     # the two phases apart: the prompt (positions known in advance: the session takes them 128 to a pass, each
     # position's logits still computed and bit-identical to its own step) and the generated tokens (one step each)
-    t_prompt = min(sess.generate(prompt, 1)["seconds"] for _ in range(2))
-    t_all = min(last["seconds"], sess.generate(prompt, n_new)["seconds"])
-    result["phases"] = {"prompt_positions_per_s": round(n_prompt / t_prompt, 1), "prompt_ms_per_position": round(t_prompt / n_prompt * 1e3, 4),
-                        "generated_tokens_per_s": round((n_new - 1) / (t_all - t_prompt), 1),
-                        "generated_ms_per_token": round((t_all - t_prompt) / (n_new - 1) * 1e3, 4)}
-    sess.set_prompt_passes(False)
-    t_steps = sess.generate(prompt, n_new)["seconds"]
-    sess.set_prompt_passes(True)
-    result["phases"]["every_position_its_own_step_tok_s"] = round(token_steps / t_steps, 1)
+    if args.no_phases:
+        t_prompt = None
+    else:
+        t_prompt = min(sess.generate(prompt, 1)["seconds"] for _ in range(2))
+    if t_prompt is not None:
+        t_all = min(last["seconds"], sess.generate(prompt, n_new)["seconds"])
+        result["phases"] = {"prompt_positions_per_s": round(n_prompt / t_prompt, 1), "prompt_ms_per_position": round(t_prompt / n_prompt * 1e3, 4),
+                            "generated_tokens_per_s": round((n_new - 1) / (t_all - t_prompt), 1),
+                            "generated_ms_per_token": round((t_all - t_prompt) / (n_new - 1) * 1e3, 4)}
+        sess.set_prompt_passes(False)
+        t_steps = sess.generate(prompt, n_new)["seconds"]
+        sess.set_prompt_passes(True)
+        result["phases"]["every_position_its_own_step_tok_s"] = round(token_steps / t_steps, 1)
     achieved = alg / per_token / 1e9
     result["roofline"] = {"bound": "hbm", "kernel": "Q8_0 GEMV kernels (4 per layer + lm_head = 113 launches per token-step)",
                           "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -1038,6 +1045,8 @@ def main():
                     help="also launch the plain copy kernel on this many MiB, 5 times, outside the timed region "
                          "(the known-size kernel that rocprofv3 --pmc traffic counters are scaled against)")
     ap.add_argument("--extra", action="store_true", help="also time the other launch modes, outside the timed region")
+    ap.add_argument("--no-phases", action="store_true",
+                    help="decode: skip the extra generations that time the prompt and the generated tokens apart")
     ap.add_argument("--no-decode", action="store_true",
                     help="projection_set only: skip the end-to-end decode figure that is attached to the JSON line")
     ap.add_argument("--no-configs", action="store_true",
@@ -1069,7 +1078,7 @@ def main():
         sub = argparse.Namespace(**vars(args))
         sub.steps, sub.warmup = 2, 1
         d = run_decode(sub, pkg, ev)
-        result["decode"] = {"value": d["value"], "unit": d["unit"], "ms_per_token_step": d["ms_per_token_step"], "phases": d["phases"],
+        result["decode"] = {"value": d["value"], "unit": d["unit"], "ms_per_token_step": d["ms_per_token_step"], "phases": d.get("phases"),
                             "workload": d["config"]["workload"], "generations_timed": sub.steps,
                             "roofline": d["roofline"], "cpu_baseline": d.get("cpu_baseline")}
     if args.workload == "projection_set" and not args.no_configs and args.batch == 1 and args.mode == "grouped" \
