@@ -4,16 +4,29 @@
 The compiler's hazard recogniser does not look into inline asm, and on this target a DPP operand must not be read
 sooner than two wait states after a vector instruction wrote that register, nor sooner than five after a vector
 instruction wrote EXEC.  This script walks the assembly (`hipcc -S --cuda-device-only`) and fails if any DPP
-instruction, hand-written or not, comes too early.  Usage: check_dpp_hazards.py file.s [minimum count of
-v_fmac_f32_dpp expected]."""
+instruction, hand-written or not, comes too early: along the text order (the fall-through path; after an
+unconditional branch this is stricter than needed, never laxer) and along every branch, i.e. from the instructions
+in front of each `s_branch` / `s_cbranch_*` to those behind its target label.  Indirect jumps (`s_setpc_b64`,
+`s_swappc_b64`) are refused: their targets are not in the text.
+
+These two rules are the hazards of the one instruction class this build writes by hand (VALU with a DPP source).
+Whoever adds another hand-written class (an `s_waitcnt`-sensitive memory instruction, an MFMA with its own
+dependency wait states, writes of M0 or VCC in front of their readers, ...) has to add that class's rules here:
+the script knows nothing of hazards it was not told about.
+
+Usage: check_dpp_hazards.py file.s [minimum count of v_fmac_f32_dpp expected]."""
 import re
 import sys
 
 
 def instructions(path):
+    """The instructions in text order; a label is yielded as ("label", name)."""
     for raw in open(path):
         line = raw.split(";")[0].split("//")[0].strip()
-        if not line or line.startswith(".") or line.endswith(":"):
+        if line.endswith(":"):  # labels first: local ones start with a dot, as directives do
+            yield ("label", line[:-1])
+            continue
+        if not line or line.startswith("."):
             continue
         yield line
 
@@ -43,31 +56,64 @@ def wait_states(ins):
     return int(m.group(1)) + 1 if m else 1
 
 
+REACH = 8  # instructions looked at on either side of a point: more than five wait states in any case
+
+
+def hazards(seq, first_checked=0):
+    """(earlier instruction, DPP instruction, wait states between) for every DPP instruction of seq from index
+    first_checked on that reads its operand too early after an instruction of seq in front of it."""
+    bad = []
+    for k in range(first_checked, len(seq)):
+        src = dpp_source(seq[k])
+        if src is None:
+            continue
+        between = 0  # wait states between an earlier instruction and this one
+        for prev in reversed(seq[max(0, k - REACH):k]):
+            if between < 2 and src in written_vgprs(prev):
+                bad.append((prev, seq[k], between))
+            if between < 5 and writes_exec(prev):
+                bad.append((prev, seq[k], between))
+            between += wait_states(prev)
+            if between >= 5:
+                break
+    return bad
+
+
+def branch_target(ins):
+    m = re.match(r"s_c?branch\w*\s+(\S+)", ins)
+    return m.group(1) if m else None
+
+
 def main():
     path = sys.argv[1]
     want = int(sys.argv[2]) if len(sys.argv) > 2 else 0
-    window, bad, n_dpp, n_fmac = [], [], 0, 0
-    for ins in instructions(path):
-        src = dpp_source(ins)
-        if src is not None:
-            n_dpp += 1
-            n_fmac += ins.startswith("v_fmac_f32_dpp")
-            between = 0  # wait states between an earlier instruction and this one
-            for prev in reversed(window):
-                if between < 2 and src in written_vgprs(prev):
-                    bad.append((prev, ins, between))
-                if between < 5 and writes_exec(prev):
-                    bad.append((prev, ins, between))
-                between += wait_states(prev)
-                if between >= 5:
-                    break
-        window.append(ins)
-        if len(window) > 8:
-            window.pop(0)
+    code, labels = [], {}
+    for item in instructions(path):
+        if isinstance(item, tuple):
+            labels[item[1]] = len(code)  # index of the first instruction behind the label
+        else:
+            code.append(item)
+    n_dpp = sum(dpp_source(ins) is not None for ins in code)
+    n_fmac = sum(ins.startswith("v_fmac_f32_dpp") for ins in code)
+    bad = hazards(code)
+    unknown = [ins for ins in code if ins.startswith(("s_setpc_b64", "s_swappc_b64"))]
+    for k, ins in enumerate(code):
+        target = branch_target(ins)
+        if target is None:
+            continue
+        if target not in labels:
+            unknown.append(ins)
+            continue
+        head = code[max(0, k + 1 - REACH):k + 1]  # up to and including the branch, which is a wait state itself
+        tail = code[labels[target]:labels[target] + REACH]
+        bad += hazards(head + tail, first_checked=len(head))
+    bad = sorted(set(bad))
     for prev, ins, between in bad[:20]:
         print("hazard: %d wait state(s) between\n    %s\nand\n    %s" % (between, prev, ins))
+    for ins in unknown[:20]:
+        print("cannot follow: %s" % ins)
     print("%s: %d DPP instructions (%d v_fmac_f32_dpp), %d hazards" % (path, n_dpp, n_fmac, len(bad)))
-    if bad or n_fmac < want:
+    if bad or unknown or n_fmac < want:
         sys.exit(1)
 
 

@@ -978,7 +978,10 @@ __global__ __launch_bounds__(kAttnSplitThreads) void attn128_weights_pv_kernel(
     __syncthreads();
     // The first wave alone hands the part's sums over: its stores, one release (the other waves have nothing in
     // flight that anybody reads), its count.  The part that counts last has every part's sums in reach after one
-    // acquire, adds them in part order and quantizes.  Nobody waits for anybody.
+    // acquire, adds them in part order and quantizes.  Nobody waits for anybody.  The pair is written in its fence
+    // form: an agent-scope fence in front of a relaxed counter update releases, the same fence behind the update that
+    // read the last count acquires; the 64 storing lanes are one wave, whose fence covers the stores of all of them.
+    // (An acq_rel update would put a second write-back in front of the acquire that nothing needs.)
     if (tid >= 64) return;
     double *mine = ws.part_sums + (size_t(head) * kAttnSplitMaxParts + part) * 128;
 #pragma unroll

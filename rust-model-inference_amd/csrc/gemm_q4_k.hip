@@ -454,7 +454,7 @@ void launch(const rmi_hip_weight *w, const float *d, const int8_t *qs, const int
 
 // Two groups of waves per tile, on the even and the odd super-blocks: where the 32-token tiles are no more than the
 // chip has compute units and each group still has eight super-blocks or more (measured at 2048 x 6144, 512 tokens:
-// 29.5 -> about 16 us).  RMI_Q4K_GEMM_GROUPS = 1 or 2 forces a count where the row allows it.
+// 29.5 -> 24.3 us).  RMI_Q4K_GEMM_GROUPS = 1 or 2 forces a count where the row allows it.
 static int gemm_q4_k_groups(const rmi_hip_weight *w, uint32_t n_tokens) {
     const uint64_t groups32 = uint64_t((w->n_out + 127) / 128) * ((n_tokens + 31) / 32);
     const char *e = getenv("RMI_Q4K_GEMM_GROUPS");

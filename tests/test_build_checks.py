@@ -53,3 +53,24 @@ def test_vector_write_of_exec_fails(tmp_path):
 def test_missing_instructions_fail(tmp_path):
     """The build names how many v_fmac_f32_dpp it expects: a compile that silently dropped them does not pass."""
     assert _run(tmp_path, ["v_mul_f32_e32 v3, v1, v2"], "1000").returncode == 1
+
+
+def test_hazard_across_a_branch_fails(tmp_path):
+    """The write sits in front of a branch and the DPP read behind its target: text order alone would not see it."""
+    body = ["v_mul_f32_e32 v3, v1, v2", "s_cbranch_scc1 .LBB0_2", "s_nop 7", "s_nop 7", "s_branch .LBB0_3",
+            ".LBB0_2:", FMAC, ".LBB0_3:"]
+    r = _run(tmp_path, body)
+    assert r.returncode == 1 and "hazard: 1 wait state(s)" in r.stdout, r.stdout
+    body[0:2] = ["v_mul_f32_e32 v3, v1, v2", "s_nop 0", "s_cbranch_scc1 .LBB0_2"]  # two wait states: enough
+    assert _run(tmp_path, body).returncode == 0
+
+
+def test_loop_back_edge_is_followed(tmp_path):
+    body = [".LBB0_1:", FMAC, "v_add_u32_e32 v20, v21, v22", "v_mul_f32_e32 v3, v1, v2", "s_cbranch_vccnz .LBB0_1"]
+    assert _run(tmp_path, body).returncode == 1
+    body = [".LBB0_1:", FMAC, "v_mul_f32_e32 v3, v1, v2", "v_add_u32_e32 v20, v21, v22", "s_cbranch_vccnz .LBB0_1"]
+    assert _run(tmp_path, body).returncode == 0
+
+
+def test_indirect_jump_is_refused(tmp_path):
+    assert _run(tmp_path, ["s_setpc_b64 s[30:31]"]).returncode == 1
