@@ -279,9 +279,9 @@ int rmi_hip_gemm_q8_0_ksplit_dev(const rmi_hip_weight *w, const int8_t *x_q8, co
 uint32_t rmi_hip_gemm_q8_0_ksplit_quads_per_part(uint32_t n_in);
 /* The prefill product for callers that ask for the reference's tolerance rather than one host's bits: the library
  * takes what it expects to be fastest for this product, the k-split kernel above (few tokens, long rows), the tiled
- * kernel of rmi_hip_gemm_q8_0_dev, or that kernel with two groups of waves per tile that take the even and the odd
- * quads of a row (a chain per group, the groups' sums added in group order), which gives a product of a few hundred
- * tokens larger tiles on every compute unit.  Every output is built from exact integer block dots, deterministic,
+ * kernel of rmi_hip_gemm_q8_0_dev, or that kernel with two or four groups of waves per tile, group g of G taking the
+ * quads g, g + G, ... of a row (a chain per group, the groups' sums added in group order), which puts every compute
+ * unit to work on a product of a few hundred tokens.  Every output is built from exact integer block dots, deterministic,
  * and within 1e-4 + 1e-4 |ref| of the CPU kernels; which chain a token's result follows depends on the token count
  * of the call.  rmi_hip_gemm_q8_0_fast_plan says which one a call would take: RMI_HIP_GEMM_PLAN_* and, in *param,
  * the quads per run (k-split) or the number of interleaved groups (tiled). */

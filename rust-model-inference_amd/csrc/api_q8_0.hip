@@ -403,7 +403,7 @@ int rmi_hip_gemm_q8_0_ksplit_dev(const rmi_hip_weight *w, const int8_t *x_q8, co
 static int fast_plan(const rmi_hip_weight *w, uint32_t n_tokens, uint32_t *param) {
     uint32_t groups = 1;
     const double tiled = rmi_gemm_q8_0_cost_us(w, n_tokens, false, &groups);
-    if (tiled < 0.0 || rmi_gemm_q8_0_ksplit_cost_us(w, n_tokens) < tiled) {
+    if (tiled < 0.0 || (!rmi_gemm_q8_0_shape_forced() && rmi_gemm_q8_0_ksplit_cost_us(w, n_tokens) < tiled)) {
         uint32_t per = 1, n_waves = 1;
         rmi_gemm_q8_0_ksplit_shape(w->n_in, &per, &n_waves);
         *param = per;

@@ -500,7 +500,9 @@ struct GemmPlan {
 // leave compute units idle.  single_chain: only the shapes that keep one f32 chain per output.
 GemmPlan plan_gemm(const rmi_hip_weight *w, uint32_t n_tokens, bool single_chain) {
     static const GemmShape shapes[] = {make_shape<3, 1, 1, 4, 2>(),    make_shape<2, 1, 1, 4, 2>(),    make_shape<1, 1, 2, 2, 3>(),
-                                       make_shape<3, 1, 1, 4, 2, 2>(), make_shape<2, 1, 1, 4, 2, 2>(), make_shape<1, 1, 2, 2, 2, 2>()};
+                                       make_shape<3, 1, 1, 4, 2, 2>(), make_shape<2, 1, 1, 4, 2, 2>(), make_shape<1, 1, 2, 2, 2, 2>(),
+                                       make_shape<1, 1, 2, 1, 2, 4>()};
+    constexpr int kShapes = int(sizeof(shapes) / sizeof(shapes[0]));
     const uint64_t cus = uint64_t(rmi_device_cus() > 0 ? rmi_device_cus() : 1);
     const uint32_t n_quads = (w->n_in / 32 + 3) / 4;
     const bool whole_quads = (w->n_in / 32) % 4 == 0;
@@ -510,10 +512,12 @@ GemmPlan plan_gemm(const rmi_hip_weight *w, uint32_t n_tokens, bool single_chain
         return e ? atoi(e) : -1;
     }();
     for (const GemmShape &g : shapes) {
-        if (forced >= 0 && !single_chain && &g != &shapes[forced % 6]) continue;
+        if (forced >= 0 && !single_chain && &g != &shapes[forced % kShapes]) continue;
         // groups pay off on long rows only (measured: 1024 x 3072 gains 10-15 % from 768 tokens on, 3072 x 1024 loses
-        // 3-10 %: a group needs about eight quads to make up for its own first loads and the last add)
-        if (g.ks > 1 && (single_chain || !whole_quads || n_quads % g.ks != 0 || n_quads / g.ks < 8)) continue;
+        // 3-10 %: a group needs about eight quads to make up for its own first loads and the last add; four groups
+        // of a 64 x 32 tile, one workgroup of eight waves a compute unit, with six quads each: 1024 x 3072 at 512
+        // tokens 11.2 us against 12.7 for the k-split kernel and 17.6 for the single chain)
+        if (g.ks > 1 && (single_chain || !whole_quads || n_quads % g.ks != 0 || (forced < 0 && n_quads / g.ks < (g.ks == 4 ? 6 : 8)))) continue;
         const uint64_t groups = uint64_t((w->n_out + g.tile_n - 1) / g.tile_n) * ((n_tokens + g.tile_t - 1) / g.tile_t);
         if (groups > 0x7fffffffull) continue;
         const double nb = double(w->n_in / 32) / double(g.ks);
@@ -539,6 +543,8 @@ GemmPlan plan_gemm(const rmi_hip_weight *w, uint32_t n_tokens, bool single_chain
 
 // the launch time the tile chooser expects for this product, in microseconds (a negative value: no shape fits), and
 // the number of groups that split the quads in the shape it takes
+bool rmi_gemm_q8_0_shape_forced() { return getenv("RMI_GEMM_SHAPE") != nullptr; }
+
 double rmi_gemm_q8_0_cost_us(const rmi_hip_weight *w, uint32_t n_tokens, bool single_chain, uint32_t *groups) {
     if (groups) *groups = 1;
     if (n_tokens == 0 || w->n_out == 0 || w->n_in < 32) return 0.0;

@@ -235,6 +235,7 @@ int rmi_launch_gemm_q8_0(const rmi_hip_weight *w, const int8_t *x_q8, const floa
 // waves' sums added in wave order (gemm_q8_0_ksplit.hip; within rounding of the single-chain result)
 void rmi_gemm_q8_0_ksplit_shape(uint32_t n_in, uint32_t *quads_per_wave, uint32_t *n_waves);
 // what either kernel expects a launch to take, in microseconds (rmi_gemm_q8_0_cost_us < 0: no tile shape fits)
+bool rmi_gemm_q8_0_shape_forced();  // measurements: RMI_GEMM_SHAPE is set, the fast plan keeps to the tiled kernel
 double rmi_gemm_q8_0_cost_us(const rmi_hip_weight *w, uint32_t n_tokens, bool single_chain, uint32_t *groups);
 int rmi_launch_gemm_q8_0_grouped(const rmi_hip_weight *w, const int8_t *x_q8, const float *x_scales, float *y,
                                  uint32_t n_tokens, uint32_t y_stride, hipStream_t s);
