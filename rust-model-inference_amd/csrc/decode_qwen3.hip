@@ -452,11 +452,13 @@ __device__ __forceinline__ double quad_sum(double v) {  // (l0 + l1) + (l2 + l3)
     v += __hiloint2double(__builtin_amdgcn_mov_dpp(hi, 0x4E, 0xf, 0xf, true), __builtin_amdgcn_mov_dpp(lo, 0x4E, 0xf, 0xf, true));
     return v;
 }
-__device__ __forceinline__ double swizzle_xor16_f64(double v) {  // the value of lane ^ 16
-    constexpr int kXor16 = 0x1f | (16 << 10);
-    return __hiloint2double(__builtin_amdgcn_ds_swizzle(__double2hiint(v), kXor16),
-                            __builtin_amdgcn_ds_swizzle(__double2loint(v), kXor16));
+template <int XOR>
+__device__ __forceinline__ double swizzle_xor_f64(double v) {  // the value of lane ^ XOR (XOR < 32)
+    constexpr int kPattern = 0x1f | (XOR << 10);
+    return __hiloint2double(__builtin_amdgcn_ds_swizzle(__double2hiint(v), kPattern),
+                            __builtin_amdgcn_ds_swizzle(__double2loint(v), kPattern));
 }
+__device__ __forceinline__ double swizzle_xor16_f64(double v) { return swizzle_xor_f64<16>(v); }
 __host__ __device__ inline size_t attn128_lds_bytes(uint32_t n_keys) {
     const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
     return n_pad * 12 + (kA128Threads / 64) * 128 * 8 + 128;  // 32 floats of room behind the scores
@@ -467,6 +469,12 @@ __host__ __device__ inline size_t attn128_lds_bytes(uint32_t n_keys) {
 // and 2 turn the head's q, its key/value head's new k and new v into f16 while the first cached keys are on their
 // way, the new key and value are used from LDS (and written to their cache row by the first query head of each
 // key/value head), the keys 0..step-1 come from the cache as before.
+// PVP > 1 (single-position launches): PVP workgroups per head.  Each computes every score, the maximum, the
+// exponentials and the sequential sum of the head for itself (exchanging them would cost more than repeating them)
+// and then the p.v sums of 128 / PVP of the output dimensions only, over four times as many key slices: the part of
+// the launch that is vector arithmetic on one compute unit shrinks by PVP.  A part's dimensions are whole 32-value
+// blocks of the quantizer.  Workgroup ids run key/value head fastest, so that on a chip of eight XCDs and a model of
+// eight key/value heads every workgroup that reads a head's cache rows shares one L2.
 struct AttnFromQkv {
     const float *qkv;                // [n_head * 128 q | n_head_kv * 128 k | n_head_kv * 128 v]
     const float *q_norm, *k_norm;    // [128] each, or null
@@ -474,7 +482,7 @@ struct AttnFromQkv {
     uint16_t *k_row, *v_row;         // the cache rows of this position, [n_head_kv][128] each
     float eps;
 };
-template <bool FROM_QKV>
+template <bool FROM_QKV, int PVP = 1>
 __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
     uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, int8_t *__restrict__ q8,
@@ -488,8 +496,14 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     q16 += size_t(blockIdx.z) * tok_q16_stride;
     q8 += size_t(blockIdx.z) * tok_out_stride;
     scales += size_t(blockIdx.z) * (tok_out_stride >> 5);
-    // grid = (query heads per key/value head, key/value heads)
-    const uint32_t kvh = blockIdx.y, head = blockIdx.y * gridDim.x + blockIdx.x, tid = threadIdx.x;
+    // grid = (query heads per key/value head, key/value heads), or with PVP parts n_head * PVP workgroups in a row:
+    // key/value head fastest, then the query head of its group, then the part
+    static_assert(PVP == 1 || PVP == 2 || PVP == 4, "a part is one, two or four blocks of 32 dimensions");
+    const uint32_t tid = threadIdx.x, hpk = n_head / n_head_kv;
+    const uint32_t kvh = PVP == 1 ? blockIdx.y : blockIdx.x % n_head_kv;
+    const uint32_t qh = PVP == 1 ? blockIdx.x : (blockIdx.x / n_head_kv) % hpk;
+    const uint32_t pv_part = PVP == 1 ? 0u : blockIdx.x / n_head_kv / hpk;
+    const uint32_t head = kvh * hpk + qh;
     const uint32_t n_keys = step + 1;
     // keys that come from the cache, and the last row there that may be read
     const uint32_t n_cached = FROM_QKV ? step : n_keys, last_row = n_cached ? n_cached - 1 : 0;
@@ -535,11 +549,13 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
         for (int c = 0; c < 4; c++) kk[c] = key[4 * c];
     }
     // values: lane = (8 dimensions dg, key slice sl): 16 consecutive lanes read the 256 bytes of one row
-    constexpr uint32_t kPre = kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40);
-    const uint32_t dg = tid & 15, sl = tid >> 4;
-    const uint32_t chunk = (n_cached + kA128Threads / 16 - 1) / (kA128Threads / 16);
+    // (with PVP parts: 16 / PVP lanes read the part's 256 / PVP bytes of a row, PVP times as many slices)
+    constexpr uint32_t kDgLanes = 16 / PVP, kSlices = kA128Threads / kDgLanes;
+    constexpr uint32_t kPre = (kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40)) / (PVP == 1 ? 1 : 2);
+    const uint32_t dg = tid % kDgLanes, sl = tid / kDgLanes;
+    const uint32_t chunk = (n_cached + kSlices - 1) / kSlices;
     const uint32_t t_begin = sl * chunk, t_end = t_begin + chunk < n_cached ? t_begin + chunk : n_cached;
-    const uint4 *vbase = reinterpret_cast<const uint4 *>(v_cache + size_t(kvh) * 128 + dg * 8);
+    const uint4 *vbase = reinterpret_cast<const uint4 *>(v_cache + size_t(kvh) * 128 + pv_part * (128 / PVP) + dg * 8);
     uint4 vp[kPre];
 #pragma unroll
     for (uint32_t j = 0; j < kPre; j++) {  // j < chunk is uniform: no lane waits on a guarded load of its own
@@ -575,7 +591,7 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
             }
             new16[which][lane] = h0;
             new16[which][lane + 64] = h1;
-            if (which && blockIdx.x == 0) {  // the first query head of the key/value head fills the cache row
+            if (which && qh == 0 && pv_part == 0) {  // the first query head of the key/value head fills the cache row
                 uint16_t *dst = (which == 1 ? fq.k_row : fq.v_row) + size_t(kvh) * 128;
                 dst[lane] = h0;
                 dst[lane + 64] = h1;
@@ -711,23 +727,25 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     if constexpr (FROM_QKV) {
         if (sl == 0) {  // this step's value, from LDS: one more exact term of the f64 sums
             const double w = wd[n_cached];
-            const half8 vh = as_half8(reinterpret_cast<const uint4 *>(new16[2])[dg]);
+            const half8 vh = as_half8(reinterpret_cast<const uint4 *>(new16[2])[pv_part * kDgLanes + dg]);
 #pragma unroll
             for (int d = 0; d < 8; d++) acc[d] = __builtin_fma(double(float(vh[d])), w, acc[d]);
         }
     }
 #pragma unroll
-    for (int d = 0; d < 8; d++) {  // the four slices of a wave: lanes 16 apart
+    for (int d = 0; d < 8; d++) {  // the slices of a wave: lanes kDgLanes apart
+        if constexpr (PVP >= 4) acc[d] += swizzle_xor_f64<4>(acc[d]);
+        if constexpr (PVP >= 2) acc[d] += swizzle_xor_f64<8>(acc[d]);
         acc[d] += swizzle_xor16_f64(acc[d]);
         acc[d] += __shfl_xor(acc[d], 32, 64);
     }
-    if ((tid & 63) < 16) {
+    if ((tid & 63) < kDgLanes) {
         double *dst = part + (tid >> 6) * 128 + dg * 8;
 #pragma unroll
         for (int d = 0; d < 8; d++) dst[d] = acc[d];
     }
     __syncthreads();
-    if (tid < 32) {  // four dimensions per lane: whole 8-lane groups for the quantizer
+    if (tid < 32 / PVP) {  // four dimensions per lane: whole 8-lane groups for the quantizer
         double o[4];
 #pragma unroll
         for (int d = 0; d < 4; d++) o[d] = part[tid * 4 + d];
@@ -737,8 +755,9 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
         }
         const float4 of = make_float4(float(o[0]), float(o[1]), float(o[2]), float(o[3]));
         float sc;
-        reinterpret_cast<uint32_t *>(q8)[(size_t(head) * 128 >> 2) + tid] = rmi_quantize_block8(of, rounding, &sc);
-        if ((tid & 7) == 0) scales[(size_t(head) * 128 >> 5) + (tid >> 3)] = sc;
+        const size_t first = size_t(head) * 128 + pv_part * (128 / PVP);  // of this workgroup's output dimensions
+        reinterpret_cast<uint32_t *>(q8)[(first >> 2) + tid] = rmi_quantize_block8(of, rounding, &sc);
+        if ((tid & 7) == 0) scales[(first >> 5) + (tid >> 3)] = sc;
     }
 }
 
@@ -1019,6 +1038,26 @@ __global__ __launch_bounds__(kAttnSplitThreads) void attn128_weights_pv_kernel(
         float sc;
         reinterpret_cast<uint32_t *>(q8)[(size_t(head) * 128 >> 2) + tid] = rmi_quantize_block8(of, rounding, &sc);
         if ((tid & 7) == 0) scales[(size_t(head) * 128 >> 5) + (tid >> 3)] = sc;
+    }
+}
+
+// One position's attention straight from its f32 q | k | v: the launch with the p.v sums of a head split over parts.
+// Four parts from 64 keys on (measured over 512..638 keys, 28 layers: 0.840 ms a generated token with one part, 0.789
+// with two, 0.779 with four); below, the p.v sums are a few terms and one workgroup a head is enough.
+static int attn_pv_parts(uint32_t n_keys) { return n_keys >= 64 ? 4 : 1; }
+static void launch_attention128_from_qkv(const uint16_t *k_cache, const uint16_t *v_cache, uint32_t step, uint32_t kv_stride,
+                                         uint32_t n_head, uint32_t n_head_kv, int8_t *q8, float *scales, int rounding,
+                                         const AttnFromQkv &fq, hipStream_t st) {
+    const size_t lds = attn128_lds_bytes(step + 1);
+    const uint16_t *no_q16 = nullptr;
+    switch (attn_pv_parts(step + 1)) {
+    case 4:
+        hipLaunchKernelGGL((attention128_quant_kernel<true, 4>), dim3(n_head * 4), dim3(kA128Threads), lds, st, no_q16, k_cache,
+                           v_cache, step, kv_stride, n_head, n_head_kv, q8, scales, rounding, fq, 0u, 0u);
+        break;
+    default:
+        hipLaunchKernelGGL((attention128_quant_kernel<true, 1>), dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, st,
+                           no_q16, k_cache, v_cache, step, kv_stride, n_head, n_head_kv, q8, scales, rounding, fq, 0u, 0u);
     }
 }
 
@@ -1340,9 +1379,8 @@ int enqueue_step(rmi_hip_qwen3 *s, uint32_t step, hipStream_t st) {
             const size_t half = 64;
             const AttnFromQkv fq{s->qkv, qn, kn, s->cos_t + size_t(step) * half, s->sin_t + size_t(step) * half,
                                  s->k_cache + row, s->v_cache + row, c.eps};
-            hipLaunchKernelGGL(attention128_quant_kernel<true>, dim3(c.n_head / c.n_head_kv, c.n_head_kv), dim3(kA128Threads),
-                               attn128_lds_bytes(step + 1), st, static_cast<const uint16_t *>(nullptr), s->k_cache + layer_base,
-                               s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv, s->act_q8, s->act_scales, rnd, fq, 0u, 0u);
+            launch_attention128_from_qkv(s->k_cache + layer_base, s->v_cache + layer_base, step, s->kv_stride, c.n_head, c.n_head_kv,
+                                         s->act_q8, s->act_scales, rnd, fq, st);
         } else if (rmi_gemv_q8_0_norm_rope_fusable(s->w_qkv[l], c.n_head, c.n_head_kv, c.head_dim_k, c.head_dim_v)) {
             // norm, q/k/v products, head norms, rotation and the cache row in one launch
             const size_t half = c.head_dim_k / 2;
@@ -1613,9 +1651,8 @@ int rmi_hip_qkv_attention_f16_quantize_q8_0_dev(const float *qkv, const float *q
                         uint32_t((48 * 1024 - (kA128Threads / 64) * 128 * 8 - 128) / 12 / kAttnPad * kAttnPad));
     const size_t row = size_t(n_keys - 1) * kv_stride;
     const AttnFromQkv fq{qkv, q_norm, k_norm, cos_row, sin_row, k_cache + row, v_cache + row, eps};
-    hipLaunchKernelGGL(attention128_quant_kernel<true>, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds,
-                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(nullptr), k_cache, v_cache, n_keys - 1,
-                       kv_stride, n_head, n_head_kv, q8, scales, rounding, fq, 0u, 0u);
+    launch_attention128_from_qkv(k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding, fq,
+                                 static_cast<hipStream_t>(stream));
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
 }
