@@ -82,6 +82,46 @@ __device__ __forceinline__ void stage_token(uint32_t *dq, const int8_t *x_q8, co
     }
 }
 
+// The same for n_tokens tokens at once, tok_dw dwords apart in LDS: the pieces of all tokens are one index space, so
+// that a workgroup of eight waves has every load of a small batch in flight before the first LDS write waits (token
+// after token, each token is a memory round trip of its own).
+template <int UNROLL>
+__device__ __forceinline__ void stage_tokens(uint32_t *dq, uint32_t tok_dw, const int8_t *x_q8, const float *x_scales,
+                                             uint32_t n_tokens, uint32_t n_oct, uint32_t nb, uint32_t tid, uint32_t n_threads) {
+    gptr_u4 xq = as_global<gptr_u4>(x_q8);
+    gptr_f32 xs = as_global<gptr_f32>(x_scales);
+    const uint32_t n_u4 = n_oct * 16, src_u4 = nb * 2, total = n_tokens * n_u4;
+    for (uint32_t base = tid; base < total; base += n_threads * UNROLL) {
+        u32x4 v[UNROLL];
+        uint32_t tok[UNROLL], idx[UNROLL];
+#pragma unroll
+        for (int j = 0; j < UNROLL; j++) {
+            const uint32_t e = base + j * n_threads < total ? base + j * n_threads : total - 1;
+            tok[j] = e / n_u4;
+            idx[j] = e - tok[j] * n_u4;
+            v[j] = xq[size_t(tok[j]) * src_u4 + (idx[j] < src_u4 ? idx[j] : src_u4 - 1)];
+        }
+#pragma unroll
+        for (int j = 0; j < UNROLL; j++) {
+            if (base + j * n_threads < total) {
+                const uint32_t i = idx[j], b = i >> 1;
+                uint32_t *d = dq + tok[j] * tok_dw + (b >> 2) * 32 + (i & 1) * 16 + (b & 3);
+                const bool live = i < src_u4;
+                d[0] = live ? v[j].x : 0u;
+                d[4] = live ? v[j].y : 0u;
+                d[8] = live ? v[j].z : 0u;
+                d[12] = live ? v[j].w : 0u;
+            }
+        }
+    }
+    const uint32_t n_sc = n_oct * 8;
+    for (uint32_t e = tid; e < n_tokens * n_sc; e += n_threads) {
+        const uint32_t t = e / n_sc, i = e - t * n_sc;
+        const float sv = xs[size_t(t) * nb + (i < nb ? i : nb - 1)];
+        reinterpret_cast<float *>(dq + t * tok_dw + n_oct * 64)[i] = i < nb ? sv : 0.0f;
+    }
+}
+
 // acc = fma(s of lane K of this lane's quad, p, acc): v_fmac_f32 takes its first factor through DPP, so the
 // broadcast costs no instruction of its own.  (The compiler does not fold a DPP move into the VOP3 fma it selects.)
 template <int K>
@@ -275,6 +315,220 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
     };
     rmi_ring_walk(ring, n_units, cur, consume);
     if (out.pending()) out.flush(yp, p.y_stride, p.tile0 + k, r, L, p.row_start, p.row_end);
+}
+
+// ---- The same GEMV for four to eight tokens with the 4-byte dots on the matrix cores.
+// The x86-64 order needs, per row, block, 4-byte slice and token, one dot of four byte pairs, its conversion and one
+// fma; at eight tokens those three vector instructions are what the kernel above is bound by.  v_mfma_i32_4x4x4_16B_i8
+// is sixteen independent 4 x 4 x 4 products: in block beta (lanes 4 beta .. 4 beta + 3) the result register v of lane
+// 4 beta + j is the dot of the four bytes in the A register of lane 4 beta + v with the four bytes in the B register of
+// lane 4 beta + j.  With four weight ROWS' slice s in the A registers of a block and four TOKENS' slice s in its B
+// registers, one instruction delivers what 4 x 4 v_dot4 did, on the other pipe.  Lane layout (j = lane & 3,
+// sl = lane >> 2 & 3, s_hi = lane >> 4 & 1, rg = lane >> 5): the lane works on slice s = 4 s_hi + sl of rows
+// 4 rg .. 4 rg + 3 for tokens j and j + 4; its A register holds row 4 rg + ((j + sl) & 3), so that its result register
+// v is row 4 rg + ((v + sl) & 3).  That rotation is what lets the scale products be shared without a lane-dependent
+// register index: lane (sl, j) multiplies f32(wd) * xs for row 4 rg + sl and its two tokens only, and the fma on result
+// register v takes the product of ITS row from the lane 4 v further on in the row of sixteen (row_ror: the lane with
+// sl' = sl + v, same j), through DPP.  The weight pieces arrive in the stream's order (lane 8 r + L: slice L of row r,
+// one full-line load per quad) and cross lanes once through the LDS crossbar (ds_bpermute, no LDS memory).  Every
+// accumulator is one (row, slice, token) chain with the blocks in sequence and the eight slices meet in hsum_ps
+// order: the same bits as the kernel above.  Finished tiles park their 64 results in LDS and leave eight tiles at a
+// time, 256 bytes a token.
+// 16-byte pieces per staged token: the 18 per octet of the kernel above, padded so that tokens lie 64 bytes (mod 256)
+// apart.  Sixteen lanes read four tokens' 64 bytes of one quad at once; with the plain stride (a multiple of 128
+// bytes for an even number of octets) two or all four of them fall on the same banks.
+__host__ __device__ inline uint32_t rmi_gemv_x4_token_u4(uint32_t n_oct) {
+    const uint32_t plain = n_oct * 18;
+    return plain + ((4 + 16 - (plain & 15)) & 15);
+}
+template <int N>
+__device__ __forceinline__ void fmac_ror4(float &acc, float s, float p);  // acc += (s of the lane 4 N on in the row) * p
+template <>
+__device__ __forceinline__ void fmac_ror4<0>(float &acc, float s, float p) {
+    acc = __builtin_fmaf(s, p, acc);
+}
+template <>
+__device__ __forceinline__ void fmac_ror4<1>(float &acc, float s, float p) {
+    asm("v_fmac_f32_dpp %0, %1, %2 row_ror:12 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(s), "v"(p));
+}
+template <>
+__device__ __forceinline__ void fmac_ror4<2>(float &acc, float s, float p) {
+    asm("v_fmac_f32_dpp %0, %1, %2 row_ror:8 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(s), "v"(p));
+}
+template <>
+__device__ __forceinline__ void fmac_ror4<3>(float &acc, float s, float p) {
+    asm("v_fmac_f32_dpp %0, %1, %2 row_ror:4 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(s), "v"(p));
+}
+constexpr int kDppRowRor4 = 0x124, kDppRowRor8 = 0x128, kDppRowRor12 = 0x12c;  // lane i reads lane i - n of its sixteen
+constexpr int kSwizzleXor16 = 0x1f | (16 << 10);
+typedef int v4i_x4 __attribute__((ext_vector_type(4)));
+
+template <int B>
+__device__ __forceinline__ void octet_fma_x4(float (&acc)[2][4], const OctetRegs &g, const uint4 *lds, uint32_t tok_u4,
+                                             uint32_t n_oct, uint32_t o, uint32_t s, uint32_t j, uint32_t src_addr) {
+    constexpr int TG = B > 4 ? 2 : 1;
+    // the lane's tokens; one past the batch takes token 0's data, and its results are not stored
+    const uint4 *xt[2] = {lds + (j < B ? j : 0) * tok_u4, lds + (j + 4 < B ? j + 4 : 0) * tok_u4};
+    // the weight pieces of row 4 rg + ((j + sl) & 3), slice s: from the lane that loaded them
+    int wq[8];
+    {
+        const uint32_t nat[8] = {g.qa.x, g.qa.y, g.qa.z, g.qa.w, g.qb.x, g.qb.y, g.qb.z, g.qb.w};
+#pragma unroll
+        for (int b = 0; b < 8; b++) wq[b] = __builtin_amdgcn_ds_bpermute(int(src_addr), int(nat[b]));
+    }
+    const uint32_t scw[4] = {g.sc.x, g.sc.y, g.sc.z, g.sc.w};  // the eight block scales of row 4 rg + sl
+    float wd[8];
+#pragma unroll
+    for (int b = 0; b < 8; b++) wd[b] = h2f((b & 1) ? scw[b >> 1] >> 16 : scw[b >> 1] & 0xffffu);
+    float pr[2][8];
+    int xq[2][8];
+#pragma unroll
+    for (int tg = 0; tg < TG; tg++) {
+        const float4 a0 = reinterpret_cast<const float4 *>(xt[tg] + n_oct * 16)[2 * o];
+        const float4 a1 = reinterpret_cast<const float4 *>(xt[tg] + n_oct * 16)[2 * o + 1];
+        const float xs[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+        for (int b = 0; b < 8; b++) pr[tg][b] = wd[b] * xs[b];
+        const uint4 xa = xt[tg][(2 * o) * 8 + s];
+        const uint4 xb = xt[tg][(2 * o + 1) * 8 + s];
+        xq[tg][0] = int(xa.x), xq[tg][1] = int(xa.y), xq[tg][2] = int(xa.z), xq[tg][3] = int(xa.w);
+        xq[tg][4] = int(xb.x), xq[tg][5] = int(xb.y), xq[tg][6] = int(xb.z), xq[tg][7] = int(xb.w);
+    }
+    // a DPP read of a register needs two wait states after the vector instruction that wrote it, and the compiler
+    // does not look into the asm statements below: all products pass this point first
+    if constexpr (TG == 2)
+        asm volatile("s_nop 1" : "+v"(pr[0][0]), "+v"(pr[0][1]), "+v"(pr[0][2]), "+v"(pr[0][3]), "+v"(pr[0][4]), "+v"(pr[0][5]), "+v"(pr[0][6]), "+v"(pr[0][7]),
+                                 "+v"(pr[1][0]), "+v"(pr[1][1]), "+v"(pr[1][2]), "+v"(pr[1][3]), "+v"(pr[1][4]), "+v"(pr[1][5]), "+v"(pr[1][6]), "+v"(pr[1][7]));
+    else
+        asm volatile("s_nop 1" : "+v"(pr[0][0]), "+v"(pr[0][1]), "+v"(pr[0][2]), "+v"(pr[0][3]), "+v"(pr[0][4]), "+v"(pr[0][5]), "+v"(pr[0][6]), "+v"(pr[0][7]));
+    const v4i_x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++) {
+            const v4i_x4 d = __builtin_amdgcn_mfma_i32_4x4x4i8(wq[b], xq[tg][b], zero4, 0, 0, 0);
+            fmac_ror4<0>(acc[tg][0], pr[tg][b], float(d[0]));
+            fmac_ror4<1>(acc[tg][1], pr[tg][b], float(d[1]));
+            fmac_ror4<2>(acc[tg][2], pr[tg][b], float(d[2]));
+            fmac_ror4<3>(acc[tg][3], pr[tg][b], float(d[3]));
+        }
+    }
+}
+
+template <int B, bool GROUPED, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_q8_0_x4_kernel(RmiGemvProblem single, const RmiGemvProblem *__restrict__ list,
+                                                           const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
+    static_assert(B >= 2 && B <= 8, "two to eight tokens");
+    constexpr int TG = B > 4 ? 2 : 1;
+    extern __shared__ uint4 lds[];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t j = lane & 3, sl = (lane >> 2) & 3, s_hi = (lane >> 4) & 1, rg = lane >> 5, s = 4 * s_hi + sl;
+    const uint32_t a_row = 4 * rg + ((j + sl) & 3);      // the row whose slice s this lane gives the matrix cores
+    const uint32_t src_addr = (8 * a_row + s) * 4;       // ... and the lane that loaded that piece (byte address of ds_bpermute)
+    const uint32_t sc_row = 4 * rg + sl;                 // the row whose scale products this lane multiplies
+    const uint32_t w_idx = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+
+    RmiGemvProblem p;
+    uint32_t k, k_end;
+    if (GROUPED) {
+        const uint4 run = runs[w_idx];
+        p = list[run.x];
+        k = run.y;
+        k_end = run.y + run.z;
+    } else {
+        p = single;
+        p.x_q8 += size_t(blockIdx.y) * B * p.n_in;  // token group blockIdx.y of the launch
+        p.x_scales += size_t(blockIdx.y) * B * (p.n_in >> 5);
+        p.y += size_t(blockIdx.y) * B * p.y_stride;
+        k = w_idx * tiles_per_wave < p.n_tiles ? w_idx * tiles_per_wave : p.n_tiles;
+        k_end = k + tiles_per_wave < p.n_tiles ? k + tiles_per_wave : p.n_tiles;
+    }
+    const uint32_t n_oct = p.n_oct;
+    const uint32_t tok_u4 = rmi_gemv_x4_token_u4(n_oct);
+    const uint32_t n_units = (k_end - k) * n_oct;
+    struct Cursor {
+        gptr_u4 sc_unit, q_unit;
+        uint32_t o, n_oct, sc_row, lane;
+        __device__ __forceinline__ void load(OctetRegs &g) const {
+            g.sc = sc_unit[sc_row];
+            g.qa = __builtin_nontemporal_load(q_unit + lane);
+            g.qb = __builtin_nontemporal_load(q_unit + 64 + lane);
+        }
+        __device__ __forceinline__ void step() {
+            sc_unit += 8;
+            q_unit += 128;
+            if (++o == n_oct) {
+                o = 0;
+                sc_unit += size_t(n_oct) * 128;
+                q_unit += size_t(n_oct) * 8;
+            }
+        }
+    } cur;
+    {
+        gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + (n_units ? k : 0)) * n_oct * kOctetBytes);
+        cur = Cursor{tile, tile + n_oct * 8, 0, n_oct, sc_row, lane};
+    }
+    RmiRing<OctetRegs> ring;
+    rmi_ring_fill(ring, n_units, cur);
+    {
+        stage_tokens<4>(reinterpret_cast<uint32_t *>(lds), tok_u4 * 4, p.x_q8, p.x_scales, B, n_oct, p.n_in >> 5, threadIdx.x,
+                        blockDim.x);
+        __syncthreads();
+    }
+    // results of finished tiles, per wave: [tile & 7][token][row of the tile]
+    float *park = reinterpret_cast<float *>(lds + size_t(B) * tok_u4) + wave * (8 * B * 8);
+
+    float acc[2][4];
+#pragma unroll
+    for (int tg = 0; tg < 2; tg++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[tg][v] = 0.0f;
+    uint32_t o = 0, tiles_done = 0, flushed = 0;
+    gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
+    auto flush = [&]() {
+        // lane l: tile l >> 3 of the group, row l & 7: a token's 64 results are 256 consecutive bytes
+        const uint32_t t8 = lane >> 3, row = (p.tile0 + k + flushed + t8) * 8 + (lane & 7);
+        const bool live = flushed + t8 < tiles_done && row >= p.row_start && row < p.row_end;
+#pragma unroll
+        for (int t = 0; t < B; t++) {
+            const float v = park[(t8 * B + t) * 8 + (lane & 7)];
+            if (live) yp[size_t(t) * p.y_stride + row] = v;
+        }
+        flushed = tiles_done;
+    };
+    auto consume = [&](const OctetRegs &g) {
+        octet_fma_x4<B>(acc, g, lds, tok_u4, n_oct, o, s, j, src_addr);
+        if (++o == n_oct) {
+            // a tile's end stays a branch of its own: the sums pass through a statement the compiler may not move,
+            // or it computes the whole combine ahead of the branch, in every unit
+            asm volatile("; tile end"
+                         : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]),
+                           "+v"(acc[1][2]), "+v"(acc[1][3]));
+            o = 0;
+#pragma unroll
+            for (int tg = 0; tg < TG; tg++) {
+                float u[4], total[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) {  // slices s and s + 4: lanes 16 apart
+                    u[v] = acc[tg][v] + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, acc[tg][v]), kSwizzleXor16));
+                    acc[tg][v] = 0.0f;
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r++) {  // (u0 + u1) + (u2 + u3) of row 4 rg + r, in the lanes with sl = 0
+                    const float a = u[r] + dpp_f32<kDppRowRor12>(u[(r + 3) & 3]);
+                    const float c = dpp_f32<kDppRowRor8>(u[(r + 2) & 3]) + dpp_f32<kDppRowRor4>(u[(r + 1) & 3]);
+                    total[r] = a + c;
+                }
+                if (sl == 0 && s_hi == 0 && j + 4 * tg < B)
+                    *reinterpret_cast<float4 *>(park + (((tiles_done & 7) * B + j + 4 * tg) * 8 + 4 * rg)) =
+                        make_float4(total[0], total[1], total[2], total[3]);
+            }
+            tiles_done++;
+            if ((tiles_done & 7) == 0) flush();
+        }
+    };
+    rmi_ring_walk(ring, n_units, cur, consume);
+    if (flushed < tiles_done) flush();
 }
 
 // Launches too small to fill the chip (one token, a matrix of at most a few thousand tiles) are bound by
@@ -640,11 +894,29 @@ template <int B>
 int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, const uint4 *d_runs, uint32_t n_waves,
                 uint32_t wpg,
                 uint32_t tiles_per_wave, uint32_t max_n_oct, hipStream_t s, uint32_t token_groups = 1) {
-    const size_t lds_bytes = size_t(B) * max_n_oct * 288;
+    size_t lds_bytes = size_t(B) * max_n_oct * 288;
     if (lds_bytes > 64 * 1024)
         return rmi_fail(RMI_HIP_E_INVALID, "activation of %d tokens x %u elements does not fit the LDS staging", B,
                         max_n_oct * 256);
     const dim3 grid_single((n_waves + wpg - 1) / wpg, token_groups), grid_group(n_waves / wpg), block(64 * wpg);
+    if constexpr (B >= 4) {
+        static const bool off = getenv("RMI_GEMV_X4_OFF") != nullptr;
+        // the kernel with the dots on the matrix cores; its waves park finished tiles behind the staged tokens
+        const size_t x4_bytes = size_t(B) * rmi_gemv_x4_token_u4(max_n_oct) * 16 + size_t(wpg) * 8 * B * 32;
+        if (!off && x4_bytes <= 64 * 1024) {
+            lds_bytes = x4_bytes;
+            if (single && wpg == 1)
+                hipLaunchKernelGGL((gemv_q8_0_x4_kernel<B, false, 64>), grid_single, block, lds_bytes, s, *single, d_list, d_runs, tiles_per_wave);
+            else if (single)
+                hipLaunchKernelGGL((gemv_q8_0_x4_kernel<B, false, 512>), grid_single, block, lds_bytes, s, *single, d_list, d_runs, tiles_per_wave);
+            else if (wpg == 1)
+                hipLaunchKernelGGL((gemv_q8_0_x4_kernel<B, true, 64>), grid_group, block, lds_bytes, s, RmiGemvProblem{}, d_list, d_runs, tiles_per_wave);
+            else
+                hipLaunchKernelGGL((gemv_q8_0_x4_kernel<B, true, 512>), grid_group, block, lds_bytes, s, RmiGemvProblem{}, d_list, d_runs, tiles_per_wave);
+            RMI_HIP_CHECK(hipGetLastError());
+            return RMI_HIP_OK;
+        }
+    }
     // the grouped run table is padded to whole workgroups
     if (single && wpg == 1)
         hipLaunchKernelGGL((gemv_q8_0_kernel<B, false, 64>), grid_single, block, lds_bytes, s, *single, d_list, d_runs,
