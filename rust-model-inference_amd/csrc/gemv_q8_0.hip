@@ -287,9 +287,10 @@ __global__ __launch_bounds__(MAXT) void gemv_q8_0_kernel(RmiGemvProblem single,
     {
         const uint32_t nb = p.n_in >> 5;
         uint32_t *lds_dw = reinterpret_cast<uint32_t *>(lds);
-        for (int t = 0; t < B; t++)
-            stage_token<4>(lds_dw + t * tok_u4 * 4, p.x_q8 + size_t(t) * p.n_in, p.x_scales + size_t(t) * nb, n_oct, nb,
-                           threadIdx.x, blockDim.x);
+        if constexpr (B == 1)
+            stage_token<4>(lds_dw, p.x_q8, p.x_scales, n_oct, nb, threadIdx.x, blockDim.x);
+        else
+            stage_tokens<4>(lds_dw, tok_u4 * 4, p.x_q8, p.x_scales, B, n_oct, nb, threadIdx.x, blockDim.x);
         __syncthreads();
     }
 
@@ -402,16 +403,18 @@ __device__ __forceinline__ void octet_fma_x4(float (&acc)[2][4], const OctetRegs
     else
         asm volatile("s_nop 1" : "+v"(pr[0][0]), "+v"(pr[0][1]), "+v"(pr[0][2]), "+v"(pr[0][3]), "+v"(pr[0][4]), "+v"(pr[0][5]), "+v"(pr[0][6]), "+v"(pr[0][7]));
     const v4i_x4 zero4 = {0, 0, 0, 0};
+    // one product ahead of the sums: the matrix cores' result of step i + 1 is on its way while step i is added
+    v4i_x4 d = __builtin_amdgcn_mfma_i32_4x4x4i8(wq[0], xq[0][0], zero4, 0, 0, 0);
 #pragma unroll
-    for (int b = 0; b < 8; b++) {
-#pragma unroll
-        for (int tg = 0; tg < TG; tg++) {
-            const v4i_x4 d = __builtin_amdgcn_mfma_i32_4x4x4i8(wq[b], xq[tg][b], zero4, 0, 0, 0);
-            fmac_ror4<0>(acc[tg][0], pr[tg][b], float(d[0]));
-            fmac_ror4<1>(acc[tg][1], pr[tg][b], float(d[1]));
-            fmac_ror4<2>(acc[tg][2], pr[tg][b], float(d[2]));
-            fmac_ror4<3>(acc[tg][3], pr[tg][b], float(d[3]));
-        }
+    for (int i = 0; i < 8 * TG; i++) {
+        const int b = i / TG, tg = i % TG;
+        v4i_x4 d_next = zero4;
+        if (i + 1 < 8 * TG) d_next = __builtin_amdgcn_mfma_i32_4x4x4i8(wq[(i + 1) / TG], xq[(i + 1) % TG][(i + 1) / TG], zero4, 0, 0, 0);
+        fmac_ror4<0>(acc[tg][0], pr[tg][b], float(d[0]));
+        fmac_ror4<1>(acc[tg][1], pr[tg][b], float(d[1]));
+        fmac_ror4<2>(acc[tg][2], pr[tg][b], float(d[2]));
+        fmac_ror4<3>(acc[tg][3], pr[tg][b], float(d[3]));
+        d = d_next;
     }
 }
 
@@ -1107,7 +1110,13 @@ int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipS
             per_group >>= 1;
             groups <<= 1;
         }
-        if (groups > 1) return dispatch_gemv(per_group, &p, nullptr, nullptr, n_waves, 1, tpw, p.n_oct, s, groups);
+        if (groups > 1) {
+            // the waves of a workgroup share the staged tokens of their group: as many as leave every compute unit
+            // two workgroups or more
+            uint32_t wpg = rmi_gemv_waves_per_group(size_t(per_group) * p.n_oct * 288, size_t(tpw) * p.n_oct * kOctetBytes);
+            while (wpg > 1 && uint64_t(n_waves / wpg) * groups < 2ull * cus) wpg >>= 1;
+            return dispatch_gemv(per_group, &p, nullptr, nullptr, n_waves, wpg, tpw, p.n_oct, s, groups);
+        }
     }
     uint32_t wpg = rmi_gemv_waves_per_group(size_t(n_tokens) * p.n_oct * 288, size_t(tpw) * p.n_oct * kOctetBytes);
     // a launch with fewer waves than would give every compute unit a workgroup of that size is bound by latency,
