@@ -215,6 +215,12 @@ def cpu_baseline(problems, batch, alg_bytes):
     }, outs
 
 
+def gemv_kernel_name(batch):
+    """The x86-64-order GEMV the library launches for this many tokens: from four on, the one with its dots on the
+    matrix cores."""
+    return "gemv_q8_0_x4_kernel" if batch >= 4 else "gemv_q8_0_kernel"
+
+
 def read_traffic(name, case=""):
     """HBM bytes per launch as rocprofv3 --pmc measured them when profiles/<name>_pmc.txt was recorded: a figure
     read back from that file, not measured by this run.  A file that covers several workloads names the case in the
@@ -326,8 +332,8 @@ def run_projection_set(args, pkg, ev):
             "bound": "hbm",
             "kernel": ("gemv_q8_0_mfma_kernel<%d,%s>" % ((batch + 15) // 16, "true" if args.mode != "per_matmul" else "false"))
                       if neon else
-                      "gemv_q8_0_kernel<%d,%s,%s>" % (batch, "true" if args.mode != "per_matmul" else "false",
-                                                       group_maxt(H, group_all) if args.mode == "grouped" else "*"),
+                      "%s<%d,%s,%s>" % (gemv_kernel_name(batch), batch, "true" if args.mode != "per_matmul" else "false",
+                                        group_maxt(H, group_all) if args.mode == "grouped" else "*"),
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -403,7 +409,7 @@ def run_small_batches(args, pkg, ev):
             "value": round(alg / wall / 1e9, 1), "unit": "GB/s", "ms_per_step": round(wall * 1e3, 4),
             "steps": steps, "warmup": warmup, "token_steps_per_s": round(batch / wall, 1), "algorithmic_bytes_per_step": alg,
             "roofline": {"bound": "hbm",
-                         "kernel": "gemv_q8_0_kernel<%d,true,%s>" % (batch, group_maxt(H, group)) if order == "avx2"
+                         "kernel": "%s<%d,true,%s>" % (gemv_kernel_name(batch), batch, group_maxt(H, group)) if order == "avx2"
                                    else "gemv_q8_0_mfma_kernel<%d,true>" % ((batch + 15) // 16),
                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_us": round(dev_ms * 1e3, 3)}}
