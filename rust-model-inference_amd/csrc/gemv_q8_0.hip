@@ -903,10 +903,10 @@ int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, cons
                         max_n_oct * 256);
     const dim3 grid_single((n_waves + wpg - 1) / wpg, token_groups), grid_group(n_waves / wpg), block(64 * wpg);
     if constexpr (B >= 4) {
-        static const bool off = getenv("RMI_GEMV_X4_OFF") != nullptr;
-        // the kernel with the dots on the matrix cores; its waves park finished tiles behind the staged tokens
+        // the kernel with the dots on the matrix cores, where its staging fits (its tokens lie further apart, and its
+        // waves park finished tiles behind them)
         const size_t x4_bytes = size_t(B) * rmi_gemv_x4_token_u4(max_n_oct) * 16 + size_t(wpg) * 8 * B * 32;
-        if (!off && x4_bytes <= 64 * 1024) {
+        if (x4_bytes <= 64 * 1024) {
             lds_bytes = x4_bytes;
             if (single && wpg == 1)
                 hipLaunchKernelGGL((gemv_q8_0_x4_kernel<B, false, 64>), grid_single, block, lds_bytes, s, *single, d_list, d_runs, tiles_per_wave);

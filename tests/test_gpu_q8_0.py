@@ -368,6 +368,21 @@ def test_prequantized_batch_bit_exact(hip, oracle, n_tokens):
         assert np.array_equal(bits(out[t]), bits(oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, A))), t
 
 
+@pytest.mark.parametrize("n_tokens,n_out,n_in", [(4, 1030, 1024), (5, 77, 2048), (6, 264, 3072), (7, 8, 6144), (8, 515, 6144),
+                                                  (8, 9, 7168), (5, 130, 7168), (4, 136, 7424), (8, 520, 1056)])
+def test_batches_of_four_to_eight_on_both_kernels(hip, oracle, n_tokens, n_out, n_in):
+    """From four tokens on the x86-64-order GEMV computes its 4-byte dots on the matrix cores; rows too long for that
+    kernel's LDS staging (7168 and 7424 elements here) keep the kernel with the dots on the vector ALU.  Both against
+    the checker's AVX2 order, every row and token, with row counts that are not multiples of eight and a row length
+    that is not a whole octet (1056)."""
+    w, x = _case(hip, 7700 + n_tokens + n_in, n_out, n_in, n_tokens)
+    q8, sc = _quantize_rows(oracle, x)
+    out = np.full((n_tokens, n_out), np.nan, np.float32)
+    hip.kernel.Q8Kernel(w, n_in, n_out).matmul_q8_0_quantized_batch(q8, sc, out, n_in, n_out, n_tokens)
+    for t in range(n_tokens):
+        assert np.array_equal(bits(out[t]), bits(oracle.matmul_q8_0_quantized(w, q8[t], sc[t], n_in, n_out, A))), t
+
+
 @pytest.mark.parametrize("n_tokens", [1, 4, 8])
 def test_forward_batched_small_is_gemv_order(hip, oracle, n_tokens):
     """Kernel::forward_batched up to 8 tokens: device quantizer + GEMV in the AVX2 order, bit-exact."""
