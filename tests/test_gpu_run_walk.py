@@ -180,3 +180,13 @@ def test_random_grouped_launches(hip, oracle, fmt, seed):
             got = ys[i].to_array(np.float32, (n_tokens, n_out))
             assert np.array_equal(bits(got), bits(refs[i])), (fmt, seed, n_tokens, i, n_out, n_units)
         H.lib.rmi_hip_gemv_group_destroy(g)
+
+
+@pytest.mark.parametrize("n_units,n_out,n_tokens", [(1, 8 * 2048 * 16 + 5, 8), (2, 8 * 2048 * 8 + 8 * 3 + 1, 4), (3, 8 * 2048 * 5 + 8 * 2, 5),
+                                                    (5, 8 * 2048 * 3 + 8 * 1 + 7, 8), (7, 8 * 2048 * 2 + 3, 6)])
+def test_long_runs_with_four_to_eight_tokens(hip, oracle, n_units, n_out, n_tokens):
+    """The Q8_0 kernel for four tokens and more (its dots on the matrix cores, its results parked in LDS and leaving
+    eight tiles at a time) over the same run lengths, and over row ranges that start and end inside a tile."""
+    _run(hip, oracle, "q8_0", 170 + n_units, n_out, n_units, n_tokens)
+    _run(hip, oracle, "q8_0", 180 + n_units, n_out, n_units, n_tokens, r0=8 * 517 + 3, r1=n_out - 8 * 11 - 6)
+    _run(hip, oracle, "q8_0", 190 + n_units, n_out, n_units, n_tokens, r0=8 * 1000 + 7, r1=8 * 1000 + 9)
