@@ -422,8 +422,14 @@ int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const fl
  * Head dimension 128 and 768 keys or more: a head's keys are spread over up to 16 workgroups in two launches
  * (scores; then weights and p.v, the parts meeting in the workgroup that arrives last).  The softmax sum is still
  * the reference's sequential f32 sum; results have the same bits as the one-workgroup-per-head kernel.  The
- * hand-over uses a scratch region of the calling host thread (allocated at the first such call, which also
- * synchronises `stream` once): calls of one host thread that overlap on different streams would share it. */
+ * hand-over uses a scratch region of the calling host thread: calls of one host thread that overlap on different
+ * streams would share it, and the thread synchronises its launches before it exits (the region goes back to the
+ * library with the thread).  rmi_hip_attention_reserve(n_head, max_keys) makes the region ahead of time (it
+ * synchronises the device, allocates and clears; no counterpart in the reference), after which no call of this
+ * thread with at most that many heads and keys allocates or synchronises; without it the first call that needs
+ * the region synchronises `stream` and allocates it.  Up to 16 384 keys (head dimension 128); otherwise what one
+ * workgroup holds in LDS (12 bytes a key of 159 KiB). */
+int rmi_hip_attention_reserve(uint32_t n_head, uint32_t max_keys);
 int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache,
                                             uint32_t n_keys, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv,
                                             uint32_t head_dim_k, uint32_t head_dim_v, int8_t *q8, float *scales,

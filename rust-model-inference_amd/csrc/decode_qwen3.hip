@@ -1009,6 +1009,7 @@ __global__ __launch_bounds__(kAttnSplitThreads) void attn128_weights_pv_kernel(
         for (uint32_t w = 1; w < kAttnSplitThreads / 64; w++) o += wave_sums[w * 128 + d];
         mine[d] = o;
     }
+    __builtin_amdgcn_wave_barrier();  // the hand-over stays inside this one wave: its stores, then its fence, then its count
     __threadfence();
     uint32_t before = 0;
     if (tid == 0) before = __hip_atomic_fetch_add(ws.arrived + head, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1591,6 +1592,28 @@ int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const fl
     return RMI_HIP_OK;
 }
 
+// The calling thread's scratch for the two-launch attention: sized for n_head heads and max_keys keys, counters zero.
+constexpr int kAttnSplitSlot = 5;
+constexpr uint32_t kAttnSplitReserveKeys = 16384;  // what the two launches hold at most: sized once for any context
+static int attn_split_reserve(RmiThreadCtx *c, uint32_t n_head, uint32_t max_keys) {
+    const size_t need = attn_split_scratch_bytes(n_head, max_keys);
+    if (c->dev_cap[kAttnSplitSlot] >= need) return RMI_HIP_OK;
+    void *fresh = rmi_dev_buf(c, kAttnSplitSlot, need);
+    if (!fresh) return RMI_HIP_E_RUNTIME;
+    RMI_HIP_CHECK(hipMemset(fresh, 0, c->dev_cap[kAttnSplitSlot]));  // the arrival counters start at zero
+    return RMI_HIP_OK;
+}
+
+int rmi_hip_attention_reserve(uint32_t n_head, uint32_t max_keys) {
+    RMI_REQUIRE_INIT();
+    if (n_head == 0 || n_head > kAttnSplitMaxHeads) return rmi_fail(RMI_HIP_E_INVALID, "1..%u heads", kAttnSplitMaxHeads);
+    RmiThreadCtx *c = rmi_thread_ctx();
+    if (!c) return RMI_HIP_E_RUNTIME;
+    (void)attn_lds_limit();  // the kernels' dynamic-LDS limit is raised here, too, not at the first launch
+    RMI_HIP_CHECK(hipDeviceSynchronize());  // a launch of this thread may still use the region this call replaces
+    return attn_split_reserve(c, n_head, max_keys < kAttnSplitReserveKeys ? kAttnSplitReserveKeys : max_keys);
+}
+
 int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache,
                                             uint32_t n_keys, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv,
                                             uint32_t head_dim_k, uint32_t head_dim_v, int8_t *q8, float *scales,
@@ -1601,29 +1624,28 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
         head_dim_k == 0 || head_dim_v == 0 || head_dim_k > 1024 || head_dim_v > 1024 || kv_stride % 8)
         return rmi_fail(RMI_HIP_E_INVALID, "bad attention shape");
     const bool d128 = head_dim_k == 128 && head_dim_v == 128;
-    const size_t lds = d128 ? attn128_lds_bytes(n_keys) : attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
-    if (lds > attn_lds_limit()) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
     if (d128 && attn128_use_split(n_keys, n_head)) {
         // The scratch of the two launches is the calling thread's (slot 5 of its staging buffers, never used by
         // the host-slice entry points): calls of one thread that overlap on different streams would share it.
+        // rmi_hip_attention_reserve makes it ahead of time; without that call it is made here, once.  (What the two
+        // launches hold in LDS is their own figure, checked where they are launched.)
         RmiThreadCtx *c = rmi_thread_ctx();
         if (!c) return RMI_HIP_E_RUNTIME;
-        constexpr int kSlot = 5;
-        const uint32_t max_keys = n_keys < 16384 ? 16384 : n_keys;  // sized once for any context the kernels hold
-        const size_t need = attn_split_scratch_bytes(n_head, max_keys);
-        if (c->dev_cap[kSlot] < need) {
+        const uint32_t max_keys = n_keys < kAttnSplitReserveKeys ? kAttnSplitReserveKeys : n_keys;
+        if (c->dev_cap[kAttnSplitSlot] < attn_split_scratch_bytes(n_head, max_keys)) {
             RMI_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));  // it may still read the old one
-            void *fresh = rmi_dev_buf(c, kSlot, need);
-            if (!fresh) return RMI_HIP_E_RUNTIME;
-            RMI_HIP_CHECK(hipMemset(fresh, 0, c->dev_cap[kSlot]));  // the arrival counters start at zero
+            const int rc = attn_split_reserve(c, n_head, max_keys);
+            if (rc != RMI_HIP_OK) return rc;
         }
         const int rc = launch_attention128_split(q16, k_cache, v_cache, n_keys, kv_stride, n_head, n_head_kv,
-                                                 attn_split_scratch_at(c->dev[kSlot], n_head, max_keys), q8, scales,
+                                                 attn_split_scratch_at(c->dev[kAttnSplitSlot], n_head, max_keys), q8, scales,
                                                  rounding, static_cast<hipStream_t>(stream));
         if (rc != RMI_HIP_OK) return rc;
         RMI_HIP_CHECK(hipGetLastError());
         return RMI_HIP_OK;
     }
+    const size_t lds = d128 ? attn128_lds_bytes(n_keys) : attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
+    if (lds > attn_lds_limit()) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
     if (d128)
         hipLaunchKernelGGL(attention128_quant_kernel<false>, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
                            q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding, AttnFromQkv{}, 0u, 0u);

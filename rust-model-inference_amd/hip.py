@@ -57,6 +57,7 @@ SIGNATURES = {
     "rmi_hip_shutdown": (None, []),
     "rmi_hip_last_error": (C.c_char_p, []),
     "rmi_hip_thread_context_count": (_sz, []),
+    "rmi_hip_attention_reserve": (C.c_int, [_u32, _u32]),
     "rmi_hip_set_forward_batched_mode": (C.c_int, [C.c_int]),
     "rmi_hip_get_forward_batched_mode": (C.c_int, []),
     "rmi_hip_device_info": (C.c_int, [C.c_char_p, _sz, C.POINTER(C.c_int), C.POINTER(_sz)]),

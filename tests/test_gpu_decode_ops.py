@@ -264,6 +264,57 @@ def test_attention_split_mixed_head_counts(hip, oracle):
             b.free()
 
 
+def test_attention_reserve_then_calls_allocate_nothing(hip, oracle):
+    """rmi_hip_attention_reserve makes the calling thread's scratch for the two-launch attention ahead of time: a call
+    over 1024 keys from a thread that reserved first leaves the device's free memory as it was (the HIP runtime is the
+    meter), and has the checker's bits.  Between the 13 000 keys one workgroup holds and the 16 384 the two launches
+    hold, the call is accepted as well (the LDS figure that is checked is that of the path taken)."""
+    import ctypes
+    import threading
+
+    H = hip.hip
+    rt = ctypes.CDLL("libamdhip64.so")
+    rt.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert rt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    rng = np.random.default_rng(91)
+    hk = hv = 128
+    for n_head, n_kv, n_keys in [(16, 8, 1024), (2, 1, 14000)]:
+        kv_stride = n_kv * hk
+        q = rng.normal(0, 1, n_head * hk).astype(np.float32)
+        kc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+        vc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
+        d_q, d_k, d_v = _dev(H, q.astype(np.float16).view(np.uint16)), _dev(H, kc), _dev(H, vc)
+        d_o, d_s = H.DeviceBuffer(n_head * hv), H.DeviceBuffer(n_head * hv // 32 * 4)
+        H.check(H.lib.rmi_hip_synchronize())
+        seen = {}
+
+        def call():
+            seen["reserve"] = H.lib.rmi_hip_attention_reserve(n_head, n_keys)
+            seen["free_before"] = free_bytes()
+            seen["rc"] = H.lib.rmi_hip_attention_f16_quantize_q8_0_dev(d_q.ptr, d_k.ptr, d_v.ptr, n_keys, kv_stride, n_head,
+                                                                      n_kv, hk, hv, d_o.ptr, d_s.ptr, A, None)
+            seen["free_after"] = free_bytes()
+            seen["sync"] = H.lib.rmi_hip_synchronize()  # before the thread, and with it its scratch, goes away
+
+        t = threading.Thread(target=call)
+        t.start()
+        t.join()
+        assert seen["reserve"] == 0 and seen["rc"] == 0 and seen["sync"] == 0, (seen, H.last_error())
+        assert seen["free_after"] == seen["free_before"], (n_head, n_keys)
+        ref = oracle.attention_f16(q, kc, vc, n_keys - 1, kv_stride, n_head, n_kv, hk, hv)
+        q_ref, s_ref = _quant(oracle, ref)
+        assert np.array_equal(d_o.to_array(np.int8, (n_head * hv,)), q_ref), (n_head, n_keys)
+        assert np.array_equal(d_s.to_array(np.float32, (n_head * hv // 32,)).view(np.uint32), s_ref.view(np.uint32))
+        for b in (d_q, d_k, d_v, d_o, d_s):
+            b.free()
+    assert H.lib.rmi_hip_attention_reserve(0, 1024) != 0
+
+
 @pytest.mark.parametrize("n_head,n_kv,with_norm", [(16, 8, True), (16, 8, False), (6, 6, True), (32, 4, True)])
 def test_qkv_attention_in_one_launch_equals_the_two_calls(hip, oracle, n_head, n_kv, with_norm):
     """rmi_hip_qkv_attention_f16_quantize_q8_0_dev against rmi_hip_qk_norm_rope_f16_dev followed by
