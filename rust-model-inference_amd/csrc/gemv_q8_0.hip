@@ -1114,11 +1114,13 @@ int rmi_launch_gemv_q8_0_single(const RmiGemvProblem &p, uint32_t n_tokens, hipS
             // the waves of a workgroup share the staged tokens of their group: as many as leave every compute unit
             // two workgroups or more
             uint32_t wpg = rmi_gemv_waves_per_group(size_t(per_group) * p.n_oct * 288, size_t(tpw) * p.n_oct * kOctetBytes);
+            if (per_group >= 4 && wpg > 4) wpg = 4;  // as in the grouped launch: four-wave workgroups turn over more evenly
             while (wpg > 1 && uint64_t(n_waves / wpg) * groups < 2ull * cus) wpg >>= 1;
             return dispatch_gemv(per_group, &p, nullptr, nullptr, n_waves, wpg, tpw, p.n_oct, s, groups);
         }
     }
     uint32_t wpg = rmi_gemv_waves_per_group(size_t(n_tokens) * p.n_oct * 288, size_t(tpw) * p.n_oct * kOctetBytes);
+    if (n_tokens >= 4 && wpg > 4) wpg = 4;
     // a launch with fewer waves than would give every compute unit a workgroup of that size is bound by latency,
     // not by the staging it shares: smaller workgroups on more compute units
     while (wpg > 1 && n_waves / wpg < cus) wpg >>= 1;
