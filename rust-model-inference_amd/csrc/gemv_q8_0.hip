@@ -342,6 +342,8 @@ __host__ __device__ inline uint32_t rmi_gemv_x4_token_u4(uint32_t n_oct) {
     const uint32_t plain = n_oct * 18;
     return plain + ((4 + 16 - (plain & 15)) & 15);
 }
+// waves that are to share a SIMD (the register budget): five fit only with spills, and measured no faster
+constexpr int kX4WavesPerSimd = 4;
 template <int N>
 __device__ __forceinline__ void fmac_ror4(float &acc, float s, float p);  // acc += (s of the lane 4 N on in the row) * p
 template <>
@@ -370,56 +372,53 @@ __device__ __forceinline__ void octet_fma_x4(float (&acc)[2][4], const OctetRegs
     constexpr int TG = B > 4 ? 2 : 1;
     // the lane's tokens; one past the batch takes token 0's data, and its results are not stored
     const uint4 *xt[2] = {lds + (j < B ? j : 0) * tok_u4, lds + (j + 4 < B ? j + 4 : 0) * tok_u4};
-    // the weight pieces of row 4 rg + ((j + sl) & 3), slice s: from the lane that loaded them
-    int wq[8];
-    {
-        const uint32_t nat[8] = {g.qa.x, g.qa.y, g.qa.z, g.qa.w, g.qb.x, g.qb.y, g.qb.z, g.qb.w};
-#pragma unroll
-        for (int b = 0; b < 8; b++) wq[b] = __builtin_amdgcn_ds_bpermute(int(src_addr), int(nat[b]));
-    }
     const uint32_t scw[4] = {g.sc.x, g.sc.y, g.sc.z, g.sc.w};  // the eight block scales of row 4 rg + sl
-    float wd[8];
-#pragma unroll
-    for (int b = 0; b < 8; b++) wd[b] = h2f((b & 1) ? scw[b >> 1] >> 16 : scw[b >> 1] & 0xffffu);
-    float pr[2][8];
-    int xq[2][8];
-#pragma unroll
-    for (int tg = 0; tg < TG; tg++) {
-        const float4 a0 = reinterpret_cast<const float4 *>(xt[tg] + n_oct * 16)[2 * o];
-        const float4 a1 = reinterpret_cast<const float4 *>(xt[tg] + n_oct * 16)[2 * o + 1];
-        const float xs[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-#pragma unroll
-        for (int b = 0; b < 8; b++) pr[tg][b] = wd[b] * xs[b];
-        const uint4 xa = xt[tg][(2 * o) * 8 + s];
-        const uint4 xb = xt[tg][(2 * o + 1) * 8 + s];
-        xq[tg][0] = int(xa.x), xq[tg][1] = int(xa.y), xq[tg][2] = int(xa.z), xq[tg][3] = int(xa.w);
-        xq[tg][4] = int(xb.x), xq[tg][5] = int(xb.y), xq[tg][6] = int(xb.z), xq[tg][7] = int(xb.w);
-    }
-    // a DPP read of a register needs two wait states after the vector instruction that wrote it, and the compiler
-    // does not look into the asm statements below: all products pass this point first
-    if constexpr (TG == 2)
-        asm volatile("s_nop 1" : "+v"(pr[0][0]), "+v"(pr[0][1]), "+v"(pr[0][2]), "+v"(pr[0][3]), "+v"(pr[0][4]), "+v"(pr[0][5]), "+v"(pr[0][6]), "+v"(pr[0][7]),
-                                 "+v"(pr[1][0]), "+v"(pr[1][1]), "+v"(pr[1][2]), "+v"(pr[1][3]), "+v"(pr[1][4]), "+v"(pr[1][5]), "+v"(pr[1][6]), "+v"(pr[1][7]));
-    else
-        asm volatile("s_nop 1" : "+v"(pr[0][0]), "+v"(pr[0][1]), "+v"(pr[0][2]), "+v"(pr[0][3]), "+v"(pr[0][4]), "+v"(pr[0][5]), "+v"(pr[0][6]), "+v"(pr[0][7]));
     const v4i_x4 zero4 = {0, 0, 0, 0};
-    // one product ahead of the sums: the matrix cores' result of step i + 1 is on its way while step i is added
-    v4i_x4 d = __builtin_amdgcn_mfma_i32_4x4x4i8(wq[0], xq[0][0], zero4, 0, 0, 0);
+    // a quad of blocks at a time: what is live at once (the weight pieces, the tokens' pieces, the scale products)
+    // stays at half an octet
 #pragma unroll
-    for (int i = 0; i < 8 * TG; i++) {
-        const int b = i / TG, tg = i % TG;
-        v4i_x4 d_next = zero4;
-        if (i + 1 < 8 * TG) d_next = __builtin_amdgcn_mfma_i32_4x4x4i8(wq[(i + 1) / TG], xq[(i + 1) % TG][(i + 1) / TG], zero4, 0, 0, 0);
-        fmac_ror4<0>(acc[tg][0], pr[tg][b], float(d[0]));
-        fmac_ror4<1>(acc[tg][1], pr[tg][b], float(d[1]));
-        fmac_ror4<2>(acc[tg][2], pr[tg][b], float(d[2]));
-        fmac_ror4<3>(acc[tg][3], pr[tg][b], float(d[3]));
-        d = d_next;
+    for (int h = 0; h < 2; h++) {
+        // the weight pieces of row 4 rg + ((j + sl) & 3), slice s: from the lane that loaded them
+        const uint32_t nat[4] = {h ? g.qb.x : g.qa.x, h ? g.qb.y : g.qa.y, h ? g.qb.z : g.qa.z, h ? g.qb.w : g.qa.w};
+        int wq[4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) wq[b] = __builtin_amdgcn_ds_bpermute(int(src_addr), int(nat[b]));
+        float wd[4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) wd[b] = h2f((b & 1) ? scw[2 * h + (b >> 1)] >> 16 : scw[2 * h + (b >> 1)] & 0xffffu);
+        float pr[2][4];
+        int xq[2][4];
+#pragma unroll
+        for (int tg = 0; tg < TG; tg++) {
+            const float4 a = reinterpret_cast<const float4 *>(xt[tg] + n_oct * 16)[2 * o + h];
+            pr[tg][0] = wd[0] * a.x, pr[tg][1] = wd[1] * a.y, pr[tg][2] = wd[2] * a.z, pr[tg][3] = wd[3] * a.w;
+            const uint4 x = xt[tg][(2 * o + h) * 8 + s];
+            xq[tg][0] = int(x.x), xq[tg][1] = int(x.y), xq[tg][2] = int(x.z), xq[tg][3] = int(x.w);
+        }
+        // a DPP read of a register needs two wait states after the vector instruction that wrote it, and the compiler
+        // does not look into the asm statements below: all products pass this point first
+        if constexpr (TG == 2)
+            asm volatile("s_nop 1" : "+v"(pr[0][0]), "+v"(pr[0][1]), "+v"(pr[0][2]), "+v"(pr[0][3]), "+v"(pr[1][0]), "+v"(pr[1][1]), "+v"(pr[1][2]), "+v"(pr[1][3]));
+        else
+            asm volatile("s_nop 1" : "+v"(pr[0][0]), "+v"(pr[0][1]), "+v"(pr[0][2]), "+v"(pr[0][3]));
+        // one product ahead of the sums: the matrix cores' result of step i + 1 is on its way while step i is added
+        v4i_x4 d = __builtin_amdgcn_mfma_i32_4x4x4i8(wq[0], xq[0][0], zero4, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4 * TG; i++) {
+            const int b = i / TG, tg = i % TG;
+            v4i_x4 d_next = zero4;
+            if (i + 1 < 4 * TG) d_next = __builtin_amdgcn_mfma_i32_4x4x4i8(wq[(i + 1) / TG], xq[(i + 1) % TG][(i + 1) / TG], zero4, 0, 0, 0);
+            fmac_ror4<0>(acc[tg][0], pr[tg][b], float(d[0]));
+            fmac_ror4<1>(acc[tg][1], pr[tg][b], float(d[1]));
+            fmac_ror4<2>(acc[tg][2], pr[tg][b], float(d[2]));
+            fmac_ror4<3>(acc[tg][3], pr[tg][b], float(d[3]));
+            d = d_next;
+        }
     }
 }
 
 template <int B, bool GROUPED, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemv_q8_0_x4_kernel(RmiGemvProblem single, const RmiGemvProblem *__restrict__ list,
+__global__ __launch_bounds__(MAXT, kX4WavesPerSimd) void gemv_q8_0_x4_kernel(RmiGemvProblem single, const RmiGemvProblem *__restrict__ list,
                                                            const uint4 *__restrict__ runs, uint32_t tiles_per_wave) {
     static_assert(B >= 2 && B <= 8, "two to eight tokens");
     constexpr int TG = B > 4 ? 2 : 1;
