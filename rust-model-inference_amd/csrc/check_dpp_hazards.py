@@ -9,7 +9,13 @@ unconditional branch this is stricter than needed, never laxer) and along every 
 in front of each `s_branch` / `s_cbranch_*` to those behind its target label.  Indirect jumps (`s_setpc_b64`,
 `s_swappc_b64`) are refused: their targets are not in the text.
 
-These two rules are the hazards of the one instruction class this build writes by hand (VALU with a DPP source).
+A third rule is for hand-written READERS: a vector instruction may not read the result registers of a
+v_mfma_*_4x4x4_* (two passes) sooner than five wait states after it.  The compiler keeps that distance for the
+instructions it emits itself, but an asm statement that takes the result as an operand is opaque to it.  Other
+matrix-core shapes have other distances: the script refuses a file that holds them until their rule is added.
+
+These rules are the hazards of what this build writes by hand: vector instructions with a DPP source, in asm
+statements next to matrix-core instructions.
 Whoever adds another hand-written class (an `s_waitcnt`-sensitive memory instruction, an MFMA with its own
 dependency wait states, writes of M0 or VCC in front of their readers, ...) has to add that class's rules here:
 the script knows nothing of hazards it was not told about.
@@ -51,6 +57,31 @@ def dpp_source(ins):
     return int(m.group(1)) if m else None
 
 
+def read_vgprs(ins):
+    """VGPRs a vector instruction reads: every register operand behind the first, and the first as well where the
+    instruction accumulates into its destination."""
+    if not ins.startswith("v_"):
+        return set()
+    ops = ins.split(None, 1)[1] if " " in ins else ""
+    first, _, rest = ops.partition(",")
+    if "UNUSED_PRESERVE" in ins or ins.startswith(("v_fmac", "v_mac", "v_dot4c")):
+        rest = first + "," + rest  # the destination is a source, too
+    regs = set()
+    for a, b in re.findall(r"v\[(\d+):(\d+)\]", rest):
+        regs.update(range(int(a), int(b) + 1))
+    regs.update(int(r) for r in re.findall(r"\bv(\d+)\b", rest))
+    return regs
+
+
+MFMA_4X4_WAIT = 5  # wait states between a two-pass matrix-core instruction and a vector read of its result
+
+
+def mfma_result(ins):
+    """The result registers of a 4x4x4 matrix-core instruction, or None."""
+    m = re.match(r"v_mfma_\w+_4x4x4\w*\s+v\[(\d+):(\d+)\]", ins)
+    return set(range(int(m.group(1)), int(m.group(2)) + 1)) if m else None
+
+
 def wait_states(ins):
     m = re.match(r"s_nop\s+(\d+)", ins)
     return int(m.group(1)) + 1 if m else 1
@@ -63,6 +94,20 @@ def hazards(seq, first_checked=0):
     """(earlier instruction, DPP instruction, wait states between) for every DPP instruction of seq from index
     first_checked on that reads its operand too early after an instruction of seq in front of it."""
     bad = []
+    for k in range(first_checked, len(seq)):
+        reads = read_vgprs(seq[k])
+        if not reads:
+            continue
+        between = 0
+        for prev in reversed(seq[max(0, k - REACH):k]):
+            res = mfma_result(prev)
+            if res and between < MFMA_4X4_WAIT and res & reads:
+                bad.append((prev, seq[k], between))
+            if written_vgprs(prev) & reads and not res:
+                reads = reads - written_vgprs(prev)  # a later writer in between: the read is of that value
+            between += wait_states(prev)
+            if between >= MFMA_4X4_WAIT:
+                break
     for k in range(first_checked, len(seq)):
         src = dpp_source(seq[k])
         if src is None:
@@ -97,6 +142,7 @@ def main():
     n_fmac = sum(ins.startswith("v_fmac_f32_dpp") for ins in code)
     bad = hazards(code)
     unknown = [ins for ins in code if ins.startswith(("s_setpc_b64", "s_swappc_b64"))]
+    unknown += [ins for ins in code if ins.startswith("v_mfma") and mfma_result(ins) is None]  # a shape without a rule
     for k, ins in enumerate(code):
         target = branch_target(ins)
         if target is None:

@@ -74,3 +74,17 @@ def test_loop_back_edge_is_followed(tmp_path):
 
 def test_indirect_jump_is_refused(tmp_path):
     assert _run(tmp_path, ["s_setpc_b64 s[30:31]"]).returncode == 1
+
+
+def test_reading_a_matrix_core_result_too_early_fails(tmp_path):
+    """An instruction (an asm statement's, for the compiler spaces its own) that reads a 4x4x4 matrix-core result
+    sooner than five wait states after it; a matrix-core shape the script has no rule for is refused."""
+    mfma = "v_mfma_f32_4x4x4_16b_f16 v[8:11], v[4:5], v[6:7], 0"
+    use = "v_fmac_f32_dpp v20, v3, v9 row_ror:12 row_mask:0xf bank_mask:0xf"
+    pad = "v_add_u32_e32 v30, v31, v32"
+    assert _run(tmp_path, [mfma, pad, pad, use]).returncode == 1
+    assert _run(tmp_path, [mfma, pad, pad, pad, pad, pad, use]).returncode == 0
+    assert _run(tmp_path, [mfma, "s_nop 4", use]).returncode == 0
+    assert _run(tmp_path, [mfma, "s_nop 3", use]).returncode == 1
+    assert _run(tmp_path, [mfma, "v_mov_b32_e32 v9, v1", use]).returncode == 0  # v9 is another value by then
+    assert _run(tmp_path, ["v_mfma_i32_32x32x32_i8 v[0:15], v[16:19], v[20:23], 0"]).returncode == 1
