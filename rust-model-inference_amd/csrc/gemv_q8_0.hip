@@ -342,6 +342,16 @@ __host__ __device__ inline uint32_t rmi_gemv_x4_token_u4(uint32_t n_oct) {
     const uint32_t plain = n_oct * 18;
     return plain + ((4 + 16 - (plain & 15)) & 15);
 }
+// Between LDS accesses by which the lanes of ONE wave hand values to each other: every lane arrives, and the compiler
+// moves no memory access across (the hardware carries a wave's LDS instructions out in order; no instruction is
+// emitted beyond the wait for the accesses in front).
+__device__ __forceinline__ void rmi_wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+// floats of LDS per wave behind the staged tokens: four tiles' results and the 8 x 33 partial sums of a tile's end
+__host__ __device__ constexpr uint32_t kX4WaveFloats(uint32_t n_tokens) { return 4 * n_tokens * 8 + 8 * 33 + 8; }
 // waves that are to share a SIMD (the register budget): five fit only with spills, and measured no faster
 constexpr int kX4WavesPerSimd = 4;
 template <int N>
@@ -362,8 +372,6 @@ template <>
 __device__ __forceinline__ void fmac_ror4<3>(float &acc, float s, float p) {
     asm("v_fmac_f32_dpp %0, %1, %2 row_ror:4 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(s), "v"(p));
 }
-constexpr int kDppRowRor4 = 0x124, kDppRowRor8 = 0x128, kDppRowRor12 = 0x12c;  // lane i reads lane i - n of its sixteen
-constexpr int kSwizzleXor16 = 0x1f | (16 << 10);
 typedef int v4i_x4 __attribute__((ext_vector_type(4)));
 
 template <int B>
@@ -477,8 +485,14 @@ __global__ __launch_bounds__(MAXT, kX4WavesPerSimd) void gemv_q8_0_x4_kernel(Rmi
                         blockDim.x);
         __syncthreads();
     }
-    // results of finished tiles, per wave: [tile & 7][token][row of the tile]
-    float *park = reinterpret_cast<float *>(lds + size_t(B) * tok_u4) + wave * (8 * B * 8);
+    // Per wave behind the staged tokens: the results of up to four finished tiles, [tile & 3][token][row of the tile],
+    // and the 8 x 32 partial sums of one group of four tokens at a tile's end, [slice][token of the group][row], rows
+    // of 33 floats (the lanes of a wave write eight different slices at once).
+    float *park = reinterpret_cast<float *>(lds + size_t(B) * tok_u4) + wave * kX4WaveFloats(B);
+    float *red = park + 4 * B * 8;
+    uint32_t red_w[4];  // where this lane's sum of result register v goes: row 4 rg + ((v + sl) & 3) of token j, slice s
+#pragma unroll
+    for (int v = 0; v < 4; v++) red_w[v] = s * 33 + j * 8 + 4 * rg + ((uint32_t(v) + sl) & 3);
 
     float acc[2][4];
 #pragma unroll
@@ -488,12 +502,12 @@ __global__ __launch_bounds__(MAXT, kX4WavesPerSimd) void gemv_q8_0_x4_kernel(Rmi
     uint32_t o = 0, tiles_done = 0, flushed = 0;
     gptr_f32_w yp = as_global<gptr_f32_w>(p.y);
     auto flush = [&]() {
-        // lane l: tile l >> 3 of the group, row l & 7: a token's 64 results are 256 consecutive bytes
-        const uint32_t t8 = lane >> 3, row = (p.tile0 + k + flushed + t8) * 8 + (lane & 7);
-        const bool live = flushed + t8 < tiles_done && row >= p.row_start && row < p.row_end;
+        // lane l < 32: tile l >> 3 of the group of four, row l & 7: a token's 32 results are 128 consecutive bytes
+        const uint32_t t4 = (lane >> 3) & 3, row = (p.tile0 + k + flushed + t4) * 8 + (lane & 7);
+        const bool live = lane < 32 && flushed + t4 < tiles_done && row >= p.row_start && row < p.row_end;
 #pragma unroll
         for (int t = 0; t < B; t++) {
-            const float v = park[(t8 * B + t) * 8 + (lane & 7)];
+            const float v = park[(t4 * B + t) * 8 + (lane & 7)];
             if (live) yp[size_t(t) * p.y_stride + row] = v;
         }
         flushed = tiles_done;
@@ -507,26 +521,30 @@ __global__ __launch_bounds__(MAXT, kX4WavesPerSimd) void gemv_q8_0_x4_kernel(Rmi
                          : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]),
                            "+v"(acc[1][2]), "+v"(acc[1][3]));
             o = 0;
+            // The eight slices of a (row, token) meet through LDS, a group of four tokens at a time: every lane leaves
+            // its four sums where lane (token, row) of the first 32 finds the eight slices of its output, and adds them
+            // in hsum_ps order, ((l0 + l4) + (l1 + l5)) + ((l2 + l6) + (l3 + l7)).  A wave's LDS instructions are
+            // carried out in order, but the compiler knows nothing of lanes that talk to each other through memory: it
+            // had moved the upper lanes' writes of the second group in front of the lower lanes' reads of the first.
+            // The wave barriers (no instruction: a point no memory access crosses, reached by all lanes) say so.
 #pragma unroll
             for (int tg = 0; tg < TG; tg++) {
-                float u[4], total[4];
 #pragma unroll
-                for (int v = 0; v < 4; v++) {  // slices s and s + 4: lanes 16 apart
-                    u[v] = acc[tg][v] + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, acc[tg][v]), kSwizzleXor16));
+                for (int v = 0; v < 4; v++) {
+                    red[red_w[v]] = acc[tg][v];
                     acc[tg][v] = 0.0f;
                 }
+                rmi_wave_lds_fence();
+                float l[8];
 #pragma unroll
-                for (int r = 0; r < 4; r++) {  // (u0 + u1) + (u2 + u3) of row 4 rg + r, in the lanes with sl = 0
-                    const float a = u[r] + dpp_f32<kDppRowRor12>(u[(r + 3) & 3]);
-                    const float c = dpp_f32<kDppRowRor8>(u[(r + 2) & 3]) + dpp_f32<kDppRowRor4>(u[(r + 1) & 3]);
-                    total[r] = a + c;
-                }
-                if (sl == 0 && s_hi == 0 && j + 4 * tg < B)
-                    *reinterpret_cast<float4 *>(park + (((tiles_done & 7) * B + j + 4 * tg) * 8 + 4 * rg)) =
-                        make_float4(total[0], total[1], total[2], total[3]);
+                for (int sx = 0; sx < 8; sx++) l[sx] = red[sx * 33 + (lane & 31)];
+                const float y = ((l[0] + l[4]) + (l[1] + l[5])) + ((l[2] + l[6]) + (l[3] + l[7]));
+                const uint32_t tok = ((lane >> 3) & 3) + 4 * tg;
+                if (lane < 32 && tok < B) park[((tiles_done & 3) * B + tok) * 8 + (lane & 7)] = y;
+                rmi_wave_lds_fence();
             }
             tiles_done++;
-            if ((tiles_done & 7) == 0) flush();
+            if ((tiles_done & 3) == 0) flush();
         }
     };
     rmi_ring_walk(ring, n_units, cur, consume);
@@ -904,7 +922,7 @@ int launch_gemv(const RmiGemvProblem *single, const RmiGemvProblem *d_list, cons
     if constexpr (B >= 4) {
         // the kernel with the dots on the matrix cores, where its staging fits (its tokens lie further apart, and its
         // waves park finished tiles behind them)
-        const size_t x4_bytes = size_t(B) * rmi_gemv_x4_token_u4(max_n_oct) * 16 + size_t(wpg) * 8 * B * 32;
+        const size_t x4_bytes = size_t(B) * rmi_gemv_x4_token_u4(max_n_oct) * 16 + size_t(wpg) * kX4WaveFloats(B) * 4;
         if (x4_bytes <= 64 * 1024) {
             lds_bytes = x4_bytes;
             if (single && wpg == 1)
