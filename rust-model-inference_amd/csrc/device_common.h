@@ -61,6 +61,14 @@ __device__ __forceinline__ void rmi_gemm_tile_of(uint32_t lin, uint32_t grid_n, 
     }
 }
 
+// Between LDS accesses by which the lanes of ONE wave hand values to each other: every lane arrives, and the compiler
+// moves no memory access across (the barrier emits no instruction; it is a point in the program that accesses stay on
+// their side of).  The hardware carries a wave's LDS instructions out in order, which is all the hand-over needs; but
+// to the compiler lanes that talk through memory without this are a race, and it has been seen to move one lane
+// group's later writes in front of another's reads.  (Fences of wavefront scope around it would do the same and
+// wait for every global load in flight as well: 7 % on a kernel that prefetches across the point.)
+__device__ __forceinline__ void rmi_wave_lds_fence() { __builtin_amdgcn_wave_barrier(); }
+
 // signed 4 x int8 dot from zero (the build turns v_dot4c off, so this is one v_dot4_i32_i8 with a literal 0)
 __device__ __forceinline__ int dot4_i8(int a, int b) {
     return __builtin_amdgcn_sdot4(a, b, 0, false);

@@ -145,6 +145,9 @@ __global__ __launch_bounds__(64 * kKsplitMaxWaves) void gemm_q8_0_ksplit_kernel(
             const u32x2 wd = ld.wd;
             const u32x4 xs = ld.xs;
             stage_quad(ld);
+            rmi_wave_lds_fence();  // the lanes read each other's pieces (the loop has no divergent branch that the next
+                                   // quad's writes could be moved past this quad's reads through; a second barrier
+                                   // behind the reads costs 7 %: it also keeps the fold's tail from overlapping them)
             load_quad(ld, q + 1 < q_end ? q + 1 : q);
             fold_quad(wd, xs, q);
         }

@@ -342,14 +342,6 @@ __host__ __device__ inline uint32_t rmi_gemv_x4_token_u4(uint32_t n_oct) {
     const uint32_t plain = n_oct * 18;
     return plain + ((4 + 16 - (plain & 15)) & 15);
 }
-// Between LDS accesses by which the lanes of ONE wave hand values to each other: every lane arrives, and the compiler
-// moves no memory access across (the hardware carries a wave's LDS instructions out in order; no instruction is
-// emitted beyond the wait for the accesses in front).
-__device__ __forceinline__ void rmi_wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 // floats of LDS per wave behind the staged tokens: four tiles' results and the 8 x 33 partial sums of a tile's end
 __host__ __device__ constexpr uint32_t kX4WaveFloats(uint32_t n_tokens) { return 4 * n_tokens * 8 + 8 * 33 + 8; }
 // waves that are to share a SIMD (the register budget): five fit only with spills, and measured no faster
