@@ -513,6 +513,8 @@ def compact(r):
             "steps": r["steps"], "roofline": r["roofline"]}
     if r.get("other_mode"):
         keep["other_mode"] = r["other_mode"]
+    if r.get("ffn_stacked_gate_up"):
+        keep["ffn_stacked_gate_up"] = r["ffn_stacked_gate_up"]
     if r.get("cpu_baseline"):
         keep["cpu_baseline"] = r["cpu_baseline"]
     return keep
@@ -566,6 +568,23 @@ def run_gemm(args, pkg, ev):
     w2, d2 = time_region(H, ev, lambda: step(other), args.steps, args.warmup)
     result["other_mode"] = {"mode": "exact (tiled kernel, single chain)" if fast else "fast (kernel chosen per product)",
                             "value": round(ops / w2 / 1e12, 1), "unit": "TOP/s", "avg_launch_us": round(d2 * 1e3 / 2, 3)}
+    # The FFN as a host runs it after fuse_vstack (src/ops/quant/fuse.rs:25-64): gate and up are one stacked weight,
+    # one product of twice the rows, then down: three products' operations in two launches.
+    kg = K.Q8Kernel(synth.q8_0_weight(synth.seed_for(2, 7), 6144, 1024), 1024, 6144)
+    d_yg = H.DeviceBuffer(M * 6144 * 4)
+
+    def ffn(fn):
+        H.check(fn(kg.w.handle, recs[0]["d_q8"].ptr, recs[0]["d_sc"].ptr, d_yg.ptr, M, 6144, None))
+        H.check(fn(recs[1]["k"].w.handle, recs[1]["d_q8"].ptr, recs[1]["d_sc"].ptr, recs[1]["d_y"].ptr, M, 1024, None))
+
+    ffn_ops = 2.0 * M * 1024 * 6144 + 2.0 * M * 3072 * 1024
+    result["ffn_stacked_gate_up"] = {"workload": f"X[Mx1024].[W_gate ; W_up][6144x1024]^T, then X[Mx3072].W_down[1024x3072]^T, M={M}: "
+                                                 "2 launches, the operations of 3 products", "ops_per_step": ffn_ops, "unit": "TOP/s"}
+    for name, fn in (("fast", H.lib.rmi_hip_gemm_q8_0_fast_dev), ("exact", H.lib.rmi_hip_gemm_q8_0_dev)):
+        wf, df = time_region(H, ev, lambda: ffn(fn), args.steps, args.warmup)
+        result["ffn_stacked_gate_up"][name] = {"value": round(ffn_ops / wf / 1e12, 1), "us_per_step": round(df * 1e3, 3)}
+    d_yg.free()
+    kg.w.free()
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
@@ -868,6 +887,23 @@ def run_q4k_gemm(args, pkg, ev):
     result["roofline"] = {"bound": "mfma", "kernel": "gemm_q4_k_kernel", "achieved": round(achieved, 1),
                           "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s", "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
                           "avg_launch_us": round(dev_ms * 1e3 / 3, 3), **read_traffic("gemm_q4_k_m512_m2048_1.7b_ffn", f"m{M}")}
+    # The FFN as a host runs it after fuse_vstack (src/ops/quant/fuse.rs:25-64): gate and up are one stacked weight of
+    # twice the rows, then down: the same operations in two launches.
+    kg = K.Q4_KKernel(synth.q4_k_weight(synth.seed_for(3, 7), 12288, 2048), 2048, 12288)
+    d_yg = H.DeviceBuffer(M * 12288 * 4)
+
+    def ffn():
+        r = recs[0]
+        H.check(H.lib.rmi_hip_gemm_q4_k_q8k_dev(kg.w.handle, r["d_d"].ptr, r["d_q"].ptr, r["d_b"].ptr, d_yg.ptr, M, 12288, None))
+        r = recs[2]
+        H.check(H.lib.rmi_hip_gemm_q4_k_q8k_dev(r["k"].w.handle, r["d_d"].ptr, r["d_q"].ptr, r["d_b"].ptr, r["d_y"].ptr, M, 2048, None))
+
+    wf, df = time_region(H, ev, ffn, args.steps, args.warmup)
+    result["ffn_stacked_gate_up"] = {"workload": f"X[Mx2048].[W_gate ; W_up][12288x2048]^T, then X[Mx6144].W_down[2048x6144]^T, M={M}: "
+                                                 "2 launches, the same operations", "ops_per_step": ops,
+                                     "value": round(ops / wf / 1e12, 1), "unit": "TOP/s", "us_per_step": round(df * 1e3, 3)}
+    d_yg.free()
+    kg.w.free()
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import rmi_oracle as oracle
