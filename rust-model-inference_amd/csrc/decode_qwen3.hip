@@ -551,7 +551,9 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     // values: lane = (8 dimensions dg, key slice sl): 16 consecutive lanes read the 256 bytes of one row
     // (with PVP parts: 16 / PVP lanes read the part's 256 / PVP bytes of a row, PVP times as many slices)
     constexpr uint32_t kDgLanes = 16 / PVP, kSlices = kA128Threads / kDgLanes;
-    constexpr uint32_t kPre = (kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40)) / (PVP == 1 ? 1 : 2);
+    // With parts a slice is short (six keys cover 768 with four parts) and its loads are unconditional: a load under
+    // a branch makes the wait for this position's q, k, v (issued first) drain most of what was issued behind them.
+    constexpr uint32_t kPre = PVP == 1 ? (kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40)) : 24 / PVP;
     const uint32_t dg = tid % kDgLanes, sl = tid / kDgLanes;
     const uint32_t chunk = (n_cached + kSlices - 1) / kSlices;
     const uint32_t t_begin = sl * chunk, t_end = t_begin + chunk < n_cached ? t_begin + chunk : n_cached;
@@ -559,7 +561,7 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     uint4 vp[kPre];
 #pragma unroll
     for (uint32_t j = 0; j < kPre; j++) {  // j < chunk is uniform: no lane waits on a guarded load of its own
-        if (j < chunk) {
+        if (PVP > 1 || j < chunk) {
             const uint32_t t = t_begin + j < n_cached ? t_begin + j : last_row;
             vp[j] = vbase[__umul24(t, row_u4)];
         }
