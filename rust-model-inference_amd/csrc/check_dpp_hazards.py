@@ -20,7 +20,12 @@ Whoever adds another hand-written class (an `s_waitcnt`-sensitive memory instruc
 dependency wait states, writes of M0 or VCC in front of their readers, ...) has to add that class's rules here:
 the script knows nothing of hazards it was not told about.
 
-Usage: check_dpp_hazards.py file.s [minimum count of v_fmac_f32_dpp expected]."""
+A compile that silently dropped the hand-written instructions must not pass either: the optional second argument
+is a regular expression, and every function of the file whose symbol matches it (the set of instantiations is the
+build's own, not a number kept by hand) has to hold at least one v_fmac_f32_dpp, and at least one function has to
+match.  A plain number is taken as the minimum count over the whole file.
+
+Usage: check_dpp_hazards.py file.s [regular expression of the symbols that must hold v_fmac_f32_dpp | minimum count]."""
 import re
 import sys
 
@@ -131,7 +136,7 @@ def branch_target(ins):
 
 def main():
     path = sys.argv[1]
-    want = int(sys.argv[2]) if len(sys.argv) > 2 else 0
+    want = sys.argv[2] if len(sys.argv) > 2 else "0"
     code, labels = [], {}
     for item in instructions(path):
         if isinstance(item, tuple):
@@ -158,8 +163,26 @@ def main():
         print("hazard: %d wait state(s) between\n    %s\nand\n    %s" % (between, prev, ins))
     for ins in unknown[:20]:
         print("cannot follow: %s" % ins)
+    missing = []
+    if want.isdigit():
+        if n_fmac < int(want):
+            missing.append("the file: %d v_fmac_f32_dpp, %s expected" % (n_fmac, want))
+    else:
+        starts = sorted((at, name) for name, at in labels.items() if not name.startswith("."))  # function symbols
+        matched = 0
+        for i, (at, name) in enumerate(starts):
+            if not re.search(want, name):
+                continue
+            matched += 1
+            end = starts[i + 1][0] if i + 1 < len(starts) else len(code)
+            if not any(ins.startswith("v_fmac_f32_dpp") for ins in code[at:end]):
+                missing.append(name)
+        if not matched:
+            missing.append("no function symbol matches %r" % want)
+    for name in missing[:20]:
+        print("no v_fmac_f32_dpp: %s" % name)
     print("%s: %d DPP instructions (%d v_fmac_f32_dpp), %d hazards" % (path, n_dpp, n_fmac, len(bad)))
-    if bad or unknown or n_fmac < want:
+    if bad or unknown or missing:
         sys.exit(1)
 
 

@@ -55,6 +55,17 @@ def test_missing_instructions_fail(tmp_path):
     assert _run(tmp_path, ["v_mul_f32_e32 v3, v1, v2"], "1000").returncode == 1
 
 
+def test_every_matching_function_must_hold_the_instruction(tmp_path):
+    """With a regular expression instead of a count the functions that must hold a v_fmac_f32_dpp are the build's
+    own instantiations: one of them without it, or no match at all, fails."""
+    two = ["v_add_u32_e32 v20, v21, v22", "v_cvt_f32_i32_e32 v7, v8", FMAC, "s_endpgm", "kernel_b:", "v_add_u32_e32 v20, v21, v22"]
+    r = _run(tmp_path, two, "kernel")
+    assert r.returncode == 1 and "kernel_b" in r.stdout
+    assert _run(tmp_path, two, "kernel$").returncode == 0  # only the first function is named
+    assert _run(tmp_path, two + ["s_nop 1", FMAC], "kernel").returncode == 0
+    assert _run(tmp_path, two, "no_such_function").returncode == 1
+
+
 def test_hazard_across_a_branch_fails(tmp_path):
     """The write sits in front of a branch and the DPP read behind its target: text order alone would not see it."""
     body = ["v_mul_f32_e32 v3, v1, v2", "s_cbranch_scc1 .LBB0_2", "s_nop 7", "s_nop 7", "s_branch .LBB0_3",
