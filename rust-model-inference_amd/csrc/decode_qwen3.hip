@@ -459,6 +459,45 @@ __device__ __forceinline__ double swizzle_xor_f64(double v) {  // the value of l
                             __builtin_amdgcn_ds_swizzle(__double2loint(v), kPattern));
 }
 __device__ __forceinline__ double swizzle_xor16_f64(double v) { return swizzle_xor_f64<16>(v); }
+// Two registers exchange lanes in one vector instruction (v_permlane32_swap: lanes 32..63 of the first with lanes
+// 0..31 of the second; v_permlane16_swap: the odd rows of sixteen of the first with the even rows of the second).
+// a + b afterwards is, in the lower half (the even rows), a summed over both halves (both rows of a pair), and in the
+// upper half (the odd rows) b summed likewise: two values to reduce become one, without the LDS crossbar.
+template <bool ROWS>
+__device__ __forceinline__ double swap_add_f64(double a, double b) {
+    const uint64_t ab = __builtin_bit_cast(uint64_t, a), bb = __builtin_bit_cast(uint64_t, b);
+    uint64_t x, y;
+    if constexpr (ROWS) {
+        const auto lo = __builtin_amdgcn_permlane16_swap(uint32_t(ab), uint32_t(bb), false, false);
+        const auto hi = __builtin_amdgcn_permlane16_swap(uint32_t(ab >> 32), uint32_t(bb >> 32), false, false);
+        x = uint64_t(lo[0]) | (uint64_t(hi[0]) << 32);
+        y = uint64_t(lo[1]) | (uint64_t(hi[1]) << 32);
+    } else {
+        const auto lo = __builtin_amdgcn_permlane32_swap(uint32_t(ab), uint32_t(bb), false, false);
+        const auto hi = __builtin_amdgcn_permlane32_swap(uint32_t(ab >> 32), uint32_t(bb >> 32), false, false);
+        x = uint64_t(lo[0]) | (uint64_t(hi[0]) << 32);
+        y = uint64_t(lo[1]) | (uint64_t(hi[1]) << 32);
+    }
+    return __builtin_bit_cast(double, x) + __builtin_bit_cast(double, y);
+}
+// The eight f64 sums of a lane (dimensions 8 dg .. 8 dg + 7, dg = lane % DG_LANES) added over the wave's 64 / DG_LANES
+// key slices (lanes DG_LANES apart; DG_LANES = 4, 8 or 16).  Halves, then rows, halve the values as they halve the
+// lanes; what is left inside a row of sixteen goes round it by DPP.  Lane l ends with two sums, those of dimensions
+// 8 dg + pv_dim_base(l) and the next one.  (f64 sums of exact terms: the order of the additions is free.)
+__device__ __forceinline__ uint32_t pv_dim_base(uint32_t lane) { return 2 * ((lane >> 4) & 1) + 4 * (lane >> 5); }
+template <int DG_LANES>
+__device__ __forceinline__ void pv_slices_sum(const double (&acc)[8], double (&u)[2]) {
+    static_assert(DG_LANES == 4 || DG_LANES == 8 || DG_LANES == 16, "slices are whole parts of a row of sixteen lanes");
+    double r[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) r[k] = swap_add_f64<false>(acc[k], acc[k + 4]);
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        u[k] = swap_add_f64<true>(r[k], r[k + 2]);
+        if constexpr (DG_LANES <= 8) u[k] += dpp_f64<0x128>(u[k]);  // row_ror:8
+        if constexpr (DG_LANES <= 4) u[k] += dpp_f64<0x124>(u[k]);  // row_ror:4
+    }
+}
 __host__ __device__ inline size_t attn128_lds_bytes(uint32_t n_keys) {
     const size_t n_pad = (size_t(n_keys) + kAttnPad - 1) / kAttnPad * kAttnPad;
     return n_pad * 12 + (kA128Threads / 64) * 128 * 8 + 128;  // 32 floats of room behind the scores
@@ -734,17 +773,14 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
             for (int d = 0; d < 8; d++) acc[d] = __builtin_fma(double(float(vh[d])), w, acc[d]);
         }
     }
-#pragma unroll
-    for (int d = 0; d < 8; d++) {  // the slices of a wave: lanes kDgLanes apart
-        if constexpr (PVP >= 4) acc[d] += swizzle_xor_f64<4>(acc[d]);
-        if constexpr (PVP >= 2) acc[d] += swizzle_xor_f64<8>(acc[d]);
-        acc[d] += swizzle_xor16_f64(acc[d]);
-        acc[d] += __shfl_xor(acc[d], 32, 64);
-    }
-    if ((tid & 63) < kDgLanes) {
-        double *dst = part + (tid >> 6) * 128 + dg * 8;
-#pragma unroll
-        for (int d = 0; d < 8; d++) dst[d] = acc[d];
+    {  // the slices of a wave: lanes kDgLanes apart
+        double u[2];
+        pv_slices_sum<kDgLanes>(acc, u);
+        if ((tid & 15) < kDgLanes) {  // one lane of each row for every dg
+            double *dst = part + (tid >> 6) * 128 + dg * 8 + pv_dim_base(tid & 63);
+            dst[0] = u[0];
+            dst[1] = u[1];
+        }
     }
     __syncthreads();
     if (tid < 32 / PVP) {  // four dimensions per lane: whole 8-lane groups for the quantizer
@@ -986,15 +1022,12 @@ __global__ __launch_bounds__(kAttnSplitThreads) void attn128_weights_pv_kernel(
             for (uint32_t j = 0; j < 8; j++) cur[j] = nxt[j];
         }
     }
-#pragma unroll
-    for (int d = 0; d < 8; d++) {  // the four slices of a wave: lanes 16 apart
-        acc[d] += swizzle_xor16_f64(acc[d]);
-        acc[d] += __shfl_xor(acc[d], 32, 64);
-    }
-    if ((tid & 63) < 16) {
-        double *dst = wave_sums + (tid >> 6) * 128 + dg * 8;
-#pragma unroll
-        for (int d = 0; d < 8; d++) dst[d] = acc[d];
+    {  // the four slices of a wave: lanes 16 apart
+        double u[2];
+        pv_slices_sum<16>(acc, u);
+        double *dst = wave_sums + (tid >> 6) * 128 + dg * 8 + pv_dim_base(tid & 63);
+        dst[0] = u[0];
+        dst[1] = u[1];
     }
     __syncthreads();
     // The first wave alone hands the part's sums over: its stores, one release (the other waves have nothing in
