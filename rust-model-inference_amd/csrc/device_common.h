@@ -82,7 +82,6 @@ constexpr int kDppRowHalfMirror = 0x141;                          // lane i <-> 
 constexpr int kDppRowMirror = 0x140;                              // lane i <-> 15 - i of each 16 lanes
 constexpr int kDppRowBcast15 = 0x142;                             // lane 15 of a row to the whole next row
 constexpr int kDppRowBcast31 = 0x143;                             // lane 31 to rows 2 and 3
-constexpr int kSwizzleXor4 = 0x1f | (4 << 10);                    // bit-mask mode: and 0x1f, or 0, xor 4
 constexpr int kSwizzleFirstOf8 = 0x18;                            // bit-mask mode: lane & ~7
 
 template <int CTRL, int ROW_MASK = 0xf>
@@ -100,10 +99,21 @@ __device__ __forceinline__ double dpp_f64(double v) {
     return __builtin_bit_cast(double, lo | (hi << 32));
 }
 
+// The value of lane ^ 4 without the LDS crossbar: lanes 0..3 and 8..11 of a row of sixteen (banks 0 and 2) read four
+// lanes up (row_shl:4), the others four lanes down (row_shr:4); two vector moves instead of a ds_swizzle, whose
+// round trip a lone wave waits out.
+constexpr int kDppRowShl4 = 0x104, kDppRowShr4 = 0x114;
+__device__ __forceinline__ float dpp_xor4_f32(float v) {
+    const int b = __builtin_bit_cast(int, v);
+    int r = __builtin_amdgcn_update_dpp(0, b, kDppRowShl4, 0xf, 0x5, false);
+    r = __builtin_amdgcn_update_dpp(r, b, kDppRowShr4, 0xf, 0xa, false);
+    return __builtin_bit_cast(float, r);
+}
+
 // ((l0+l4)+(l1+l5))+((l2+l6)+(l3+l7)) of the eight lanes of a row (src/ops/dot.rs:447-456); every lane of the
 // row ends up with the sum (a + b and b + a are the same bits).
 __device__ __forceinline__ float hsum8_lanes(float a) {
-    a = a + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, a), kSwizzleXor4));
+    a = a + dpp_xor4_f32(a);
     a = a + dpp_f32<kDppQuadXor1>(a);
     a = a + dpp_f32<kDppQuadXor2>(a);
     return a;
