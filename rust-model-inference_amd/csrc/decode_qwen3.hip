@@ -521,8 +521,11 @@ struct AttnFromQkv {
     uint16_t *k_row, *v_row;         // the cache rows of this position, [n_head_kv][128] each
     float eps;
 };
-template <bool FROM_QKV, int PVP = 1>
-__global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
+// DENSE: for launches of many workgroups (a prompt pass: positions x heads).  Every phase below is a stretch of
+// dependent instructions, so one workgroup leaves its compute unit idle most of the time; with the registers held
+// to 128 (a short value prefetch) two workgroups share a unit and fill each other's waits.
+template <bool FROM_QKV, int PVP = 1, bool DENSE = false>
+__global__ __launch_bounds__(kA128Threads, DENSE ? 4 : 2) void attention128_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
     uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, int8_t *__restrict__ q8,
     float *__restrict__ scales, int rounding, AttnFromQkv fq, uint32_t tok_q16_stride, uint32_t tok_out_stride) {
@@ -592,7 +595,7 @@ __global__ __launch_bounds__(kA128Threads) void attention128_quant_kernel(
     constexpr uint32_t kDgLanes = 16 / PVP, kSlices = kA128Threads / kDgLanes;
     // With parts a slice is short (six keys cover 768 with four parts) and its loads are unconditional: a load under
     // a branch makes the wait for this position's q, k, v (issued first) drain most of what was issued behind them.
-    constexpr uint32_t kPre = PVP == 1 ? (kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40)) : 24 / PVP;
+    constexpr uint32_t kPre = DENSE ? 4 : (PVP == 1 ? (kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40)) : 24 / PVP);
     const uint32_t dg = tid % kDgLanes, sl = tid / kDgLanes;
     const uint32_t chunk = (n_cached + kSlices - 1) / kSlices;
     const uint32_t t_begin = sl * chunk, t_end = t_begin + chunk < n_cached ? t_begin + chunk : n_cached;
@@ -1510,7 +1513,8 @@ int enqueue_prompt_pass(rmi_hip_qwen3 *s, uint32_t step0, uint32_t n, hipStream_
         hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(c.n_head + 2 * c.n_head_kv, n), dim3(64), 0, st, s->qkvb, qn, kn,
                            s->cos_t, s->sin_t, step0, s->q16b, s->k_cache + row, s->v_cache + row, c.n_head, c.n_head_kv,
                            c.head_dim_k, c.head_dim_v, c.eps, TokStride3{n_qkv, s->n_q, s->kv_stride});
-        hipLaunchKernelGGL(attention128_quant_kernel<false>, dim3(c.n_head / c.n_head_kv, c.n_head_kv, n), dim3(kA128Threads),
+        // (a pass ends short of the split's first position, far below the 64 KiB of LDS a launch may take unasked)
+        hipLaunchKernelGGL((attention128_quant_kernel<false, 1, true>), dim3(c.n_head / c.n_head_kv, c.n_head_kv, n), dim3(kA128Threads),
                            attn128_lds_bytes(step0 + n), st, s->q16b, s->k_cache + layer_base, s->v_cache + layer_base, step0,
                            s->kv_stride, c.n_head, c.n_head_kv, s->act_q8b, s->act_scalesb, rnd, AttnFromQkv{}, s->n_q, s->n_attn);
         rc = rmi_gemv_q8_0_tokens(s->w_o[l], s->act_q8b, s->act_scalesb, s->residb, n, c.n_embd, 0, c.n_embd, st);
