@@ -524,8 +524,9 @@ struct AttnFromQkv {
 // DENSE: for launches of many workgroups (a prompt pass: positions x heads).  Every phase below is a stretch of
 // dependent instructions, so one workgroup leaves its compute unit idle most of the time; with the registers held
 // to 128 (a short value prefetch) two workgroups share a unit and fill each other's waits.
+constexpr int kDenseWaves = 6, kDenseBatch = 2;
 template <bool FROM_QKV, int PVP = 1, bool DENSE = false>
-__global__ __launch_bounds__(kA128Threads, DENSE ? 4 : 2) void attention128_quant_kernel(
+__global__ __launch_bounds__(kA128Threads, DENSE ? kDenseWaves : 2) void attention128_quant_kernel(
     const uint16_t *__restrict__ q16, const uint16_t *__restrict__ k_cache, const uint16_t *__restrict__ v_cache,
     uint32_t step, uint32_t kv_stride, uint32_t n_head, uint32_t n_head_kv, int8_t *__restrict__ q8,
     float *__restrict__ scales, int rounding, AttnFromQkv fq, uint32_t tok_q16_stride, uint32_t tok_out_stride) {
@@ -595,7 +596,8 @@ __global__ __launch_bounds__(kA128Threads, DENSE ? 4 : 2) void attention128_quan
     constexpr uint32_t kDgLanes = 16 / PVP, kSlices = kA128Threads / kDgLanes;
     // With parts a slice is short (six keys cover 768 with four parts) and its loads are unconditional: a load under
     // a branch makes the wait for this position's q, k, v (issued first) drain most of what was issued behind them.
-    constexpr uint32_t kPre = DENSE ? 4 : (PVP == 1 ? (kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40)) : 24 / PVP);
+    constexpr uint32_t kPre = DENSE ? 1 : (PVP == 1 ? (kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40)) : 24 / PVP);
+    constexpr uint32_t kBatch = DENSE ? kDenseBatch : 8;  // keys of a slice in flight beyond the first kPre
     const uint32_t dg = tid % kDgLanes, sl = tid / kDgLanes;
     const uint32_t chunk = (n_cached + kSlices - 1) / kSlices;
     const uint32_t t_begin = sl * chunk, t_end = t_begin + chunk < n_cached ? t_begin + chunk : n_cached;
@@ -695,14 +697,15 @@ __global__ __launch_bounds__(kA128Threads, DENSE ? 4 : 2) void attention128_quan
     if (tid == 0) {  // the reference adds the weights one after the other in f32; the padding zeros change nothing
         // one lane, one dependent chain of adds; the LDS reads run 32 values ahead of it (two buffers, no copies)
         float acc = 0.0f;
-        float4 a[8], b[8];
+        constexpr int kAhead = DENSE ? 4 : 8;  // float4 of each buffer
+        float4 a[kAhead], b[kAhead];
 #pragma unroll
-        for (int j = 0; j < 8; j++) a[j] = reinterpret_cast<const float4 *>(scores)[j];
-        for (uint32_t t = 0; t < n_pad; t += 64) {  // n_pad is a multiple of 64
+        for (int j = 0; j < kAhead; j++) a[j] = reinterpret_cast<const float4 *>(scores)[j];
+        for (uint32_t t = 0; t < n_pad; t += 8 * kAhead) {  // n_pad is a multiple of 64
 #pragma unroll
-            for (int j = 0; j < 8; j++) b[j] = reinterpret_cast<const float4 *>(scores + t + 32)[j];
+            for (int j = 0; j < kAhead; j++) b[j] = reinterpret_cast<const float4 *>(scores + t + 4 * kAhead)[j];
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
+            for (int j = 0; j < kAhead; j++) {
                 acc += a[j].x;
                 acc += a[j].y;
                 acc += a[j].z;
@@ -711,9 +714,9 @@ __global__ __launch_bounds__(kA128Threads, DENSE ? 4 : 2) void attention128_quan
             // unconditional (the array has 32 floats of room behind n_pad): under a branch the registers would be
             // copied every round, on the chain's own lane
 #pragma unroll
-            for (int j = 0; j < 8; j++) a[j] = reinterpret_cast<const float4 *>(scores + t + 64)[j];
+            for (int j = 0; j < kAhead; j++) a[j] = reinterpret_cast<const float4 *>(scores + t + 8 * kAhead)[j];
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
+            for (int j = 0; j < kAhead; j++) {
                 acc += b[j].x;
                 acc += b[j].y;
                 acc += b[j].z;
@@ -742,21 +745,21 @@ __global__ __launch_bounds__(kA128Threads, DENSE ? 4 : 2) void attention128_quan
             for (int d = 0; d < 8; d++) acc[d] = __builtin_fma(double(float(vh[d])), w, acc[d]);
         }
     }
-    if (t_begin + kPre < t_end) {  // longer slices: batches of 8 keys, the next one in flight while one is added
-        uint4 cur[8], nxt[8];
+    if (t_begin + kPre < t_end) {  // longer slices: batches of kBatch keys, the next one in flight while one is added
+        uint4 cur[kBatch], nxt[kBatch];
 #pragma unroll
-        for (uint32_t j = 0; j < 8; j++) {
+        for (uint32_t j = 0; j < kBatch; j++) {
             const uint32_t t = t_begin + kPre + j;
             cur[j] = vbase[__umul24(t < n_cached ? t : last_row, row_u4)];
         }
-        for (uint32_t t0 = t_begin + kPre; t0 < t_end; t0 += 8) {
+        for (uint32_t t0 = t_begin + kPre; t0 < t_end; t0 += kBatch) {
 #pragma unroll
-            for (uint32_t j = 0; j < 8; j++) {
-                const uint32_t t = t0 + 8 + j;
+            for (uint32_t j = 0; j < kBatch; j++) {
+                const uint32_t t = t0 + kBatch + j;
                 nxt[j] = vbase[__umul24(t < n_cached ? t : last_row, row_u4)];
             }
 #pragma unroll
-            for (uint32_t j = 0; j < 8; j++) {
+            for (uint32_t j = 0; j < kBatch; j++) {
                 if (t0 + j < t_end) {
                     const double w = wd[t0 + j];
                     const half8 vh = as_half8(cur[j]);
@@ -765,7 +768,7 @@ __global__ __launch_bounds__(kA128Threads, DENSE ? 4 : 2) void attention128_quan
                 }
             }
 #pragma unroll
-            for (uint32_t j = 0; j < 8; j++) cur[j] = nxt[j];
+            for (uint32_t j = 0; j < kBatch; j++) cur[j] = nxt[j];
         }
     }
     if constexpr (FROM_QKV) {
