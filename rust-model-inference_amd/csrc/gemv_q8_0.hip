@@ -217,6 +217,48 @@ __device__ __forceinline__ void octet_fma(float (&acc)[B], const OctetRegs &g, c
     }
 }
 
+// One token's staged operands of an octet, as a lane reads them from LDS.
+struct OctetX {
+    uint4 xa, xb;   // bytes 4L..4L+3 of blocks 8o..8o+3 and 8o+4..8o+7
+    float4 s0, s1;  // the eight block scales
+};
+__device__ __forceinline__ OctetX load_octet_x(const uint4 *lds, uint32_t n_oct, uint32_t o, uint32_t L) {
+    OctetX x;
+    x.xa = lds[(2 * o) * 8 + L];
+    x.xb = lds[(2 * o + 1) * 8 + L];
+    x.s0 = reinterpret_cast<const float4 *>(lds + n_oct * 16)[2 * o];
+    x.s1 = reinterpret_cast<const float4 *>(lds + n_oct * 16)[2 * o + 1];
+    return x;
+}
+// The NOCT octets of a tile whose weights are in registers already, one token: the LDS reads of octet o + 1 go out
+// before octet o is multiplied.  A wave that has its compute unit to itself otherwise waits out an LDS round trip
+// per octet (the reads of an octet and the wait for the first of them stood back to back).  Same arithmetic and
+// order as octet_fma<1>.
+template <int NOCT>
+__device__ __forceinline__ void octets_fma_ahead(float &acc, const OctetRegs (&g)[NOCT], const uint4 *lds, uint32_t L) {
+    OctetX x = load_octet_x(lds, NOCT, 0, L);
+    float a = acc;
+#pragma unroll
+    for (int o = 0; o < NOCT; o++) {
+        OctetX nx = x;
+        if (o + 1 < NOCT) nx = load_octet_x(lds, NOCT, o + 1, L);
+        // The sum passes a point that no memory access moves across: the reads of octet o + 1 stay in front of
+        // the multiply-adds of octet o.  (Left to itself the compiler moves them back down to their uses.)
+        asm volatile("" : "+v"(a) : : "memory");
+        const OctetRegs &w = g[o];
+        block_fma<true>(a, w.sc.x & 0xffffu, x.s0.x, int(w.qa.x), int(x.xa.x));
+        block_fma<true>(a, w.sc.x >> 16, x.s0.y, int(w.qa.y), int(x.xa.y));
+        block_fma<true>(a, w.sc.y & 0xffffu, x.s0.z, int(w.qa.z), int(x.xa.z));
+        block_fma<true>(a, w.sc.y >> 16, x.s0.w, int(w.qa.w), int(x.xa.w));
+        block_fma<true>(a, w.sc.z & 0xffffu, x.s1.x, int(w.qb.x), int(x.xb.x));
+        block_fma<true>(a, w.sc.z >> 16, x.s1.y, int(w.qb.y), int(x.xb.y));
+        block_fma<true>(a, w.sc.w & 0xffffu, x.s1.z, int(w.qb.z), int(x.xb.z));
+        block_fma<true>(a, w.sc.w >> 16, x.s1.w, int(w.qb.w), int(x.xb.w));
+        x = nx;
+    }
+    acc = a;
+}
+
 // A wave owns a short run of consecutive 8-row tiles of ONE matrix (about 34 KiB of
 // weights) and walks it four octets deep (device_run_ring.h).  A launch has far more
 // waves than fit on the chip at once: the dispatcher hands out runs as waves retire,
@@ -559,8 +601,7 @@ __global__ __launch_bounds__(64) void gemv_q8_0_deep_kernel(RmiGemvProblem p) {
     stage_token<(NOCT + 3) / 4>(reinterpret_cast<uint32_t *>(lds), p.x_q8, p.x_scales, NOCT, p.n_in >> 5, lane, 64);
     __syncthreads();
     float acc[1] = {0.0f};
-#pragma unroll
-    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
+    octets_fma_ahead<NOCT>(acc[0], g, lds, L);
     const uint32_t row = (p.tile0 + k) * kTileRows + r;
     const float y = hsum8_lanes(acc[0]);
     if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
@@ -638,8 +679,7 @@ __global__ __launch_bounds__(64) void gemv_q8_0_norm_deep_kernel(RmiGemvProblem 
     }
     __syncthreads();
     float acc[1] = {0.0f};
-#pragma unroll
-    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
+    octets_fma_ahead<NOCT>(acc[0], g, lds, L);
     const uint32_t row = (p.tile0 + k) * kTileRows + r;
     const float y = hsum8_lanes(acc[0]);
     if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
@@ -716,8 +756,7 @@ __global__ __launch_bounds__(512) void gemv_q8_0_norm_silu_kernel(const uint8_t 
     }
     __syncthreads();
     float acc[1] = {0.0f};
-#pragma unroll
-    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
+    octets_fma_ahead<NOCT>(acc[0], g, lds, L);
     const float y = hsum8_lanes(acc[0]);
     if (L == 0) gu[wave * 8 + r] = y;  // [0,32): gate rows of this block, [32,64): up rows
     __syncthreads();
@@ -833,10 +872,8 @@ __global__ __launch_bounds__(512) void gemv_q8_0_norm_rope_kernel(const uint8_t 
     }
     __syncthreads();
     float acc[1] = {0.0f}, acc2[1] = {0.0f};
-#pragma unroll
-    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc, g[o], lds, NOCT * 18, NOCT, o, L);
-#pragma unroll
-    for (int o = 0; o < NOCT; o++) octet_fma<1>(acc2, g2[o], lds, NOCT * 18, NOCT, o, L);
+    octets_fma_ahead<NOCT>(acc[0], g, lds, L);
+    octets_fma_ahead<NOCT>(acc2[0], g2, lds, L);
     const float y = hsum8_lanes(acc[0]), y2 = hsum8_lanes(acc2[0]);
     if (L == 0) {
         yl[wave * 16 + r] = y;
