@@ -589,16 +589,69 @@ __global__ __launch_bounds__(MAXT, kX4WavesPerSimd) void gemv_q8_0_x4_kernel(Rmi
 // latency, not bandwidth: one wave per tile, and all loads of the tile's NOCT octets go out at once, before
 // the activation is staged, so the wave sees one memory round trip instead of one per pipeline refill.
 // Same arithmetic and order as the streaming kernel above.
+// stage_token for one wave and NOCT <= 16 octets in two halves, so that other loads can go out between the
+// activation's loads and the LDS writes that wait for them.
+template <int NOCT>
+struct TokenRegs {
+    u32x4 v[(NOCT + 3) / 4];
+    float sv0, sv1;
+};
+template <int NOCT>
+__device__ __forceinline__ void wave_token_load(TokenRegs<NOCT> &t, const int8_t *x_q8, const float *x_scales, uint32_t nb,
+                                                uint32_t lane) {
+    gptr_u4 xq = as_global<gptr_u4>(x_q8);
+    gptr_f32 xs = as_global<gptr_f32>(x_scales);
+    const uint32_t src_u4 = nb * 2, s0 = lane, s1 = lane + 64;
+#pragma unroll
+    for (int j = 0; j < (NOCT + 3) / 4; j++) {
+        const uint32_t i = lane + j * 64;
+        t.v[j] = xq[i < src_u4 ? i : src_u4 - 1];
+    }
+    t.sv0 = xs[s0 < nb ? s0 : nb - 1];
+    t.sv1 = xs[s1 < nb ? s1 : nb - 1];
+}
+template <int NOCT>
+__device__ __forceinline__ void wave_token_store(const TokenRegs<NOCT> &t, uint32_t *dq, uint32_t nb, uint32_t lane) {
+    static_assert(NOCT <= 16, "two scales a lane cover 128 blocks");
+    const uint32_t n_u4 = NOCT * 16, src_u4 = nb * 2, s0 = lane, s1 = lane + 64;
+#pragma unroll
+    for (int j = 0; j < (NOCT + 3) / 4; j++) {
+        const uint32_t i = lane + j * 64;
+        if (i < n_u4) {
+            const uint32_t b = i >> 1;  // block; this uint4 holds its dwords l = 4*(i&1) .. +3
+            uint32_t *d = dq + (b >> 2) * 32 + (i & 1) * 16 + (b & 3);
+            const bool live = i < src_u4;
+            d[0] = live ? t.v[j].x : 0u;
+            d[4] = live ? t.v[j].y : 0u;
+            d[8] = live ? t.v[j].z : 0u;
+            d[12] = live ? t.v[j].w : 0u;
+        }
+    }
+    float *ds = reinterpret_cast<float *>(dq + NOCT * 64);
+    if (s0 < NOCT * 8) ds[s0] = s0 < nb ? t.sv0 : 0.0f;
+    if (s1 < NOCT * 8) ds[s1] = s1 < nb ? t.sv1 : 0.0f;
+}
+
+// The activation's loads go out first and the weights' behind them: loads come back in the order they were issued,
+// so the activation is staged while the weights arrive and octet o is multiplied as soon as ITS pieces are there
+// (a compute unit takes in a lone wave's 1 KiB loads one every 30 clocks or so, and an octet takes 200 clocks to
+// multiply: with the activation last, nothing started before the last piece had arrived).
 template <int NOCT>
 __global__ __launch_bounds__(64) void gemv_q8_0_deep_kernel(RmiGemvProblem p) {
     extern __shared__ uint4 lds[];
     const uint32_t lane = threadIdx.x, r = lane >> 3, L = lane & 7;
     const uint32_t k = blockIdx.x;
+    TokenRegs<NOCT> tok;
+    wave_token_load<NOCT>(tok, p.x_q8, p.x_scales, p.n_in >> 5, lane);
+    asm volatile("" : : : "memory");  // the compiler keeps this order of the loads (it had moved one of these behind the weights)
     gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * NOCT * kOctetBytes);
     OctetRegs g[NOCT];
 #pragma unroll
-    for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
-    stage_token<(NOCT + 3) / 4>(reinterpret_cast<uint32_t *>(lds), p.x_q8, p.x_scales, NOCT, p.n_in >> 5, lane, 64);
+    for (int o = 0; o < NOCT; o++) {  // octet after octet, in the order they are multiplied
+        load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+        asm volatile("" : : : "memory");
+    }
+    wave_token_store<NOCT>(tok, reinterpret_cast<uint32_t *>(lds), p.n_in >> 5, lane);
     __syncthreads();
     float acc[1] = {0.0f};
     octets_fma_ahead<NOCT>(acc[0], g, lds, L);
@@ -638,7 +691,10 @@ __global__ __launch_bounds__(64) void gemv_q8_0_norm_deep_kernel(RmiGemvProblem 
     gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * NOCT * kOctetBytes);
     OctetRegs g[NOCT];
 #pragma unroll
-    for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+    for (int o = 0; o < NOCT; o++) {  // octet after octet, in the order they are multiplied
+        load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+        asm volatile("" : : : "memory");
+    }
 
     double part = 0.0;
 #pragma unroll
@@ -717,7 +773,10 @@ __global__ __launch_bounds__(512) void gemv_q8_0_norm_silu_kernel(const uint8_t 
     gptr_u4 tile = as_global<gptr_u4>(w + size_t(tile_idx) * NOCT * kOctetBytes);
     OctetRegs g[NOCT];
 #pragma unroll
-    for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+    for (int o = 0; o < NOCT; o++) {  // octet after octet, in the order they are multiplied
+        load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+        asm volatile("" : : : "memory");
+    }
 
     if (owner) {
         if (na.resid) {
@@ -819,9 +878,15 @@ __global__ __launch_bounds__(512) void gemv_q8_0_norm_rope_kernel(const uint8_t 
     gptr_u4 tile2 = tile + NOCT * (kOctetBytes / 16);
     OctetRegs g[NOCT], g2[NOCT];
 #pragma unroll
-    for (int o = 0; o < NOCT; o++) load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+    for (int o = 0; o < NOCT; o++) {  // octet after octet, in the order they are multiplied
+        load_octet(g[o], tile + r, tile + NOCT * 8 + lane, o);
+        asm volatile("" : : : "memory");
+    }
 #pragma unroll
-    for (int o = 0; o < NOCT; o++) load_octet(g2[o], tile2 + r, tile2 + NOCT * 8 + lane, o);
+    for (int o = 0; o < NOCT; o++) {
+        load_octet(g2[o], tile2 + r, tile2 + NOCT * 8 + lane, o);
+        asm volatile("" : : : "memory");
+    }
     // what the first wave needs at the end: out now, used after the products
     const bool is_q = head < ra.n_head, is_v = head >= ra.n_head + ra.n_head_kv;
     const float *nw = is_q ? ra.q_norm : ra.k_norm;
