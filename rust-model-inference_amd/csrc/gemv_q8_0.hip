@@ -235,13 +235,14 @@ __device__ __forceinline__ OctetX load_octet_x(const uint4 *lds, uint32_t n_oct,
 // per octet (the reads of an octet and the wait for the first of them stood back to back).  Same arithmetic and
 // order as octet_fma<1>.
 template <int NOCT>
-__device__ __forceinline__ void octets_fma_ahead(float &acc, const OctetRegs (&g)[NOCT], const uint4 *lds, uint32_t L) {
-    OctetX x = load_octet_x(lds, NOCT, 0, L);
+__device__ __forceinline__ void octets_fma_ahead(float &acc, const OctetRegs (&g)[NOCT], const uint4 *lds, uint32_t L,
+                                                 uint32_t n_staged = NOCT) {  // octets staged in LDS (NOCT or more)
+    OctetX x = load_octet_x(lds, n_staged, 0, L);
     float a = acc;
 #pragma unroll
     for (int o = 0; o < NOCT; o++) {
         OctetX nx = x;
-        if (o + 1 < NOCT) nx = load_octet_x(lds, NOCT, o + 1, L);
+        if (o + 1 < NOCT) nx = load_octet_x(lds, n_staged, o + 1, L);
         // The sum passes a point that no memory access moves across: the reads of octet o + 1 stay in front of
         // the multiply-adds of octet o.  (Left to itself the compiler moves them back down to their uses.)
         asm volatile("" : "+v"(a) : : "memory");
@@ -979,6 +980,96 @@ int launch_gemv_norm_rope(const rmi_hip_weight *w, const RmiNormArgs &na, const 
     return RMI_HIP_OK;
 }
 
+// The same tile on W waves, for launches that leave most of the chip idle anyway.  A lone wave multiplies an octet
+// in about 200 clocks (36 vector instructions, dependent ones eight clocks apart), and only one in four of them is
+// the row sums' own chain: fma(scale product, float(dot), acc), block after block.  Wave w loads the octets
+// [w N, (w + 1) N), N = NOCT / W; waves 1.. multiply theirs down to the two factors of every block's fma and leave
+// them in LDS; wave 0 multiplies the first N octets as before and then only adds: the same operations on the same
+// values in the same order, a quarter of them on the critical path.  Every wave issues a quarter of the loads.
+template <int NOCT, int W>
+__global__ __launch_bounds__(64 * W) void gemv_q8_0_deep_split_kernel(RmiGemvProblem p) {
+    static_assert(NOCT % W == 0 && NOCT * 16 <= 64 * W, "whole octets a wave, one piece of the activation a thread");
+    constexpr int N = NOCT / W;
+    extern __shared__ uint4 lds[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, r = lane >> 3, L = lane & 7;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t k = blockIdx.x, nb = p.n_in >> 5;
+    // the activation: thread t takes the 16-byte piece t and the block scale t (zeros beyond the nb source blocks)
+    gptr_u4 xq = as_global<gptr_u4>(p.x_q8);
+    gptr_f32 xs = as_global<gptr_f32>(p.x_scales);
+    const uint32_t src_u4 = nb * 2;
+    const u32x4 xv = xq[tid < src_u4 ? tid : src_u4 - 1];
+    const float xsv = xs[tid < nb ? tid : nb - 1];
+    asm volatile("" : : : "memory");  // the activation's loads stay in front of the weights'
+    gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * NOCT * kOctetBytes);
+    OctetRegs g[N];
+#pragma unroll
+    for (int i = 0; i < N; i++) {  // octet after octet, in the order they are multiplied
+        load_octet(g[i], tile + r, tile + NOCT * 8 + lane, wave * N + i);
+        asm volatile("" : : : "memory");
+    }
+    uint32_t *dq = reinterpret_cast<uint32_t *>(lds);
+    if (tid < NOCT * 16) {
+        const uint32_t b = tid >> 1;  // block; this piece holds its dwords l = 4*(tid&1) .. +3
+        uint32_t *d = dq + (b >> 2) * 32 + (tid & 1) * 16 + (b & 3);
+        const bool live = tid < src_u4;
+        d[0] = live ? xv.x : 0u;
+        d[4] = live ? xv.y : 0u;
+        d[8] = live ? xv.z : 0u;
+        d[12] = live ? xv.w : 0u;
+    }
+    if (tid < NOCT * 8) reinterpret_cast<float *>(dq + NOCT * 64)[tid] = tid < nb ? xsv : 0.0f;
+    __syncthreads();
+    // the factors of the octets N .. NOCT - 1: [octet - N][pair of blocks q][lane] = {s, float(dot), s', float(dot')}
+    float4 *hand = reinterpret_cast<float4 *>(lds + NOCT * 18);
+    if (wave != 0) {
+        OctetX x = load_octet_x(lds, NOCT, wave * N, L);
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            OctetX nx = x;
+            if (i + 1 < N) nx = load_octet_x(lds, NOCT, wave * N + i + 1, L);
+            const OctetRegs &w = g[i];
+            float4 *dst = hand + ((wave - 1) * N + i) * 4 * 64 + lane;
+            dst[0] = make_float4(h2f_times<true>(w.sc.x & 0xffffu, x.s0.x), float(dot4_i8(int(w.qa.x), int(x.xa.x))),
+                                 h2f_times<true>(w.sc.x >> 16, x.s0.y), float(dot4_i8(int(w.qa.y), int(x.xa.y))));
+            dst[64] = make_float4(h2f_times<true>(w.sc.y & 0xffffu, x.s0.z), float(dot4_i8(int(w.qa.z), int(x.xa.z))),
+                                  h2f_times<true>(w.sc.y >> 16, x.s0.w), float(dot4_i8(int(w.qa.w), int(x.xa.w))));
+            dst[128] = make_float4(h2f_times<true>(w.sc.z & 0xffffu, x.s1.x), float(dot4_i8(int(w.qb.x), int(x.xb.x))),
+                                   h2f_times<true>(w.sc.z >> 16, x.s1.y), float(dot4_i8(int(w.qb.y), int(x.xb.y))));
+            dst[192] = make_float4(h2f_times<true>(w.sc.w & 0xffffu, x.s1.z), float(dot4_i8(int(w.qb.z), int(x.xb.z))),
+                                   h2f_times<true>(w.sc.w >> 16, x.s1.w), float(dot4_i8(int(w.qb.w), int(x.xb.w))));
+            x = nx;
+        }
+    }
+    float acc = 0.0f;
+    if (wave == 0) octets_fma_ahead<N>(acc, g, lds, L, NOCT);
+    __syncthreads();
+    if (wave != 0) return;
+    {
+        const float4 *src = hand + lane;
+        float4 f[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) f[q] = src[q * 64];
+#pragma unroll
+        for (int o = 0; o < NOCT - N; o++) {
+            float4 nf[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) nf[q] = o + 1 < NOCT - N ? src[((o + 1) * 4 + q) * 64] : f[q];
+            asm volatile("" : "+v"(acc) : : "memory");  // the next octet's reads stay in front of this octet's sums
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                acc = __builtin_fmaf(f[q].x, f[q].y, acc);
+                acc = __builtin_fmaf(f[q].z, f[q].w, acc);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) f[q] = nf[q];
+        }
+    }
+    const uint32_t row = (p.tile0 + k) * kTileRows + r;
+    const float y = hsum8_lanes(acc);
+    if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
+}
+
 template <int NOCT>
 int launch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
     hipLaunchKernelGGL((gemv_q8_0_deep_kernel<NOCT>), dim3(p.n_tiles), dim3(64), size_t(NOCT) * 288, s, p);
@@ -987,7 +1078,25 @@ int launch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
 }
 
 constexpr uint32_t kDeepMaxOct = 12, kDeepMaxTiles = 4096;
+template <int NOCT, int W>
+int launch_gemv_deep_split(const RmiGemvProblem &p, hipStream_t s) {
+    constexpr size_t kLds = size_t(NOCT) * 288 + size_t(NOCT - NOCT / W) * 4 * 64 * 16;
+    static_assert(kLds <= 64 * 1024, "staged activation and handed-over factors");
+    hipLaunchKernelGGL((gemv_q8_0_deep_split_kernel<NOCT, W>), dim3(p.n_tiles), dim3(64 * W), kLds, s, p);
+    RMI_HIP_CHECK(hipGetLastError());
+    return RMI_HIP_OK;
+}
+
+// From this many tiles on a launch fills the chip with one-wave workgroups and the split has nothing to gain.
+constexpr uint32_t kDeepSplitMaxTiles = 1024;
 int dispatch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
+    if (p.n_tiles <= kDeepSplitMaxTiles) {
+        switch (p.n_oct) {
+            case 8: return launch_gemv_deep_split<8, 4>(p, s);  // (four octets: 3.3 us a launch either way)
+            case 12: return launch_gemv_deep_split<12, 4>(p, s);
+            default: break;
+        }
+    }
     switch (p.n_oct) {
         case 1: return launch_gemv_deep<1>(p, s);
         case 2: return launch_gemv_deep<2>(p, s);

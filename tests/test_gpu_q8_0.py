@@ -222,6 +222,28 @@ def test_gemv_batched_tiny_and_huge_scales(hip, oracle, n_tokens):
     assert np.count_nonzero((prod != 0) & (np.abs(prod) < 1.17549435e-38)) > 100
 
 
+@pytest.mark.parametrize("n_out,n_in", [(1021, 2048), (517, 3072), (40, 1984), (99, 2944), (8, 1824), (3, 2848)])
+def test_gemv_with_a_tile_on_four_waves(hip, oracle, n_out, n_in):
+    """Rows of 8 or 12 octets (1793 to 2048 and 2817 to 3072 elements) in matrices of up to 1024 tiles: a tile's
+    octets are multiplied by four waves and summed in block order by the first.  Row lengths that end inside the
+    last octet, row counts that end inside a tile, and (ith, nth) slices that begin and end inside tiles."""
+    w, x = _case(hip, 900 + n_out + n_in, n_out, n_in)
+    q8, sc = oracle.quantize_q8_0(x[0], A)
+    kernel = hip.kernel.Q8Kernel(w, n_in, n_out)
+    ref = oracle.matmul_q8_0_quantized(w, q8, sc, n_in, n_out, A)
+    out = np.zeros(n_out, np.float32)
+    kernel.forward_prequantized(q8, sc, out, n_in, n_out, 0, 1)
+    assert np.array_equal(bits(out), bits(ref))
+    nth = 3
+    for ith in range(nth):
+        single = np.full(n_out, -1.0, np.float32)
+        kernel.forward_prequantized(q8, sc, single, n_in, n_out, ith, nth)
+        per = -(-n_out // nth)
+        lo, hi = min(ith * per, n_out), min(ith * per + per, n_out)
+        assert np.all(single[:lo] == -1.0) and np.all(single[hi:] == -1.0)
+        assert np.array_equal(bits(single[lo:hi]), bits(ref[lo:hi]))
+
+
 @pytest.mark.parametrize("nth", [1, 2, 3, 4, 8, 16])
 def test_thread_partition_bit_exact(hip, oracle, nth):
     """tests/q8_0_parallel_matmul.rs:82-145: every (ith, nth) slice of the full output."""
