@@ -260,6 +260,52 @@ __device__ __forceinline__ void octets_fma_ahead(float &acc, const OctetRegs (&g
     acc = a;
 }
 
+// A wave's N octets (the staged octets first .. first + N - 1) multiplied down to the two factors of every block's
+// fma, for another wave to add: dst[(4 i + q) * 64] = {s, float(dot), s', float(dot')} of blocks 2q and 2q + 1 of its
+// octet i (dst already points at this lane's float4).
+template <int N>
+__device__ __forceinline__ void octets_to_factors(const OctetRegs (&g)[N], const uint4 *lds, uint32_t n_staged,
+                                                  uint32_t first, uint32_t L, float4 *dst) {
+    OctetX x = load_octet_x(lds, n_staged, first, L);
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        OctetX nx = x;
+        if (i + 1 < N) nx = load_octet_x(lds, n_staged, first + i + 1, L);
+        const OctetRegs &w = g[i];
+        float4 *d = dst + i * 4 * 64;
+        d[0] = make_float4(h2f_times<true>(w.sc.x & 0xffffu, x.s0.x), float(dot4_i8(int(w.qa.x), int(x.xa.x))),
+                           h2f_times<true>(w.sc.x >> 16, x.s0.y), float(dot4_i8(int(w.qa.y), int(x.xa.y))));
+        d[64] = make_float4(h2f_times<true>(w.sc.y & 0xffffu, x.s0.z), float(dot4_i8(int(w.qa.z), int(x.xa.z))),
+                            h2f_times<true>(w.sc.y >> 16, x.s0.w), float(dot4_i8(int(w.qa.w), int(x.xa.w))));
+        d[128] = make_float4(h2f_times<true>(w.sc.z & 0xffffu, x.s1.x), float(dot4_i8(int(w.qb.x), int(x.xb.x))),
+                             h2f_times<true>(w.sc.z >> 16, x.s1.y), float(dot4_i8(int(w.qb.y), int(x.xb.y))));
+        d[192] = make_float4(h2f_times<true>(w.sc.w & 0xffffu, x.s1.z), float(dot4_i8(int(w.qb.z), int(x.xb.z))),
+                             h2f_times<true>(w.sc.w >> 16, x.s1.w), float(dot4_i8(int(w.qb.w), int(x.xb.w))));
+        x = nx;
+    }
+}
+// ... and the M octets' factors added to a lane's sum in block order (src points at this lane's float4 of the first)
+template <int M>
+__device__ __forceinline__ void factors_sum(float &acc, const float4 *src) {
+    float4 f[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) f[q] = src[q * 64];
+#pragma unroll
+    for (int o = 0; o < M; o++) {
+        float4 nf[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) nf[q] = o + 1 < M ? src[((o + 1) * 4 + q) * 64] : f[q];
+        asm volatile("" : "+v"(acc) : : "memory");  // the next octet's reads stay in front of this octet's sums
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            acc = __builtin_fmaf(f[q].x, f[q].y, acc);
+            acc = __builtin_fmaf(f[q].z, f[q].w, acc);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) f[q] = nf[q];
+    }
+}
+
 // A wave owns a short run of consecutive 8-row tiles of ONE matrix (about 34 KiB of
 // weights) and walks it four octets deep (device_run_ring.h).  A launch has far more
 // waves than fit on the chip at once: the dispatcher hands out runs as waves retire,
@@ -742,8 +788,98 @@ __global__ __launch_bounds__(64) void gemv_q8_0_norm_deep_kernel(RmiGemvProblem 
     if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
 }
 
+// The norm in front of a tile on four waves (gemv_q8_0_deep_split_kernel): every wave normalises and quantizes a
+// quarter of the activation (a lone wave's 400 instructions of it stood between the activation's arrival and the
+// first product), multiplies a quarter of the tile's octets, and the first wave adds.  n_in = NOCT * 256, NOCT = 4 or 8.
+template <int NOCT>
+__global__ __launch_bounds__(256) void gemv_q8_0_norm_deep_split_kernel(RmiGemvProblem p, RmiNormArgs na) {
+    static_assert(NOCT % 4 == 0, "whole octets a wave, whole float4s a thread");
+    constexpr int N = NOCT / 4, R = NOCT / 4;  // octets a wave, float4s of the activation a thread
+    extern __shared__ uint4 lds[];
+    __shared__ double red[4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, r = lane >> 3, L = lane & 7;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t k = blockIdx.x;
+    const float4 *xin = reinterpret_cast<const float4 *>(na.x_in), *rin = reinterpret_cast<const float4 *>(na.resid),
+                 *win = reinterpret_cast<const float4 *>(na.weight);
+    float4 v[R], a[R], wv[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) {  // thread owns the float4s tid, tid + 256, ...: element blocks stay in 8 lanes
+        v[j] = xin[tid + 256 * j];
+        if (na.resid) a[j] = rin[tid + 256 * j];
+        wv[j] = win[tid + 256 * j];
+    }
+    asm volatile("" : : : "memory");  // the activation's loads stay in front of the weights'
+    gptr_u4 tile = as_global<gptr_u4>(p.w + size_t(p.tile0 + k) * NOCT * kOctetBytes);
+    OctetRegs g[N];
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        load_octet(g[i], tile + r, tile + NOCT * 8 + lane, wave * N + i);
+        asm volatile("" : : : "memory");
+    }
+    double part = 0.0;
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        if (na.resid) {
+            v[j].x += a[j].x;
+            v[j].y += a[j].y;
+            v[j].z += a[j].z;
+            v[j].w += a[j].w;
+        }
+        const float s0 = v[j].x * v[j].x, s1 = v[j].y * v[j].y, s2 = v[j].z * v[j].z, s3 = v[j].w * v[j].w;
+        part += double(s0);
+        part += double(s1);
+        part += double(s2);
+        part += double(s3);
+    }
+    if (k == 0) {
+#pragma unroll
+        for (int j = 0; j < R; j++) reinterpret_cast<float4 *>(na.x_out)[tid + 256 * j] = v[j];
+    }
+    part = wave_sum_f64(part);
+    if (lane == 0) red[wave] = part;
+    __syncthreads();
+    const double total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float mean_sq = float(total / double(NOCT * 256));
+    const float scale = 1.0f / sqrtf(mean_sq + na.eps);
+    uint32_t *dq = reinterpret_cast<uint32_t *>(lds);
+    float *ds = reinterpret_cast<float *>(dq + NOCT * 64);
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        float4 o;
+        o.x = (v[j].x * scale) * wv[j].x;
+        o.y = (v[j].y * scale) * wv[j].y;
+        o.z = (v[j].z * scale) * wv[j].z;
+        o.w = (v[j].w * scale) * wv[j].w;
+        float sc;
+        const uint32_t q = rmi_quantize_block8(o, na.rounding, &sc);
+        const uint32_t b = (tid >> 3) + 32 * j;  // block of this float4; L = its dword inside the block
+        dq[(b >> 2) * 32 + L * 4 + (b & 3)] = q;
+        if (L == 0) ds[b] = sc;
+    }
+    __syncthreads();
+    float4 *hand = reinterpret_cast<float4 *>(lds + NOCT * 18);
+    if (wave != 0) octets_to_factors<N>(g, lds, NOCT, wave * N, L, hand + (wave - 1) * N * 4 * 64 + lane);
+    float acc = 0.0f;
+    if (wave == 0) octets_fma_ahead<N>(acc, g, lds, L, NOCT);
+    __syncthreads();
+    if (wave != 0) return;
+    factors_sum<NOCT - N>(acc, hand + lane);
+    const uint32_t row = (p.tile0 + k) * kTileRows + r;
+    const float y = hsum8_lanes(acc);
+    if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
+}
+
 template <int NOCT>
 int launch_gemv_norm_deep(const RmiGemvProblem &p, const RmiNormArgs &na, hipStream_t s) {
+    if constexpr (NOCT % 4 == 0) {
+        if (p.n_tiles <= 1024) {  // beyond, one-wave workgroups fill the chip by themselves
+            constexpr size_t kLds = size_t(NOCT) * 288 + size_t(NOCT - NOCT / 4) * 4 * 64 * 16;
+            hipLaunchKernelGGL((gemv_q8_0_norm_deep_split_kernel<NOCT>), dim3(p.n_tiles), dim3(256), kLds, s, p, na);
+            RMI_HIP_CHECK(hipGetLastError());
+            return RMI_HIP_OK;
+        }
+    }
     hipLaunchKernelGGL((gemv_q8_0_norm_deep_kernel<NOCT>), dim3(p.n_tiles), dim3(64), size_t(NOCT) * 288, s, p, na);
     RMI_HIP_CHECK(hipGetLastError());
     return RMI_HIP_OK;
@@ -1022,49 +1158,12 @@ __global__ __launch_bounds__(64 * W) void gemv_q8_0_deep_split_kernel(RmiGemvPro
     __syncthreads();
     // the factors of the octets N .. NOCT - 1: [octet - N][pair of blocks q][lane] = {s, float(dot), s', float(dot')}
     float4 *hand = reinterpret_cast<float4 *>(lds + NOCT * 18);
-    if (wave != 0) {
-        OctetX x = load_octet_x(lds, NOCT, wave * N, L);
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            OctetX nx = x;
-            if (i + 1 < N) nx = load_octet_x(lds, NOCT, wave * N + i + 1, L);
-            const OctetRegs &w = g[i];
-            float4 *dst = hand + ((wave - 1) * N + i) * 4 * 64 + lane;
-            dst[0] = make_float4(h2f_times<true>(w.sc.x & 0xffffu, x.s0.x), float(dot4_i8(int(w.qa.x), int(x.xa.x))),
-                                 h2f_times<true>(w.sc.x >> 16, x.s0.y), float(dot4_i8(int(w.qa.y), int(x.xa.y))));
-            dst[64] = make_float4(h2f_times<true>(w.sc.y & 0xffffu, x.s0.z), float(dot4_i8(int(w.qa.z), int(x.xa.z))),
-                                  h2f_times<true>(w.sc.y >> 16, x.s0.w), float(dot4_i8(int(w.qa.w), int(x.xa.w))));
-            dst[128] = make_float4(h2f_times<true>(w.sc.z & 0xffffu, x.s1.x), float(dot4_i8(int(w.qb.x), int(x.xb.x))),
-                                   h2f_times<true>(w.sc.z >> 16, x.s1.y), float(dot4_i8(int(w.qb.y), int(x.xb.y))));
-            dst[192] = make_float4(h2f_times<true>(w.sc.w & 0xffffu, x.s1.z), float(dot4_i8(int(w.qb.z), int(x.xb.z))),
-                                   h2f_times<true>(w.sc.w >> 16, x.s1.w), float(dot4_i8(int(w.qb.w), int(x.xb.w))));
-            x = nx;
-        }
-    }
+    if (wave != 0) octets_to_factors<N>(g, lds, NOCT, wave * N, L, hand + (wave - 1) * N * 4 * 64 + lane);
     float acc = 0.0f;
     if (wave == 0) octets_fma_ahead<N>(acc, g, lds, L, NOCT);
     __syncthreads();
     if (wave != 0) return;
-    {
-        const float4 *src = hand + lane;
-        float4 f[4];
-#pragma unroll
-        for (int q = 0; q < 4; q++) f[q] = src[q * 64];
-#pragma unroll
-        for (int o = 0; o < NOCT - N; o++) {
-            float4 nf[4];
-#pragma unroll
-            for (int q = 0; q < 4; q++) nf[q] = o + 1 < NOCT - N ? src[((o + 1) * 4 + q) * 64] : f[q];
-            asm volatile("" : "+v"(acc) : : "memory");  // the next octet's reads stay in front of this octet's sums
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                acc = __builtin_fmaf(f[q].x, f[q].y, acc);
-                acc = __builtin_fmaf(f[q].z, f[q].w, acc);
-            }
-#pragma unroll
-            for (int q = 0; q < 4; q++) f[q] = nf[q];
-        }
-    }
+    factors_sum<NOCT - N>(acc, hand + lane);
     const uint32_t row = (p.tile0 + k) * kTileRows + r;
     const float y = hsum8_lanes(acc);
     if (L == 0 && row >= p.row_start && row < p.row_end) as_global<gptr_f32_w>(p.y)[row] = y;
