@@ -873,7 +873,7 @@ __global__ __launch_bounds__(256) void gemv_q8_0_norm_deep_split_kernel(RmiGemvP
 template <int NOCT>
 int launch_gemv_norm_deep(const RmiGemvProblem &p, const RmiNormArgs &na, hipStream_t s) {
     if constexpr (NOCT % 4 == 0) {
-        if (p.n_tiles <= 1024) {  // beyond, one-wave workgroups fill the chip by themselves
+        if (p.n_tiles <= 512) {  // two workgroups a compute unit; beyond, one-wave workgroups fill the chip by themselves
             constexpr size_t kLds = size_t(NOCT) * 288 + size_t(NOCT - NOCT / 4) * 4 * 64 * 16;
             hipLaunchKernelGGL((gemv_q8_0_norm_deep_split_kernel<NOCT>), dim3(p.n_tiles), dim3(256), kLds, s, p, na);
             RMI_HIP_CHECK(hipGetLastError());
@@ -1186,8 +1186,10 @@ int launch_gemv_deep_split(const RmiGemvProblem &p, hipStream_t s) {
     return RMI_HIP_OK;
 }
 
-// From this many tiles on a launch fills the chip with one-wave workgroups and the split has nothing to gain.
-constexpr uint32_t kDeepSplitMaxTiles = 1024;
+// Up to a workgroup a compute unit.  Beyond, one-wave workgroups fill the chip and the split only adds work
+// (independent launches back to back, 512 tiles of 12 octets: 4.4 us against 4.1; 128 tiles: the same either way,
+// and in a chain of dependent launches, which is where such a matrix is found, the split is the faster one).
+constexpr uint32_t kDeepSplitMaxTiles = 256;
 int dispatch_gemv_deep(const RmiGemvProblem &p, hipStream_t s) {
     if (p.n_tiles <= kDeepSplitMaxTiles) {
         switch (p.n_oct) {

@@ -46,7 +46,7 @@ def test_rms_norm_quantize(hip, oracle, n):
 @pytest.mark.parametrize("n_in,n_out", [(1024, 4096), (1024, 6144), (256, 13), (2048, 1000), (1024, 8320), (1536, 520)])
 def test_rms_norm_gemv_fused(hip, oracle, n_in, n_out):
     """add + rms_norm + quantize folded into the Q8_0 product (src/models/qwen3.rs:719-774): the same bits
-    as the three restated steps followed by the restated AVX2 matmul.  (Rows of 4 or 8 octets in up to 1024 tiles
+    as the three restated steps followed by the restated AVX2 matmul.  (Rows of 4 or 8 octets in up to 512 tiles
     take a tile on four waves, the others a wave a tile.)"""
     H, K = hip.hip, hip.kernel
     rng = np.random.default_rng(n_in + n_out)

@@ -222,10 +222,10 @@ def test_gemv_batched_tiny_and_huge_scales(hip, oracle, n_tokens):
     assert np.count_nonzero((prod != 0) & (np.abs(prod) < 1.17549435e-38)) > 100
 
 
-@pytest.mark.parametrize("n_out,n_in", [(1021, 2048), (517, 3072), (40, 1984), (99, 2944), (8, 1824), (3, 2848)])
+@pytest.mark.parametrize("n_out,n_in", [(1021, 2048), (517, 3072), (40, 1984), (99, 2944), (8, 1824), (3, 2848), (2048, 3072), (2056, 2048)])
 def test_gemv_with_a_tile_on_four_waves(hip, oracle, n_out, n_in):
-    """Rows of 8 or 12 octets (1793 to 2048 and 2817 to 3072 elements) in matrices of up to 1024 tiles: a tile's
-    octets are multiplied by four waves and summed in block order by the first.  Row lengths that end inside the
+    """Rows of 8 or 12 octets (1793 to 2048 and 2817 to 3072 elements) in matrices of up to 256 tiles: a tile's
+    octets are multiplied by four waves and summed in block order by the first (the last shape is one tile beyond).  Row lengths that end inside the
     last octet, row counts that end inside a tile, and (ith, nth) slices that begin and end inside tiles."""
     w, x = _case(hip, 900 + n_out + n_in, n_out, n_in)
     q8, sc = oracle.quantize_q8_0(x[0], A)
