@@ -251,11 +251,42 @@ def copy_calibration(H, args):
     dst.free()
 
 
-def time_region(H, ev, fn, steps, warmup):
-    """W untimed warm-up steps, then exactly K timed steps between a device synchronisation on both sides.
+SETTLE_MS = 60.0  # least device time of the settling phase, ms
+# Untimed steps of the last time_region call that asked for settled clocks (beyond its W warm-up steps).
+LAST_SETTLE_STEPS = 0
+
+
+def settle(H, ev, fn, min_ms, max_ms=800.0, chunk=20):
+    """Untimed steps until the device's clocks have settled under this load: chunks of `chunk` steps until at least
+    `min_ms` of device time have passed and two chunks in a row differ by under 1 % (at most `max_ms`).  The chip
+    raises its clocks over the first tens of milliseconds of a compute-bound load: the tiled GEMM at 2048 tokens
+    takes 53 us a step in its second 50 steps and 43.5 us from the 600th on; an HBM-bound launch does not change."""
+    ev_a, ev_b = ev.create(), ev.create()
+    total, n, prev = 0.0, 0, None
+    while total < max_ms:
+        ev.record(ev_a)
+        for _ in range(chunk):
+            fn()
+        ev.record(ev_b)
+        H.check(H.lib.rmi_hip_synchronize())
+        ms = ev.elapsed_ms(ev_a, ev_b)
+        total += ms
+        n += chunk
+        per = ms / chunk
+        if total >= min_ms and prev is not None and abs(per - prev) <= 0.01 * prev:
+            break
+        prev = per
+    return n
+
+
+def time_region(H, ev, fn, steps, warmup, settle_ms=0.0):
+    """W untimed warm-up steps (and, with settle_ms, further untimed steps until the clocks have settled: their
+    number is left in LAST_SETTLE_STEPS), then exactly K timed steps between a device synchronisation on both sides.
     Returns (host wall seconds per step, device ms per step from two HIP events on the launch stream)."""
+    global LAST_SETTLE_STEPS
     for _ in range(warmup):
         fn()
+    LAST_SETTLE_STEPS = settle(H, ev, fn, settle_ms) if settle_ms else 0
     ev_a, ev_b = ev.create(), ev.create()
     H.check(H.lib.rmi_hip_synchronize())
     t0 = time.perf_counter()
@@ -306,7 +337,8 @@ def run_projection_set(args, pkg, ev):
     copy_calibration(H, args)
 
     fn, launches = modes[args.mode]
-    wall, dev_ms = time_region(H, ev, fn, args.steps, args.warmup)
+    wall, dev_ms = time_region(H, ev, fn, args.steps, args.warmup, args.settle_ms if batch > 1 else 0.0)
+    settled = LAST_SETTLE_STEPS
     value = alg_bytes / wall / 1e9
     achieved = alg_bytes / (dev_ms * 1e-3) / 1e9  # bytes per launch / average launch duration, summed over the step
     result = base_result(args, "Q8_0 GEMV HBM GB/s, Qwen3-0.6B shapes, 1 GPU", "GB/s", round(value, 1), wall,
@@ -323,6 +355,7 @@ def run_projection_set(args, pkg, ev):
         "device": dev_name.strip(),
         "compute_units": cus,
     })
+    result["warmup"] = args.warmup + settled  # untimed steps in all (batches of two and more wait for settled clocks)
     result.update({
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "gbs_by_reference_convention": round(result["config"]["reference_convention_bytes_per_step"] / wall / 1e9, 1),
@@ -397,9 +430,11 @@ def run_small_batches(args, pkg, ev):
         def step(g=group):
             H.check(H.lib.rmi_hip_gemv_group_run_dev(g, None))
 
-        # a step is 0.13 ms: 200 of them after 50 untimed ones, so that the figure is the steady state
+        # a step is 0.13 ms: 200 of them after 50 untimed ones and as many more as the clocks take to settle (the
+        # launches of four tokens and more are bound by the vector ALU), so that the figure is the steady state
         steps, warmup = 200, 50
-        wall, dev_ms = time_region(H, ev, step, steps, warmup)
+        wall, dev_ms = time_region(H, ev, step, steps, warmup, SETTLE_MS)
+        warmup += LAST_SETTLE_STEPS
         alg = sum(synth.q8_0_gemv_bytes(r["n_out"], r["n_in"], batch) for r in problems)
         achieved = alg / (dev_ms * 1e-3) / 1e9
         out[label] = {
@@ -510,7 +545,7 @@ def run_single_gemv(args, pkg, ev):
 def compact(r):
     """A sub-record of the default line: the figure, its workload, its roofline and its CPU leg."""
     keep = {"workload": r["config"]["workload"], "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
-            "steps": r["steps"], "roofline": r["roofline"]}
+            "steps": r["steps"], "warmup": r["warmup"], "roofline": r["roofline"]}
     if r.get("other_mode"):
         keep["other_mode"] = r["other_mode"]
     if r.get("ffn_stacked_gate_up"):
@@ -548,7 +583,8 @@ def run_gemm(args, pkg, ev):
             H.check(fn(r["k"].w.handle, r["d_q8"].ptr, r["d_sc"].ptr, r["d_y"].ptr, M, r["n_out"], None))
 
     copy_calibration(H, args)
-    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
+    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup, args.settle_ms)
+    settled = LAST_SETTLE_STEPS
     ops = sum(2.0 * M * r["n_in"] * r["n_out"] for r in recs)
     value = ops / wall / 1e12
     achieved = ops / (dev_ms * 1e-3) / 1e12
@@ -565,7 +601,8 @@ def run_gemm(args, pkg, ev):
                           "avg_launch_us": round(dev_ms * 1e3 / 2, 3),
                           **(read_traffic("gemm_q8_0_m2048_qwen3_0.6b_ffn") if M == 2048 else
                              read_traffic("gemm_q8_0_m64_m512_qwen3_0.6b_ffn", f"m{M}"))}
-    w2, d2 = time_region(H, ev, lambda: step(other), args.steps, args.warmup)
+    result["warmup"] = args.warmup + settled  # untimed steps in all: the W asked for and those the clocks took to settle
+    w2, d2 = time_region(H, ev, lambda: step(other), args.steps, args.warmup, args.settle_ms)
     result["other_mode"] = {"mode": "exact (tiled kernel, single chain)" if fast else "fast (kernel chosen per product)",
                             "value": round(ops / w2 / 1e12, 1), "unit": "TOP/s", "avg_launch_us": round(d2 * 1e3 / 2, 3)}
     # The FFN as a host runs it after fuse_vstack (src/ops/quant/fuse.rs:25-64): gate and up are one stacked weight,
@@ -581,7 +618,7 @@ def run_gemm(args, pkg, ev):
     result["ffn_stacked_gate_up"] = {"workload": f"X[Mx1024].[W_gate ; W_up][6144x1024]^T, then X[Mx3072].W_down[1024x3072]^T, M={M}: "
                                                  "2 launches, the operations of 3 products", "ops_per_step": ffn_ops, "unit": "TOP/s"}
     for name, fn in (("fast", H.lib.rmi_hip_gemm_q8_0_fast_dev), ("exact", H.lib.rmi_hip_gemm_q8_0_dev)):
-        wf, df = time_region(H, ev, lambda: ffn(fn), args.steps, args.warmup)
+        wf, df = time_region(H, ev, lambda: ffn(fn), args.steps, args.warmup, args.settle_ms)
         result["ffn_stacked_gate_up"][name] = {"value": round(ffn_ops / wf / 1e12, 1), "us_per_step": round(df * 1e3, 3)}
     d_yg.free()
     kg.w.free()
@@ -877,7 +914,8 @@ def run_q4k_gemm(args, pkg, ev):
                                                     r["d_y"].ptr, M, r["n_out"], None))
 
     copy_calibration(H, args)
-    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup)
+    wall, dev_ms = time_region(H, ev, step, args.steps, args.warmup, args.settle_ms)
+    settled = LAST_SETTLE_STEPS
     ops = sum(2.0 * M * r["n_in"] * r["n_out"] for r in recs)
     achieved = ops / (dev_ms * 1e-3) / 1e12
     result = base_result(args, "Q4_K x Q8_K prefill GEMM TOP/s (int8 MFMA), 1.7B-class FFN shapes, 1 GPU", "TOP/s",
@@ -898,7 +936,8 @@ def run_q4k_gemm(args, pkg, ev):
         r = recs[2]
         H.check(H.lib.rmi_hip_gemm_q4_k_q8k_dev(r["k"].w.handle, r["d_d"].ptr, r["d_q"].ptr, r["d_b"].ptr, r["d_y"].ptr, M, 2048, None))
 
-    wf, df = time_region(H, ev, ffn, args.steps, args.warmup)
+    result["warmup"] = args.warmup + settled  # untimed steps in all: the W asked for and those the clocks took to settle
+    wf, df = time_region(H, ev, ffn, args.steps, args.warmup, args.settle_ms)
     result["ffn_stacked_gate_up"] = {"workload": f"X[Mx2048].[W_gate ; W_up][12288x2048]^T, then X[Mx6144].W_down[2048x6144]^T, M={M}: "
                                                  "2 launches, the same operations", "ops_per_step": ops,
                                      "value": round(ops / wf / 1e12, 1), "unit": "TOP/s", "us_per_step": round(df * 1e3, 3)}
@@ -1074,7 +1113,10 @@ def main():
     ap.add_argument("--steps", type=int, default=None,
                     help="timed steps (default 50; 500 for the q4_0 / q4k / q6k GEMV workloads, whose compute-heavy kernels "
                          "read 10-15 %% slower until the clocks have settled, a few hundred launches in)")
-    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before (default 10; 100 for q4_0 / q4k / q6k)")
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps before (default 10; 100 for q4_0 / q4k / q6k).  Left at its default, the compute-bound "
+                         "workloads (GEMM, Q4_K GEMM, batches of two and more) add untimed steps until the clocks have "
+                         "settled and report the total as `warmup`; given, it is exactly the number asked for")
     ap.add_argument("--workload", choices=["projection_set", "single_gemv", "gemm", "q4_0", "q4k", "q6k", "q4k_gemm", "qlinear", "attention", "decode"], default="projection_set",
                     help="projection_set: the headline Q8_0 decode GEMV workload (default); gemm: Q8_0 prefill GEMM; "
                          "q4_0: Q4_0 x Q8_0 decode GEMV; q4k / q6k: Q4_K / Q6_K x Q8_K decode GEMV; q4k_gemm: Q4_K prefill GEMM (M = --tokens); qlinear: QuantizedLinear::forward (Q4_K dequantise-and-dot, f32 activation); decode: end-to-end device-resident greedy decode "
@@ -1107,6 +1149,9 @@ def main():
     args = ap.parse_args()
     global THREADS_OVERRIDE
     THREADS_OVERRIDE = args.threads or None
+    # compute-bound workloads wait for settled clocks unless the warm-up is given on the command line (then it is
+    # exactly the W asked for)
+    args.settle_ms = SETTLE_MS if args.warmup is None else 0.0
     long_run = args.workload in ("q4_0", "q4k", "q6k")
     if args.steps is None:
         args.steps = 500 if long_run else 50
@@ -1143,13 +1188,13 @@ def main():
         configs.update(run_small_batches(args, pkg, ev))
         for m in (64, 512, 2048):
             sub = argparse.Namespace(**vars(args))
-            sub.tokens, sub.steps, sub.warmup, sub.copy_calibration_mb = m, 50, 10, 0
+            sub.tokens, sub.steps, sub.warmup, sub.copy_calibration_mb, sub.settle_ms = m, 50, 10, 0, SETTLE_MS
             configs[f"gemm_m{m}"] = compact(run_gemm(sub, pkg, ev))
         sub = argparse.Namespace(**vars(args))
         sub.steps, sub.warmup, sub.batch, sub.copy_calibration_mb = 300, 100, 1, 0
         configs["q4k_gemv"] = compact(run_q4k(sub, pkg, ev))
         sub = argparse.Namespace(**vars(args))
-        sub.tokens, sub.steps, sub.warmup, sub.copy_calibration_mb = 512, 50, 10, 0
+        sub.tokens, sub.steps, sub.warmup, sub.copy_calibration_mb, sub.settle_ms = 512, 50, 10, 0, SETTLE_MS
         configs["q4k_gemm_m512"] = compact(run_q4k_gemm(sub, pkg, ev))
         result["configs"] = configs
         log(f"[bench] other configurations measured in {time.time() - t_cfg:.1f}s")
