@@ -251,18 +251,18 @@ def copy_calibration(H, args):
     dst.free()
 
 
-SETTLE_MS = 60.0  # least device time of the settling phase, ms
+SETTLE_MS = 150.0  # least device time of the settling phase, ms
 # Untimed steps of the last time_region call that asked for settled clocks (beyond its W warm-up steps).
 LAST_SETTLE_STEPS = 0
 
 
-def settle(H, ev, fn, min_ms, max_ms=800.0, chunk=20):
+def settle(H, ev, fn, min_ms, max_ms=1000.0, chunk=20):
     """Untimed steps until the device's clocks have settled under this load: chunks of `chunk` steps until at least
-    `min_ms` of device time have passed and two chunks in a row differ by under 1 % (at most `max_ms`).  The chip
+    `min_ms` of device time have passed and three chunks in a row lie within 1 % (at most `max_ms`).  The chip
     raises its clocks over the first tens of milliseconds of a compute-bound load: the tiled GEMM at 2048 tokens
     takes 53 us a step in its second 50 steps and 43.5 us from the 600th on; an HBM-bound launch does not change."""
     ev_a, ev_b = ev.create(), ev.create()
-    total, n, prev = 0.0, 0, None
+    total, n, last = 0.0, 0, []
     while total < max_ms:
         ev.record(ev_a)
         for _ in range(chunk):
@@ -272,10 +272,9 @@ def settle(H, ev, fn, min_ms, max_ms=800.0, chunk=20):
         ms = ev.elapsed_ms(ev_a, ev_b)
         total += ms
         n += chunk
-        per = ms / chunk
-        if total >= min_ms and prev is not None and abs(per - prev) <= 0.01 * prev:
+        last = (last + [ms / chunk])[-3:]
+        if total >= min_ms and len(last) == 3 and max(last) - min(last) <= 0.01 * min(last):
             break
-        prev = per
     return n
 
 
