@@ -419,7 +419,7 @@ int rmi_hip_qk_norm_rope_f16_dev(const float *qkv, const float *q_norm, const fl
                                  uint32_t n_head_kv, uint32_t head_dim_k, uint32_t head_dim_v, float eps, void *stream);
 /* Attention of one token over keys 0..n_keys-1 of an F16 cache [t][kv_stride] (src/models/qwen3.rs:876-933,
  * dot_f16 src/ops/dot.rs:99-119, softmax src/ops/attention.rs:28-38); the output leaves quantized to Q8_0.
- * Head dimension 128 and 768 keys or more: a head's keys are spread over up to 16 workgroups in two launches
+ * Head dimension 128 and 1280 keys or more: a head's keys are spread over up to 16 workgroups in two launches
  * (scores; then weights and p.v, the parts meeting in the workgroup that arrives last).  The softmax sum is still
  * the reference's sequential f32 sum; results have the same bits as the one-workgroup-per-head kernel.  The
  * hand-over uses a scratch region of the calling host thread: calls of one host thread that overlap on different
@@ -453,7 +453,7 @@ void rmi_hip_qwen3_destroy(rmi_hip_qwen3 *s);
  * default.  At most 16. */
 int rmi_hip_qwen3_set_stop_ids(rmi_hip_qwen3 *s, const uint32_t *ids, uint32_t n_ids);
 /* Prompt positions are known in advance, so rmi_hip_qwen3_generate takes them 128 to a pass while it can (head
- * dimension 128, contexts short of the split attention's 768 keys): every product is one launch for all of them
+ * dimension 128, contexts short of the split attention's 1280 keys): every product is one launch for all of them
  * (eight tokens to a workgroup, the x86-64 order's bits for each), the other kernels run once per position inside
  * one launch; each position's logits, argmax and cache rows are what the step-by-step run gives, bit for bit.
  * enabled = 1 (the default): 128 positions a pass; 0: every position its own step; n > 1: n positions a pass (at

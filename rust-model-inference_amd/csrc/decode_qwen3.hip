@@ -594,7 +594,8 @@ __global__ __launch_bounds__(kA128Threads, DENSE ? kDenseWaves : 2) void attenti
     // values: lane = (8 dimensions dg, key slice sl): 16 consecutive lanes read the 256 bytes of one row
     // (with PVP parts: 16 / PVP lanes read the part's 256 / PVP bytes of a row, PVP times as many slices)
     constexpr uint32_t kDgLanes = 16 / PVP, kSlices = kA128Threads / kDgLanes;
-    // With parts a slice is short (six keys cover 768 with four parts) and its loads are unconditional: a load under
+    // With parts a slice is short (six keys a slice cover 768 keys with four parts; longer slices go on in the batches
+    // further down) and its loads are unconditional: a load under
     // a branch makes the wait for this position's q, k, v (issued first) drain most of what was issued behind them.
     constexpr uint32_t kPre = DENSE ? 1 : (PVP == 1 ? (kA128Threads >= 1024 ? 12 : (kA128Threads >= 512 ? 20 : 40)) : 24 / PVP);
     constexpr uint32_t kBatch = DENSE ? kDenseBatch : 8;  // keys of a slice in flight beyond the first kPre
@@ -1122,9 +1123,10 @@ size_t attn_lds_limit() {
 }
 
 // From this many keys on a head's keys are split over workgroups (measured: below, the second launch and the
-// hand-over through HBM cost more than the other compute units save).
+// hand-over through HBM cost more than the other compute units save; with four workgroups a head in the single
+// launch the two meet between 1024 keys, 14.3 us against 14.7, and 1536, 18.6 against 17.2).
 #ifndef RMI_ATTN_SPLIT_MIN_KEYS
-#define RMI_ATTN_SPLIT_MIN_KEYS 768
+#define RMI_ATTN_SPLIT_MIN_KEYS 1280
 #endif
 constexpr uint32_t kAttnSplitMinKeys = RMI_ATTN_SPLIT_MIN_KEYS;
 inline bool attn128_use_split(uint32_t n_keys, uint32_t n_head);
@@ -1688,7 +1690,10 @@ int rmi_hip_attention_f16_quantize_q8_0_dev(const uint16_t *q16, const uint16_t 
     }
     const size_t lds = d128 ? attn128_lds_bytes(n_keys) : attn_lds_bytes(n_keys, head_dim_k, head_dim_v);
     if (lds > attn_lds_limit()) return rmi_fail(RMI_HIP_E_INVALID, "%u keys exceed what the kernel holds in LDS", n_keys);
-    if (d128)
+    if (d128 && attn_pv_parts(n_keys) == 4 && lds <= 64 * 1024)  // four workgroups a head, as in the session's own launch
+        hipLaunchKernelGGL((attention128_quant_kernel<false, 4>), dim3(n_head * 4), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
+                           q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding, AttnFromQkv{}, 0u, 0u);
+    else if (d128)
         hipLaunchKernelGGL(attention128_quant_kernel<false>, dim3(n_head / n_head_kv, n_head_kv), dim3(kA128Threads), lds, static_cast<hipStream_t>(stream),
                            q16, k_cache, v_cache, n_keys - 1, kv_stride, n_head, n_head_kv, q8, scales, rounding, AttnFromQkv{}, 0u, 0u);
     else

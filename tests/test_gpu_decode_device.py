@@ -120,17 +120,17 @@ def test_create_rejects_null_and_overflowing_shapes(hip):
 
 
 def test_long_context_device_decode_crosses_the_attention_split(hip, oracle, tmp_path):
-    """From 768 cached positions on, the head-dimension-128 attention of the device-resident step runs as two
+    """From 1280 cached positions on, the head-dimension-128 attention of the device-resident step runs as two
     launches with a head's keys split over workgroups; logits before, at and after the switch equal the CPU loop's."""
     kw = dict(n_layer=2, n_embd=256, n_head=4, n_head_kv=2, head_dim=128, n_ff=512, vocab=2000, n_ctx=4096)
     f = _write_model(hip, tmp_path, **kw)
     pool = oracle.Pool(8)
-    prompt = np.random.default_rng(9).integers(0, 2000, 700, dtype=np.uint32)
-    steps = [0, 699, 765, 766, 767, 768, 769, 832, 833, 899]
+    prompt = np.random.default_rng(9).integers(0, 2000, 1210, dtype=np.uint32)
+    steps = [0, 1209, 1277, 1278, 1279, 1280, 1281, 1344, 1345, 1409]
     cpu = oracle.Qwen3Decoder(f.metadata, _tensors(f), pool).generate(prompt, 201, dump_steps=steps)
-    sess = hip.decode.Qwen3Session(f.metadata, _tensors(f), capacity=901)
+    sess = hip.decode.Qwen3Session(f.metadata, _tensors(f), capacity=1411)
     gpu = sess.generate(prompt, 201, dump_steps=steps)
-    assert gpu["steps"] == 900
+    assert gpu["steps"] == 1410
     worst, same = _compare(cpu, gpu, "long context")
     print(f"\nlong context: {same}/{len(steps)} dumped steps bit-identical, worst error {worst:.3g} of tolerance")
     again = sess.generate(prompt, 201, dump_steps=steps)  # the split's arrival counters were left at zero

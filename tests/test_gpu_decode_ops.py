@@ -218,9 +218,10 @@ def test_attention_f16_quantize(hip, oracle, hk, n_head, n_kv):
     rng = np.random.default_rng(hk + 1)
     hv = hk
     kv_stride = n_kv * hk
-    # 5000 and 12000 keys take more than the default 64 KiB of LDS per workgroup; from 768 keys on, head dimension
-    # 128 goes through the launches that split a head's keys over workgroups (2 to 16 parts of whole 64-key groups)
-    for n_keys in [1, 2, 7, 8, 9, 36, 63, 64, 255, 256, 257, 383, 640, 767, 768, 769, 833, 1025, 2048, 4097, 5000, 12000]:
+    # 5000 and 12000 keys take more than the default 64 KiB of LDS per workgroup; from 1280 keys on, head dimension
+    # 128 goes through the launches that split a head's keys over workgroups (5 to 16 parts of whole 64-key groups);
+    # from 64 keys up to there a head is four workgroups of one launch, whose key slices outgrow their prefetch at 768
+    for n_keys in [1, 2, 7, 8, 9, 36, 63, 64, 255, 256, 257, 383, 640, 767, 768, 769, 833, 1025, 1279, 1280, 1281, 2048, 4097, 5000, 12000]:
         for trial in range(3 if n_keys < 1000 else 1):
             scale = rng.choice([0.3, 1.0, 3.0])
             q = (rng.normal(0, 1, n_head * hk) * scale).astype(np.float32)
@@ -241,12 +242,12 @@ def test_attention_f16_quantize(hip, oracle, hk, n_head, n_kv):
 
 
 def test_attention_split_mixed_head_counts(hip, oracle):
-    """Head dimension 128 from 768 keys on: launches with different head counts and key counts in turn share the
+    """Head dimension 128 from 1280 keys on: launches with different head counts and key counts in turn share the
     calling thread's scratch region (partial sums, arrival counters); every result has the checker's bits."""
     H = hip.hip
     rng = np.random.default_rng(77)
     hk = hv = 128
-    for n_head, n_kv, n_keys in [(32, 8, 4097), (6, 2, 1500), (16, 8, 769), (32, 4, 768), (6, 6, 2300), (16, 8, 640), (32, 8, 1024)]:
+    for n_head, n_kv, n_keys in [(32, 8, 4097), (6, 2, 1500), (16, 8, 1281), (32, 4, 1280), (6, 6, 2300), (16, 8, 640), (32, 8, 1024), (8, 8, 1344)]:
         kv_stride = n_kv * hk
         q = rng.normal(0, 1, n_head * hk).astype(np.float32)
         kc = rng.normal(0, 1, (n_keys, kv_stride)).astype(np.float16).view(np.uint16)
@@ -326,7 +327,7 @@ def test_qkv_attention_in_one_launch_equals_the_two_calls(hip, oracle, n_head, n
     rng = np.random.default_rng(n_head * 31 + n_kv)
     hd = 128
     kv_stride = n_kv * hd + 8  # rows wider than the heads: the stride is not the width
-    for n_keys in [1, 2, 3, 16, 17, 33, 127, 128, 129, 257, 512, 640, 767, 1024]:
+    for n_keys in [1, 2, 3, 16, 17, 33, 127, 128, 129, 257, 512, 640, 767, 769, 1024, 1279]:
         scale = rng.choice([0.3, 1.0, 3.0])
         qkv = (rng.normal(0, 1, (n_head + 2 * n_kv) * hd) * scale).astype(np.float32)
         qn = rng.normal(1, 0.2, hd).astype(np.float32)
